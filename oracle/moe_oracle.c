@@ -1,0 +1,555 @@
+/*
+ * moe_oracle.c -- CPU restatement of the reference's mixture-of-experts layer
+ * forward (per-token, f32 storage, f64 accumulation).
+ *
+ * THIS IS TEST INFRASTRUCTURE, NOT PRODUCT CODE.  Only the test-suite, the
+ * smoke check and the benchmark's CPU-baseline leg may load it, and only as
+ * the checker / the reported CPU baseline.  The shipped HIP path never calls
+ * into this file and has no CPU fallback.
+ *
+ * Every function cites the reference source it restates (paths relative to
+ * the reference checkout).  The reference is Rust; it cannot be compiled in
+ * this image (no cargo/rustc), so there is no oracle/_ref build.  What pins
+ * each function (golden fixtures, known-answer tests of the reference's own
+ * test modules, closed forms) is listed next to it; the tests that do the
+ * pinning live in tests/test_oracle_*.py.
+ *
+ * Parity status
+ *   pinned   : ora_matvec, ora_silu, ora_softmax, ora_top_k_routing_with,
+ *              ora_combine_selected, ora_expert_forward, ora_sigmoid_dot,
+ *              ora_layer_forward_with, ora_execute_layer, ora_seeded,
+ *              ora_quantize_per_row_i8, ora_dequantize_per_row_i8,
+ *              ora_absmax_per_channel_symmetric, ora_int8_to_bf16_per_channel,
+ *              ora_f32_to_bf16_bits / ora_bf16_bits_to_f32,
+ *              ora_numerical_metrics, ora_layer_forward_f64, ora_permute
+ *              (brute force), ora_matvec_f32acc.
+ *   parity unpinned (no reference counterpart; defined by this build):
+ *              the `router_bias` term of ora_route (the reference router has
+ *              no bias, dense.rs:333).  With router_bias == NULL ora_route is
+ *              pinned like the rest.
+ *   platform note: exp() is the host libm's; the reference uses Rust's
+ *              f64::exp (also the platform libm).  Last-ulp differences of
+ *              exp between platforms are not pinned by any fixture.
+ *
+ * Build: see oracle/Makefile (gcc -O2 -fopenmp -ffp-contract=off).
+ * -ffp-contract=off is REQUIRED: the reference performs separate multiply and
+ * add roundings in its f32 loops (Rust never contracts).
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define ORA_OK 0
+#define ORA_ERR_DIM -1               /* DimMismatch (dense.rs:31-49)            */
+#define ORA_ERR_ZERO_K -2            /* MoeSparseError::ZeroK (sparse.rs:35-50) */
+#define ORA_ERR_K_EXCEEDS -3         /* KExceedsExperts                         */
+#define ORA_ERR_NON_FINITE -4        /* NonFiniteWeight{index}                  */
+#define ORA_ERR_NEGATIVE -5          /* NegativeWeight{index}                   */
+#define ORA_ERR_SUM_NON_POSITIVE -6  /* SelectedSumNonPositive                  */
+
+/* dense.rs:84 -- rows*cols at or above which matvec runs rows in parallel. */
+#define ORA_MATVEC_PAR_THRESHOLD (1u << 16)
+
+/* Number of threads the row-parallel matvec may use (1 = serial everywhere).
+ * Thread count never changes results: each row is the same sequential sum. */
+static int g_threads = 1;
+void ora_set_threads(int n) { g_threads = n < 1 ? 1 : n; }
+int ora_get_threads(void) { return g_threads; }
+int ora_hw_threads(void) {
+#ifdef _OPENMP
+  return omp_get_num_procs();
+#else
+  return 1;
+#endif
+}
+
+/* ---- tensor.rs:294-308 : bf16 <-> f32 (truncation, lossless upcast) ------ */
+uint16_t ora_f32_to_bf16_bits(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  return (uint16_t)(u >> 16);
+}
+float ora_bf16_bits_to_f32(uint16_t b) {
+  uint32_t u = ((uint32_t)b) << 16;
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+
+/* ---- dense.rs:368-379 : deterministic xorshift fixture generator --------- */
+void ora_seeded(uint64_t seed, size_t n, float* out) {
+  uint64_t state = seed * 0x9E3779B97F4A7C15ull + 1ull;
+  for (size_t i = 0; i < n; ++i) {
+    state ^= state << 13;
+    state ^= state >> 7;
+    state ^= state << 17;
+    uint32_t u = (uint32_t)(state >> 11);
+    out[i] = ((float)u / (float)UINT32_MAX) * 2.0f - 1.0f;
+  }
+}
+
+/* ---- dense.rs:74-77 : silu in f64, returned as f32 ----------------------- */
+float ora_silu(float x) {
+  double xd = (double)x;
+  return (float)(xd / (1.0 + exp(-xd)));
+}
+
+/* ---- dense.rs:97-115 : y = W x, W row-major [rows, cols], f64 accumulate,
+ * each row one sequential c-ascending sum; rows in parallel above the
+ * threshold (dense.rs:106-109). ------------------------------------------- */
+static inline float ora_row_f64(const float* w, const float* x, size_t cols) {
+  double acc = 0.0;
+  for (size_t c = 0; c < cols; ++c) acc += (double)w[c] * (double)x[c];
+  return (float)acc;
+}
+void ora_matvec(const float* w, size_t rows, size_t cols, const float* x, float* y) {
+  if (g_threads > 1 && rows * cols >= ORA_MATVEC_PAR_THRESHOLD) {
+#pragma omp parallel for schedule(static) num_threads(g_threads)
+    for (long r = 0; r < (long)rows; ++r) y[r] = ora_row_f64(w + (size_t)r * cols, x, cols);
+  } else {
+    for (size_t r = 0; r < rows; ++r) y[r] = ora_row_f64(w + r * cols, x, cols);
+  }
+}
+
+/* ---- dense.rs:120-135 : f32-accumulating matvec (Strict policy) ---------- */
+void ora_matvec_f32acc(const float* w, size_t rows, size_t cols, const float* x, float* y) {
+  for (size_t r = 0; r < rows; ++r) {
+    float acc = 0.0f;
+    const float* wr = w + r * cols;
+    for (size_t c = 0; c < cols; ++c) acc += wr[c] * x[c];
+    y[r] = acc;
+  }
+}
+
+/* ---- dense.rs:172-187 : softmax.  max is an f32 fold from -inf that skips
+ * NaN (f32::max); the subtraction is f32, exp and the sum are f64, the sum is
+ * a sequential fold, the result is (e * (1/sum)) rounded to f32. ----------- */
+void ora_softmax(const float* logits, size_t n, float* out) {
+  if (n == 0) return;
+  float mx = -INFINITY;
+  for (size_t i = 0; i < n; ++i) mx = fmaxf(mx, logits[i]);
+  double* e = (double*)malloc(n * sizeof(double));
+  double sum = 0.0;
+  for (size_t i = 0; i < n; ++i) e[i] = exp((double)(logits[i] - mx));
+  for (size_t i = 0; i < n; ++i) sum += e[i];
+  double inv = sum > 0.0 ? 1.0 / sum : 0.0;
+  for (size_t i = 0; i < n; ++i) out[i] = (float)(e[i] * inv);
+  free(e);
+}
+
+/* ---- sparse.rs:142-191 : top-k by (f32 weight desc, index asc); selected
+ * indices returned ASCENDING; weights renormalised in f64 when asked.
+ * err_index receives the offending expert for NON_FINITE / NEGATIVE. ------- */
+int ora_top_k_routing_with(const float* weights, size_t n, size_t k, int renormalize,
+                           int32_t* idx_out, float* w_out, int32_t* err_index) {
+  if (err_index) *err_index = -1;
+  if (k == 0) return ORA_ERR_ZERO_K;
+  if (k > n) return ORA_ERR_K_EXCEEDS;
+  for (size_t i = 0; i < n; ++i) {
+    if (!isfinite(weights[i])) {
+      if (err_index) *err_index = (int32_t)i;
+      return ORA_ERR_NON_FINITE;
+    }
+    if (weights[i] < 0.0f) {
+      if (err_index) *err_index = (int32_t)i;
+      return ORA_ERR_NEGATIVE;
+    }
+  }
+  /* The comparator is a strict total order on finite weights, so a stable
+   * sort and k rounds of arg-best select the same set. */
+  uint8_t* taken = (uint8_t*)calloc(n, 1);
+  for (size_t r = 0; r < k; ++r) {
+    size_t best = n;
+    for (size_t i = 0; i < n; ++i) {
+      if (taken[i]) continue;
+      if (best == n || weights[i] > weights[best]) best = i; /* ties keep lower i */
+    }
+    taken[best] = 1;
+  }
+  size_t m = 0;
+  for (size_t i = 0; i < n; ++i)
+    if (taken[i]) idx_out[m++] = (int32_t)i; /* ascending (sparse.rs:175) */
+  free(taken);
+  double sum = 0.0;
+  for (size_t j = 0; j < k; ++j) sum += (double)weights[idx_out[j]];
+  if (sum <= 0.0) return ORA_ERR_SUM_NON_POSITIVE;
+  double scale = renormalize ? 1.0 / sum : 1.0;
+  for (size_t j = 0; j < k; ++j) w_out[j] = (float)((double)weights[idx_out[j]] * scale);
+  return ORA_OK;
+}
+
+/* ---- sparse.rs:87-116 : combine_selected --------------------------------- */
+int ora_combine_selected(const int32_t* indices, const float* weights, size_t k,
+                         const float* expert_outputs, size_t n_outputs, size_t d_model,
+                         float* out) {
+  for (size_t d = 0; d < d_model; ++d) out[d] = 0.0f;
+  for (size_t slot = 0; slot < k; ++slot) {
+    size_t base = (size_t)indices[slot] * d_model;
+    if (base + d_model > n_outputs) return ORA_ERR_DIM;
+    float w = weights[slot];
+    for (size_t d = 0; d < d_model; ++d) out[d] += w * expert_outputs[base + d];
+  }
+  return ORA_OK;
+}
+
+/* ---- dense.rs:253-270 : SwiGLU expert.  policy 0 = Certified (f64 acc),
+ * 1 = Strict (f32 acc).  h = silu(gate)*up is an f32 product. -------------- */
+void ora_expert_forward(const float* w_gate, const float* w_up, const float* w_down,
+                        size_t d_model, size_t d_ff, const float* x, float* y, int policy) {
+  float* gate = (float*)malloc(d_ff * sizeof(float));
+  float* up = (float*)malloc(d_ff * sizeof(float));
+  float* h = (float*)malloc(d_ff * sizeof(float));
+  if (policy == 1) {
+    ora_matvec_f32acc(w_gate, d_ff, d_model, x, gate);
+    ora_matvec_f32acc(w_up, d_ff, d_model, x, up);
+  } else {
+    ora_matvec(w_gate, d_ff, d_model, x, gate);
+    ora_matvec(w_up, d_ff, d_model, x, up);
+  }
+  for (size_t i = 0; i < d_ff; ++i) h[i] = ora_silu(gate[i]) * up[i];
+  if (policy == 1)
+    ora_matvec_f32acc(w_down, d_model, d_ff, h, y);
+  else
+    ora_matvec(w_down, d_model, d_ff, h, y);
+  free(gate);
+  free(up);
+  free(h);
+}
+
+/* ---- layer.rs:436-443 : sigmoid(g . x) with f64 accumulation ------------- */
+float ora_sigmoid_dot(const float* g, const float* x, size_t n) {
+  double acc = 0.0;
+  for (size_t i = 0; i < n; ++i) acc += (double)g[i] * (double)x[i];
+  return (float)(1.0 / (1.0 + exp(-acc)));
+}
+
+/* Layer description shared by the oracle entry points below.  Mirrors
+ * RealMoeLayer (layer.rs:200-212) with flat arrays: experts packed
+ * [E, f, d] / [E, d, f]. */
+typedef struct {
+  int32_t num_experts;   /* E */
+  int32_t top_k;         /* k  = experts_per_token */
+  int32_t d_model;       /* d */
+  int32_t d_ff;          /* f */
+  int32_t d_ff_shared;   /* f_s, 0 = no shared expert */
+  int32_t convention;    /* 0 = Atenia, 1 = HuggingFaceQwen (layer.rs:185-195) */
+  const float* w_router; /* [E, d] */
+  const float* router_bias; /* [E] or NULL; extension, added to the f32 logits */
+  const float* w_gate;   /* [E, f, d] */
+  const float* w_up;     /* [E, f, d] */
+  const float* w_down;   /* [E, d, f] */
+  const float* s_gate;   /* [f_s, d] */
+  const float* s_up;     /* [f_s, d] */
+  const float* s_down;   /* [d, f_s] */
+  const float* shared_gate; /* [d] or NULL */
+} OraLayer;
+
+/* ---- dense.rs:325-337 : route = softmax(matvec(W_r, x)) ------------------ */
+void ora_route(const OraLayer* L, const float* x, float* logits, float* weights) {
+  size_t E = (size_t)L->num_experts, d = (size_t)L->d_model;
+  /* The router matvec is serial below the threshold and row-parallel above;
+   * identical arithmetic either way (dense.rs:89-96). */
+  ora_matvec(L->w_router, E, d, x, logits);
+  if (L->router_bias)
+    for (size_t e = 0; e < E; ++e) logits[e] = logits[e] + L->router_bias[e];
+  ora_softmax(logits, E, weights);
+}
+
+/* ---- sparse.rs:218-238 + layer.rs:405-431 : one token through the layer.
+ * idx_out / w_out (k entries each) receive the routing when non-NULL. ------ */
+int ora_layer_forward_with(const OraLayer* L, const float* x, int convention, int policy,
+                           float* out, int32_t* idx_out, float* w_out, int32_t* err_index) {
+  size_t E = (size_t)L->num_experts, d = (size_t)L->d_model, f = (size_t)L->d_ff;
+  size_t k = (size_t)L->top_k;
+  float* logits = (float*)malloc(E * sizeof(float));
+  float* weights = (float*)malloc(E * sizeof(float));
+  int32_t* idx = (int32_t*)malloc((k ? k : 1) * sizeof(int32_t));
+  float* selw = (float*)malloc((k ? k : 1) * sizeof(float));
+  float* y = (float*)malloc(d * sizeof(float));
+  ora_route(L, x, logits, weights);
+  int renormalize = (convention == 0);
+  int rc = ora_top_k_routing_with(weights, E, k, renormalize, idx, selw, err_index);
+  if (rc == ORA_OK) {
+    for (size_t i = 0; i < d; ++i) out[i] = 0.0f;
+    for (size_t slot = 0; slot < k; ++slot) {
+      size_t e = (size_t)idx[slot];
+      ora_expert_forward(L->w_gate + e * f * d, L->w_up + e * f * d, L->w_down + e * d * f, d, f,
+                         x, y, policy);
+      float w = selw[slot];
+      for (size_t i = 0; i < d; ++i) out[i] += w * y[i]; /* sparse.rs:230-232 */
+    }
+    if (L->d_ff_shared > 0) { /* layer.rs:415-429 */
+      size_t fs = (size_t)L->d_ff_shared;
+      ora_expert_forward(L->s_gate, L->s_up, L->s_down, d, fs, x, y, policy);
+      float scale = 1.0f;
+      if (convention == 1 && L->shared_gate) scale = ora_sigmoid_dot(L->shared_gate, x, d);
+      for (size_t i = 0; i < d; ++i) out[i] += scale * y[i];
+    }
+    if (idx_out) memcpy(idx_out, idx, k * sizeof(int32_t));
+    if (w_out) memcpy(w_out, selw, k * sizeof(float));
+  }
+  free(logits);
+  free(weights);
+  free(idx);
+  free(selw);
+  free(y);
+  return rc;
+}
+
+/* ---- graph_op.rs:327-350 : the op applies the layer row by row ----------- */
+int ora_execute_layer(const OraLayer* L, const float* input, size_t n_tokens, int policy,
+                      float* out, int32_t* idx_out, float* w_out, int32_t* err_token,
+                      int32_t* err_index) {
+  size_t d = (size_t)L->d_model, k = (size_t)L->top_k;
+  for (size_t t = 0; t < n_tokens; ++t) {
+    int rc = ora_layer_forward_with(L, input + t * d, L->convention, policy, out + t * d,
+                                    idx_out ? idx_out + t * k : NULL,
+                                    w_out ? w_out + t * k : NULL, err_index);
+    if (rc != ORA_OK) {
+      if (err_token) *err_token = (int32_t)t;
+      return rc;
+    }
+  }
+  return ORA_OK;
+}
+
+/* Routing only (router -> softmax -> top-k) for n_tokens rows. */
+int ora_route_tokens(const OraLayer* L, const float* input, size_t n_tokens, int32_t* idx_out,
+                     float* w_out, float* logits_out, int32_t* err_token, int32_t* err_index) {
+  size_t E = (size_t)L->num_experts, d = (size_t)L->d_model, k = (size_t)L->top_k;
+  float* logits = (float*)malloc(E * sizeof(float));
+  float* weights = (float*)malloc(E * sizeof(float));
+  int rc = ORA_OK;
+  for (size_t t = 0; t < n_tokens && rc == ORA_OK; ++t) {
+    ora_route(L, input + t * d, logits, weights);
+    if (logits_out) memcpy(logits_out + t * E, logits, E * sizeof(float));
+    rc = ora_top_k_routing_with(weights, E, k, L->convention == 0, idx_out + t * k,
+                                w_out + t * k, err_index);
+    if (rc != ORA_OK && err_token) *err_token = (int32_t)t;
+  }
+  free(logits);
+  free(weights);
+  return rc;
+}
+
+/* ---- derived contract (no reference code): expert-grouping permutation.
+ * Pairs (t, slot) are enumerated token-major, slot-minor -- the order the
+ * reference visits them (graph_op.rs:345-348 outer loop, sparse.rs:175
+ * ascending experts inside a token).  counts[e] = pairs routed to e;
+ * offsets = exclusive scan; perm[pos] = pair id t*k+slot, a STABLE counting
+ * sort by expert. ---------------------------------------------------------- */
+void ora_permute(const int32_t* idx, size_t n_tokens, size_t k, size_t E, int32_t* counts,
+                 int32_t* offsets, int32_t* perm) {
+  for (size_t e = 0; e < E; ++e) counts[e] = 0;
+  for (size_t p = 0; p < n_tokens * k; ++p) counts[idx[p]]++;
+  offsets[0] = 0;
+  for (size_t e = 0; e < E; ++e) offsets[e + 1] = offsets[e] + counts[e];
+  int32_t* cur = (int32_t*)malloc(E * sizeof(int32_t));
+  for (size_t e = 0; e < E; ++e) cur[e] = offsets[e];
+  for (size_t p = 0; p < n_tokens * k; ++p) perm[cur[idx[p]]++] = (int32_t)p;
+  free(cur);
+}
+
+/* ---- disk_tier.rs:231-248 : per-row symmetric int8 quantisation ---------- */
+void ora_quantize_per_row_i8(const float* data, size_t rows, size_t cols, int8_t* q,
+                             float* scales) {
+  for (size_t r = 0; r < rows; ++r) {
+    const float* row = data + r * cols;
+    float amax = 0.0f;
+    for (size_t c = 0; c < cols; ++c) amax = fmaxf(amax, fabsf(row[c]));
+    float scale = amax > 0.0f ? amax / 127.0f : 1.0f;
+    scales[r] = scale;
+    float inv = 1.0f / scale;
+    for (size_t c = 0; c < cols; ++c) {
+      float v = roundf(row[c] * inv); /* Rust round(): half away from zero */
+      if (v < -127.0f) v = -127.0f;
+      if (v > 127.0f) v = 127.0f;
+      q[r * cols + c] = (int8_t)v;
+    }
+  }
+}
+/* ---- disk_tier.rs:250-259 ------------------------------------------------ */
+void ora_dequantize_per_row_i8(const int8_t* q, const float* scales, size_t rows, size_t cols,
+                               float* out) {
+  for (size_t r = 0; r < rows; ++r)
+    for (size_t c = 0; c < cols; ++c) out[r * cols + c] = (float)q[r * cols + c] * scales[r];
+}
+
+/* ---- quantizer.rs:67-117 : per-COLUMN symmetric int8 of a [K, N] weight -- */
+void ora_absmax_per_channel_symmetric(const float* w, size_t k, size_t n, int8_t* q,
+                                      float* scales) {
+  for (size_t col = 0; col < n; ++col) {
+    float max_abs = 0.0f;
+    for (size_t row = 0; row < k; ++row) {
+      float v = fabsf(w[row * n + col]);
+      if (v > max_abs) max_abs = v;
+    }
+    scales[col] = fmaxf(max_abs / 127.0f, 1e-12f);
+  }
+  for (size_t row = 0; row < k; ++row)
+    for (size_t col = 0; col < n; ++col) {
+      float qf = roundf(w[row * n + col] / scales[col]);
+      if (qf < -127.0f) qf = -127.0f;
+      if (qf > 127.0f) qf = 127.0f;
+      q[row * n + col] = (int8_t)(int32_t)qf;
+    }
+}
+/* ---- cuda/int8_to_bf16.cu:24-40 : bf16 = truncate(float(q) * scale[col]) - */
+void ora_int8_to_bf16_per_channel(const int8_t* q, const float* scales, size_t k, size_t n,
+                                  uint16_t* out_bf16) {
+  for (size_t i = 0; i < k * n; ++i)
+    out_bf16[i] = ora_f32_to_bf16_bits((float)q[i] * scales[i % n]);
+}
+
+/* ---- numerical.rs:40-88 : comparison metrics, f64 accumulation ----------- */
+typedef struct {
+  double max_abs_diff, mean_abs_diff, rmse;
+  int32_t argmax_match;
+} OraMetrics;
+static size_t ora_argmax(const float* v, size_t n) {
+  size_t best = 0;
+  double bv = (double)v[0];
+  for (size_t i = 1; i < n; ++i)
+    if ((double)v[i] > bv) {
+      bv = (double)v[i];
+      best = i;
+    }
+  return best;
+}
+int ora_numerical_metrics(const float* a, const float* r, size_t n, OraMetrics* m) {
+  if (n == 0) return ORA_ERR_DIM;
+  double mx = 0, sa = 0, sq = 0;
+  for (size_t i = 0; i < n; ++i) {
+    double dd = (double)a[i] - (double)r[i];
+    double ad = fabs(dd);
+    if (ad > mx) mx = ad;
+    sa += ad;
+    sq += dd * dd;
+  }
+  m->max_abs_diff = mx;
+  m->mean_abs_diff = sa / (double)n;
+  m->rmse = sqrt(sq / (double)n);
+  m->argmax_match = ora_argmax(a, n) == ora_argmax(r, n);
+  return ORA_OK;
+}
+
+/* ---- all-f64 reference of one token (fixtures/moe/generate_reference.py
+ * atenia_moe_block, text lines 55-95): weights upcast to f64, nothing rounded
+ * to f32 in between.  If fixed_idx != NULL the expert set is taken from it
+ * (ascending), otherwise selected from the f64 softmax with the same
+ * (weight desc, index asc) rule. -------------------------------------------- */
+static void ora_expert_f64(const float* wg, const float* wu, const float* wd, size_t d, size_t f,
+                           const float* x, double* y, double* h) {
+  if (g_threads > 1) {
+#pragma omp parallel for schedule(static) num_threads(g_threads)
+    for (long i = 0; i < (long)f; ++i) {
+      double g = 0, u = 0;
+      for (size_t c = 0; c < d; ++c) {
+        g += (double)wg[(size_t)i * d + c] * (double)x[c];
+        u += (double)wu[(size_t)i * d + c] * (double)x[c];
+      }
+      h[i] = (g / (1.0 + exp(-g))) * u;
+    }
+#pragma omp parallel for schedule(static) num_threads(g_threads)
+    for (long r = 0; r < (long)d; ++r) {
+      double a = 0;
+      for (size_t c = 0; c < f; ++c) a += (double)wd[(size_t)r * f + c] * h[c];
+      y[r] = a;
+    }
+    return;
+  }
+  for (size_t i = 0; i < f; ++i) {
+    double g = 0, u = 0;
+    for (size_t c = 0; c < d; ++c) {
+      g += (double)wg[i * d + c] * (double)x[c];
+      u += (double)wu[i * d + c] * (double)x[c];
+    }
+    h[i] = (g / (1.0 + exp(-g))) * u;
+  }
+  for (size_t r = 0; r < d; ++r) {
+    double a = 0;
+    for (size_t c = 0; c < f; ++c) a += (double)wd[r * f + c] * h[c];
+    y[r] = a;
+  }
+}
+int ora_layer_forward_f64(const OraLayer* L, const float* x, const int32_t* fixed_idx,
+                          double* out) {
+  size_t E = (size_t)L->num_experts, d = (size_t)L->d_model, f = (size_t)L->d_ff;
+  size_t k = (size_t)L->top_k;
+  if (k == 0 || k > E) return ORA_ERR_DIM;
+  double* w = (double*)malloc(E * sizeof(double));
+  double mx = -INFINITY;
+  for (size_t e = 0; e < E; ++e) {
+    double a = 0;
+    for (size_t c = 0; c < d; ++c) a += (double)L->w_router[e * d + c] * (double)x[c];
+    if (L->router_bias) a += (double)L->router_bias[e];
+    w[e] = a;
+    if (a > mx) mx = a;
+  }
+  double sum = 0;
+  for (size_t e = 0; e < E; ++e) {
+    w[e] = exp(w[e] - mx);
+    sum += w[e];
+  }
+  for (size_t e = 0; e < E; ++e) w[e] /= sum;
+  int32_t* idx = (int32_t*)malloc(k * sizeof(int32_t));
+  if (fixed_idx) {
+    memcpy(idx, fixed_idx, k * sizeof(int32_t));
+  } else {
+    uint8_t* taken = (uint8_t*)calloc(E, 1);
+    for (size_t r = 0; r < k; ++r) {
+      size_t best = E;
+      for (size_t e = 0; e < E; ++e)
+        if (!taken[e] && (best == E || w[e] > w[best])) best = e;
+      taken[best] = 1;
+    }
+    size_t m = 0;
+    for (size_t e = 0; e < E; ++e)
+      if (taken[e]) idx[m++] = (int32_t)e;
+    free(taken);
+  }
+  double ssel = 0;
+  for (size_t j = 0; j < k; ++j) ssel += w[idx[j]];
+  size_t fmax = f > (size_t)L->d_ff_shared ? f : (size_t)L->d_ff_shared;
+  double* y = (double*)malloc(d * sizeof(double));
+  double* h = (double*)malloc(fmax * sizeof(double));
+  for (size_t i = 0; i < d; ++i) out[i] = 0.0;
+  for (size_t j = 0; j < k; ++j) {
+    size_t e = (size_t)idx[j];
+    double wj = L->convention == 0 ? w[e] / ssel : w[e];
+    ora_expert_f64(L->w_gate + e * f * d, L->w_up + e * f * d, L->w_down + e * d * f, d, f, x, y,
+                   h);
+    for (size_t i = 0; i < d; ++i) out[i] += wj * y[i];
+  }
+  if (L->d_ff_shared > 0) {
+    ora_expert_f64(L->s_gate, L->s_up, L->s_down, d, (size_t)L->d_ff_shared, x, y, h);
+    double scale = 1.0;
+    if (L->convention == 1 && L->shared_gate) {
+      double a = 0;
+      for (size_t c = 0; c < d; ++c) a += (double)L->shared_gate[c] * (double)x[c];
+      scale = 1.0 / (1.0 + exp(-a));
+    }
+    for (size_t i = 0; i < d; ++i) out[i] += scale * y[i];
+  }
+  free(w);
+  free(idx);
+  free(y);
+  free(h);
+  return ORA_OK;
+}
+
+/* One expert's SwiGLU output in f64 (per-expert parity obligation; the
+ * reference's decomposition generator computes h = silu(g@x)*(u@x); y = d@h
+ * one expert at a time, fixtures/moe/generate_qwen_moe_decomposition_reference.py
+ * compute_layer, text lines 101-123). */
+void ora_expert_forward_f64(const float* wg, const float* wu, const float* wd, size_t d,
+                            size_t f, const float* x, double* y) {
+  double* h = (double*)malloc(f * sizeof(double));
+  ora_expert_f64(wg, wu, wd, d, f, x, y, h);
+  free(h);
+}
