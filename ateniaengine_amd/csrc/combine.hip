@@ -1,0 +1,70 @@
+// Kernel 4: weighted combine back to token order.
+//
+// out[t] = sum over the token's slots (ascending expert id) of w[t,slot] * y[t,slot], then
+// += scale[t] * y_shared[t]      (src/moe/sparse.rs:226-233, src/moe/layer.rs:415-429).
+// The reference multiplies and adds in f32 with two roundings and a fixed order; the same
+// sequence is kept here (no fused multiply-add, no atomics), so given equal expert outputs
+// the combine is bit-identical.  Expert outputs are stored by pair id t*k+slot, so a token's
+// k rows are adjacent and every read and write is a coalesced float4.
+#include "moe_internal.h"
+
+namespace atenia_moe {
+
+namespace {
+
+__global__ __launch_bounds__(256) void combine_kernel(int T, int k, int d,
+                                                      const float* __restrict__ w,
+                                                      const float* __restrict__ y, int y_stride,
+                                                      const float* __restrict__ y_shared,
+                                                      const float* __restrict__ sgate,
+                                                      float* __restrict__ out) {
+  const int chunks = (d + 1023) / 1024;
+  const int t = blockIdx.x / chunks;
+  const int c = ((blockIdx.x - t * chunks) * 256 + threadIdx.x) * 4;
+  if (c >= d) return;
+  const bool vec = (c + 3 < d) && ((y_stride & 3) == 0) && ((d & 3) == 0);
+  float o[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int slot = 0; slot < k; ++slot) {
+    const float ws = w[(size_t)t * k + slot];
+    const float* yr = y + ((size_t)t * k + slot) * y_stride + c;
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    if (vec) {
+      float4 q = *(const float4*)yr;
+      v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+    } else {
+      for (int j = 0; j < 4 && c + j < d; ++j) v[j] = yr[j];
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) o[j] = __fadd_rn(o[j], __fmul_rn(ws, v[j]));
+  }
+  if (y_shared) {
+    const float sc = sgate ? sgate[t] : 1.0f;
+    const float* yr = y_shared + (size_t)t * y_stride + c;
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    if (vec) {
+      float4 q = *(const float4*)yr;
+      v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+    } else {
+      for (int j = 0; j < 4 && c + j < d; ++j) v[j] = yr[j];
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) o[j] = __fadd_rn(o[j], __fmul_rn(sc, v[j]));
+  }
+  float* orow = out + (size_t)t * d + c;
+  if (vec) {
+    *(float4*)orow = make_float4(o[0], o[1], o[2], o[3]);
+  } else {
+    for (int j = 0; j < 4 && c + j < d; ++j) orow[j] = o[j];
+  }
+}
+
+}  // namespace
+
+hipError_t launch_combine(const CombineArgs& a, hipStream_t s) {
+  const unsigned grid = (unsigned)((a.d + 1023) / 1024) * (unsigned)a.T;
+  combine_kernel<<<grid, 256, 0, s>>>(a.T, a.k, a.d, a.w, a.y, a.y_stride, a.y_shared, a.sgate,
+                                      a.out);
+  return hipGetLastError();
+}
+
+}  // namespace atenia_moe

@@ -1,0 +1,351 @@
+// Kernel 3, weight-streaming form: grouped SwiGLU expert projections for small row counts
+// (decode).  Computes, per expert e and per row of tokens routed to it,
+//   gate = W_g x, up = W_u x, h = silu(gate) * up        (src/moe/dense.rs:253-266)
+//   y    = W_d h                                          (src/moe/dense.rs:267-269)
+// with bf16 MFMA (f32 accumulate).  INT8 W8A16 weights (per-output-row scales,
+// src/tensor/disk_tier.rs:231-259) are widened to bf16 in registers -- an int8 value is exact
+// in bf16 -- and the row scale is applied to the f32 accumulator, which equals
+// sum_k (q*scale) x_k of the reference's dequantised weight up to f32 rounding.
+//
+// The bound here is HBM: every weight byte of an active expert is read exactly once per
+// launch, straight from global memory into the MFMA B-operand registers (the weights are
+// stored in that register layout, see moe_internal.h), 1 KiB per wave per load, several
+// loads in flight.  A workgroup owns one 16-row strip of W_g and W_u (or of W_d); its four
+// waves split K and reduce through LDS.  Token rows (A operand) come from L2.
+#include "moe_internal.h"
+
+#include "../../include/atenia_moe_hip.h"
+
+namespace atenia_moe {
+
+namespace {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+
+constexpr int kThreads = 256;
+constexpr int kWavesPerWg = 4;
+
+struct StreamParams {
+  const uint4* wa;      // gate (up phase) or down blocks
+  const uint4* wb;      // up blocks (up phase only)
+  const float* sa;      // int8 row scales of wa, [G, n_rows]
+  const float* sb;
+  int64_t w_stride_u4;  // uint4 between experts
+  int n_rows;           // unpadded N
+  int nkb;              // K blocks per strip
+  const uint16_t* a;    // bf16 rows: x [T, a_stride] (up) or h [rows, a_stride] (down)
+  int a_stride;
+  void* out;            // up: h bf16 [rows, out_stride]; down: y f32 [pairs, out_stride]
+  int out_stride;
+  GroupDesc g;
+};
+
+__device__ inline uint16_t bf16_rne(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+__device__ inline uint32_t pack_i8_pair(uint32_t w, int sh) {
+  float f0 = (float)(int8_t)((w >> sh) & 0xff);
+  float f1 = (float)(int8_t)((w >> (sh + 8)) & 0xff);
+  // |q| <= 127 is exact in bf16, so dropping the low 16 bits loses nothing.
+  return (__float_as_uint(f0) >> 16) | (__float_as_uint(f1) & 0xffff0000u);
+}
+__device__ inline void widen_i8x16(uint4 q, bf16x8& lo, bf16x8& hi) {
+  uint4 l, h;
+  l.x = pack_i8_pair(q.x, 0);
+  l.y = pack_i8_pair(q.x, 16);
+  l.z = pack_i8_pair(q.y, 0);
+  l.w = pack_i8_pair(q.y, 16);
+  h.x = pack_i8_pair(q.z, 0);
+  h.y = pack_i8_pair(q.z, 16);
+  h.z = pack_i8_pair(q.w, 0);
+  h.w = pack_i8_pair(q.w, 16);
+  lo = *(bf16x8*)&l;
+  hi = *(bf16x8*)&h;
+}
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+// Streaming (non-temporal) 16-byte load: the weights are read once per launch.
+__device__ inline uint4 load_stream(const uint4* p) {
+  u32x4 v = __builtin_nontemporal_load((const u32x4*)p);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+__device__ inline f32x4 mfma(uint4 a, uint4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(bf16x8*)&a, *(bf16x8*)&b, c, 0, 0, 0);
+}
+__device__ inline f32x4 mfma(bf16x8 a, bf16x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+// MT  : 16-row tiles of tokens held per workgroup
+// INT8: weights are int8 blocks (64 k per block) instead of bf16 blocks (32 k per block)
+// UP  : gate/up phase with SwiGLU epilogue, else down phase
+template <int MT, bool INT8, bool UP>
+__global__ __launch_bounds__(kThreads) void ffn_stream_kernel(StreamParams p) {
+  const int u = blockIdx.y;
+  if (u >= *p.g.n_active) return;
+  const int e = p.g.active[u];
+  const int base = p.g.offsets[e];
+  const int cnt = p.g.offsets[e + 1] - base;
+  const int m0 = blockIdx.z * 16 * MT;
+  if (m0 >= cnt) return;
+  const int nb = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int kq = lane >> 4, mm = lane & 15;
+  constexpr int KB = INT8 ? kKbInt8 : kKbBf16;  // k per block
+  constexpr int NACC = UP ? 2 : 1;
+
+  const uint16_t* arow[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) {
+    int pos = m0 + 16 * i + mm;
+    if (pos < cnt) {
+      if (UP) {
+        int pair = p.g.perm[base + pos];
+        arow[i] = p.a + (size_t)(pair / p.g.pair_div) * p.a_stride + (KB / 4) * kq;
+      } else {
+        arow[i] = p.a + (size_t)(base + pos) * p.a_stride + (KB / 4) * kq;
+      }
+    } else {
+      arow[i] = nullptr;
+    }
+  }
+
+  const int kb_per = (p.nkb + kWavesPerWg - 1) / kWavesPerWg;
+  const int kb0 = wave * kb_per;
+  const int kb1 = min(p.nkb, kb0 + kb_per);
+  const uint4* pa = p.wa + (size_t)e * p.w_stride_u4 + (size_t)nb * p.nkb * 64 + lane;
+  const uint4* pb = UP ? p.wb + (size_t)e * p.w_stride_u4 + (size_t)nb * p.nkb * 64 + lane
+                       : nullptr;
+
+  f32x4 acc[NACC][MT];
+#pragma unroll
+  for (int n = 0; n < NACC; ++n)
+#pragma unroll
+    for (int i = 0; i < MT; ++i) acc[n][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  constexpr int U = INT8 ? 4 : 8;  // blocks in flight per projection per wave
+  const uint4 zero4 = make_uint4(0, 0, 0, 0);
+  int kb = kb0;
+  for (; kb + U <= kb1; kb += U) {
+    uint4 ba[U], bb[U];
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      ba[j] = load_stream(pa + (size_t)(kb + j) * 64);
+      if (UP) bb[j] = load_stream(pb + (size_t)(kb + j) * 64);
+    }
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      if (INT8) {
+        bf16x8 al, ah, bl, bh;
+        widen_i8x16(ba[j], al, ah);
+        if (UP) widen_i8x16(bb[j], bl, bh);
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+          uint4 x0 = zero4, x1 = zero4;
+          if (arow[i]) {
+            const uint4* ap = (const uint4*)(arow[i] + (size_t)(kb + j) * KB);
+            x0 = ap[0];
+            x1 = ap[1];
+          }
+          acc[0][i] = mfma(*(bf16x8*)&x0, al, acc[0][i]);
+          acc[0][i] = mfma(*(bf16x8*)&x1, ah, acc[0][i]);
+          if (UP) {
+            acc[NACC - 1][i] = mfma(*(bf16x8*)&x0, bl, acc[NACC - 1][i]);
+            acc[NACC - 1][i] = mfma(*(bf16x8*)&x1, bh, acc[NACC - 1][i]);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+          uint4 x0 = zero4;
+          if (arow[i]) x0 = *(const uint4*)(arow[i] + (size_t)(kb + j) * KB);
+          acc[0][i] = mfma(x0, ba[j], acc[0][i]);
+          if (UP) acc[NACC - 1][i] = mfma(x0, bb[j], acc[NACC - 1][i]);
+        }
+      }
+    }
+  }
+  for (; kb < kb1; ++kb) {
+    uint4 ba = pa[(size_t)kb * 64];
+    uint4 bb = UP ? pb[(size_t)kb * 64] : zero4;
+    if (INT8) {
+      bf16x8 al, ah, bl, bh;
+      widen_i8x16(ba, al, ah);
+      if (UP) widen_i8x16(bb, bl, bh);
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        uint4 x0 = zero4, x1 = zero4;
+        if (arow[i]) {
+          const uint4* ap = (const uint4*)(arow[i] + (size_t)kb * KB);
+          x0 = ap[0];
+          x1 = ap[1];
+        }
+        acc[0][i] = mfma(*(bf16x8*)&x0, al, acc[0][i]);
+        acc[0][i] = mfma(*(bf16x8*)&x1, ah, acc[0][i]);
+        if (UP) {
+          acc[NACC - 1][i] = mfma(*(bf16x8*)&x0, bl, acc[NACC - 1][i]);
+          acc[NACC - 1][i] = mfma(*(bf16x8*)&x1, bh, acc[NACC - 1][i]);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        uint4 x0 = zero4;
+        if (arow[i]) x0 = *(const uint4*)(arow[i] + (size_t)kb * KB);
+        acc[0][i] = mfma(x0, ba, acc[0][i]);
+        if (UP) acc[NACC - 1][i] = mfma(x0, bb, acc[NACC - 1][i]);
+      }
+    }
+  }
+
+  // Reduce the four K-slices through LDS; wave 0 finishes.
+  __shared__ f32x4 red[kWavesPerWg - 1][NACC][MT][64];
+  if (wave > 0) {
+#pragma unroll
+    for (int n = 0; n < NACC; ++n)
+#pragma unroll
+      for (int i = 0; i < MT; ++i) red[wave - 1][n][i][lane] = acc[n][i];
+  }
+  __syncthreads();
+  if (wave != 0) return;
+#pragma unroll
+  for (int w = 0; w < kWavesPerWg - 1; ++w)
+#pragma unroll
+    for (int n = 0; n < NACC; ++n)
+#pragma unroll
+      for (int i = 0; i < MT; ++i) acc[n][i] += red[w][n][i][lane];
+
+  // D layout: lane holds rows 4*kq + r (r = 0..3) of column mm.
+  const int n = nb * 16 + mm;
+  float sa = 1.f, sb = 1.f;
+  if (INT8) {
+    sa = n < p.n_rows ? p.sa[(size_t)e * p.n_rows + n] : 0.f;
+    if (UP) sb = n < p.n_rows ? p.sb[(size_t)e * p.n_rows + n] : 0.f;
+  }
+#pragma unroll
+  for (int i = 0; i < MT; ++i) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      int pos = m0 + 16 * i + 4 * kq + r;
+      if (pos >= cnt) continue;
+      if (UP) {
+        float g = acc[0][i][r] * sa;
+        float uu = acc[NACC - 1][i][r] * sb;
+        float h = (g / (1.f + __expf(-g))) * uu;
+        ((uint16_t*)p.out)[(size_t)(base + pos) * p.out_stride + n] = bf16_rne(h);
+      } else if (n < p.n_rows) {
+        int pair = p.g.perm[base + pos];
+        ((float*)p.out)[(size_t)pair * p.out_stride + n] = acc[0][i][r] * sa;
+      }
+    }
+  }
+}
+
+template <bool INT8, bool UP>
+hipError_t launch_stream(const StreamParams& p, int n_pad, int n_groups, int rows_max,
+                         hipStream_t s) {
+  int mt = rows_max <= 16 ? 1 : rows_max <= 32 ? 2 : 4;
+  dim3 grid(n_pad / 16, n_groups, (rows_max + 16 * mt - 1) / (16 * mt));
+  if (mt == 1)
+    ffn_stream_kernel<1, INT8, UP><<<grid, kThreads, 0, s>>>(p);
+  else if (mt == 2)
+    ffn_stream_kernel<2, INT8, UP><<<grid, kThreads, 0, s>>>(p);
+  else
+    ffn_stream_kernel<4, INT8, UP><<<grid, kThreads, 0, s>>>(p);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_ffn_up_f32(const FfnArgs& a, hipStream_t s);
+hipError_t launch_ffn_down_f32(const FfnArgs& a, hipStream_t s);
+
+hipError_t launch_ffn_up(const FfnArgs& a, hipStream_t s) {
+  if (a.wdtype == ATENIA_MOE_WEIGHT_F32) return launch_ffn_up_f32(a, s);
+  const bool int8 = a.wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
+  StreamParams p;
+  p.wa = (const uint4*)a.gate.w;
+  p.wb = (const uint4*)a.up.w;
+  p.sa = a.gate.scale;
+  p.sb = a.up.scale;
+  p.w_stride_u4 = a.gate.expert_stride / 16;
+  p.n_rows = a.gate.n_rows;
+  p.nkb = a.gate.k_pad / (int8 ? kKbInt8 : kKbBf16);
+  p.a = (const uint16_t*)a.x;
+  p.a_stride = a.x_stride;
+  p.out = a.h;
+  p.out_stride = a.h_stride;
+  p.g = a.g;
+  return int8 ? launch_stream<true, true>(p, a.gate.n_pad, a.n_groups_max, a.rows_max, s)
+              : launch_stream<false, true>(p, a.gate.n_pad, a.n_groups_max, a.rows_max, s);
+}
+
+hipError_t launch_ffn_down(const FfnArgs& a, hipStream_t s) {
+  if (a.wdtype == ATENIA_MOE_WEIGHT_F32) return launch_ffn_down_f32(a, s);
+  const bool int8 = a.wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
+  StreamParams p;
+  p.wa = (const uint4*)a.down.w;
+  p.wb = nullptr;
+  p.sa = a.down.scale;
+  p.sb = nullptr;
+  p.w_stride_u4 = a.down.expert_stride / 16;
+  p.n_rows = a.down.n_rows;
+  p.nkb = a.down.k_pad / (int8 ? kKbInt8 : kKbBf16);
+  p.a = (const uint16_t*)a.h;
+  p.a_stride = a.h_stride;
+  p.out = a.y;
+  p.out_stride = a.y_stride;
+  p.g = a.g;
+  return int8 ? launch_stream<true, false>(p, a.down.n_pad, a.n_groups_max, a.rows_max, s)
+              : launch_stream<false, false>(p, a.down.n_pad, a.n_groups_max, a.rows_max, s);
+}
+
+// ---- load-time repack of a row-major matrix into B blocks -------------------------------
+namespace {
+// One thread writes one 16-byte lane slot of one block.
+__global__ void repack_blocks_kernel(const uint8_t* __restrict__ src, uint4* __restrict__ dst,
+                                     int n_rows, int k_cols, int n_pad, int k_pad,
+                                     int elem_bytes) {
+  const int epl = 16 / elem_bytes;       // elements per lane slot
+  const int KB = 4 * epl;                // k per block
+  const int nkb = k_pad / KB;
+  size_t slot = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  size_t total = (size_t)(n_pad / 16) * nkb * 64;
+  if (slot >= total) return;
+  int lane = slot & 63;
+  size_t blk = slot >> 6;
+  int kb = blk % nkb;
+  int nb = blk / nkb;
+  int row = nb * 16 + (lane & 15);
+  int k0 = kb * KB + epl * (lane >> 4);
+  alignas(16) uint8_t buf[16];
+  for (int j = 0; j < 16; ++j) buf[j] = 0;
+  if (row < n_rows) {
+    for (int j = 0; j < epl; ++j) {
+      int kk = k0 + j;
+      if (kk < k_cols)
+        for (int b = 0; b < elem_bytes; ++b)
+          buf[j * elem_bytes + b] = src[((size_t)row * k_cols + kk) * elem_bytes + b];
+    }
+  }
+  dst[slot] = *(const uint4*)buf;
+}
+}  // namespace
+
+hipError_t launch_repack_blocks(const void* src, void* dst, int n_rows, int k_cols, int n_pad,
+                                int k_pad, int elem_bytes, hipStream_t s) {
+  const int KB = 4 * (16 / elem_bytes);
+  size_t total = (size_t)(n_pad / 16) * (k_pad / KB) * 64;
+  int blocks = (int)((total + 255) / 256);
+  repack_blocks_kernel<<<blocks, 256, 0, s>>>((const uint8_t*)src, (uint4*)dst, n_rows, k_cols,
+                                              n_pad, k_pad, elem_bytes);
+  return hipGetLastError();
+}
+
+}  // namespace atenia_moe

@@ -1,0 +1,703 @@
+// extern "C" surface of libatenia_moe_hip.so: layer handles, weight upload, workspace and the
+// forward pipeline  router -> permute -> expert gate/up -> expert down -> combine.
+//
+// The handle plays the part of the reference's registry entry (src/moe/graph_op.rs:207-232):
+// it owns the layer, here resident in HBM.  The reference's residency tiers
+// (src/moe/residency.rs) collapse to this single tier.
+#include "../../include/atenia_moe_hip.h"
+
+#include <climits>
+#include <cstdarg>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "moe_internal.h"
+
+using namespace atenia_moe;
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int rc, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  g_last_error = buf;
+  return rc;
+}
+
+int hip_rc(hipError_t e, const char* what) {
+  if (e == hipSuccess) return ATENIA_MOE_OK;
+  int rc = e == hipErrorOutOfMemory ? ATENIA_MOE_ERR_OOM : ATENIA_MOE_ERR_LAUNCH;
+  return fail(rc, "%s: %s", what, hipGetErrorString(e));
+}
+
+#define HIP_TRY(expr)                               \
+  do {                                              \
+    int rc__ = hip_rc((expr), #expr);               \
+    if (rc__ != ATENIA_MOE_OK) return rc__;         \
+  } while (0)
+
+struct DevBuf {
+  void* p = nullptr;
+  size_t bytes = 0;
+  ~DevBuf() { release(); }
+  void release() {
+    if (p) (void)hipFree(p);
+    p = nullptr;
+    bytes = 0;
+  }
+  // Grow-only; contents are zeroed on (re)allocation.
+  int ensure(size_t want) {
+    if (want <= bytes) return ATENIA_MOE_OK;
+    release();
+    HIP_TRY(hipMalloc(&p, want));
+    HIP_TRY(hipMemset(p, 0, want));
+    bytes = want;
+    return ATENIA_MOE_OK;
+  }
+  template <typename T>
+  T* as() const { return (T*)p; }
+};
+
+size_t elem_bytes_of(int wdtype) {
+  return wdtype == ATENIA_MOE_WEIGHT_F32 ? 4 : wdtype == ATENIA_MOE_WEIGHT_BF16 ? 2 : 1;
+}
+int kb_of(int wdtype) { return wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16 ? kKbInt8 : kKbBf16; }
+
+}  // namespace
+
+struct AteniaMoeLayer {
+  uint32_t magic = 0x4d6f4541u;
+  int E = 0, k = 0, d = 0, f = 0, fs = 0, conv = 0, wdtype = 0;
+  int d_kpad = 0;   // K padding of x rows (gate/up projections)
+  int f_kpad = 0;   // K padding of h rows (down projection)
+  int fs_kpad = 0;
+  int device = 0;
+
+  DevBuf w_router, router_bias, shared_gate;
+  DevBuf wg, wu, wd, sg, su, sd;        // routed experts
+  DevBuf swg, swu, swd, ssg, ssu, ssd;  // shared expert
+  WeightSet gate{}, up{}, down{}, s_gate{}, s_up{}, s_down{};
+  int64_t bytes_per_expert = 0;
+
+  // workspace (grow-only in tokens)
+  int cap_tokens = 0;
+  DevBuf x_in, out, xb, idx, w, sgate, counts, offsets, active, n_active, perm, inv, blk_counts,
+      shared_desc, ident, h, hs, y, ys, status;
+  int last_T = 0;
+
+  hipStream_t stream = nullptr;
+  std::mutex mu;
+
+  bool profiling = false;
+  hipEvent_t ev[ATENIA_MOE_N_STAGES] = {};
+  bool ev_valid = false;
+  int32_t launches[ATENIA_MOE_N_STAGES] = {};
+};
+
+namespace {
+
+bool valid_handle(const AteniaMoeLayer* L) { return L && L->magic == 0x4d6f4541u; }
+
+// Uploads one projection family [G, n_rows, k_cols] (row-major per expert at
+// host + g*host_stride) into `dst` and fills `ws`.
+int upload_family(const void* host, size_t host_stride_elems, int G, int n_rows, int k_cols,
+                  int wdtype, DevBuf& dst, WeightSet& ws, DevBuf& staging) {
+  const size_t eb = elem_bytes_of(wdtype);
+  ws.n_rows = n_rows;
+  ws.k_cols = k_cols;
+  if (wdtype == ATENIA_MOE_WEIGHT_F32) {
+    ws.n_pad = n_rows;
+    ws.k_pad = k_cols;
+    ws.expert_stride = (int64_t)n_rows * k_cols;
+    int rc = dst.ensure((size_t)G * n_rows * k_cols * 4);
+    if (rc) return rc;
+    for (int g = 0; g < G; ++g)
+      HIP_TRY(hipMemcpy((float*)dst.p + (size_t)g * ws.expert_stride,
+                        (const float*)host + (size_t)g * host_stride_elems,
+                        (size_t)n_rows * k_cols * 4, hipMemcpyHostToDevice));
+    ws.w = dst.p;
+    return ATENIA_MOE_OK;
+  }
+  const int KB = kb_of(wdtype);
+  ws.n_pad = round_up(n_rows, 16);
+  ws.k_pad = round_up(k_cols, KB);
+  ws.expert_stride = (int64_t)ws.n_pad * ws.k_pad * (int64_t)eb;  // bytes
+  int rc = dst.ensure((size_t)G * ws.expert_stride);
+  if (rc) return rc;
+  rc = staging.ensure((size_t)n_rows * k_cols * eb);
+  if (rc) return rc;
+  for (int g = 0; g < G; ++g) {
+    HIP_TRY(hipMemcpy(staging.p, (const uint8_t*)host + (size_t)g * host_stride_elems * eb,
+                      (size_t)n_rows * k_cols * eb, hipMemcpyHostToDevice));
+    HIP_TRY(launch_repack_blocks(staging.p, (uint8_t*)dst.p + (size_t)g * ws.expert_stride,
+                                 n_rows, k_cols, ws.n_pad, ws.k_pad, (int)eb, nullptr));
+    HIP_TRY(hipDeviceSynchronize());
+  }
+  ws.w = dst.p;
+  return ATENIA_MOE_OK;
+}
+
+int upload_f32(const float* host, size_t n, DevBuf& dst) {
+  int rc = dst.ensure(n * 4);
+  if (rc) return rc;
+  HIP_TRY(hipMemcpy(dst.p, host, n * 4, hipMemcpyHostToDevice));
+  return ATENIA_MOE_OK;
+}
+
+int ensure_workspace(AteniaMoeLayer* L, int T) {
+  if (T <= L->cap_tokens) return ATENIA_MOE_OK;
+  const size_t P = (size_t)T * L->k;
+  const bool f32w = L->wdtype == ATENIA_MOE_WEIGHT_F32;
+  const size_t act = f32w ? 4 : 2;
+  int rc = 0;
+#define ENS(buf, bytes)                 \
+  if ((rc = L->buf.ensure(bytes))) return rc;
+  ENS(x_in, (size_t)T * L->d * 4)
+  ENS(out, (size_t)T * L->d * 4)
+  if (!f32w) ENS(xb, (size_t)T * L->d_kpad * 2)
+  ENS(idx, P * 4)
+  ENS(w, P * 4)
+  ENS(sgate, (size_t)T * 4)
+  ENS(counts, (size_t)L->E * 4)
+  ENS(offsets, (size_t)(L->E + 1) * 4)
+  ENS(active, (size_t)L->E * 4)
+  ENS(n_active, 4)
+  ENS(perm, P * 4)
+  ENS(inv, P * 4)
+  ENS(blk_counts, ((P + kPermuteBlock - 1) / kPermuteBlock) * L->E * 4)
+  ENS(shared_desc, 16)  // [0..1] offsets {0,T}, [2] active {0}, [3] n_active {1}
+  ENS(ident, (size_t)T * 4)
+  ENS(h, P * (size_t)L->f_kpad * act)
+  ENS(y, P * (size_t)L->d * 4)
+  if (L->fs > 0) {
+    ENS(hs, (size_t)T * L->fs_kpad * act)
+    ENS(ys, (size_t)T * L->d * 4)
+  }
+  ENS(status, 8)
+#undef ENS
+  HIP_TRY(launch_fill_i32(L->ident.as<int32_t>(), T, 0, 1, nullptr));
+  int32_t sd[4] = {0, 0, 0, 1};
+  HIP_TRY(hipMemcpy(L->shared_desc.p, sd, 16, hipMemcpyHostToDevice));
+  int32_t st[2] = {0, INT_MAX};
+  HIP_TRY(hipMemcpy(L->status.p, st, 8, hipMemcpyHostToDevice));
+  HIP_TRY(hipDeviceSynchronize());
+  L->cap_tokens = T;
+  return ATENIA_MOE_OK;
+}
+
+struct StageTimer {
+  AteniaMoeLayer* L;
+  hipStream_t s;
+  int next = 0;
+  void mark() {
+    if (L->profiling && next < ATENIA_MOE_N_STAGES) (void)hipEventRecord(L->ev[next], s);
+    ++next;
+  }
+};
+
+// Runs the pipeline on `s`.  stop_after: 0 = all, 1 = router only.
+int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d_out,
+                hipStream_t s, int stop_after) {
+  const bool f32w = L->wdtype == ATENIA_MOE_WEIGHT_F32;
+  if (f32w && x_dtype != ATENIA_MOE_ACT_F32)
+    return fail(ATENIA_MOE_ERR_UNSUPPORTED, "f32 weights need f32 activations");
+  StageTimer tm{L, s};
+  for (int i = 0; i < ATENIA_MOE_N_STAGES; ++i) L->launches[i] = 0;
+  tm.mark();  // ev[0]: start
+
+  const bool x_bf16 = x_dtype == ATENIA_MOE_ACT_BF16;
+  const bool need_xb = !f32w && !(x_bf16 && L->d_kpad == L->d);
+  RouterArgs ra{};
+  ra.x = d_x;
+  ra.x_is_bf16 = x_bf16;
+  ra.T = T;
+  ra.d = L->d;
+  ra.E = L->E;
+  ra.k = L->k;
+  ra.renorm = L->conv == ATENIA_MOE_CONVENTION_ATENIA;
+  ra.w_router = L->w_router.as<float>();
+  ra.router_bias = L->router_bias.as<float>();
+  const bool gated = L->fs > 0 && L->conv == ATENIA_MOE_CONVENTION_HUGGINGFACE_QWEN &&
+                     L->shared_gate.p != nullptr;
+  ra.shared_gate = gated ? L->shared_gate.as<float>() : nullptr;
+  ra.idx = L->idx.as<int32_t>();
+  ra.w = L->w.as<float>();
+  ra.sgate = L->sgate.as<float>();
+  ra.xb = need_xb ? L->xb.as<uint16_t>() : nullptr;
+  ra.d_pad = L->d_kpad;
+  ra.status = L->status.as<int32_t>();
+  HIP_TRY(launch_router(ra, s));
+  L->launches[0] = 1;
+  tm.mark();  // ev[1]: router done
+  L->last_T = T;
+  if (stop_after == 1) return ATENIA_MOE_OK;
+
+  PermuteArgs pa{};
+  pa.idx = L->idx.as<int32_t>();
+  pa.T = T;
+  pa.k = L->k;
+  pa.E = L->E;
+  pa.counts = L->counts.as<int32_t>();
+  pa.offsets = L->offsets.as<int32_t>();
+  pa.perm = L->perm.as<int32_t>();
+  pa.inv = L->inv.as<int32_t>();
+  pa.active = L->active.as<int32_t>();
+  pa.n_active = L->n_active.as<int32_t>();
+  pa.blk_counts = L->blk_counts.as<int32_t>();
+  pa.shared_offsets = L->shared_desc.as<int32_t>();
+  int nl = 0;
+  HIP_TRY(launch_permute(pa, s, &nl));
+  L->launches[1] = nl;
+  tm.mark();  // ev[2]: permute done
+
+  const void* a_x = f32w ? d_x : (need_xb ? (const void*)L->xb.p : d_x);
+  const int a_stride = f32w ? L->d : L->d_kpad;
+
+  FfnArgs fa{};
+  fa.wdtype = L->wdtype;
+  fa.g.offsets = L->offsets.as<int32_t>();
+  fa.g.active = L->active.as<int32_t>();
+  fa.g.n_active = L->n_active.as<int32_t>();
+  fa.g.perm = L->perm.as<int32_t>();
+  fa.g.pair_div = L->k;
+  fa.n_groups_max = (int)std::min<long long>(L->E, (long long)T * L->k);
+  fa.rows_max = T;
+  fa.gate = L->gate;
+  fa.up = L->up;
+  fa.down = L->down;
+  fa.x = a_x;
+  fa.x_stride = a_stride;
+  fa.h = L->h.p;
+  fa.h_stride = L->f_kpad;
+  fa.y = L->y.as<float>();
+  fa.y_stride = L->d;
+
+  FfnArgs fsd{};
+  if (L->fs > 0) {
+    fsd = fa;
+    const int32_t* sd = L->shared_desc.as<int32_t>();
+    fsd.g.offsets = sd;
+    fsd.g.active = sd + 2;
+    fsd.g.n_active = sd + 3;
+    fsd.g.perm = L->ident.as<int32_t>();
+    fsd.g.pair_div = 1;
+    fsd.n_groups_max = 1;
+    fsd.rows_max = T;
+    fsd.gate = L->s_gate;
+    fsd.up = L->s_up;
+    fsd.down = L->s_down;
+    fsd.h = L->hs.p;
+    fsd.h_stride = L->fs_kpad;
+    fsd.y = L->ys.as<float>();
+  }
+
+  HIP_TRY(launch_ffn_up(fa, s));
+  L->launches[2] = 1;
+  if (L->fs > 0) {
+    HIP_TRY(launch_ffn_up(fsd, s));
+    L->launches[2] = 2;
+  }
+  tm.mark();  // ev[3]: gate/up done
+  HIP_TRY(launch_ffn_down(fa, s));
+  L->launches[3] = 1;
+  if (L->fs > 0) {
+    HIP_TRY(launch_ffn_down(fsd, s));
+    L->launches[3] = 2;
+  }
+  tm.mark();  // ev[4]: down done
+
+  CombineArgs ca{};
+  ca.T = T;
+  ca.k = L->k;
+  ca.d = L->d;
+  ca.w = L->w.as<float>();
+  ca.y = L->y.as<float>();
+  ca.y_stride = L->d;
+  ca.y_shared = L->fs > 0 ? L->ys.as<float>() : nullptr;
+  ca.sgate = gated ? L->sgate.as<float>() : nullptr;
+  ca.out = d_out;
+  HIP_TRY(launch_combine(ca, s));
+  L->launches[4] = 1;
+  tm.mark();  // ev[5]: combine done
+  L->launches[5] = L->launches[0] + L->launches[1] + L->launches[2] + L->launches[3] + 1;
+  return ATENIA_MOE_OK;
+}
+
+int read_status(AteniaMoeLayer* L, hipStream_t s, int32_t* token, int32_t* expert) {
+  if (hipStreamSynchronize(s) != hipSuccess)
+    return fail(ATENIA_MOE_ERR_SYNC, "stream synchronisation failed");
+  int32_t st[2] = {0, INT_MAX};
+  if (!L->status.p) return ATENIA_MOE_OK;
+  HIP_TRY(hipMemcpy(st, L->status.p, 8, hipMemcpyDeviceToHost));
+  if (st[0] == 0) return ATENIA_MOE_OK;
+  int tk = st[1] >> 10, ex = st[1] & 1023;
+  if (token) *token = tk;
+  if (expert) *expert = ex;
+  int32_t reset[2] = {0, INT_MAX};
+  HIP_TRY(hipMemcpy(L->status.p, reset, 8, hipMemcpyHostToDevice));
+  return fail(ATENIA_MOE_ERR_NON_FINITE, "non-finite routing weight at token %d, expert %d", tk,
+              ex);
+}
+
+}  // namespace
+
+extern "C" {
+
+int atenia_moe_hip_available(void) {
+  static int cached = [] {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) return 0;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, 0) != hipSuccess) return 0;
+    return strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : 0;
+  }();
+  return cached;
+}
+
+const char* atenia_moe_hip_last_error_string(void) { return g_last_error.c_str(); }
+
+int atenia_moe_hip_layer_create(const AteniaMoeLayerDesc* D, AteniaMoeLayer** out_layer) {
+  if (!D || !out_layer) return fail(ATENIA_MOE_ERR_DIM, "null descriptor or output pointer");
+  *out_layer = nullptr;
+  if (D->num_experts < 1 || D->d_model < 1 || D->d_ff < 1 || D->d_ff_shared < 0)
+    return fail(ATENIA_MOE_ERR_DIM, "bad dimensions E=%d d=%d f=%d f_s=%d", D->num_experts,
+                D->d_model, D->d_ff, D->d_ff_shared);
+  if (D->top_k < 1 || D->top_k > D->num_experts)
+    return fail(ATENIA_MOE_ERR_K, "bad k=%d for %d experts", D->top_k, D->num_experts);
+  if (D->convention != ATENIA_MOE_CONVENTION_ATENIA &&
+      D->convention != ATENIA_MOE_CONVENTION_HUGGINGFACE_QWEN)
+    return fail(ATENIA_MOE_ERR_DIM, "unknown convention %d", D->convention);
+  if (D->weight_dtype < 0 || D->weight_dtype > 2)
+    return fail(ATENIA_MOE_ERR_DIM, "unknown weight dtype %d", D->weight_dtype);
+  if (!D->w_router || !D->w_gate || !D->w_down)
+    return fail(ATENIA_MOE_ERR_DIM, "router / gate / down weights are required");
+  const bool int8 = D->weight_dtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
+  if (int8 && (!D->scale_gate || !D->scale_up || !D->scale_down))
+    return fail(ATENIA_MOE_ERR_DIM, "int8 weights need per-row scales");
+  if (D->d_ff_shared > 0) {
+    if (!D->s_gate || !D->s_up || !D->s_down)
+      return fail(ATENIA_MOE_ERR_DIM, "shared expert weights missing");
+    if (int8 && (!D->s_scale_gate || !D->s_scale_up || !D->s_scale_down))
+      return fail(ATENIA_MOE_ERR_DIM, "int8 shared expert needs per-row scales");
+  }
+  if (D->num_experts + 1 > kMaxRouterRows)
+    return fail(ATENIA_MOE_ERR_UNSUPPORTED, "at most %d experts", kMaxRouterRows - 1);
+  if (!atenia_moe_hip_available())
+    return fail(ATENIA_MOE_ERR_LAUNCH, "no gfx950 device available");
+
+  AteniaMoeLayer* L = new (std::nothrow) AteniaMoeLayer();
+  if (!L) return fail(ATENIA_MOE_ERR_OOM, "host allocation failed");
+  L->E = D->num_experts;
+  L->k = D->top_k;
+  L->d = D->d_model;
+  L->f = D->d_ff;
+  L->fs = D->d_ff_shared;
+  L->conv = D->convention;
+  L->wdtype = D->weight_dtype;
+  const int KB = L->wdtype == ATENIA_MOE_WEIGHT_F32 ? 1 : kb_of(L->wdtype);
+  L->d_kpad = round_up(L->d, KB);
+  L->f_kpad = round_up(L->f, KB);
+  L->fs_kpad = round_up(L->fs, KB);
+
+  int rc = ATENIA_MOE_OK;
+  auto bail = [&](int code) {
+    delete L;
+    return code;
+  };
+  if (hipStreamCreate(&L->stream) != hipSuccess)
+    return bail(fail(ATENIA_MOE_ERR_LAUNCH, "hipStreamCreate failed"));
+  const size_t E = L->E, d = L->d, f = L->f, fs = L->fs;
+  if ((rc = upload_f32(D->w_router, E * d, L->w_router))) return bail(rc);
+  if (D->router_bias && (rc = upload_f32(D->router_bias, E, L->router_bias))) return bail(rc);
+  if (D->shared_gate && (rc = upload_f32(D->shared_gate, d, L->shared_gate))) return bail(rc);
+
+  DevBuf staging;
+  const size_t eb = elem_bytes_of(L->wdtype);
+  const bool packed = D->w_up == nullptr;
+  const void* gate_h = D->w_gate;
+  const void* up_h = packed ? (const void*)((const uint8_t*)D->w_gate + f * d * eb) : D->w_up;
+  const size_t gu_stride = packed ? 2 * f * d : f * d;
+  if ((rc = upload_family(gate_h, gu_stride, L->E, L->f, L->d, L->wdtype, L->wg, L->gate,
+                          staging)))
+    return bail(rc);
+  if ((rc = upload_family(up_h, gu_stride, L->E, L->f, L->d, L->wdtype, L->wu, L->up, staging)))
+    return bail(rc);
+  if ((rc = upload_family(D->w_down, d * f, L->E, L->d, L->f, L->wdtype, L->wd, L->down,
+                          staging)))
+    return bail(rc);
+  if (int8) {
+    if ((rc = upload_f32(D->scale_gate, E * f, L->sg))) return bail(rc);
+    if ((rc = upload_f32(D->scale_up, E * f, L->su))) return bail(rc);
+    if ((rc = upload_f32(D->scale_down, E * d, L->sd))) return bail(rc);
+    L->gate.scale = L->sg.as<float>();
+    L->up.scale = L->su.as<float>();
+    L->down.scale = L->sd.as<float>();
+  }
+  if (fs > 0) {
+    if ((rc = upload_family(D->s_gate, fs * d, 1, L->fs, L->d, L->wdtype, L->swg, L->s_gate,
+                            staging)))
+      return bail(rc);
+    if ((rc = upload_family(D->s_up, fs * d, 1, L->fs, L->d, L->wdtype, L->swu, L->s_up,
+                            staging)))
+      return bail(rc);
+    if ((rc = upload_family(D->s_down, d * fs, 1, L->d, L->fs, L->wdtype, L->swd, L->s_down,
+                            staging)))
+      return bail(rc);
+    if (int8) {
+      if ((rc = upload_f32(D->s_scale_gate, fs, L->ssg))) return bail(rc);
+      if ((rc = upload_f32(D->s_scale_up, fs, L->ssu))) return bail(rc);
+      if ((rc = upload_f32(D->s_scale_down, d, L->ssd))) return bail(rc);
+      L->s_gate.scale = L->ssg.as<float>();
+      L->s_up.scale = L->ssu.as<float>();
+      L->s_down.scale = L->ssd.as<float>();
+    }
+  }
+  // Algorithmic bytes of one routed expert as stored (weights + int8 scales).
+  L->bytes_per_expert = (int64_t)(3 * d * f * eb) + (int8 ? (int64_t)(2 * f + d) * 4 : 0);
+  if (D->max_tokens_hint > 0 && (rc = ensure_workspace(L, D->max_tokens_hint))) return bail(rc);
+  if (hipDeviceSynchronize() != hipSuccess)
+    return bail(fail(ATENIA_MOE_ERR_SYNC, "device synchronisation failed after upload"));
+  *out_layer = L;
+  return ATENIA_MOE_OK;
+}
+
+int atenia_moe_hip_layer_destroy(AteniaMoeLayer* L) {
+  if (!valid_handle(L)) return fail(ATENIA_MOE_ERR_HANDLE, "invalid layer handle");
+  {
+    std::lock_guard<std::mutex> lock(L->mu);
+    (void)hipDeviceSynchronize();
+    if (L->ev_valid)
+      for (auto& e : L->ev) (void)hipEventDestroy(e);
+    if (L->stream) (void)hipStreamDestroy(L->stream);
+    L->magic = 0;
+  }
+  delete L;
+  return ATENIA_MOE_OK;
+}
+
+int atenia_moe_hip_layer_forward_device(AteniaMoeLayer* L, const void* d_x, int x_dtype,
+                                        int n_tokens, float* d_out, void* stream) {
+  if (!valid_handle(L)) return fail(ATENIA_MOE_ERR_HANDLE, "invalid layer handle");
+  if (n_tokens < 0) return fail(ATENIA_MOE_ERR_DIM, "negative token count");
+  if (n_tokens == 0) return ATENIA_MOE_OK;
+  if (!d_x || !d_out) return fail(ATENIA_MOE_ERR_DIM, "null activation pointer");
+  if (x_dtype != ATENIA_MOE_ACT_F32 && x_dtype != ATENIA_MOE_ACT_BF16)
+    return fail(ATENIA_MOE_ERR_DIM, "unknown activation dtype %d", x_dtype);
+  if ((long long)n_tokens * L->k > (long long)INT_MAX / 4)
+    return fail(ATENIA_MOE_ERR_DIM, "too many tokens");
+  std::lock_guard<std::mutex> lock(L->mu);
+  int rc = ensure_workspace(L, n_tokens);
+  if (rc) return rc;
+  return run_forward(L, d_x, x_dtype, n_tokens, d_out, (hipStream_t)stream, 0);
+}
+
+int atenia_moe_hip_layer_forward(AteniaMoeLayer* L, const float* x_host, int n_tokens,
+                                 float* out_host) {
+  if (!valid_handle(L)) return fail(ATENIA_MOE_ERR_HANDLE, "invalid layer handle");
+  if (n_tokens < 0) return fail(ATENIA_MOE_ERR_DIM, "negative token count");
+  if (n_tokens == 0) return ATENIA_MOE_OK;
+  if (!x_host || !out_host) return fail(ATENIA_MOE_ERR_DIM, "null activation pointer");
+  std::lock_guard<std::mutex> lock(L->mu);
+  int rc = ensure_workspace(L, n_tokens);
+  if (rc) return rc;
+  const size_t bytes = (size_t)n_tokens * L->d * 4;
+  HIP_TRY(hipMemcpyAsync(L->x_in.p, x_host, bytes, hipMemcpyHostToDevice, L->stream));
+  rc = run_forward(L, L->x_in.p, ATENIA_MOE_ACT_F32, n_tokens, L->out.as<float>(), L->stream, 0);
+  if (rc) return rc;
+  HIP_TRY(hipMemcpyAsync(out_host, L->out.p, bytes, hipMemcpyDeviceToHost, L->stream));
+  return read_status(L, L->stream, nullptr, nullptr);
+}
+
+int atenia_moe_hip_layer_status(AteniaMoeLayer* L, void* stream, int32_t* token,
+                                int32_t* expert) {
+  if (!valid_handle(L)) return fail(ATENIA_MOE_ERR_HANDLE, "invalid layer handle");
+  std::lock_guard<std::mutex> lock(L->mu);
+  return read_status(L, (hipStream_t)stream, token, expert);
+}
+
+int atenia_moe_hip_layer_route(AteniaMoeLayer* L, const float* x_host, int n_tokens,
+                               int32_t* idx_host, float* w_host) {
+  if (!valid_handle(L)) return fail(ATENIA_MOE_ERR_HANDLE, "invalid layer handle");
+  if (n_tokens < 0) return fail(ATENIA_MOE_ERR_DIM, "negative token count");
+  if (n_tokens == 0) return ATENIA_MOE_OK;
+  if (!x_host || !idx_host || !w_host) return fail(ATENIA_MOE_ERR_DIM, "null pointer");
+  std::lock_guard<std::mutex> lock(L->mu);
+  int rc = ensure_workspace(L, n_tokens);
+  if (rc) return rc;
+  HIP_TRY(hipMemcpyAsync(L->x_in.p, x_host, (size_t)n_tokens * L->d * 4, hipMemcpyHostToDevice,
+                         L->stream));
+  rc = run_forward(L, L->x_in.p, ATENIA_MOE_ACT_F32, n_tokens, nullptr, L->stream, 1);
+  if (rc) return rc;
+  rc = read_status(L, L->stream, nullptr, nullptr);
+  if (rc) return rc;
+  const size_t P = (size_t)n_tokens * L->k;
+  HIP_TRY(hipMemcpy(idx_host, L->idx.p, P * 4, hipMemcpyDeviceToHost));
+  HIP_TRY(hipMemcpy(w_host, L->w.p, P * 4, hipMemcpyDeviceToHost));
+  return ATENIA_MOE_OK;
+}
+
+int atenia_moe_hip_layer_permute(AteniaMoeLayer* L, const int32_t* idx_host, int n_tokens,
+                                 int32_t* counts_host, int32_t* offsets_host,
+                                 int32_t* perm_host) {
+  if (!valid_handle(L)) return fail(ATENIA_MOE_ERR_HANDLE, "invalid layer handle");
+  if (n_tokens < 0) return fail(ATENIA_MOE_ERR_DIM, "negative token count");
+  if (!idx_host || !counts_host || !offsets_host || (n_tokens > 0 && !perm_host))
+    return fail(ATENIA_MOE_ERR_DIM, "null pointer");
+  if (n_tokens == 0) {
+    for (int e = 0; e < L->E; ++e) counts_host[e] = 0;
+    for (int e = 0; e <= L->E; ++e) offsets_host[e] = 0;
+    return ATENIA_MOE_OK;
+  }
+  const size_t P = (size_t)n_tokens * L->k;
+  for (size_t p = 0; p < P; ++p)
+    if (idx_host[p] < 0 || idx_host[p] >= L->E)
+      return fail(ATENIA_MOE_ERR_DIM, "expert index %d out of range at pair %zu", idx_host[p], p);
+  std::lock_guard<std::mutex> lock(L->mu);
+  int rc = ensure_workspace(L, n_tokens);
+  if (rc) return rc;
+  HIP_TRY(hipMemcpyAsync(L->idx.p, idx_host, P * 4, hipMemcpyHostToDevice, L->stream));
+  PermuteArgs pa{};
+  pa.idx = L->idx.as<int32_t>();
+  pa.T = n_tokens;
+  pa.k = L->k;
+  pa.E = L->E;
+  pa.counts = L->counts.as<int32_t>();
+  pa.offsets = L->offsets.as<int32_t>();
+  pa.perm = L->perm.as<int32_t>();
+  pa.inv = L->inv.as<int32_t>();
+  pa.active = L->active.as<int32_t>();
+  pa.n_active = L->n_active.as<int32_t>();
+  pa.blk_counts = L->blk_counts.as<int32_t>();
+  pa.shared_offsets = nullptr;
+  HIP_TRY(launch_permute(pa, L->stream, nullptr));
+  if (hipStreamSynchronize(L->stream) != hipSuccess)
+    return fail(ATENIA_MOE_ERR_SYNC, "stream synchronisation failed");
+  HIP_TRY(hipMemcpy(counts_host, L->counts.p, (size_t)L->E * 4, hipMemcpyDeviceToHost));
+  HIP_TRY(hipMemcpy(offsets_host, L->offsets.p, (size_t)(L->E + 1) * 4, hipMemcpyDeviceToHost));
+  HIP_TRY(hipMemcpy(perm_host, L->perm.p, P * 4, hipMemcpyDeviceToHost));
+  L->last_T = 0;  // the workspace no longer describes a forward
+  return ATENIA_MOE_OK;
+}
+
+int atenia_moe_hip_layer_last_routing(AteniaMoeLayer* L, int32_t* idx_host, float* w_host,
+                                      int32_t* counts_host, int32_t* offsets_host,
+                                      int32_t* perm_host) {
+  if (!valid_handle(L)) return fail(ATENIA_MOE_ERR_HANDLE, "invalid layer handle");
+  std::lock_guard<std::mutex> lock(L->mu);
+  if (L->last_T <= 0) return fail(ATENIA_MOE_ERR_DIM, "no forward has run on this handle");
+  if (hipDeviceSynchronize() != hipSuccess)
+    return fail(ATENIA_MOE_ERR_SYNC, "device synchronisation failed");
+  const size_t P = (size_t)L->last_T * L->k;
+  if (idx_host) HIP_TRY(hipMemcpy(idx_host, L->idx.p, P * 4, hipMemcpyDeviceToHost));
+  if (w_host) HIP_TRY(hipMemcpy(w_host, L->w.p, P * 4, hipMemcpyDeviceToHost));
+  if (counts_host)
+    HIP_TRY(hipMemcpy(counts_host, L->counts.p, (size_t)L->E * 4, hipMemcpyDeviceToHost));
+  if (offsets_host)
+    HIP_TRY(hipMemcpy(offsets_host, L->offsets.p, (size_t)(L->E + 1) * 4, hipMemcpyDeviceToHost));
+  if (perm_host) HIP_TRY(hipMemcpy(perm_host, L->perm.p, P * 4, hipMemcpyDeviceToHost));
+  return ATENIA_MOE_OK;
+}
+
+int atenia_moe_hip_layer_last_expert_outputs(AteniaMoeLayer* L, float* y_host,
+                                             float* y_shared_host) {
+  if (!valid_handle(L)) return fail(ATENIA_MOE_ERR_HANDLE, "invalid layer handle");
+  std::lock_guard<std::mutex> lock(L->mu);
+  if (L->last_T <= 0) return fail(ATENIA_MOE_ERR_DIM, "no forward has run on this handle");
+  if (hipDeviceSynchronize() != hipSuccess)
+    return fail(ATENIA_MOE_ERR_SYNC, "device synchronisation failed");
+  const size_t P = (size_t)L->last_T * L->k;
+  if (y_host) HIP_TRY(hipMemcpy(y_host, L->y.p, P * L->d * 4, hipMemcpyDeviceToHost));
+  if (y_shared_host && L->fs > 0)
+    HIP_TRY(hipMemcpy(y_shared_host, L->ys.p, (size_t)L->last_T * L->d * 4,
+                      hipMemcpyDeviceToHost));
+  return ATENIA_MOE_OK;
+}
+
+int atenia_moe_hip_layer_set_profiling(AteniaMoeLayer* L, int enabled) {
+  if (!valid_handle(L)) return fail(ATENIA_MOE_ERR_HANDLE, "invalid layer handle");
+  std::lock_guard<std::mutex> lock(L->mu);
+  if (enabled && !L->ev_valid) {
+    for (auto& e : L->ev) HIP_TRY(hipEventCreate(&e));
+    L->ev_valid = true;
+  }
+  L->profiling = enabled != 0;
+  return ATENIA_MOE_OK;
+}
+
+int atenia_moe_hip_layer_stage_ms(AteniaMoeLayer* L, float ms[ATENIA_MOE_N_STAGES]) {
+  if (!valid_handle(L)) return fail(ATENIA_MOE_ERR_HANDLE, "invalid layer handle");
+  if (!ms) return fail(ATENIA_MOE_ERR_DIM, "null pointer");
+  std::lock_guard<std::mutex> lock(L->mu);
+  if (!L->profiling || !L->ev_valid || L->last_T <= 0)
+    return fail(ATENIA_MOE_ERR_DIM, "profiling is off or no forward has run");
+  if (hipEventSynchronize(L->ev[ATENIA_MOE_N_STAGES - 1]) != hipSuccess)
+    return fail(ATENIA_MOE_ERR_SYNC, "event synchronisation failed");
+  for (int i = 0; i < ATENIA_MOE_N_STAGES - 1; ++i)
+    HIP_TRY(hipEventElapsedTime(&ms[i], L->ev[i], L->ev[i + 1]));
+  HIP_TRY(hipEventElapsedTime(&ms[ATENIA_MOE_N_STAGES - 1], L->ev[0],
+                              L->ev[ATENIA_MOE_N_STAGES - 1]));
+  return ATENIA_MOE_OK;
+}
+
+int atenia_moe_hip_layer_stage_launches(AteniaMoeLayer* L, int32_t n[ATENIA_MOE_N_STAGES]) {
+  if (!valid_handle(L)) return fail(ATENIA_MOE_ERR_HANDLE, "invalid layer handle");
+  if (!n) return fail(ATENIA_MOE_ERR_DIM, "null pointer");
+  std::lock_guard<std::mutex> lock(L->mu);
+  for (int i = 0; i < ATENIA_MOE_N_STAGES; ++i) n[i] = L->launches[i];
+  return ATENIA_MOE_OK;
+}
+
+int atenia_moe_hip_layer_info(const AteniaMoeLayer* L, int64_t info[8]) {
+  if (!valid_handle(L)) return fail(ATENIA_MOE_ERR_HANDLE, "invalid layer handle");
+  if (!info) return fail(ATENIA_MOE_ERR_DIM, "null pointer");
+  info[0] = L->E;
+  info[1] = L->k;
+  info[2] = L->d;
+  info[3] = L->f;
+  info[4] = L->fs;
+  info[5] = L->conv;
+  info[6] = L->wdtype;
+  info[7] = L->bytes_per_expert;
+  return ATENIA_MOE_OK;
+}
+
+int atenia_moe_quantize_per_row_i8(const float* w, size_t rows, size_t cols, int8_t* q,
+                                   float* scales) {
+  if (!w || !q || !scales) return fail(ATENIA_MOE_ERR_DIM, "null pointer");
+  for (size_t r = 0; r < rows; ++r) {
+    const float* row = w + r * cols;
+    float amax = 0.0f;
+    for (size_t c = 0; c < cols; ++c) amax = fmaxf(amax, fabsf(row[c]));
+    const float scale = amax > 0.0f ? amax / 127.0f : 1.0f;
+    scales[r] = scale;
+    const float inv = 1.0f / scale;
+    for (size_t c = 0; c < cols; ++c) {
+      float v = roundf(row[c] * inv);
+      v = v < -127.0f ? -127.0f : (v > 127.0f ? 127.0f : v);
+      q[r * cols + c] = (int8_t)v;
+    }
+  }
+  return ATENIA_MOE_OK;
+}
+
+int atenia_moe_f32_to_bf16_trunc(const float* src, size_t n, uint16_t* dst) {
+  if (!src || !dst) return fail(ATENIA_MOE_ERR_DIM, "null pointer");
+  for (size_t i = 0; i < n; ++i) {
+    uint32_t u;
+    memcpy(&u, src + i, 4);
+    dst[i] = (uint16_t)(u >> 16);
+  }
+  return ATENIA_MOE_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,114 @@
+// Internal declarations shared by the HIP translation units of libatenia_moe_hip.so.
+// gfx950 (MI355X, wave64) only.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace atenia_moe {
+
+// ---- limits ------------------------------------------------------------------------------
+constexpr int kMaxRouterRows = 256;  // E (+1 for the shared-expert gate row) handled per block
+constexpr int kPermuteBlock = 1024;  // pairs per permute block
+
+// ---- weight storage in HBM ---------------------------------------------------------------
+// bf16 and int8 expert matrices W[N, K] ("[out, in]", K contiguous in the reference layout)
+// are stored as 1 KiB "B blocks": block (nb, kb) covers rows 16*nb .. 16*nb+15 and KB
+// consecutive k (KB = 32 for bf16, 64 for int8).  Inside a block, lane l of a wavefront
+// owns 16 bytes: row 16*nb + (l & 15), k = KB*kb + (KB/4)*(l >> 4) .. + KB/4 - 1.  That is
+// the register layout of the B operand of v_mfma_f32_16x16x32_bf16, so a wave streams a row
+// strip with one fully contiguous 1 KiB load per block.  Blocks are ordered [nb][kb].
+// N is padded to a multiple of 16 and K to a multiple of KB with zeros.
+constexpr int kBlockBytes = 1024;
+constexpr int kKbBf16 = 32;
+constexpr int kKbInt8 = 64;
+
+static inline int round_up(int v, int m) { return (v + m - 1) / m * m; }
+
+// A set of row groups (one group per expert) for the expert kernels.  All device pointers.
+struct GroupDesc {
+  const int32_t* offsets;   // [G+1] first row of each group in grouped order
+  const int32_t* active;    // [<=G] ids of the groups that have rows, ascending
+  const int32_t* n_active;  // [1]
+  const int32_t* perm;      // [rows] pair id (token*pair_div + slot) of each grouped row
+  int pair_div;             // token = pair id / pair_div
+};
+
+// One expert projection family as stored on the device.
+struct WeightSet {
+  const void* w;            // blocks (bf16/int8) or row-major f32
+  const float* scale;       // int8: per output row, [G, N] (unpadded N stride = n_rows)
+  int64_t expert_stride;    // elements (f32) or bytes (blocked) between experts
+  int n_rows;               // N (unpadded)
+  int n_pad;                // padded N
+  int k_cols;               // K (unpadded)
+  int k_pad;                // padded K
+};
+
+// ---- stage launchers (each returns a hipError_t from the launch) --------------------------
+struct RouterArgs {
+  const void* x;        // [T, d] f32 or bf16
+  int x_is_bf16;
+  int T, d, E, k, renorm;
+  const float* w_router;     // [E, d]
+  const float* router_bias;  // [E] or null
+  const float* shared_gate;  // [d] or null
+  int32_t* idx;              // [T, k]
+  float* w;                  // [T, k]
+  float* sgate;              // [T] (written when shared_gate != null)
+  uint16_t* xb;              // [T, d_pad] bf16 copy of x (null = do not write)
+  int d_pad;
+  int32_t* status;           // [2]: code, (token << 10 | expert)
+};
+hipError_t launch_router(const RouterArgs& a, hipStream_t s);
+
+struct PermuteArgs {
+  const int32_t* idx;  // [P] expert of each pair, P = T*k
+  int T, k, E;
+  int32_t* counts;     // [E]
+  int32_t* offsets;    // [E+1]
+  int32_t* perm;       // [P]
+  int32_t* inv;        // [P] position of each pair in grouped order
+  int32_t* active;     // [E]
+  int32_t* n_active;   // [1]
+  int32_t* blk_counts; // [nblk, E] scratch (multi-block path)
+  int32_t* shared_offsets;  // [2] = {0, T} (may be null)
+};
+hipError_t launch_permute(const PermuteArgs& a, hipStream_t s, int* n_launches);
+
+struct FfnArgs {
+  int wdtype;          // ATENIA_MOE_WEIGHT_*
+  GroupDesc g;
+  int n_groups_max;    // upper bound of *n_active (grid sizing)
+  int rows_max;        // upper bound of rows in any one group (grid sizing)
+  // gate/up phase: x -> h
+  WeightSet gate, up;
+  const void* x;       // bf16 [T, x_stride] (blocked weights) or f32 [T, x_stride]
+  int x_stride;
+  void* h;             // bf16 [rows, h_stride] or f32
+  int h_stride;
+  // down phase: h -> y
+  WeightSet down;
+  float* y;            // f32 [rows, y_stride] indexed by PAIR id (token*pair_div+slot)
+  int y_stride;
+};
+hipError_t launch_ffn_up(const FfnArgs& a, hipStream_t s);
+hipError_t launch_ffn_down(const FfnArgs& a, hipStream_t s);
+
+struct CombineArgs {
+  int T, k, d;
+  const float* w;        // [T, k]
+  const float* y;        // [T*k, y_stride] pair order
+  int y_stride;
+  const float* y_shared; // [T, y_stride] or null
+  const float* sgate;    // [T] or null (scale 1)
+  float* out;            // [T, d]
+};
+hipError_t launch_combine(const CombineArgs& a, hipStream_t s);
+
+// Rewrites a row-major [n_rows, k_cols] matrix (bf16 bits or int8) into B blocks.
+hipError_t launch_repack_blocks(const void* src, void* dst, int n_rows, int k_cols, int n_pad,
+                                int k_pad, int elem_bytes, hipStream_t s);
+hipError_t launch_fill_i32(int32_t* p, int n, int32_t v, int32_t step, hipStream_t s);
+
+}  // namespace atenia_moe

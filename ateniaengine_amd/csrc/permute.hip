@@ -1,0 +1,202 @@
+// Kernel 2: histogram, prefix scan and stable permutation that groups (token, slot) pairs
+// by expert.
+//
+// The reference has no such step: it visits tokens one after another
+// (src/moe/graph_op.rs:345-348) and, inside a token, the selected experts in ascending
+// index order (src/moe/sparse.rs:175).  The grouping contract is derived from that visiting
+// order: pairs are numbered p = t*k + slot, counts[e] is the number of pairs routed to e,
+// offsets is the exclusive scan of counts, and perm lists the pair ids expert by expert,
+// ascending in p inside each expert (a stable counting sort).  All integer work; results are
+// unique, so they must match the CPU oracle bit for bit.
+//
+// Small batches (P <= 1024 pairs) take one launch of one block.  Larger ones take three:
+// per-block histograms, one block that scans them, and a scatter pass that recomputes each
+// block's stable ranks.
+#include "moe_internal.h"
+
+namespace atenia_moe {
+
+namespace {
+
+constexpr int kWaves = kPermuteBlock / 64;
+
+// Stable rank of this thread's pair among the pairs of the same expert inside the block.
+// sWaveCnt: [kWaves][E] scratch.  On return sWaveCnt[w][e] holds the exclusive prefix over
+// waves and sBlkCnt[e] the block total.  All threads of the block must call.
+__device__ int block_stable_rank(int e, bool valid, int E, int32_t* sWaveCnt,
+                                 int32_t* sBlkCnt) {
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  for (int j = tid; j < kWaves * E; j += kPermuteBlock) sWaveCnt[j] = 0;
+  __syncthreads();
+  int my_rank = 0;
+  unsigned long long todo = __ballot(valid);
+  const unsigned long long lt = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  while (todo) {
+    int leader = __ffsll((long long)todo) - 1;
+    int e0 = __shfl(e, leader);
+    unsigned long long m = __ballot(valid && e == e0);
+    if (valid && e == e0) my_rank = __popcll(m & lt);
+    if (lane == leader) sWaveCnt[wave * E + e0] = __popcll(m);
+    todo &= ~m;
+  }
+  __syncthreads();
+  for (int ee = tid; ee < E; ee += kPermuteBlock) {
+    int run = 0;
+    for (int w = 0; w < kWaves; ++w) {
+      int c = sWaveCnt[w * E + ee];
+      sWaveCnt[w * E + ee] = run;
+      run += c;
+    }
+    sBlkCnt[ee] = run;
+  }
+  __syncthreads();
+  return valid ? sWaveCnt[wave * E + e] + my_rank : 0;
+}
+
+// counts -> offsets / active list, done by one thread (E <= a few hundred).
+__device__ void finish_offsets(int E, const int32_t* counts, int32_t* offsets, int32_t* active,
+                               int32_t* n_active, int32_t* shared_offsets, int T) {
+  int run = 0, na = 0;
+  for (int e = 0; e < E; ++e) {
+    offsets[e] = run;
+    int c = counts[e];
+    if (c > 0) active[na++] = e;
+    run += c;
+  }
+  offsets[E] = run;
+  *n_active = na;
+  if (shared_offsets) {
+    shared_offsets[0] = 0;
+    shared_offsets[1] = T;
+  }
+}
+
+__global__ __launch_bounds__(kPermuteBlock) void permute_single_kernel(
+    const int32_t* __restrict__ idx, int P, int E, int T, int32_t* counts, int32_t* offsets,
+    int32_t* perm, int32_t* inv, int32_t* active, int32_t* n_active, int32_t* shared_offsets) {
+  extern __shared__ int32_t sm[];
+  int32_t* sWaveCnt = sm;               // [kWaves][E]
+  int32_t* sBlkCnt = sm + kWaves * E;   // [E]
+  int32_t* sOff = sBlkCnt + E;          // [E+1]
+  const int p = threadIdx.x;
+  const bool valid = p < P;
+  const int e = valid ? idx[p] : 0;
+  int rank = block_stable_rank(e, valid, E, sWaveCnt, sBlkCnt);
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int ee = 0; ee < E; ++ee) {
+      sOff[ee] = run;
+      run += sBlkCnt[ee];
+    }
+    sOff[E] = run;
+  }
+  __syncthreads();
+  for (int ee = threadIdx.x; ee < E; ee += kPermuteBlock) counts[ee] = sBlkCnt[ee];
+  if (threadIdx.x == 0)
+    finish_offsets(E, sBlkCnt, offsets, active, n_active, shared_offsets, T);
+  if (valid) {
+    int pos = sOff[e] + rank;
+    perm[pos] = p;
+    inv[p] = pos;
+  }
+}
+
+__global__ __launch_bounds__(kPermuteBlock) void permute_hist_kernel(
+    const int32_t* __restrict__ idx, int P, int E, int32_t* __restrict__ blk_counts) {
+  extern __shared__ int32_t sm[];
+  for (int j = threadIdx.x; j < E; j += kPermuteBlock) sm[j] = 0;
+  __syncthreads();
+  int p = blockIdx.x * kPermuteBlock + threadIdx.x;
+  if (p < P) atomicAdd(&sm[idx[p]], 1);
+  __syncthreads();
+  for (int j = threadIdx.x; j < E; j += kPermuteBlock)
+    blk_counts[(size_t)blockIdx.x * E + j] = sm[j];
+}
+
+// One block: for every expert, turn the per-block counts into per-block bases.
+__global__ __launch_bounds__(kPermuteBlock) void permute_scan_kernel(
+    int E, int nblk, int T, int32_t* __restrict__ blk_counts, int32_t* counts,
+    int32_t* offsets, int32_t* active, int32_t* n_active, int32_t* shared_offsets) {
+  extern __shared__ int32_t sm[];  // [E] totals, [E+1] offsets
+  int32_t* sTot = sm;
+  int32_t* sOff = sm + E;
+  for (int e = threadIdx.x; e < E; e += kPermuteBlock) {
+    int run = 0;
+    for (int b = 0; b < nblk; ++b) run += blk_counts[(size_t)b * E + e];
+    sTot[e] = run;
+    counts[e] = run;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int e = 0; e < E; ++e) {
+      sOff[e] = run;
+      run += sTot[e];
+    }
+    sOff[E] = run;
+    finish_offsets(E, sTot, offsets, active, n_active, shared_offsets, T);
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += kPermuteBlock) {
+    int run = sOff[e];
+    for (int b = 0; b < nblk; ++b) {
+      int c = blk_counts[(size_t)b * E + e];
+      blk_counts[(size_t)b * E + e] = run;  // becomes the block's base for expert e
+      run += c;
+    }
+  }
+}
+
+__global__ __launch_bounds__(kPermuteBlock) void permute_scatter_kernel(
+    const int32_t* __restrict__ idx, int P, int E, const int32_t* __restrict__ blk_base,
+    int32_t* __restrict__ perm, int32_t* __restrict__ inv) {
+  extern __shared__ int32_t sm[];
+  int32_t* sWaveCnt = sm;
+  int32_t* sBlkCnt = sm + kWaves * E;
+  const int p = blockIdx.x * kPermuteBlock + threadIdx.x;
+  const bool valid = p < P;
+  const int e = valid ? idx[p] : 0;
+  int rank = block_stable_rank(e, valid, E, sWaveCnt, sBlkCnt);
+  if (valid) {
+    int pos = blk_base[(size_t)blockIdx.x * E + e] + rank;
+    perm[pos] = p;
+    inv[p] = pos;
+  }
+}
+
+__global__ void fill_i32_kernel(int32_t* p, int n, int32_t v, int32_t step) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v + step * i;
+}
+
+}  // namespace
+
+hipError_t launch_permute(const PermuteArgs& a, hipStream_t s, int* n_launches) {
+  const int P = a.T * a.k, E = a.E;
+  if (P <= 0) return hipErrorInvalidValue;
+  if (P <= kPermuteBlock) {
+    size_t sm = ((size_t)kWaves * E + E + E + 1) * sizeof(int32_t);
+    permute_single_kernel<<<1, kPermuteBlock, sm, s>>>(a.idx, P, E, a.T, a.counts, a.offsets,
+                                                       a.perm, a.inv, a.active, a.n_active,
+                                                       a.shared_offsets);
+    if (n_launches) *n_launches = 1;
+    return hipGetLastError();
+  }
+  const int nblk = (P + kPermuteBlock - 1) / kPermuteBlock;
+  permute_hist_kernel<<<nblk, kPermuteBlock, (size_t)E * sizeof(int32_t), s>>>(a.idx, P, E,
+                                                                                 a.blk_counts);
+  permute_scan_kernel<<<1, kPermuteBlock, ((size_t)2 * E + 1) * sizeof(int32_t), s>>>(
+      E, nblk, a.T, a.blk_counts, a.counts, a.offsets, a.active, a.n_active, a.shared_offsets);
+  permute_scatter_kernel<<<nblk, kPermuteBlock, ((size_t)kWaves * E + E) * sizeof(int32_t), s>>>(
+      a.idx, P, E, a.blk_counts, a.perm, a.inv);
+  if (n_launches) *n_launches = 3;
+  return hipGetLastError();
+}
+
+hipError_t launch_fill_i32(int32_t* p, int n, int32_t v, int32_t step, hipStream_t s) {
+  if (n <= 0) return hipSuccess;
+  fill_i32_kernel<<<(n + 255) / 256, 256, 0, s>>>(p, n, v, step);
+  return hipGetLastError();
+}
+
+}  // namespace atenia_moe

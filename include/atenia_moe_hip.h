@@ -1,0 +1,201 @@
+/*
+ * atenia_moe_hip.h -- C ABI of the MI355X (gfx950) mixture-of-experts layer forward.
+ *
+ * This is the boundary a host (Rust via `extern "C"`, C++, Python/ctypes) binds to run the
+ * reference's MoE layer op on one GPU.  It takes the place of the reference's `src/cuda`
+ * FFI for this path: plain pointers, `int` dimensions, `int` return codes, no exceptions
+ * and no unwinding across the boundary -- the conventions of the reference's launchers
+ * (`matmul_f32_launch_device`, src/cuda/matmul_kernel.cu:28-55 and src/cuda/matmul.rs:21-32;
+ * `launch_linear_f32_device_ptrs`, src/cuda/linear_cuda.cu:36-73;
+ * `int8_to_bf16_per_channel_launch_device`, src/cuda/int8_to_bf16.cu:42-71).
+ *
+ * Return codes (every entry point that returns `int`):
+ *    0  success
+ *    1  a stream/device synchronisation failed          (linear_cuda.cu:60-70 uses 1)
+ *    2  a kernel launch or runtime call failed          (linear_cuda.cu:44-45 uses 2)
+ *   -1  bad dimensions / null pointer / length mismatch (MoeDenseError::DimMismatch,
+ *                                                        src/moe/dense.rs:31-49)
+ *   -2  bad k: k == 0 or k > num_experts                (MoeSparseError::ZeroK /
+ *                                                        KExceedsExperts, src/moe/sparse.rs:35-50)
+ *   -3  a routing weight is not finite                  (MoeSparseError::NonFiniteWeight{index},
+ *                                                        src/moe/sparse.rs:156-160); token and
+ *                                                        expert via atenia_moe_hip_layer_status
+ *   -4  out of device memory
+ *   -5  invalid handle / unknown layer                  (MoeBindingError::LayerNotFound)
+ *   -6  configuration not supported by this build
+ * A non-zero code leaves the outputs unspecified; the reference's wrappers treat a non-zero
+ * launcher code as "fall back to the CPU path" (src/cuda/matmul.rs:131-150) and a host
+ * keeps that choice.  This library itself never computes on the CPU.
+ *
+ * Threading: any thread may call; one handle is NOT re-entrant (it owns one workspace) and
+ * calls on the same handle are serialised by an internal mutex, as the reference serialises
+ * forwards behind its registry mutex (src/moe/graph_op.rs:304-316).  Different handles may
+ * run concurrently.
+ */
+#ifndef ATENIA_MOE_HIP_H
+#define ATENIA_MOE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* MoeExecutionConvention (src/moe/layer.rs:185-195). */
+#define ATENIA_MOE_CONVENTION_ATENIA 0           /* renormalise top-k weights; ungated shared */
+#define ATENIA_MOE_CONVENTION_HUGGINGFACE_QWEN 1 /* raw softmax weights; sigmoid-gated shared */
+
+/* Storage type of the expert weights, on the host side of `create` and in HBM. */
+#define ATENIA_MOE_WEIGHT_F32 0        /* TensorStorage::Cpu      (src/tensor/tensor.rs:93-160) */
+#define ATENIA_MOE_WEIGHT_BF16 1       /* TensorStorage::CpuBf16, raw u16 bit patterns          */
+#define ATENIA_MOE_WEIGHT_INT8_W8A16 2 /* per-output-row int8 + f32 scales
+                                          (src/tensor/disk_tier.rs:231-259)                     */
+
+/* Element type of device activations handed to `forward_device`. */
+#define ATENIA_MOE_ACT_F32 0
+#define ATENIA_MOE_ACT_BF16 1
+
+#define ATENIA_MOE_OK 0
+#define ATENIA_MOE_ERR_SYNC 1
+#define ATENIA_MOE_ERR_LAUNCH 2
+#define ATENIA_MOE_ERR_DIM (-1)
+#define ATENIA_MOE_ERR_K (-2)
+#define ATENIA_MOE_ERR_NON_FINITE (-3)
+#define ATENIA_MOE_ERR_OOM (-4)
+#define ATENIA_MOE_ERR_HANDLE (-5)
+#define ATENIA_MOE_ERR_UNSUPPORTED (-6)
+
+typedef struct AteniaMoeLayer AteniaMoeLayer; /* opaque; owns weights + workspace in HBM */
+
+/*
+ * Everything `create` needs; all pointers are HOST pointers borrowed for the call only
+ * (the reference's launch helpers borrow host slices the same way,
+ * src/cuda/pool_helpers.rs:118-128).  Mirrors RealMoeLayer + MoeLayerConfig
+ * (src/moe/layer.rs:37-43,200-212) with flat arrays.
+ *
+ * Expert weights are row-major "[out, in]" exactly as the reference holds them
+ * (src/moe/dense.rs:203-210): gate/up `[E, f, d]`, down `[E, d, f]`.  The packed checkpoint
+ * layout `[E, 2f, d]` (gate = rows 0..f, up = rows f..2f; src/moe/binding.rs:384-413) is
+ * passed as `w_gate` with `w_up == NULL`.
+ */
+typedef struct AteniaMoeLayerDesc {
+  int32_t num_experts;     /* E  >= 1                                                    */
+  int32_t top_k;           /* k  = experts_per_token, 1 <= k <= E                        */
+  int32_t d_model;         /* d                                                          */
+  int32_t d_ff;            /* f  (routed expert width)                                   */
+  int32_t d_ff_shared;     /* f_s, 0 = no shared expert                                  */
+  int32_t convention;      /* ATENIA_MOE_CONVENTION_*                                    */
+  int32_t weight_dtype;    /* ATENIA_MOE_WEIGHT_* (applies to routed and shared experts) */
+  int32_t max_tokens_hint; /* workspace is sized for this many tokens up front (0 = lazy) */
+
+  const float* w_router;    /* f32 [E, d]; the router is always f32 (src/moe/dense.rs:325-337) */
+  const float* router_bias; /* f32 [E] added to the f32 logits before softmax, or NULL.
+                               Extension with no counterpart in the reference router.    */
+
+  const void* w_gate;       /* [E, f, d], or packed [E, 2f, d] when w_up == NULL         */
+  const void* w_up;         /* [E, f, d] or NULL                                         */
+  const void* w_down;       /* [E, d, f]                                                 */
+  const float* scale_gate;  /* int8 only: f32 [E, f]  one scale per output row           */
+  const float* scale_up;    /* int8 only: f32 [E, f]                                     */
+  const float* scale_down;  /* int8 only: f32 [E, d]                                     */
+
+  const void* s_gate;       /* shared expert [f_s, d]  (NULL when f_s == 0)              */
+  const void* s_up;         /* [f_s, d]                                                  */
+  const void* s_down;       /* [d, f_s]                                                  */
+  const float* s_scale_gate; /* int8 only: f32 [f_s]                                     */
+  const float* s_scale_up;   /* int8 only: f32 [f_s]                                     */
+  const float* s_scale_down; /* int8 only: f32 [d]                                       */
+  const float* shared_gate; /* f32 [d] sigmoid gate vector (src/moe/layer.rs:436-443) or NULL */
+} AteniaMoeLayerDesc;
+
+/* 1 when a gfx950 device is present and usable, else 0.  Replaces `cuda_available()`
+ * (src/cuda/mod.rs:61-70); the result is computed once per process. */
+int atenia_moe_hip_available(void);
+
+/* Human-readable text of the calling thread's most recent failure ("" if none). */
+const char* atenia_moe_hip_last_error_string(void);
+
+/* Uploads the layer once; the handle owns the device copies, as the reference registry owns
+ * its `Arc<RealMoeLayer>` (src/moe/graph_op.rs:228-232).  Replaces the per-call H->D upload of
+ * the `Fast` policy (src/moe/dense.rs:146-152 -> src/cuda/matmul.rs:131-203). */
+int atenia_moe_hip_layer_create(const AteniaMoeLayerDesc* desc, AteniaMoeLayer** out_layer);
+int atenia_moe_hip_layer_destroy(AteniaMoeLayer* layer);
+
+/* The op: `[T*d]` f32 in host memory -> `[T*d]` f32 in host memory, the WHOLE batch in one
+ * call.  Replaces the per-row loop of `execute_real_moe_layer`
+ * (src/moe/graph_op.rs:327-350) and everything below it (src/moe/layer.rs:405-431,
+ * src/moe/sparse.rs:218-238, src/moe/dense.rs:253-270).  Synchronous.  T == 0 is a no-op. */
+int atenia_moe_hip_layer_forward(AteniaMoeLayer* layer, const float* x_host, int n_tokens,
+                                 float* out_host);
+
+/* Same op on device-resident activations, asynchronous on `stream` (a hipStream_t; NULL =
+ * the default stream).  x: [T, d] of `x_dtype`; out: [T, d] f32.  The call allocates only
+ * when the workspace has to grow (n_tokens above every earlier call and the create hint).
+ * Errors detected on the device (-3) are reported by atenia_moe_hip_layer_status. */
+int atenia_moe_hip_layer_forward_device(AteniaMoeLayer* layer, const void* d_x, int x_dtype,
+                                        int n_tokens, float* d_out, void* stream);
+
+/* Waits for the handle's last forward and returns its device-side status: 0, or -3 with the
+ * first offending token / expert (either pointer may be NULL). */
+int atenia_moe_hip_layer_status(AteniaMoeLayer* layer, void* stream, int32_t* token,
+                                int32_t* expert);
+
+/* Parity taps -------------------------------------------------------------------------- */
+
+/* Router + softmax + top-k only (src/moe/dense.rs:325-337, src/moe/sparse.rs:142-191):
+ * idx[T*k] ascending per token, w[T*k] the (re)normalised f32 weights; host buffers. */
+int atenia_moe_hip_layer_route(AteniaMoeLayer* layer, const float* x_host, int n_tokens,
+                               int32_t* idx_host, float* w_host);
+
+/* Expert grouping of a given routing: counts[E], offsets[E+1], perm[T*k] (pair ids t*k+slot
+ * in expert-major order, stable in pair id); host buffers.  No reference counterpart: the
+ * contract is derived from the reference's visiting order (src/moe/graph_op.rs:345-348,
+ * src/moe/sparse.rs:175). */
+int atenia_moe_hip_layer_permute(AteniaMoeLayer* layer, const int32_t* idx_host, int n_tokens,
+                                 int32_t* counts_host, int32_t* offsets_host,
+                                 int32_t* perm_host);
+
+/* Routing/grouping of the handle's most recent forward, copied to host buffers (any pointer
+ * may be NULL): idx[T*k], w[T*k], counts[E], offsets[E+1], perm[T*k]. */
+int atenia_moe_hip_layer_last_routing(AteniaMoeLayer* layer, int32_t* idx_host, float* w_host,
+                                      int32_t* counts_host, int32_t* offsets_host,
+                                      int32_t* perm_host);
+
+/* Per-(token, slot) expert outputs of the most recent forward, before the weighted combine:
+ * y[T*k, d] f32 in pair order (row t*k+slot = expert idx[t,slot] applied to token t), and the
+ * shared expert's y_shared[T, d] (NULL to skip / when there is none).  Host buffers.  Serves
+ * the per-expert parity obligation of the reference's certification ladder
+ * (docs/decisions/ADR-007-moe-certification-ladder.md:62-73). */
+int atenia_moe_hip_layer_last_expert_outputs(AteniaMoeLayer* layer, float* y_host,
+                                             float* y_shared_host);
+
+/* Stage timing with HIP events recorded on the forward's own stream.  After
+ * `set_profiling(layer, 1)` every forward records an event before/after each stage;
+ * `stage_ms` waits for the last forward and returns that forward's durations in
+ * milliseconds: [0] router, [1] permute, [2] expert gate/up (+shared), [3] expert down
+ * (+shared), [4] combine, [5] whole forward.  `stage_launches` returns the kernel count of
+ * each stage so a per-launch mean can be formed. */
+#define ATENIA_MOE_N_STAGES 6
+int atenia_moe_hip_layer_set_profiling(AteniaMoeLayer* layer, int enabled);
+int atenia_moe_hip_layer_stage_ms(AteniaMoeLayer* layer, float ms[ATENIA_MOE_N_STAGES]);
+int atenia_moe_hip_layer_stage_launches(AteniaMoeLayer* layer, int32_t n[ATENIA_MOE_N_STAGES]);
+
+/* Layer facts a host needs to size buffers: writes E, k, d, f, f_s, convention,
+ * weight_dtype, bytes of expert weights per routed expert as stored in HBM. */
+int atenia_moe_hip_layer_info(const AteniaMoeLayer* layer, int64_t info[8]);
+
+/* Host-side weight preparation (load time, no GPU involved) ------------------------------ */
+
+/* Per-output-row symmetric int8 quantisation, bit-identical to `quantize_per_row_i8`
+ * (src/tensor/disk_tier.rs:231-248): scale = amax/127 (1 for an all-zero row),
+ * q = clamp(round_half_away(w * (1/scale)), -127, 127). */
+int atenia_moe_quantize_per_row_i8(const float* w, size_t rows, size_t cols, int8_t* q,
+                                   float* scales);
+/* f32 -> bf16 bit patterns by truncation (`f32_to_bf16_bits`, src/tensor/tensor.rs:306-308). */
+int atenia_moe_f32_to_bf16_trunc(const float* src, size_t n, uint16_t* dst);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ATENIA_MOE_HIP_H */

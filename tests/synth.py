@@ -1,0 +1,81 @@
+"""Synthetic layers shared by the parity tests: the same host arrays feed the CPU oracle and
+the HIP library, so both see identical stored weight values."""
+import numpy as np
+
+from ateniaengine_amd import capi
+
+
+def bf16_round_trip(a):
+    """f32 -> bf16 (truncation, reference src/tensor/tensor.rs:306-308) -> f32."""
+    bits = capi.f32_to_bf16_trunc(a)
+    return bits, (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+def make_weights(seed, E, d, f, f_s=0, gated=False, w_std=0.02, router_std=None, bias=None,
+                 outlier_frac=0.0):
+    rng = np.random.default_rng(seed)
+    n = lambda *s: rng.standard_normal(s, dtype=np.float32)
+    W = dict(
+        w_router=n(E, d) * (router_std if router_std is not None else w_std),
+        w_gate=n(E, f, d) * w_std, w_up=n(E, f, d) * w_std, w_down=n(E, d, f) * w_std)
+    if f_s:
+        W.update(s_gate=n(f_s, d) * w_std, s_up=n(f_s, d) * w_std, s_down=n(d, f_s) * w_std)
+        if gated:
+            W["shared_gate"] = n(d) * w_std
+    if bias is not None:
+        W["router_bias"] = np.asarray(bias, dtype=np.float32)
+    if outlier_frac > 0:
+        for name in ("w_gate", "w_up", "w_down"):
+            a = W[name].reshape(-1, W[name].shape[-1])
+            rows = rng.choice(a.shape[0], size=max(1, int(a.shape[0] * outlier_frac)),
+                              replace=False)
+            a[rows] *= 8.0
+    return W
+
+
+def build_pair(ora, W, top_k, convention, weight_dtype, max_tokens_hint=0):
+    """Returns (oracle Layer on the stored values, capi Layer)."""
+    proj = ["w_gate", "w_up", "w_down"] + (["s_gate", "s_up", "s_down"] if "s_gate" in W else [])
+    stored, dev, scales = {}, {}, {}
+    for name in proj:
+        w = np.ascontiguousarray(W[name], dtype=np.float32)
+        if weight_dtype == capi.WEIGHT_F32:
+            stored[name] = dev[name] = w
+        elif weight_dtype == capi.WEIGHT_BF16:
+            dev[name], stored[name] = bf16_round_trip(w)
+        else:
+            q, s = capi.quantize_per_row_i8(w)
+            dev[name], scales[name] = q, s
+            stored[name] = (q.astype(np.float32) * s[..., None]).astype(np.float32)
+    if weight_dtype == capi.WEIGHT_F32:
+        router = W["w_router"]
+    else:  # a bf16 checkpoint stores a bf16 router as well
+        router = bf16_round_trip(W["w_router"])[1]
+    common = dict(top_k=top_k, convention=convention, shared_gate=W.get("shared_gate"),
+                  router_bias=W.get("router_bias"))
+    oracle_layer = ora.Layer(w_router=router, w_gate=stored["w_gate"], w_up=stored["w_up"],
+                             w_down=stored["w_down"], s_gate=stored.get("s_gate"),
+                             s_up=stored.get("s_up"), s_down=stored.get("s_down"), **common)
+    kw = {}
+    if weight_dtype == capi.WEIGHT_INT8_W8A16:
+        kw = dict(scale_gate=scales["w_gate"], scale_up=scales["w_up"],
+                  scale_down=scales["w_down"])
+        if "s_gate" in W:
+            kw.update(s_scale_gate=scales["s_gate"], s_scale_up=scales["s_up"],
+                      s_scale_down=scales["s_down"])
+    gpu_layer = capi.Layer(w_router=router, w_gate=dev["w_gate"], w_up=dev["w_up"],
+                           w_down=dev["w_down"], s_gate=dev.get("s_gate"), s_up=dev.get("s_up"),
+                           s_down=dev.get("s_down"), weight_dtype=weight_dtype,
+                           max_tokens_hint=max_tokens_hint, **common, **kw)
+    return oracle_layer, gpu_layer
+
+
+def make_tokens(seed, T, d, bf16=True):
+    x = np.random.default_rng(seed).standard_normal((T, d), dtype=np.float32)
+    return bf16_round_trip(x)[1] if bf16 else x
+
+
+def rel_err(a, ref):
+    """max|a - ref| / max|ref| -- the layer-output metric of the parity bar."""
+    ref = np.asarray(ref, dtype=np.float64)
+    return float(np.abs(np.asarray(a, dtype=np.float64) - ref).max() / np.abs(ref).max())

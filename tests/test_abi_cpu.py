@@ -1,0 +1,54 @@
+"""CPU-side checks of the C-ABI library: it loads, exports every symbol the header declares,
+and its host-only helpers (no GPU involved) match the oracle bit for bit."""
+import os
+import re
+
+import numpy as np
+
+from ateniaengine_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "atenia_moe_hip.h")).read()
+    declared = set(re.findall(r"\b(atenia_moe_\w+)\s*\(", header))
+    assert declared == set(capi.EXPORTS)
+    L = capi.lib()
+    for name in declared:
+        assert hasattr(L, name), f"{name} is declared but not exported"
+
+
+def test_last_error_string_and_bad_handles():
+    L = capi.lib()
+    assert L.atenia_moe_hip_layer_destroy(None) == capi.ERR_HANDLE
+    assert b"invalid layer handle" in L.atenia_moe_hip_last_error_string()
+    assert L.atenia_moe_hip_layer_forward(None, None, 1, None) == capi.ERR_HANDLE
+    assert L.atenia_moe_hip_layer_create(None, None) == capi.ERR_DIM
+
+
+def test_host_quantiser_matches_oracle(ora):
+    rng = np.random.default_rng(0)
+    w = (rng.standard_normal((64, 129)) * 0.02).astype(np.float32)
+    w[5] = 0
+    w[7] *= 8
+    q, s = capi.quantize_per_row_i8(w)
+    oq, os_ = ora.quantize_per_row_i8(w)
+    assert (q == oq).all() and s.tobytes() == os_.tobytes()
+
+
+def test_host_bf16_truncation_matches_oracle(ora):
+    a = np.random.default_rng(1).standard_normal(4097).astype(np.float32)
+    assert (capi.f32_to_bf16_trunc(a) == ora.f32_to_bf16_bits(a)).all()
+
+
+def test_missing_gpu_fails_loudly():
+    """Without a GPU the product path refuses to run; it never computes on the CPU."""
+    if capi.available():
+        return
+    import pytest
+    with pytest.raises(capi.MoeHipError) as e:
+        capi.Layer(w_router=np.zeros((2, 4), np.float32), w_gate=np.zeros((2, 4, 4), np.float32),
+                   w_up=np.zeros((2, 4, 4), np.float32), w_down=np.zeros((2, 4, 4), np.float32),
+                   top_k=1)
+    assert e.value.rc == capi.ERR_LAUNCH and "no gfx950 device" in str(e.value)
