@@ -1,0 +1,225 @@
+#!/usr/bin/env python3
+"""Benchmark of the MoE layer hot path on one MI355X.
+
+Workload (BASELINE config 2): Mixtral-8x7B-shape layer, d_model 4096, 8 experts, top-2 with
+renormalisation, expert d_ff 14336, bf16 weights resident in HBM (2.8 GB), bf16 activations
+already on the device.  A step is one layer forward over one batch of T tokens through the
+C ABI (`atenia_moe_hip_layer_forward_device`).  The default run times the prefill point
+T=4096 (the headline tokens/s, MFMA-bound) and the decode point T=1 (HBM-bound);
+`--sweep 1,16,128,512,4096` adds more batch sizes.
+
+Prints ONE JSON line.  `roofline` describes the dominant kernel of the headline batch, timed
+live with HIP events on the launch stream; `decode.roofline` the same for T=1;
+`cpu_baseline` is the CPU oracle (a C restatement of the reference's certified per-token
+path, not the reference binary) timed on this box's host cores on a bounded token sample.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+D_MODEL, N_EXPERTS, TOP_K, D_FF = 4096, 8, 2, 14336
+W_STD = 0.02
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, GB/s
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, TFLOP/s
+
+
+def make_weights(torch, np, seed):
+    """~N(0, 0.02) weights generated on the GPU, truncated to bf16 (the reference's storage
+    convention, src/tensor/tensor.rs:306-308), returned as host uint16 arrays."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+
+    def bf16_bits(shape):
+        w = torch.randn(shape, generator=g, device="cuda", dtype=torch.float32) * W_STD
+        bits = (w.view(torch.int32) >> 16).to(torch.int16)
+        return bits.cpu().numpy().view(np.uint16)
+
+    gate = np.stack([bf16_bits((D_FF, D_MODEL)) for _ in range(N_EXPERTS)])
+    up = np.stack([bf16_bits((D_FF, D_MODEL)) for _ in range(N_EXPERTS)])
+    down = np.stack([bf16_bits((D_MODEL, D_FF)) for _ in range(N_EXPERTS)])
+    router = bf16_bits((N_EXPERTS, D_MODEL))
+    return router, gate, up, down
+
+
+def upcast(np, bits):
+    return (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+def measure(torch, np, capi, layer, T, steps, warmup, seed):
+    """Times `steps` forwards of a T-token batch; returns a dict of figures."""
+    n_buf = 8 if T <= 64 else 3
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed + T)
+    xs = [torch.randn((T, D_MODEL), generator=g, device="cuda", dtype=torch.float32)
+          .to(torch.bfloat16) for _ in range(n_buf)]
+    out = torch.empty((T, D_MODEL), device="cuda", dtype=torch.float32)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def step(i):
+        layer.forward_device(xs[i % n_buf].data_ptr(), capi.ACT_BF16, T, out.data_ptr(), stream)
+
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(i)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+
+    # Per-stage durations: HIP events recorded by the library on the launch stream.
+    layer.set_profiling(True)
+    acc = np.zeros(capi.N_STAGES, dtype=np.float64)
+    active = 0
+    for i in range(steps):
+        step(i)
+        acc += layer.stage_ms()
+        _, _, counts, _, _ = layer.last_routing(T)
+        active += int((counts > 0).sum())
+    layer.set_profiling(False)
+    stage_ms = acc / steps
+    launches = layer.stage_launches()
+    rc, tok, ex = layer.status(stream)
+    if rc != 0:
+        raise RuntimeError(f"device status {rc} at token {tok}, expert {ex}")
+    U = active / steps  # experts with at least one token (mean over steps)
+
+    eb = 2  # bytes per bf16 weight
+    bytes_up = U * 2 * D_FF * D_MODEL * eb
+    bytes_down = U * D_MODEL * D_FF * eb
+    bytes_fwd = (U * 3 * D_FF * D_MODEL * eb + N_EXPERTS * D_MODEL * 4
+                 + T * D_MODEL * (2 + 4))
+    P = T * TOP_K
+    flops_up = 4.0 * P * D_MODEL * D_FF
+    flops_down = 2.0 * P * D_MODEL * D_FF
+    flops_fwd = T * (2.0 * D_MODEL * N_EXPERTS + 6.0 * TOP_K * D_MODEL * D_FF)
+    r = dict(
+        tokens=T, ms_per_step=wall_ms, tokens_per_s=T / (wall_ms * 1e-3),
+        active_experts=U,
+        stage_ms={n: float(v) for n, v in zip(capi.STAGES, stage_ms)},
+        stage_launches={n: int(v) for n, v in zip(capi.STAGES, launches)},
+        forward_gbs=bytes_fwd / (wall_ms * 1e-3) / 1e9,
+        forward_tflops=flops_fwd / (wall_ms * 1e-3) / 1e12,
+        forward_hbm_frac=bytes_fwd / (wall_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+        forward_mfma_frac=flops_fwd / (wall_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+        algorithmic_bytes=bytes_fwd, algorithmic_flops=flops_fwd,
+    )
+    up_ms, down_ms = stage_ms[2], stage_ms[3]
+    dom, dom_ms, dom_bytes, dom_flops = (
+        ("expert_gate_up", up_ms, bytes_up, flops_up) if up_ms >= down_ms
+        else ("expert_down", down_ms, bytes_down, flops_down))
+    # HBM-bound while the weights outweigh the arithmetic: below ~300 rows per expert.
+    hbm_bound = (dom_flops / (PEAK_BF16_TFLOPS * 1e12)) < (dom_bytes / (PEAK_HBM_GBS * 1e9))
+    if hbm_bound:
+        ach = dom_bytes / (dom_ms * 1e-3) / 1e9
+        r["roofline"] = dict(bound="hbm", kernel=dom, achieved=ach, peak=PEAK_HBM_GBS,
+                             unit="GB/s", frac=ach / PEAK_HBM_GBS, traffic=None,
+                             kernel_ms=float(dom_ms), algorithmic_bytes=dom_bytes)
+    else:
+        ach = dom_flops / (dom_ms * 1e-3) / 1e12
+        r["roofline"] = dict(bound="mfma", kernel=dom, achieved=ach, peak=PEAK_BF16_TFLOPS,
+                             unit="TFLOP/s", frac=ach / PEAK_BF16_TFLOPS, traffic=None,
+                             kernel_ms=float(dom_ms), algorithmic_flops=dom_flops)
+    return r, xs[0], out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--tokens", type=int, default=4096, help="headline batch size T")
+    ap.add_argument("--decode-tokens", type=int, default=1, help="decode batch (0 = skip)")
+    ap.add_argument("--sweep", type=str, default="", help="extra batch sizes, comma separated")
+    ap.add_argument("--cpu-tokens", type=int, default=16,
+                    help="tokens of the CPU-baseline sample (0 = skip)")
+    ap.add_argument("--seed", type=int, default=1234)
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py: this path runs on one GPU (all experts resident in one HBM, no "
+              "collectives); --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    from ateniaengine_amd import capi
+
+    if not capi.available():
+        print("bench.py: no gfx950 device; the HIP path has no fallback", file=sys.stderr)
+        sys.exit(3)
+    torch.cuda.set_device(0)
+    router, gate, up, down = make_weights(torch, np, a.seed)
+    router_f32 = upcast(np, router)
+    tmax = max([a.tokens, a.decode_tokens] + [int(t) for t in a.sweep.split(",") if t])
+    layer = capi.Layer(w_router=router_f32, w_gate=gate, w_up=up, w_down=down, top_k=TOP_K,
+                       convention=capi.CONVENTION_ATENIA, weight_dtype=capi.WEIGHT_BF16,
+                       max_tokens_hint=tmax)
+
+    head, x_head, out_head = measure(torch, np, capi, layer, a.tokens, a.steps, a.warmup, a.seed)
+    decode = None
+    if a.decode_tokens > 0:
+        decode, _, _ = measure(torch, np, capi, layer, a.decode_tokens, max(a.steps, 50),
+                               max(a.warmup, 10), a.seed)
+    sweep = []
+    for t in [int(t) for t in a.sweep.split(",") if t]:
+        r, _, _ = measure(torch, np, capi, layer, t, a.steps if t >= 512 else max(a.steps, 50),
+                          a.warmup, a.seed)
+        sweep.append(r)
+
+    cpu = None
+    parity = None
+    if a.cpu_tokens > 0:
+        from oracle import moe_oracle as ora  # checker + reported CPU baseline only
+        n = min(a.cpu_tokens, a.tokens)
+        # the headline batch, recomputed once so `out_head` matches `x_head`
+        layer.forward_device(x_head.data_ptr(), capi.ACT_BF16, a.tokens, out_head.data_ptr(),
+                             torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        idx_gpu, *_ = layer.last_routing(a.tokens)
+        xs = x_head[:n].to(torch.float32).cpu().numpy()
+        got = out_head[:n].cpu().numpy()
+        oL = ora.Layer(w_router=router_f32, w_gate=upcast(np, gate), w_up=upcast(np, up),
+                       w_down=upcast(np, down), top_k=TOP_K, convention=ora.ATENIA)
+        cores = ora.hw_threads()
+        ora.set_threads(cores)
+        oL.execute(xs[:1])  # warm the pages
+        t0 = time.perf_counter()
+        ref, o_idx, _ = oL.execute(xs)
+        dt = time.perf_counter() - t0
+        cpu = dict(value=n / dt, unit="tokens/s", cores=cores, kind="port",
+                   sample=f"{n} tokens of the T={a.tokens} batch, certified policy "
+                          "(f32 weights, f64 accumulation), rows parallel over all cores")
+        o_all, _ = oL.route_tokens(x_head.to(torch.float32).cpu().numpy())
+        parity = dict(
+            routing_mismatched_tokens=int((idx_gpu != o_all).any(axis=1).sum()),
+            tokens_routed=int(a.tokens),
+            max_rel_err_vs_cpu_path=float(np.abs(got - ref).max() / np.abs(ref).max()),
+            sample_tokens=n)
+
+    line = {
+        "metric": "Mixtral-shape MoE layer tok/s; decode HBM GB/s and prefill MFMA TFLOPS",
+        "value": head["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": a.steps,
+        "warmup": a.warmup, "ms_per_step": head["ms_per_step"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"mixtral-8x7b-shape MoE layer, d_model={D_MODEL}, "
+                               f"experts={N_EXPERTS}, top_k={TOP_K}, d_ff={D_FF}, bf16 weights "
+                               f"resident in HBM, T={a.tokens} tokens per step",
+                   "tokens_per_step": a.tokens},
+        "roofline": head["roofline"],
+        "cpu_baseline": cpu,
+        "prefill": head,
+        "decode": decode,
+        "sweep": sweep,
+        "parity": parity,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

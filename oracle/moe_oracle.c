@@ -62,7 +62,7 @@ void ora_set_threads(int n) { g_threads = n < 1 ? 1 : n; }
 int ora_get_threads(void) { return g_threads; }
 int ora_hw_threads(void) {
 #ifdef _OPENMP
-  return omp_get_num_procs();
+  return omp_get_max_threads(); /* honours OMP_NUM_THREADS */
 #else
   return 1;
 #endif
