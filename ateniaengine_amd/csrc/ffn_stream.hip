@@ -268,6 +268,7 @@ hipError_t launch_ffn_down_f32(const FfnArgs& a, hipStream_t s);
 
 hipError_t launch_ffn_up(const FfnArgs& a, hipStream_t s) {
   if (a.wdtype == ATENIA_MOE_WEIGHT_F32) return launch_ffn_up_f32(a, s);
+  if (a.use_tiled) return launch_ffn_up_tiled(a, s);
   const bool int8 = a.wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
   StreamParams p;
   p.wa = (const uint4*)a.gate.w;
@@ -288,6 +289,7 @@ hipError_t launch_ffn_up(const FfnArgs& a, hipStream_t s) {
 
 hipError_t launch_ffn_down(const FfnArgs& a, hipStream_t s) {
   if (a.wdtype == ATENIA_MOE_WEIGHT_F32) return launch_ffn_down_f32(a, s);
+  if (a.use_tiled) return launch_ffn_down_tiled(a, s);
   const bool int8 = a.wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
   StreamParams p;
   p.wa = (const uint4*)a.down.w;

@@ -1,0 +1,354 @@
+// Kernel 3, tiled form: grouped SwiGLU expert GEMMs for large row counts (prefill).
+//
+//   gate/up : H[rows of e, f] = silu(X_e W_g^T) * (X_e W_u^T)     (src/moe/dense.rs:253-266)
+//   down    : Y[rows of e, d] = H_e W_d^T                         (src/moe/dense.rs:267-269)
+// on v_mfma_f32_16x16x32_bf16 with f32 accumulation.  The bound is the matrix pipeline.
+//
+// A workgroup (4 waves, one per SIMD) owns a 256 x 256 output tile of one expert: 256
+// grouped token rows by 256 weight rows (gate/up phase: 128 gate rows plus the SAME 128 up
+// rows, so silu(g)*u is formed in registers).  Each wave owns 128 x 128 of it as 8 x 8 MFMA
+// tiles (256 accumulator registers); per 32-wide k step it reads 8 A and 8 B fragments from
+// LDS for 64 MFMAs, which keeps LDS at half its bandwidth.
+//
+// LDS holds both operands as 1 KiB chunks already in MFMA register order (lane l owns bytes
+// 16*l), so every fragment read is one conflict-free ds_read_b128.  Weights are stored in HBM
+// in that same chunk layout (moe_internal.h), so a B chunk is a straight 1 KiB copy; token
+// rows are gathered through the permutation while they are loaded (no permuted copy of X is
+// ever written).  INT8 W8A16 weights are widened to bf16 on their way into LDS and the
+// per-row scale is applied to the accumulator.
+//
+// Two LDS stages of 64 k each: global loads of stage i+1 are issued into registers before
+// the MFMAs of stage i and stored to the other LDS buffer after them.
+#include "moe_internal.h"
+
+#include "../../include/atenia_moe_hip.h"
+
+namespace atenia_moe {
+
+namespace {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+
+constexpr int kThreads = 256;
+constexpr int TM = kTileM;   // 256 token rows
+constexpr int TNB = 256;     // B rows per tile (gate/up: 128 + 128)
+constexpr int TK = 64;       // k per LDS stage
+constexpr int kChunk = 1024; // bytes
+constexpr int kAStage = (TM / 16) * (TK / 32) * kChunk;   // 32 KiB
+constexpr int kBStage = (TNB / 16) * (TK / 32) * kChunk;  // 32 KiB
+constexpr int kStage = kAStage + kBStage;
+constexpr int kLdsBytes = 2 * kStage;                     // 128 KiB
+
+struct TiledParams {
+  const uint4* wa;      // gate (up phase) or down blocks
+  const uint4* wb;      // up blocks
+  const float* sa;      // int8 row scales [G, n_rows]
+  const float* sb;
+  int64_t w_stride_u4;
+  int n_rows;           // unpadded N
+  int n_blocks;         // n_pad / 16
+  int nkb;              // K blocks per strip (32 k each for bf16, 64 k for int8)
+  int k_pad;
+  const uint16_t* a;    // bf16 rows
+  int a_stride;
+  void* out;
+  int out_stride;
+  GroupDesc g;
+  const int32_t* tile_group;  // [n_tiles] expert of each row tile
+  const int32_t* tile_m0;     // [n_tiles] first row (relative to the group) of each row tile
+  const int32_t* n_tiles;     // [1]
+  int n_col_tiles;
+};
+
+__device__ inline uint16_t bf16_rne(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+__device__ inline uint32_t pack_i8_pair(uint32_t w, int sh) {
+  float f0 = (float)(int8_t)((w >> sh) & 0xff);
+  float f1 = (float)(int8_t)((w >> (sh + 8)) & 0xff);
+  return (__float_as_uint(f0) >> 16) | (__float_as_uint(f1) & 0xffff0000u);
+}
+__device__ inline void widen_i8x16(uint4 q, uint4& lo, uint4& hi) {
+  lo.x = pack_i8_pair(q.x, 0);
+  lo.y = pack_i8_pair(q.x, 16);
+  lo.z = pack_i8_pair(q.y, 0);
+  lo.w = pack_i8_pair(q.y, 16);
+  hi.x = pack_i8_pair(q.z, 0);
+  hi.y = pack_i8_pair(q.z, 16);
+  hi.z = pack_i8_pair(q.w, 0);
+  hi.w = pack_i8_pair(q.w, 16);
+}
+
+__device__ inline f32x4 mfma(uint4 a, uint4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(bf16x8*)&a, *(bf16x8*)&b, c, 0, 0, 0);
+}
+
+template <bool INT8, bool UP>
+__global__ __launch_bounds__(kThreads) void ffn_tiled_kernel(TiledParams p) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  // XCD-aware order: hardware deals consecutive workgroups round-robin to the 8 XCDs, so
+  // give each XCD a contiguous run of logical tiles; neighbours in that run share a weight
+  // tile (row tiles of one expert are innermost) and meet in the same L2.
+  const int n_row_tiles = *p.n_tiles;
+  const int total = n_row_tiles * p.n_col_tiles;
+  const int per_xcd = (total + 7) / 8;
+  const int slot = blockIdx.x / 8;
+  const int logical = (blockIdx.x % 8) * per_xcd + slot;
+  if (slot >= per_xcd || logical >= total) return;
+  // logical -> (column tile, row tile), row tile fastest.
+  const int ct = logical / n_row_tiles;
+  const int rt = logical - ct * n_row_tiles;
+
+  const int e = p.tile_group[rt];
+  const int tm0 = p.tile_m0[rt];
+  const int base = p.g.offsets[e];
+  const int cnt = p.g.offsets[e + 1] - base;
+  const int rows_here = min(TM, cnt - tm0);
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int kq = lane >> 4, mm = lane & 15;
+  const int wm = wave >> 1, wn = wave & 1;
+  constexpr int BROWS = UP ? 128 : 256;  // distinct weight rows per tile
+  const int nb0 = ct * (BROWS / 16);     // first 16-row weight block of the tile
+
+  // ---- what this thread loads each stage -------------------------------------------------
+  // A: chunks c = wave*8 + j  ->  (msub = c >> 1, k32 = c & 1); 4 distinct rows per thread.
+  const uint16_t* arow[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    int m = (wave * 4 + q) * 16 + mm;
+    if (m >= rows_here) m = 0;  // clamp: such rows are computed but never stored
+    int src;
+    if (UP) src = p.g.perm[base + tm0 + m] / p.g.pair_div;
+    else src = base + tm0 + m;
+    arow[q] = p.a + (size_t)src * p.a_stride + (INT8 ? 16 * kq : 8 * kq);
+  }
+  // B (bf16): chunks c = wave*8 + j -> (nsub = c >> 1, k32 = c & 1), a straight block copy.
+  // B (int8): blocks nsub = wave*4 + j, one 64-k block each, widened into two chunks.
+  constexpr int NBL = INT8 ? 4 : 8;  // B loads per thread per stage
+  const uint4* bptr[INT8 ? 4 : 4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    int nsub = wave * 4 + q;
+    int nb;
+    const uint4* wbase;
+    if (UP) {
+      wbase = nsub < 8 ? p.wa : p.wb;
+      nb = nb0 + (nsub & 7);
+    } else {
+      wbase = p.wa;
+      nb = nb0 + nsub;
+    }
+    if (nb >= p.n_blocks) nb = p.n_blocks - 1;  // clamp: columns past N are never stored
+    bptr[q] = wbase + (size_t)e * p.w_stride_u4 + (size_t)nb * p.nkb * 64 + lane;
+  }
+
+  uint4 ra[8], rb[NBL];
+  auto load_stage = [&](int ks) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int q = j >> 1, k32 = j & 1;
+      const int koff = ks * TK + (INT8 ? 8 * k32 : 32 * k32);
+      ra[j] = *(const uint4*)(arow[q] + koff);
+    }
+    if (INT8) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) rb[q] = bptr[q][(size_t)ks * 64];
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) rb[j] = bptr[j >> 1][(size_t)(ks * 2 + (j & 1)) * 64];
+    }
+  };
+  auto store_stage = [&](int buf) {
+    uint8_t* sA = lds + buf * kStage;
+    uint8_t* sB = sA + kAStage;
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      *(uint4*)(sA + (wave * 8 + j) * kChunk + lane * 16) = ra[j];
+    if (INT8) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        uint4 lo, hi;
+        widen_i8x16(rb[q], lo, hi);
+        *(uint4*)(sB + ((wave * 4 + q) * 2 + 0) * kChunk + lane * 16) = lo;
+        *(uint4*)(sB + ((wave * 4 + q) * 2 + 1) * kChunk + lane * 16) = hi;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        *(uint4*)(sB + (wave * 8 + j) * kChunk + lane * 16) = rb[j];
+    }
+  };
+
+  f32x4 acc[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // Row sub-tiles of this wave that hold real rows (uniform per wave).
+  const int my_rows = rows_here - wm * 128;
+  const int mt = my_rows <= 0 ? 0 : min(8, (my_rows + 15) >> 4);
+
+  const int nks = p.k_pad / TK;
+  load_stage(0);
+  store_stage(0);
+  __syncthreads();
+  for (int ks = 0; ks < nks; ++ks) {
+    const bool more = ks + 1 < nks;
+    if (more) load_stage(ks + 1);
+    const uint8_t* sA = lds + (ks & 1) * kStage;
+    const uint8_t* sB = sA + kAStage;
+#pragma unroll
+    for (int k32 = 0; k32 < 2; ++k32) {
+      uint4 bf[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        // gate/up: j < 4 gate sub-tiles 4*wn+j, j >= 4 the matching up sub-tiles
+        int nsub = UP ? ((j < 4 ? 0 : 8) + 4 * wn + (j & 3)) : (8 * wn + j);
+        bf[j] = *(const uint4*)(sB + (nsub * 2 + k32) * kChunk + lane * 16);
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if (i < mt) {
+          uint4 af = *(const uint4*)(sA + ((wm * 8 + i) * 2 + k32) * kChunk + lane * 16);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) acc[i][j] = mfma(af, bf[j], acc[i][j]);
+        }
+      }
+    }
+    if (more) store_stage((ks + 1) & 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue ----------------------------------------------------------------------------
+  // D layout: lane holds rows 4*kq + r (r = 0..3) of column mm of each 16 x 16 tile.
+  if (UP) {
+    uint16_t* h = (uint16_t*)p.out;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = (nb0 + 4 * wn + j) * 16 + mm;
+      const bool n_ok = n < p.n_blocks * 16;
+      float sa = 1.f, sb = 1.f;
+      if (INT8) {
+        sa = n < p.n_rows ? p.sa[(size_t)e * p.n_rows + n] : 0.f;
+        sb = n < p.n_rows ? p.sb[(size_t)e * p.n_rows + n] : 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if (i >= mt) continue;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int m = wm * 128 + i * 16 + 4 * kq + r;
+          if (m < rows_here && n_ok) {
+            float g = acc[i][j][r] * sa;
+            float u = acc[i][j + 4][r] * sb;
+            float hv = (g / (1.f + __expf(-g))) * u;
+            h[(size_t)(base + tm0 + m) * p.out_stride + n] = bf16_rne(hv);
+          }
+        }
+      }
+    }
+  } else {
+    float* y = (float*)p.out;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (i >= mt) continue;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = wm * 128 + i * 16 + 4 * kq + r;
+        if (m >= rows_here) continue;
+        const int pair = p.g.perm[base + tm0 + m];
+        float* yr = y + (size_t)pair * p.out_stride;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int n = (nb0 + 8 * wn + j) * 16 + mm;
+          if (n < p.n_rows) {
+            float s = INT8 ? p.sa[(size_t)e * p.n_rows + n] : 1.f;
+            yr[n] = acc[i][j][r] * s;
+          }
+        }
+      }
+    }
+  }
+}
+
+template <bool INT8, bool UP>
+hipError_t launch_tiled(const TiledParams& p, int max_row_tiles, hipStream_t s) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)ffn_tiled_kernel<INT8, UP>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    if (e != hipSuccess) return e;
+    attr_set = true;
+  }
+  // Upper bound of the grid; workgroups past the real tile count return at once.
+  int n_wg = max_row_tiles * p.n_col_tiles;
+  n_wg = (n_wg + 7) / 8 * 8;
+  ffn_tiled_kernel<INT8, UP><<<n_wg, kThreads, kLdsBytes, s>>>(p);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+bool tiled_supported(const WeightSet& w, int wdtype) {
+  if (wdtype == ATENIA_MOE_WEIGHT_F32) return false;
+  return w.k_pad % TK == 0;
+}
+
+hipError_t launch_ffn_up_tiled(const FfnArgs& a, hipStream_t s) {
+  const bool int8 = a.wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
+  TiledParams p{};
+  p.wa = (const uint4*)a.gate.w;
+  p.wb = (const uint4*)a.up.w;
+  p.sa = a.gate.scale;
+  p.sb = a.up.scale;
+  p.w_stride_u4 = a.gate.expert_stride / 16;
+  p.n_rows = a.gate.n_rows;
+  p.n_blocks = a.gate.n_pad / 16;
+  p.nkb = a.gate.k_pad / (int8 ? kKbInt8 : kKbBf16);
+  p.k_pad = a.gate.k_pad;
+  p.a = (const uint16_t*)a.x;
+  p.a_stride = a.x_stride;
+  p.out = a.h;
+  p.out_stride = a.h_stride;
+  p.g = a.g;
+  p.tile_group = a.tile_group;
+  p.tile_m0 = a.tile_m0;
+  p.n_tiles = a.n_tiles;
+  p.n_col_tiles = (a.gate.n_pad + 127) / 128;
+  return int8 ? launch_tiled<true, true>(p, a.max_row_tiles, s)
+              : launch_tiled<false, true>(p, a.max_row_tiles, s);
+}
+
+hipError_t launch_ffn_down_tiled(const FfnArgs& a, hipStream_t s) {
+  const bool int8 = a.wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
+  TiledParams p{};
+  p.wa = (const uint4*)a.down.w;
+  p.wb = nullptr;
+  p.sa = a.down.scale;
+  p.sb = nullptr;
+  p.w_stride_u4 = a.down.expert_stride / 16;
+  p.n_rows = a.down.n_rows;
+  p.n_blocks = a.down.n_pad / 16;
+  p.nkb = a.down.k_pad / (int8 ? kKbInt8 : kKbBf16);
+  p.k_pad = a.down.k_pad;
+  p.a = (const uint16_t*)a.h;
+  p.a_stride = a.h_stride;
+  p.out = a.y;
+  p.out_stride = a.y_stride;
+  p.g = a.g;
+  p.tile_group = a.tile_group;
+  p.tile_m0 = a.tile_m0;
+  p.n_tiles = a.n_tiles;
+  p.n_col_tiles = (a.down.n_pad + 255) / 256;
+  return int8 ? launch_tiled<true, false>(p, a.max_row_tiles, s)
+              : launch_tiled<false, false>(p, a.max_row_tiles, s);
+}
+
+}  // namespace atenia_moe

@@ -92,7 +92,7 @@ struct AteniaMoeLayer {
   // workspace (grow-only in tokens)
   int cap_tokens = 0;
   DevBuf x_in, out, xb, idx, w, sgate, counts, offsets, active, n_active, perm, inv, blk_counts,
-      shared_desc, ident, h, hs, y, ys, status;
+      shared_desc, ident, h, hs, y, ys, status, tile_group, tile_m0, s_tile_group, s_tile_m0;
   int last_T = 0;
 
   hipStream_t stream = nullptr;
@@ -105,6 +105,9 @@ struct AteniaMoeLayer {
 };
 
 namespace {
+
+// Largest batch served by the weight-streaming expert kernels.
+constexpr int kStreamMaxTokens = 128;
 
 bool valid_handle(const AteniaMoeLayer* L) { return L && L->magic == 0x4d6f4541u; }
 
@@ -175,7 +178,13 @@ int ensure_workspace(AteniaMoeLayer* L, int T) {
   ENS(perm, P * 4)
   ENS(inv, P * 4)
   ENS(blk_counts, ((P + kPermuteBlock - 1) / kPermuteBlock) * L->E * 4)
-  ENS(shared_desc, 16)  // [0..1] offsets {0,T}, [2] active {0}, [3] n_active {1}
+  ENS(shared_desc, 32)  // [0..1] offsets {0,T}, [2] active {0}, [3] n_active {1},
+                        // [4] routed row tiles, [5] shared row tiles
+  const size_t max_tiles = (P + kTileM - 1) / kTileM + L->E;
+  ENS(tile_group, max_tiles * 4)
+  ENS(tile_m0, max_tiles * 4)
+  ENS(s_tile_group, ((size_t)T / kTileM + 1) * 4)
+  ENS(s_tile_m0, ((size_t)T / kTileM + 1) * 4)
   ENS(ident, (size_t)T * 4)
   ENS(h, P * (size_t)L->f_kpad * act)
   ENS(y, P * (size_t)L->d * 4)
@@ -186,8 +195,9 @@ int ensure_workspace(AteniaMoeLayer* L, int T) {
   ENS(status, 8)
 #undef ENS
   HIP_TRY(launch_fill_i32(L->ident.as<int32_t>(), T, 0, 1, nullptr));
-  int32_t sd[4] = {0, 0, 0, 1};
-  HIP_TRY(hipMemcpy(L->shared_desc.p, sd, 16, hipMemcpyHostToDevice));
+  HIP_TRY(launch_fill_i32(L->s_tile_m0.as<int32_t>(), T / kTileM + 1, 0, kTileM, nullptr));
+  int32_t sd[8] = {0, 0, 0, 1, 0, 0, 0, 0};
+  HIP_TRY(hipMemcpy(L->shared_desc.p, sd, 32, hipMemcpyHostToDevice));
   int32_t st[2] = {0, INT_MAX};
   HIP_TRY(hipMemcpy(L->status.p, st, 8, hipMemcpyHostToDevice));
   HIP_TRY(hipDeviceSynchronize());
@@ -255,6 +265,10 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   pa.n_active = L->n_active.as<int32_t>();
   pa.blk_counts = L->blk_counts.as<int32_t>();
   pa.shared_offsets = L->shared_desc.as<int32_t>();
+  pa.tile_group = L->tile_group.as<int32_t>();
+  pa.tile_m0 = L->tile_m0.as<int32_t>();
+  pa.n_tiles = L->shared_desc.as<int32_t>() + 4;
+  pa.shared_n_tiles = L->shared_desc.as<int32_t>() + 5;
   int nl = 0;
   HIP_TRY(launch_permute(pa, s, &nl));
   L->launches[1] = nl;
@@ -281,6 +295,16 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   fa.h_stride = L->f_kpad;
   fa.y = L->y.as<float>();
   fa.y_stride = L->d;
+  // Tiled (MFMA-bound) kernels once an expert can see more rows than the streaming kernel
+  // keeps in registers; below that the weights are streamed once (HBM-bound).
+  const bool tiled = T > kStreamMaxTokens && tiled_supported(L->gate, L->wdtype) &&
+                     tiled_supported(L->down, L->wdtype);
+  fa.use_tiled = tiled;
+  fa.tile_group = L->tile_group.as<int32_t>();
+  fa.tile_m0 = L->tile_m0.as<int32_t>();
+  fa.n_tiles = L->shared_desc.as<int32_t>() + 4;
+  fa.max_row_tiles = (int)(((size_t)T * L->k + kTileM - 1) / kTileM +
+                           std::min<long long>(L->E, (long long)T * L->k));
 
   FfnArgs fsd{};
   if (L->fs > 0) {
@@ -299,6 +323,12 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
     fsd.h = L->hs.p;
     fsd.h_stride = L->fs_kpad;
     fsd.y = L->ys.as<float>();
+    fsd.use_tiled = T > kStreamMaxTokens && tiled_supported(L->s_gate, L->wdtype) &&
+                    tiled_supported(L->s_down, L->wdtype);
+    fsd.tile_group = L->s_tile_group.as<int32_t>();
+    fsd.tile_m0 = L->s_tile_m0.as<int32_t>();
+    fsd.n_tiles = L->shared_desc.as<int32_t>() + 5;
+    fsd.max_row_tiles = (T + kTileM - 1) / kTileM;
   }
 
   HIP_TRY(launch_ffn_up(fa, s));
@@ -579,6 +609,10 @@ int atenia_moe_hip_layer_permute(AteniaMoeLayer* L, const int32_t* idx_host, int
   pa.n_active = L->n_active.as<int32_t>();
   pa.blk_counts = L->blk_counts.as<int32_t>();
   pa.shared_offsets = nullptr;
+  pa.tile_group = nullptr;
+  pa.tile_m0 = nullptr;
+  pa.n_tiles = nullptr;
+  pa.shared_n_tiles = nullptr;
   HIP_TRY(launch_permute(pa, L->stream, nullptr));
   if (hipStreamSynchronize(L->stream) != hipSuccess)
     return fail(ATENIA_MOE_ERR_SYNC, "stream synchronisation failed");

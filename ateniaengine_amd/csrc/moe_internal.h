@@ -10,6 +10,7 @@ namespace atenia_moe {
 // ---- limits ------------------------------------------------------------------------------
 constexpr int kMaxRouterRows = 256;  // E (+1 for the shared-expert gate row) handled per block
 constexpr int kPermuteBlock = 1024;  // pairs per permute block
+constexpr int kTileM = 256;          // token rows per tile of the tiled expert kernels
 
 // ---- weight storage in HBM ---------------------------------------------------------------
 // bf16 and int8 expert matrices W[N, K] ("[out, in]", K contiguous in the reference layout)
@@ -73,6 +74,12 @@ struct PermuteArgs {
   int32_t* n_active;   // [1]
   int32_t* blk_counts; // [nblk, E] scratch (multi-block path)
   int32_t* shared_offsets;  // [2] = {0, T} (may be null)
+  // Row tiles of kTileM rows for the tiled expert kernels: expert and first row (relative to
+  // the expert's group) of each tile, experts ascending; may be null.
+  int32_t* tile_group;      // [<= ceil(P / kTileM) + E]
+  int32_t* tile_m0;
+  int32_t* n_tiles;         // [1]
+  int32_t* shared_n_tiles;  // [1] = ceil(T / kTileM) (may be null)
 };
 hipError_t launch_permute(const PermuteArgs& a, hipStream_t s, int* n_launches);
 
@@ -91,7 +98,16 @@ struct FfnArgs {
   WeightSet down;
   float* y;            // f32 [rows, y_stride] indexed by PAIR id (token*pair_div+slot)
   int y_stride;
+  // tiled kernels only
+  int use_tiled;
+  const int32_t* tile_group;
+  const int32_t* tile_m0;
+  const int32_t* n_tiles;
+  int max_row_tiles;   // upper bound of *n_tiles (grid sizing)
 };
+bool tiled_supported(const WeightSet& w, int wdtype);
+hipError_t launch_ffn_up_tiled(const FfnArgs& a, hipStream_t s);
+hipError_t launch_ffn_down_tiled(const FfnArgs& a, hipStream_t s);
 hipError_t launch_ffn_up(const FfnArgs& a, hipStream_t s);
 hipError_t launch_ffn_down(const FfnArgs& a, hipStream_t s);
 

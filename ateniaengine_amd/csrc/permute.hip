@@ -54,17 +54,32 @@ __device__ int block_stable_rank(int e, bool valid, int E, int32_t* sWaveCnt,
 }
 
 // counts -> offsets / active list, done by one thread (E <= a few hundred).
+struct TileOut {
+  int32_t* tile_group;
+  int32_t* tile_m0;
+  int32_t* n_tiles;
+  int32_t* shared_n_tiles;
+};
+
 __device__ void finish_offsets(int E, const int32_t* counts, int32_t* offsets, int32_t* active,
-                               int32_t* n_active, int32_t* shared_offsets, int T) {
-  int run = 0, na = 0;
+                               int32_t* n_active, int32_t* shared_offsets, int T, TileOut to) {
+  int run = 0, na = 0, nt = 0;
   for (int e = 0; e < E; ++e) {
     offsets[e] = run;
     int c = counts[e];
     if (c > 0) active[na++] = e;
+    if (to.tile_group)
+      for (int m0 = 0; m0 < c; m0 += kTileM) {
+        to.tile_group[nt] = e;
+        to.tile_m0[nt] = m0;
+        ++nt;
+      }
     run += c;
   }
   offsets[E] = run;
   *n_active = na;
+  if (to.n_tiles) *to.n_tiles = nt;
+  if (to.shared_n_tiles) *to.shared_n_tiles = (T + kTileM - 1) / kTileM;
   if (shared_offsets) {
     shared_offsets[0] = 0;
     shared_offsets[1] = T;
@@ -73,7 +88,8 @@ __device__ void finish_offsets(int E, const int32_t* counts, int32_t* offsets, i
 
 __global__ __launch_bounds__(kPermuteBlock) void permute_single_kernel(
     const int32_t* __restrict__ idx, int P, int E, int T, int32_t* counts, int32_t* offsets,
-    int32_t* perm, int32_t* inv, int32_t* active, int32_t* n_active, int32_t* shared_offsets) {
+    int32_t* perm, int32_t* inv, int32_t* active, int32_t* n_active, int32_t* shared_offsets,
+    TileOut to) {
   extern __shared__ int32_t sm[];
   int32_t* sWaveCnt = sm;               // [kWaves][E]
   int32_t* sBlkCnt = sm + kWaves * E;   // [E]
@@ -93,7 +109,7 @@ __global__ __launch_bounds__(kPermuteBlock) void permute_single_kernel(
   __syncthreads();
   for (int ee = threadIdx.x; ee < E; ee += kPermuteBlock) counts[ee] = sBlkCnt[ee];
   if (threadIdx.x == 0)
-    finish_offsets(E, sBlkCnt, offsets, active, n_active, shared_offsets, T);
+    finish_offsets(E, sBlkCnt, offsets, active, n_active, shared_offsets, T, to);
   if (valid) {
     int pos = sOff[e] + rank;
     perm[pos] = p;
@@ -116,7 +132,7 @@ __global__ __launch_bounds__(kPermuteBlock) void permute_hist_kernel(
 // One block: for every expert, turn the per-block counts into per-block bases.
 __global__ __launch_bounds__(kPermuteBlock) void permute_scan_kernel(
     int E, int nblk, int T, int32_t* __restrict__ blk_counts, int32_t* counts,
-    int32_t* offsets, int32_t* active, int32_t* n_active, int32_t* shared_offsets) {
+    int32_t* offsets, int32_t* active, int32_t* n_active, int32_t* shared_offsets, TileOut to) {
   extern __shared__ int32_t sm[];  // [E] totals, [E+1] offsets
   int32_t* sTot = sm;
   int32_t* sOff = sm + E;
@@ -134,7 +150,7 @@ __global__ __launch_bounds__(kPermuteBlock) void permute_scan_kernel(
       run += sTot[e];
     }
     sOff[E] = run;
-    finish_offsets(E, sTot, offsets, active, n_active, shared_offsets, T);
+    finish_offsets(E, sTot, offsets, active, n_active, shared_offsets, T, to);
   }
   __syncthreads();
   for (int e = threadIdx.x; e < E; e += kPermuteBlock) {
@@ -174,11 +190,12 @@ __global__ void fill_i32_kernel(int32_t* p, int n, int32_t v, int32_t step) {
 hipError_t launch_permute(const PermuteArgs& a, hipStream_t s, int* n_launches) {
   const int P = a.T * a.k, E = a.E;
   if (P <= 0) return hipErrorInvalidValue;
+  TileOut to{a.tile_group, a.tile_m0, a.n_tiles, a.shared_n_tiles};
   if (P <= kPermuteBlock) {
     size_t sm = ((size_t)kWaves * E + E + E + 1) * sizeof(int32_t);
     permute_single_kernel<<<1, kPermuteBlock, sm, s>>>(a.idx, P, E, a.T, a.counts, a.offsets,
                                                        a.perm, a.inv, a.active, a.n_active,
-                                                       a.shared_offsets);
+                                                       a.shared_offsets, to);
     if (n_launches) *n_launches = 1;
     return hipGetLastError();
   }
@@ -186,7 +203,8 @@ hipError_t launch_permute(const PermuteArgs& a, hipStream_t s, int* n_launches) 
   permute_hist_kernel<<<nblk, kPermuteBlock, (size_t)E * sizeof(int32_t), s>>>(a.idx, P, E,
                                                                                  a.blk_counts);
   permute_scan_kernel<<<1, kPermuteBlock, ((size_t)2 * E + 1) * sizeof(int32_t), s>>>(
-      E, nblk, a.T, a.blk_counts, a.counts, a.offsets, a.active, a.n_active, a.shared_offsets);
+      E, nblk, a.T, a.blk_counts, a.counts, a.offsets, a.active, a.n_active, a.shared_offsets,
+      to);
   permute_scatter_kernel<<<nblk, kPermuteBlock, ((size_t)kWaves * E + E) * sizeof(int32_t), s>>>(
       a.idx, P, E, a.blk_counts, a.perm, a.inv);
   if (n_launches) *n_launches = 3;

@@ -79,3 +79,39 @@ def rel_err(a, ref):
     """max|a - ref| / max|ref| -- the layer-output metric of the parity bar."""
     ref = np.asarray(ref, dtype=np.float64)
     return float(np.abs(np.asarray(a, dtype=np.float64) - ref).max() / np.abs(ref).max())
+
+
+def bf16_rne(a):
+    """f32 -> nearest-even bf16 -> f32 (the rounding the expert kernels apply to h)."""
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    u = u + 0x7FFF + ((u >> 16) & 1)
+    return ((u >> 16) << 16).astype(np.uint32).view(np.float32)
+
+
+def emulate_bf16_kernels(oL, x, idx, w):
+    """NumPy model of the bf16/int8 HIP path's arithmetic on the oracle layer's stored
+    weights: exact products with wide accumulation, gate/up rounded to f32, h = silu(g)*u in
+    f32 rounded to bf16 (nearest even), f32 combine with separate multiply and add.  The GPU
+    result must sit within ~1e-3 of this model (differences: f32 accumulation order and a
+    rare bf16 rounding flip of an h element); the distance of either from the all-f64
+    reference is the bf16 rounding of h, ~2e-3 at real layer sizes."""
+    T, d = x.shape
+    out = np.zeros((T, d), dtype=np.float32)
+
+    def expert(g, u, dn, xv):
+        gg = (g.astype(np.float64) @ xv).astype(np.float32)
+        uu = (u.astype(np.float64) @ xv).astype(np.float32)
+        h = bf16_rne((gg / (np.float32(1) + np.exp(-gg, dtype=np.float32))) * uu)
+        return (dn.astype(np.float64) @ h.astype(np.float64)).astype(np.float32)
+
+    for t in range(T):
+        xv = x[t].astype(np.float64)
+        for s_, e in enumerate(idx[t]):
+            out[t] = out[t] + w[t, s_] * expert(oL.w_gate[e], oL.w_up[e], oL.w_down[e], xv)
+        if oL.f_s:
+            sc = np.float32(1.0)
+            if oL.convention == 1 and oL.shared_gate is not None:
+                acc = float(oL.shared_gate.astype(np.float64) @ xv)
+                sc = np.float32(1.0 / (1.0 + np.exp(-acc)))
+            out[t] = out[t] + sc * expert(oL.s_gate, oL.s_up, oL.s_down, xv)
+    return out
