@@ -278,6 +278,197 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_kernel(TiledParams p) {
   }
 }
 
+// ---- bf16 form with direct global->LDS loads and a four-stage ring -------------------------
+// Same tiling.  Each stage holds 32 k of both operands (16 KiB + 16 KiB); a wave fills a
+// 1 KiB chunk with one global_load_lds_dwordx4 (lane l's 16 bytes land at chunk + 16*l), so
+// no operand passes through registers on its way to LDS and three stages (about 3 * 64 MFMAs
+// of work) are always in flight behind the one being multiplied.  The four stage buffers are
+// separate arrays and the k loop is unrolled by four, so each fragment read names its buffer
+// statically.
+typedef __attribute__((address_space(1))) const void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+constexpr int kDmaStageU4 = 2 * 16 * 64;  // uint4 per stage: 16 A chunks + 16 B chunks
+
+__device__ inline void wait_vmcnt(int n) {
+  // s_waitcnt with only vmcnt active: vmcnt[3:0] in bits 3:0, vmcnt[5:4] in bits 15:14.
+  if (n >= 16) __builtin_amdgcn_s_waitcnt(0x4F70);
+  else if (n >= 8) __builtin_amdgcn_s_waitcnt(0x0F78);
+  else __builtin_amdgcn_s_waitcnt(0x0F70);
+}
+
+// One wave-wide 16-byte-per-lane load from global memory straight into LDS: lane l's bytes
+// land at lds_addr + 16*l.  Written as inline assembly so that the compiler's wait-count
+// insertion does not tie later LDS reads to these loads (it would drain all stages); the
+// kernel waits for exactly the stage it needs with wait_vmcnt() before its barrier.
+__device__ inline void dma16(const void* gaddr, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off"
+               :
+               : "v"(gaddr), "s"(lds_addr)
+               : "memory", "m0");
+}
+
+template <bool UP>
+__global__ __launch_bounds__(kThreads) void ffn_tiled_dma_kernel(TiledParams p) {
+  __shared__ uint4 S0[kDmaStageU4], S1[kDmaStageU4], S2[kDmaStageU4], S3[kDmaStageU4];
+  const int n_row_tiles = *p.n_tiles;
+  const int total = n_row_tiles * p.n_col_tiles;
+  const int per_xcd = (total + 7) / 8;
+  const int slot = blockIdx.x / 8;
+  const int logical = (blockIdx.x % 8) * per_xcd + slot;
+  if (slot >= per_xcd || logical >= total) return;
+  const int ct = logical / n_row_tiles;
+  const int rt = logical - ct * n_row_tiles;
+
+  const int e = p.tile_group[rt];
+  const int tm0 = p.tile_m0[rt];
+  const int base = p.g.offsets[e];
+  const int cnt = p.g.offsets[e + 1] - base;
+  const int rows_here = min(TM, cnt - tm0);
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept scalar
+  const int kq = lane >> 4, mm = lane & 15;
+  const int wm = wave >> 1, wn = wave & 1;
+  constexpr int BROWS = UP ? 128 : 256;
+  const int nb0 = ct * (BROWS / 16);
+
+  // Per stage this wave fills A chunks msub = 4*wave + q and B chunks nsub = 4*wave + q.
+  const uint16_t* arow[4];
+  const uint4* bptr[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    int m = (wave * 4 + q) * 16 + mm;
+    if (m >= rows_here) m = 0;
+    int src;
+    if (UP) src = p.g.perm[base + tm0 + m] / p.g.pair_div;
+    else src = base + tm0 + m;
+    arow[q] = p.a + (size_t)src * p.a_stride + 8 * kq;
+    int nsub = wave * 4 + q;
+    int nb;
+    const uint4* wbase;
+    if (UP) {
+      wbase = nsub < 8 ? p.wa : p.wb;
+      nb = nb0 + (nsub & 7);
+    } else {
+      wbase = p.wa;
+      nb = nb0 + nsub;
+    }
+    if (nb >= p.n_blocks) nb = p.n_blocks - 1;
+    bptr[q] = wbase + (size_t)e * p.w_stride_u4 + (size_t)nb * p.nkb * 64 + lane;
+  }
+
+  f32x4 acc[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int my_rows = rows_here - wm * 128;
+  const int mt = my_rows <= 0 ? 0 : min(8, (my_rows + 15) >> 4);
+  const int nks = p.k_pad / 32;
+
+  // LDS byte address of this wave's first A chunk inside a stage (wave-uniform -> SGPR).
+  const uint32_t wave_chunk = wave * 4 * kChunk;
+  auto issue = [&](uint4* S, int ks) {
+    const uint32_t sbase = (uint32_t)(uintptr_t)(lptr_t)S + wave_chunk;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      dma16(arow[q] + (size_t)ks * 32, sbase + q * kChunk);
+      dma16(bptr[q] + (size_t)ks * 64, sbase + (16 + q) * kChunk);
+    }
+  };
+  auto compute = [&](const uint4* S) {
+    uint4 bf[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      int nsub = UP ? ((j < 4 ? 0 : 8) + 4 * wn + (j & 3)) : (8 * wn + j);
+      bf[j] = S[(16 + nsub) * 64 + lane];
+    }
+    // Rows past the end of a partial tile were clamped to a real row when loading; their
+    // products are computed and dropped, which keeps this loop free of per-row branches.
+    if (mt > 0) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        uint4 af = S[(wm * 8 + i) * 64 + lane];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = mfma(af, bf[j], acc[i][j]);
+      }
+    }
+  };
+  // One k step: make stage `ks` visible to the whole workgroup, refill the buffer that was
+  // read in the previous step, multiply.
+  auto step = [&](const uint4* cur, uint4* refill, int ks) {
+    const int ahead = min(2, nks - 1 - ks);  // stages issued after `ks` and still in flight
+    wait_vmcnt(ahead * 8);
+    // A bare barrier: __syncthreads() would also drain every outstanding load (its fence
+    // counts the LDS-bound loads of the later stages), which is exactly what must stay in
+    // flight.  The explicit vmcnt wait above covers the stage that is about to be read.
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (ks + 3 < nks) issue(refill, ks + 3);
+    compute(cur);
+  };
+
+  issue(S0, 0);
+  if (nks > 1) issue(S1, 1);
+  if (nks > 2) issue(S2, 2);
+  for (int ks = 0; ks < nks; ks += 4) {
+    step(S0, S3, ks);
+    if (ks + 1 < nks) step(S1, S0, ks + 1);
+    if (ks + 2 < nks) step(S2, S1, ks + 2);
+    if (ks + 3 < nks) step(S3, S2, ks + 3);
+  }
+
+  if (UP) {
+    uint16_t* h = (uint16_t*)p.out;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = (nb0 + 4 * wn + j) * 16 + mm;
+      const bool n_ok = n < p.n_blocks * 16;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if (i >= mt) continue;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int m = wm * 128 + i * 16 + 4 * kq + r;
+          if (m < rows_here && n_ok) {
+            float g = acc[i][j][r];
+            float u = acc[i][j + 4][r];
+            float hv = (g / (1.f + __expf(-g))) * u;
+            h[(size_t)(base + tm0 + m) * p.out_stride + n] = bf16_rne(hv);
+          }
+        }
+      }
+    }
+  } else {
+    float* y = (float*)p.out;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (i >= mt) continue;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = wm * 128 + i * 16 + 4 * kq + r;
+        if (m >= rows_here) continue;
+        const int pair = p.g.perm[base + tm0 + m];
+        float* yr = y + (size_t)pair * p.out_stride;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int n = (nb0 + 8 * wn + j) * 16 + mm;
+          if (n < p.n_rows) yr[n] = acc[i][j][r];
+        }
+      }
+    }
+  }
+}
+
+template <bool UP>
+hipError_t launch_tiled_dma(const TiledParams& p, int max_row_tiles, hipStream_t s) {
+  int n_wg = max_row_tiles * p.n_col_tiles;
+  n_wg = (n_wg + 7) / 8 * 8;
+  ffn_tiled_dma_kernel<UP><<<n_wg, kThreads, 0, s>>>(p);
+  return hipGetLastError();
+}
+
 template <bool INT8, bool UP>
 hipError_t launch_tiled(const TiledParams& p, int max_row_tiles, hipStream_t s) {
   static bool attr_set = false;
@@ -322,6 +513,7 @@ hipError_t launch_ffn_up_tiled(const FfnArgs& a, hipStream_t s) {
   p.tile_m0 = a.tile_m0;
   p.n_tiles = a.n_tiles;
   p.n_col_tiles = (a.gate.n_pad + 127) / 128;
+  if (!int8 && p.k_pad % 32 == 0) return launch_tiled_dma<true>(p, a.max_row_tiles, s);
   return int8 ? launch_tiled<true, true>(p, a.max_row_tiles, s)
               : launch_tiled<false, true>(p, a.max_row_tiles, s);
 }
@@ -347,6 +539,7 @@ hipError_t launch_ffn_down_tiled(const FfnArgs& a, hipStream_t s) {
   p.tile_m0 = a.tile_m0;
   p.n_tiles = a.n_tiles;
   p.n_col_tiles = (a.down.n_pad + 255) / 256;
+  if (!int8 && p.k_pad % 32 == 0) return launch_tiled_dma<false>(p, a.max_row_tiles, s);
   return int8 ? launch_tiled<true, false>(p, a.max_row_tiles, s)
               : launch_tiled<false, false>(p, a.max_row_tiles, s);
 }
