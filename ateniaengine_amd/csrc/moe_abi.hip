@@ -108,6 +108,8 @@ namespace {
 
 // Largest batch served by the weight-streaming expert kernels.
 constexpr int kStreamMaxTokens = 128;
+// Largest batch routed by the one-workgroup-per-token router kernel.
+constexpr int kRouterTokenKernelMaxTokens = 512;
 
 bool valid_handle(const AteniaMoeLayer* L) { return L && L->magic == 0x4d6f4541u; }
 
@@ -246,6 +248,9 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   ra.xb = need_xb ? L->xb.as<uint16_t>() : nullptr;
   ra.d_pad = L->d_kpad;
   ra.status = L->status.as<int32_t>();
+  // f32-valued operands almost never satisfy the exactness test of the per-token kernel, so
+  // f32 layers always take the sequential-order kernel.
+  ra.token_kernel_max_tokens = f32w ? 0 : kRouterTokenKernelMaxTokens;
   HIP_TRY(launch_router(ra, s));
   L->launches[0] = 1;
   tm.mark();  // ev[1]: router done

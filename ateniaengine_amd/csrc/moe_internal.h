@@ -60,6 +60,7 @@ struct RouterArgs {
   uint16_t* xb;              // [T, d_pad] bf16 copy of x (null = do not write)
   int d_pad;
   int32_t* status;           // [2]: code, (token << 10 | expert)
+  int token_kernel_max_tokens;  // batches up to this size use the one-workgroup-per-token kernel
 };
 hipError_t launch_router(const RouterArgs& a, hipStream_t s);
 

@@ -11,8 +11,20 @@
 //   shared-expert gate                  src/moe/layer.rs:436-443  sigmoid(f64 dot)
 //
 // Products of two f32 values are exact in f64, so fma(w, x, acc) rounds exactly like the
-// reference's separate multiply and add.  Each (token, row) pair is owned by one thread
-// that walks c = 0..d-1 in order, so the f64 sum is the reference's sum, not merely close.
+// reference's separate multiply and add.  Two kernels compute the dot products:
+//
+//  * router_tile_kernel (any batch): each (token, row) pair is owned by one thread that walks
+//    c = 0..d-1 in order, so the f64 sum IS the reference's sum.
+//  * router_token_kernel (small batches, where that serial chain would dominate the layer):
+//    one workgroup per token, every row split over a wavefront and reduced with shuffles.
+//    A different summation order is only allowed when it provably cannot change the result:
+//    every product is an integer multiple of 2^q (q = the smallest exponent of a product's
+//    lowest set bit) and every partial sum of any subset is bounded by A = sum |product|;
+//    if A < 2^(q+53) every such partial sum is exactly representable in f64, so EVERY
+//    summation order -- the reference's included -- is free of rounding and yields the same
+//    exact value.  The kernel checks this per row (true for bf16-valued operands in
+//    practice); when it fails for any row of the token, the token's rows are recomputed in
+//    the reference's order.
 #include "moe_internal.h"
 
 namespace atenia_moe {
@@ -22,6 +34,8 @@ namespace {
 constexpr int kRouterThreads = 256;
 constexpr int kKc = 32;            // columns staged per step
 constexpr int kLd = kKc + 1;       // padded LDS row stride (words)
+constexpr int kTokenThreads = 1024;
+constexpr int kNoLsb = 32767;      // lsb exponent marker of a zero
 
 __device__ inline float load_x(const float* x, size_t i) { return x[i]; }
 __device__ inline float load_x(const uint16_t* x, size_t i) {
@@ -36,8 +50,80 @@ __device__ inline uint16_t f32_to_bf16_rne(float f) {
   return (uint16_t)(u >> 16);
 }
 
+// Exponent of the lowest set bit of a finite f32 (v = odd * 2^result); kNoLsb for zero,
+// and a hugely negative value for inf/NaN so that no exactness claim survives them.
+__device__ inline int lsb_exponent(float v) {
+  uint32_t b = __float_as_uint(v);
+  int e = (b >> 23) & 0xff;
+  uint32_t m = b & 0x7fffffu;
+  if (e == 0xff) return -100000;
+  if (e == 0) {
+    if (m == 0) return kNoLsb;
+    return -149 + (__ffs((int)m) - 1);
+  }
+  m |= 0x800000u;
+  return e - 150 + (__ffs((int)m) - 1);
+}
+
+// Softmax + top-k + renormalisation of ONE token by the threads r = 0..E-1 that call with
+// `on`; every thread of the workgroup must call (barriers inside).  lg: [E] f32 logits,
+// ex: [E] f64, wt: [E] f32, sel: [E] i32 scratch of this token.
+__device__ inline void softmax_topk(bool on, int r, int E, int k, int renorm, int token,
+                                    const float* lg, double* ex, float* wt, int32_t* sel,
+                                    int32_t* __restrict__ idx_out, float* __restrict__ w_out,
+                                    int32_t* __restrict__ status) {
+  float my_logit = 0.f;
+  if (on) {
+    float mx = -INFINITY;
+    for (int e = 0; e < E; ++e) mx = fmaxf(mx, lg[e]);  // skips NaN like f32::max
+    my_logit = lg[r];
+    ex[r] = exp((double)(my_logit - mx));                // f32 subtraction, then f64 exp
+  }
+  __syncthreads();
+  float my_w = 0.f;
+  if (on) {
+    double sum = 0.0;
+    for (int e = 0; e < E; ++e) sum += ex[e];            // sequential fold, e ascending
+    double inv = sum > 0.0 ? 1.0 / sum : 0.0;
+    my_w = (float)(ex[r] * inv);
+    wt[r] = my_w;
+    if (!isfinite(my_w) || my_w < 0.f) {
+      atomicMin(&status[0], -3);
+      atomicMin(&status[1], (token << 10) | r);
+    }
+  }
+  __syncthreads();
+  bool selected = false;
+  if (on) {
+    int rank = 0;  // experts that sort before me under (weight desc, index asc)
+    for (int e = 0; e < E; ++e) {
+      float we = wt[e];
+      rank += (we > my_w) || (we == my_w && e < r);
+    }
+    selected = rank < k;
+    sel[r] = selected ? 1 : 0;
+  }
+  __syncthreads();
+  if (on && selected) {
+    int slot = 0;
+    double sum = 0.0;
+    for (int e = 0; e < E; ++e) {
+      if (sel[e]) {
+        slot += e < r;
+        sum += (double)wt[e];  // ascending e, as the reference sums the sorted selection
+      }
+    }
+    double scale = renorm ? 1.0 / sum : 1.0;
+    if (slot < k) {
+      size_t o = (size_t)token * k + slot;
+      idx_out[o] = r;
+      w_out[o] = (float)((double)my_w * scale);
+    }
+  }
+}
+
 template <typename XT>
-__global__ __launch_bounds__(kRouterThreads) void router_kernel(
+__global__ __launch_bounds__(kRouterThreads) void router_tile_kernel(
     const XT* __restrict__ x, int T, int d, int E, int k, int renorm,
     const float* __restrict__ w_router, const float* __restrict__ bias,
     const float* __restrict__ gate_vec, int32_t* __restrict__ idx_out,
@@ -103,61 +189,95 @@ __global__ __launch_bounds__(kRouterThreads) void router_kernel(
     }
   }
   __syncthreads();
+  const int tls = owner ? tl : 0;
+  softmax_topk(owner && r < E, r, E, k, renorm, t0 + tls, sLogit + tls * R, sExp + tls * E,
+               sWt + tls * E, sSel + tls * E, idx_out, w_out, status);
+}
 
-  const bool expert_owner = owner && r < E;
-  float my_logit = 0.f;
-  if (expert_owner) {
-    const float* lg = sLogit + tl * R;
-    float mx = -INFINITY;
-    for (int e = 0; e < E; ++e) mx = fmaxf(mx, lg[e]);  // skips NaN like f32::max
-    my_logit = lg[r];
-    sExp[tl * E + r] = exp((double)(my_logit - mx));    // f32 subtraction, then f64 exp
+template <typename XT>
+__global__ __launch_bounds__(kTokenThreads) void router_token_kernel(
+    const XT* __restrict__ x, int T, int d, int E, int k, int renorm,
+    const float* __restrict__ w_router, const float* __restrict__ bias,
+    const float* __restrict__ gate_vec, int32_t* __restrict__ idx_out,
+    float* __restrict__ w_out, float* __restrict__ sgate_out, uint16_t* __restrict__ xb,
+    int d_pad, int32_t* __restrict__ status) {
+  const int R = E + (gate_vec ? 1 : 0);
+  const int t = blockIdx.x;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  constexpr int NW = kTokenThreads / 64;
+
+  extern __shared__ double smem_d[];
+  double* sAcc = smem_d;                       // [R]
+  double* sExp = sAcc + R;                     // [E]
+  float* sX = (float*)(sExp + E);              // [d]
+  float* sLogit = sX + d;                      // [E]
+  float* sWt = sLogit + E;                     // [E]
+  int32_t* sSel = (int32_t*)(sWt + E);         // [E]
+  int32_t* sBad = sSel + E;                    // [1]
+  int16_t* sLx = (int16_t*)(sBad + 1);         // [d]
+
+  if (tid == 0) *sBad = 0;
+  const int c_end = xb ? (d_pad > d ? d_pad : d) : d;
+  for (int c = tid; c < c_end; c += kTokenThreads) {
+    float v = c < d ? load_x(x, (size_t)t * d + c) : 0.f;
+    if (c < d) {
+      sX[c] = v;
+      sLx[c] = (int16_t)max(lsb_exponent(v), -32000);
+    }
+    if (xb && c < d_pad) xb[(size_t)t * d_pad + c] = f32_to_bf16_rne(v);
   }
   __syncthreads();
-  float my_w = 0.f;
-  if (expert_owner) {
-    const double* ex = sExp + tl * E;
-    double sum = 0.0;
-    for (int e = 0; e < E; ++e) sum += ex[e];           // sequential fold, e ascending
-    double inv = sum > 0.0 ? 1.0 / sum : 0.0;
-    my_w = (float)(ex[r] * inv);
-    sWt[tl * E + r] = my_w;
-    if (!isfinite(my_w) || my_w < 0.f) {
-      atomicMin(&status[0], -3);
-      atomicMin(&status[1], ((t0 + tl) << 10) | r);
+
+  for (int r = wave; r < R; r += NW) {
+    const float* wr = r < E ? w_router + (size_t)r * d : gate_vec;
+    double acc = 0.0, asum = 0.0;
+    int qmin = kNoLsb;
+    for (int c = lane; c < d; c += 64) {
+      float wv = wr[c], xv = sX[c];
+      double wd = (double)wv, xd = (double)xv;
+      acc = fma(wd, xd, acc);
+      asum = fma(fabs(wd), fabs(xd), asum);
+      int lx = sLx[c];
+      int lw = lsb_exponent(wv);
+      if (lx != kNoLsb && lw != kNoLsb) qmin = min(qmin, lx + lw);
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+      acc += __shfl_xor(acc, off);
+      asum += __shfl_xor(asum, off);
+      qmin = min(qmin, __shfl_xor(qmin, off));
+    }
+    if (lane == 0) {
+      // Exact in every order iff sum|p| < 2^(q+53); asum itself carries a relative error of
+      // at most d * 2^-53, covered by the margin.
+      bool exact = qmin == kNoLsb || (qmin > -2000 && asum * 1.000001 < ldexp(1.0, qmin + 53));
+      sAcc[r] = acc;
+      if (!exact) *sBad = 1;
     }
   }
   __syncthreads();
-  bool selected = false;
-  if (expert_owner) {
-    const float* wt = sWt + tl * E;
-    int rank = 0;  // experts that sort before me under (weight desc, index asc)
-    for (int e = 0; e < E; ++e) {
-      float we = wt[e];
-      rank += (we > my_w) || (we == my_w && e < r);
+  if (*sBad) {
+    // The reference's own order: one sequential c-ascending f64 sum per row.
+    for (int r = tid; r < R; r += kTokenThreads) {
+      const float* wr = r < E ? w_router + (size_t)r * d : gate_vec;
+      double acc = 0.0;
+      for (int c = 0; c < d; ++c) acc = fma((double)wr[c], (double)sX[c], acc);
+      sAcc[r] = acc;
     }
-    selected = rank < k;
-    sSel[tl * E + r] = selected ? 1 : 0;
+    __syncthreads();
+  }
+  if (tid < R) {
+    double acc = sAcc[tid];
+    if (tid < E) {
+      float logit = (float)acc;
+      if (bias) logit = logit + bias[tid];
+      sLogit[tid] = logit;
+    } else {
+      sgate_out[t] = (float)(1.0 / (1.0 + exp(-acc)));
+    }
   }
   __syncthreads();
-  if (expert_owner && selected) {
-    const int32_t* sel = sSel + tl * E;
-    const float* wt = sWt + tl * E;
-    int slot = 0;
-    double sum = 0.0;
-    for (int e = 0; e < E; ++e) {
-      if (sel[e]) {
-        slot += e < r;
-        sum += (double)wt[e];  // ascending e, as the reference sums the sorted selection
-      }
-    }
-    double scale = renorm ? 1.0 / sum : 1.0;
-    if (slot < k) {
-      size_t o = (size_t)(t0 + tl) * k + slot;
-      idx_out[o] = r;
-      w_out[o] = (float)((double)my_w * scale);
-    }
-  }
+  softmax_topk(tid < E, tid, E, k, renorm, t, sLogit, sExp, sWt, sSel, idx_out, w_out, status);
 }
 
 }  // namespace
@@ -165,6 +285,21 @@ __global__ __launch_bounds__(kRouterThreads) void router_kernel(
 hipError_t launch_router(const RouterArgs& a, hipStream_t s) {
   const int R = a.E + (a.shared_gate ? 1 : 0);
   if (R > kMaxRouterRows || a.T <= 0) return hipErrorInvalidValue;
+  if (a.T <= a.token_kernel_max_tokens) {
+    size_t smem = ((size_t)R + a.E) * 8 + (size_t)a.d * 4 + (size_t)a.E * 12 + 4 +
+                  (size_t)a.d * 2 + 16;
+    if (smem <= 64 * 1024) {
+      if (a.x_is_bf16)
+        router_token_kernel<uint16_t><<<a.T, kTokenThreads, smem, s>>>(
+            (const uint16_t*)a.x, a.T, a.d, a.E, a.k, a.renorm, a.w_router, a.router_bias,
+            a.shared_gate, a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status);
+      else
+        router_token_kernel<float><<<a.T, kTokenThreads, smem, s>>>(
+            (const float*)a.x, a.T, a.d, a.E, a.k, a.renorm, a.w_router, a.router_bias,
+            a.shared_gate, a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status);
+      return hipGetLastError();
+    }
+  }
   int TT = kRouterThreads / R;
   if (TT < 1) TT = 1;
   // Keep enough blocks in flight for small batches.
@@ -174,11 +309,11 @@ hipError_t launch_router(const RouterArgs& a, hipStream_t s) {
   size_t post_bytes = (((size_t)TT * R + 1) & ~(size_t)1) * 4 + (size_t)TT * a.E * (8 + 4 + 4);
   size_t smem = dot_bytes > post_bytes ? dot_bytes : post_bytes;
   if (a.x_is_bf16) {
-    router_kernel<uint16_t><<<blocks, kRouterThreads, smem, s>>>(
+    router_tile_kernel<uint16_t><<<blocks, kRouterThreads, smem, s>>>(
         (const uint16_t*)a.x, a.T, a.d, a.E, a.k, a.renorm, a.w_router, a.router_bias,
         a.shared_gate, a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status, TT);
   } else {
-    router_kernel<float><<<blocks, kRouterThreads, smem, s>>>(
+    router_tile_kernel<float><<<blocks, kRouterThreads, smem, s>>>(
         (const float*)a.x, a.T, a.d, a.E, a.k, a.renorm, a.w_router, a.router_bias,
         a.shared_gate, a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status, TT);
   }

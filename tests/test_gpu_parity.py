@@ -116,6 +116,27 @@ def test_router_bit_exact(ora, E, k, d, T, conv, bf16, bias, gated):
         assert ul.max() <= 1, f"routing weights differ by {ul.max()} ulp"
 
 
+def test_router_token_kernel_inexact_rows_fall_back(ora):
+    """bf16 layer fed f32-valued activations with a wide exponent spread: the per-token
+    router kernel's exactness test fails and it must recompute in the reference's order."""
+    E, k, d, T = 8, 2, 1024, 24
+    W = S.make_weights(7, E, d, 16, router_std=1.0)
+    oL, gL = S.build_pair(ora, W, k, 0, capi.WEIGHT_BF16)
+    rng = np.random.default_rng(8)
+    x = (rng.standard_normal((T, d)) * np.exp2(rng.integers(-30, 30, size=(T, d)))).astype(
+        np.float32)
+    with gL:
+        idx, w = gL.route(x)
+        o_idx, o_w, o_lo = oL.route_tokens(x, want_logits=True)
+        assert (idx == o_idx).all() and ulp_diff(w, o_w).max() <= 1
+    # same layer, exactly representable sums: the shuffle-reduced path must agree too
+    with S.build_pair(ora, W, k, 0, capi.WEIGHT_BF16)[1] as gL2:
+        xb = S.make_tokens(9, T, d)
+        idx, w = gL2.route(xb)
+        o_idx, o_w = oL.route_tokens(xb)
+        assert (idx == o_idx).all() and ulp_diff(w, o_w).max() <= 1
+
+
 def test_router_engineered_ties(ora):
     """Duplicate router rows give exactly equal weights; the lower index must win."""
     E, k, d, T = 8, 2, 64, 40
