@@ -138,6 +138,8 @@ def main():
     ap.add_argument("--sweep", type=str, default="", help="extra batch sizes, comma separated")
     ap.add_argument("--cpu-tokens", type=int, default=16,
                     help="tokens of the CPU-baseline sample (0 = skip)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy (reference point for HBM counters)")
     ap.add_argument("--seed", type=int, default=1234)
     a = ap.parse_args()
     if a.gpus != 1:
@@ -160,6 +162,15 @@ def main():
     layer = capi.Layer(w_router=router_f32, w_gate=gate, w_up=up, w_down=down, top_k=TOP_K,
                        convention=capi.CONVENTION_ATENIA, weight_dtype=capi.WEIGHT_BF16,
                        max_tokens_hint=tmax)
+
+    if a.calibrate_copy:
+        src = torch.empty(1 << 28, device="cuda", dtype=torch.float32)  # 1 GiB
+        src.fill_(1.0)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     head, x_head, out_head = measure(torch, np, capi, layer, a.tokens, a.steps, a.warmup, a.seed)
     decode = None
