@@ -19,6 +19,8 @@
 //
 // Two LDS stages of 64 k each: global loads of stage i+1 are issued into registers before
 // the MFMAs of stage i and stored to the other LDS buffer after them.
+#include <type_traits>
+
 #include "moe_internal.h"
 
 #include "../../include/atenia_moe_hip.h"
@@ -88,21 +90,53 @@ __device__ inline f32x4 mfma(uint4 a, uint4 b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(bf16x8*)&a, *(bf16x8*)&b, c, 0, 0, 0);
 }
 
-template <bool INT8, bool UP>
-__global__ __launch_bounds__(kThreads) void ffn_tiled_kernel(TiledParams p) {
-  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-  // XCD-aware order: hardware deals consecutive workgroups round-robin to the 8 XCDs, so
-  // give each XCD a contiguous run of logical tiles; neighbours in that run share a weight
-  // tile (row tiles of one expert are innermost) and meet in the same L2.
+// Which (row tile, column tile) a workgroup computes.
+//
+// XCD-aware order: hardware deals consecutive workgroup ids round-robin to the 8 XCDs, each
+// with its own L2, so XCD x is given the contiguous run [x*per_xcd, (x+1)*per_xcd) of the
+// logical tile order.  In that order an expert's tiles are contiguous and walked in patches of
+// (all row tiles of the expert) x (8 column tiles): the ~32 workgroups an XCD runs at a time
+// share ~4 activation tiles and 8 weight tiles instead of streaming 64 different ones.
+constexpr int kColGroup = 8;
+__device__ inline bool tile_of_workgroup(const TiledParams& p, int& rt, int& ct) {
   const int n_row_tiles = *p.n_tiles;
-  const int total = n_row_tiles * p.n_col_tiles;
+  const int nct = p.n_col_tiles;
+  const int total = n_row_tiles * nct;
   const int per_xcd = (total + 7) / 8;
   const int slot = blockIdx.x / 8;
   const int logical = (blockIdx.x % 8) * per_xcd + slot;
-  if (slot >= per_xcd || logical >= total) return;
-  // logical -> (column tile, row tile), row tile fastest.
-  const int ct = logical / n_row_tiles;
-  const int rt = logical - ct * n_row_tiles;
+  if (slot >= per_xcd || logical >= total) return false;
+  // Row tiles are sorted by expert, so the expert owning this logical id is the expert of
+  // row tile logical / nct; that tile's m0 tells where the expert's tiles start.
+  const int rt_any = logical / nct;
+  const int e = p.tile_group[rt_any];
+  const int first = rt_any - p.tile_m0[rt_any] / TM;
+  const int cnt = p.g.offsets[e + 1] - p.g.offsets[e];
+  const int nt = (cnt + TM - 1) / TM;
+  int local = logical - first * nct;
+  const int full = nct / kColGroup;
+  const int patch = nt * kColGroup;
+  int cg, gw;
+  if (local < full * patch) {
+    cg = local / patch;
+    local -= cg * patch;
+    gw = kColGroup;
+  } else {
+    local -= full * patch;
+    cg = full;
+    gw = nct - full * kColGroup;
+  }
+  const int rl = local / gw;
+  rt = first + rl;
+  ct = cg * kColGroup + (local - rl * gw);
+  return true;
+}
+
+template <bool INT8, bool UP>
+__global__ __launch_bounds__(kThreads) void ffn_tiled_kernel(TiledParams p) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  int rt, ct;
+  if (!tile_of_workgroup(p, rt, ct)) return;
 
   const int e = p.tile_group[rt];
   const int tm0 = p.tile_m0[rt];
@@ -290,10 +324,14 @@ typedef __attribute__((address_space(3))) void* lptr_t;
 constexpr int kDmaStageU4 = 2 * 16 * 64;  // uint4 per stage: 16 A chunks + 16 B chunks
 
 __device__ inline void wait_vmcnt(int n) {
-  // s_waitcnt with only vmcnt active: vmcnt[3:0] in bits 3:0, vmcnt[5:4] in bits 15:14.
-  if (n >= 16) __builtin_amdgcn_s_waitcnt(0x4F70);
-  else if (n >= 8) __builtin_amdgcn_s_waitcnt(0x0F78);
-  else __builtin_amdgcn_s_waitcnt(0x0F70);
+  // s_waitcnt vmcnt(n) lgkmcnt(0): vmcnt[3:0] in bits 3:0, vmcnt[5:4] in bits 15:14, expcnt
+  // (bits 6:4) left at "no wait", lgkmcnt (bits 11:8) = 0.  lgkmcnt(0) makes sure this wave's
+  // own LDS reads of the previous step have returned before it passes the barrier after
+  // which other waves refill that buffer.
+  if (n >= 16) __builtin_amdgcn_s_waitcnt(0x4070);
+  else if (n >= 8) __builtin_amdgcn_s_waitcnt(0x0078);
+  else if (n >= 4) __builtin_amdgcn_s_waitcnt(0x0074);
+  else __builtin_amdgcn_s_waitcnt(0x0070);
 }
 
 // One wave-wide 16-byte-per-lane load from global memory straight into LDS: lane l's bytes
@@ -307,17 +345,29 @@ __device__ inline void dma16(const void* gaddr, uint32_t lds_addr) {
                : "memory", "m0");
 }
 
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+
+// v_mfma_f32_32x32x16_bf16 operand layout: A lane l holds row l%32, k = 8*(l/32)..+7 of a
+// 32 x 16 fragment; B the same with columns; D register r of lane l is element
+// (row 8*(r/4) + 4*(l/32) + r%4, column l%32).  Measured on MI355X the 32x32x16 form sustains
+// about 1.35x the rate of 16x16x32 in this kind of loop, so the tiled kernel uses it: an LDS
+// chunk (1 KiB) is one 32 x 16 fragment.
+__device__ inline f32x16 mfma32(uint4 a, uint4 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8*)&a, *(bf16x8*)&b, c, 0, 0, 0);
+}
+
 template <bool UP>
 __global__ __launch_bounds__(kThreads) void ffn_tiled_dma_kernel(TiledParams p) {
-  __shared__ uint4 S0[kDmaStageU4], S1[kDmaStageU4], S2[kDmaStageU4], S3[kDmaStageU4];
-  const int n_row_tiles = *p.n_tiles;
-  const int total = n_row_tiles * p.n_col_tiles;
-  const int per_xcd = (total + 7) / 8;
-  const int slot = blockIdx.x / 8;
-  const int logical = (blockIdx.x % 8) * per_xcd + slot;
-  if (slot >= per_xcd || logical >= total) return;
-  const int ct = logical / n_row_tiles;
-  const int rt = logical - ct * n_row_tiles;
+  // B ring: four stages of 32 k, chunk c = (32-row group ng = c/2, k half c%2), 16 KiB each.
+  // A ring: two stages of 64 k (32 KiB each).  An A chunk is 8 rows x 64 k: one load
+  // instruction reads eight full 128-byte lines (a 32-row x 16-k fragment would touch 32
+  // lines for 32 bytes each and starve the load path).  Inside a chunk the 16-byte segment
+  // s of row r is stored at slot r*8 + (s ^ r ^ (chunk & 1)), which makes the 32-row
+  // fragment reads below free of LDS bank conflicts.
+  __shared__ uint4 A0[2048], A1[2048];
+  __shared__ uint4 B0[1024], B1[1024], B2[1024], B3[1024];
+  int rt, ct;
+  if (!tile_of_workgroup(p, rt, ct)) return;
 
   const int e = p.tile_group[rt];
   const int tm0 = p.tile_m0[rt];
@@ -327,113 +377,164 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_dma_kernel(TiledParams p) 
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept scalar
-  const int kq = lane >> 4, mm = lane & 15;
+  const int kh = lane >> 5, l32 = lane & 31;
   const int wm = wave >> 1, wn = wave & 1;
   constexpr int BROWS = UP ? 128 : 256;
   const int nb0 = ct * (BROWS / 16);
 
-  // Per stage this wave fills A chunks msub = 4*wave + q and B chunks nsub = 4*wave + q.
-  const uint16_t* arow[4];
-  const uint4* bptr[4];
+  // ---- loads issued by this thread --------------------------------------------------------
+  // A: per 64-k stage this wave fills chunks 8*wave .. 8*wave+7 (rows 64*wave .. +63); lane l
+  // fetches row l/8 of the chunk, segment (l%8) ^ (l/8) ^ (chunk&1).
+  const uint16_t* arow[8];
+  {
+    const int r8 = lane >> 3, pslot = lane & 7;
 #pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    int m = (wave * 4 + q) * 16 + mm;
-    if (m >= rows_here) m = 0;
-    int src;
-    if (UP) src = p.g.perm[base + tm0 + m] / p.g.pair_div;
-    else src = base + tm0 + m;
-    arow[q] = p.a + (size_t)src * p.a_stride + 8 * kq;
-    int nsub = wave * 4 + q;
-    int nb;
+    for (int q = 0; q < 8; ++q) {
+      int m = (wave * 8 + q) * 8 + r8;
+      if (m >= rows_here) m = 0;  // clamp: such rows are computed but never stored
+      int src;
+      if (UP) src = p.g.perm[base + tm0 + m] / p.g.pair_div;
+      else src = base + tm0 + m;
+      const int seg = pslot ^ r8 ^ (q & 1);
+      arow[q] = p.a + (size_t)src * p.a_stride + seg * 8;
+    }
+  }
+  // B: per 32-k stage this wave fills chunks 4*wave .. 4*wave+3 (row groups 2*wave, 2*wave+1,
+  // both k halves).  Inside a stored 16-row x 32-k block the lane slot is (k quarter)*16 +
+  // row%16 with k quarter = 2*half + kh.
+  const uint4* bptr[2];
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    int ng = wave * 2 + q;
+    int brow;
     const uint4* wbase;
     if (UP) {
-      wbase = nsub < 8 ? p.wa : p.wb;
-      nb = nb0 + (nsub & 7);
+      wbase = ng < 4 ? p.wa : p.wb;
+      brow = (ng & 3) * 32 + l32;
     } else {
       wbase = p.wa;
-      nb = nb0 + nsub;
+      brow = ng * 32 + l32;
     }
-    if (nb >= p.n_blocks) nb = p.n_blocks - 1;
-    bptr[q] = wbase + (size_t)e * p.w_stride_u4 + (size_t)nb * p.nkb * 64 + lane;
+    int nb = nb0 + (brow >> 4);
+    if (nb >= p.n_blocks) nb = p.n_blocks - 1;  // clamp: columns past N are never stored
+    bptr[q] = wbase + (size_t)e * p.w_stride_u4 + (size_t)nb * p.nkb * 64 + kh * 16 + (brow & 15);
+  }
+  // ---- fragment read offsets (uint4 units) ------------------------------------------------
+  // A fragment (row group mg = 4*wm + i, k16 index u of the stage): row m32 of the group is
+  // chunk mg*4 + m32/8, row m32%8; segment 2u + kh.
+  int aoff[4];
+  {
+    const int r8 = l32 & 7, cpar = (l32 >> 3) & 1;
+    const int rowbase = (wm * 16 + (l32 >> 3)) * 64 + r8 * 8;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) aoff[u] = rowbase + ((2 * u + kh) ^ r8 ^ cpar);
   }
 
-  f32x4 acc[8][8];
+  f32x16 acc[4][4];
 #pragma unroll
-  for (int i = 0; i < 8; ++i)
+  for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
   const int my_rows = rows_here - wm * 128;
-  const int mt = my_rows <= 0 ? 0 : min(8, (my_rows + 15) >> 4);
   const int nks = p.k_pad / 32;
 
-  // LDS byte address of this wave's first A chunk inside a stage (wave-uniform -> SGPR).
-  const uint32_t wave_chunk = wave * 4 * kChunk;
-  auto issue = [&](uint4* S, int ks) {
-    const uint32_t sbase = (uint32_t)(uintptr_t)(lptr_t)S + wave_chunk;
+  auto issue_a = [&](uint4* A, int t) {  // 64-k stage t
+    const uint32_t sbase = (uint32_t)(uintptr_t)(lptr_t)A + wave * 8 * kChunk;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      dma16(arow[q] + (size_t)ks * 32, sbase + q * kChunk);
-      dma16(bptr[q] + (size_t)ks * 64, sbase + (16 + q) * kChunk);
-    }
+    for (int q = 0; q < 8; ++q) dma16(arow[q] + (size_t)t * 64, sbase + q * kChunk);
   };
-  auto compute = [&](const uint4* S) {
-    uint4 bf[8];
+  auto issue_b = [&](uint4* B, int ks) {  // 32-k stage ks
+    const uint32_t sbase = (uint32_t)(uintptr_t)(lptr_t)B + wave * 4 * kChunk;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      int nsub = UP ? ((j < 4 ? 0 : 8) + 4 * wn + (j & 3)) : (8 * wn + j);
-      bf[j] = S[(16 + nsub) * 64 + lane];
-    }
-    // Rows past the end of a partial tile were clamped to a real row when loading; their
-    // products are computed and dropped, which keeps this loop free of per-row branches.
-    if (mt > 0) {
+    for (int q = 0; q < 2; ++q)
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        uint4 af = S[(wm * 8 + i) * 64 + lane];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) acc[i][j] = mfma(af, bf[j], acc[i][j]);
-      }
-    }
+      for (int h = 0; h < 2; ++h)
+        dma16(bptr[q] + (size_t)ks * 64 + 32 * h, sbase + (q * 2 + h) * kChunk);
   };
-  // One k step: make stage `ks` visible to the whole workgroup, refill the buffer that was
-  // read in the previous step, multiply.
-  auto step = [&](const uint4* cur, uint4* refill, int ks) {
-    const int ahead = min(2, nks - 1 - ks);  // stages issued after `ks` and still in flight
-    wait_vmcnt(ahead * 8);
-    // A bare barrier: __syncthreads() would also drain every outstanding load (its fence
-    // counts the LDS-bound loads of the later stages), which is exactly what must stay in
-    // flight.  The explicit vmcnt wait above covers the stage that is about to be read.
+  // One 32-k step.  Per wave the loads are issued in the order
+  //   A(0) B(0) B(1) B(2) | step 0: A(1) B(3) | step 1: B(4) | step 2: A(2) B(5) | ...
+  // (8 instructions per A stage, 4 per B stage) and complete in order, so before the
+  // barrier of an even step at most 8 younger loads may be pending and before an odd step
+  // 16; WAIT carries that count (smaller at the very end).  A bare s_barrier is used:
+  // __syncthreads() would also drain every outstanding load, and the later stages must stay
+  // in flight.  ODD / ISSUE_A / ISSUE_B / MUL are compile-time: a step is straight-line code.
+  auto step = [&](auto odd_c, auto wait_c, auto issue_a_c, auto issue_b_c, auto mul_c,
+                  const uint4* Acur, uint4* Anext, const uint4* Bcur, uint4* Brefill, int ks) {
+    wait_vmcnt(decltype(wait_c)::value);
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    if (ks + 3 < nks) issue(refill, ks + 3);
-    compute(cur);
+    uint4 fa[2][4], fb[2][4];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        // gate/up: j < 2 gate groups 2*wn+j, j >= 2 the matching up groups
+        int ng = UP ? ((j < 2 ? 0 : 4) + 2 * wn + (j & 1)) : (4 * wn + j);
+        fb[h][j] = Bcur[(ng * 2 + h) * 64 + lane];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        fa[h][i] = Acur[i * 256 + aoff[2 * decltype(odd_c)::value + h]];
+    }
+    if (decltype(issue_a_c)::value) issue_a(Anext, ks / 2 + 1);
+    if (decltype(issue_b_c)::value) issue_b(Brefill, ks + 3);
+    // Rows past the end of a partial tile were clamped to a real row when loading; their
+    // products are computed and dropped, which keeps this loop free of per-row branches.
+    if (decltype(mul_c)::value) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc[i][j] = mfma32(fa[h][i], fb[h][j], acc[i][j]);
+    }
   };
-
-  issue(S0, 0);
-  if (nks > 1) issue(S1, 1);
-  if (nks > 2) issue(S2, 2);
-  for (int ks = 0; ks < nks; ks += 4) {
-    step(S0, S3, ks);
-    if (ks + 1 < nks) step(S1, S0, ks + 1);
-    if (ks + 2 < nks) step(S2, S1, ks + 2);
-    if (ks + 3 < nks) step(S3, S2, ks + 3);
-  }
+  using std::integral_constant;
+  typedef integral_constant<bool, true> yes;
+  typedef integral_constant<bool, false> no;
+  typedef integral_constant<int, 16> w16;
+  typedef integral_constant<int, 8> w8;
+  typedef integral_constant<int, 4> w4;
+  typedef integral_constant<int, 0> w0;
+  auto run = [&](auto mul_c) {
+    issue_a(A0, 0);
+    issue_b(B0, 0);
+    issue_b(B1, 1);
+    issue_b(B2, 2);
+    int ks = 0;
+    for (; ks + 4 < nks; ks += 4) {
+      step(no{}, w8{}, yes{}, yes{}, mul_c, A0, A1, B0, B3, ks);
+      step(yes{}, w16{}, no{}, yes{}, mul_c, A0, A1, B1, B0, ks + 1);
+      step(no{}, w8{}, yes{}, yes{}, mul_c, A1, A0, B2, B1, ks + 2);
+      step(yes{}, w16{}, no{}, yes{}, mul_c, A1, A0, B3, B2, ks + 3);
+    }
+    step(no{}, w8{}, yes{}, yes{}, mul_c, A0, A1, B0, B3, ks);
+    step(yes{}, w16{}, no{}, no{}, mul_c, A0, A1, B1, B0, ks + 1);
+    step(no{}, w4{}, no{}, no{}, mul_c, A1, A0, B2, B1, ks + 2);
+    step(yes{}, w0{}, no{}, no{}, mul_c, A1, A0, B3, B2, ks + 3);
+  };
+  // nks is a multiple of 4 and at least 8 (checked by the launcher).  A wave whose half of
+  // a partial tile holds no rows still feeds LDS and meets the barriers, without MFMAs.
+  if (my_rows > 0) run(yes{});
+  else run(no{});
 
   if (UP) {
     uint16_t* h = (uint16_t*)p.out;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int n = (nb0 + 4 * wn + j) * 16 + mm;
+    for (int j = 0; j < 2; ++j) {
+      const int n = nb0 * 16 + (2 * wn + j) * 32 + l32;
       const bool n_ok = n < p.n_blocks * 16;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        if (i >= mt) continue;
+      for (int i = 0; i < 4; ++i) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int m = wm * 128 + i * 16 + 4 * kq + r;
+        for (int r = 0; r < 16; ++r) {
+          const int m = wm * 128 + i * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
           if (m < rows_here && n_ok) {
             float g = acc[i][j][r];
-            float u = acc[i][j + 4][r];
+            float u = acc[i][j + 2][r];
             float hv = (g / (1.f + __expf(-g))) * u;
             h[(size_t)(base + tm0 + m) * p.out_stride + n] = bf16_rne(hv);
           }
@@ -443,17 +544,16 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_dma_kernel(TiledParams p) 
   } else {
     float* y = (float*)p.out;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      if (i >= mt) continue;
+    for (int i = 0; i < 4; ++i) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int m = wm * 128 + i * 16 + 4 * kq + r;
+      for (int r = 0; r < 16; ++r) {
+        const int m = wm * 128 + i * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
         if (m >= rows_here) continue;
         const int pair = p.g.perm[base + tm0 + m];
         float* yr = y + (size_t)pair * p.out_stride;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int n = (nb0 + 8 * wn + j) * 16 + mm;
+        for (int j = 0; j < 4; ++j) {
+          const int n = nb0 * 16 + (4 * wn + j) * 32 + l32;
           if (n < p.n_rows) yr[n] = acc[i][j][r];
         }
       }
@@ -513,7 +613,7 @@ hipError_t launch_ffn_up_tiled(const FfnArgs& a, hipStream_t s) {
   p.tile_m0 = a.tile_m0;
   p.n_tiles = a.n_tiles;
   p.n_col_tiles = (a.gate.n_pad + 127) / 128;
-  if (!int8 && p.k_pad % 32 == 0) return launch_tiled_dma<true>(p, a.max_row_tiles, s);
+  if (!int8 && p.k_pad % 128 == 0 && p.k_pad >= 256) return launch_tiled_dma<true>(p, a.max_row_tiles, s);
   return int8 ? launch_tiled<true, true>(p, a.max_row_tiles, s)
               : launch_tiled<false, true>(p, a.max_row_tiles, s);
 }
@@ -539,7 +639,7 @@ hipError_t launch_ffn_down_tiled(const FfnArgs& a, hipStream_t s) {
   p.tile_m0 = a.tile_m0;
   p.n_tiles = a.n_tiles;
   p.n_col_tiles = (a.down.n_pad + 255) / 256;
-  if (!int8 && p.k_pad % 32 == 0) return launch_tiled_dma<false>(p, a.max_row_tiles, s);
+  if (!int8 && p.k_pad % 128 == 0 && p.k_pad >= 256) return launch_tiled_dma<false>(p, a.max_row_tiles, s);
   return int8 ? launch_tiled<true, false>(p, a.max_row_tiles, s)
               : launch_tiled<false, false>(p, a.max_row_tiles, s);
 }
