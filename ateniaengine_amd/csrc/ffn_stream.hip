@@ -23,8 +23,6 @@ namespace {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 
-constexpr int kThreads = 256;
-constexpr int kWavesPerWg = 4;
 
 struct StreamParams {
   const uint4* wa;      // gate (up phase) or down blocks
@@ -85,8 +83,10 @@ __device__ inline f32x4 mfma(bf16x8 a, bf16x8 b, f32x4 c) {
 // MT  : 16-row tiles of tokens held per workgroup
 // INT8: weights are int8 blocks (64 k per block) instead of bf16 blocks (32 k per block)
 // UP  : gate/up phase with SwiGLU epilogue, else down phase
-template <int MT, bool INT8, bool UP>
-__global__ __launch_bounds__(kThreads) void ffn_stream_kernel(StreamParams p) {
+// WAVES: waves per workgroup = K slices of the strip
+template <int MT, bool INT8, bool UP, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p) {
+  constexpr int kWavesPerWg = WAVES;
   const int u = blockIdx.y;
   if (u >= *p.g.n_active) return;
   const int e = p.g.active[u];
@@ -252,12 +252,15 @@ hipError_t launch_stream(const StreamParams& p, int n_pad, int n_groups, int row
                          hipStream_t s) {
   int mt = rows_max <= 16 ? 1 : rows_max <= 32 ? 2 : 4;
   dim3 grid(n_pad / 16, n_groups, (rows_max + 16 * mt - 1) / (16 * mt));
+  // The down projection has few strips (d / 16) and a long K (f): eight K slices per strip
+  // keep enough loads in flight; gate/up has 2f / 16 strips and uses four.
+  constexpr int W = UP ? 4 : 8;
   if (mt == 1)
-    ffn_stream_kernel<1, INT8, UP><<<grid, kThreads, 0, s>>>(p);
+    ffn_stream_kernel<1, INT8, UP, W><<<grid, 64 * W, 0, s>>>(p);
   else if (mt == 2)
-    ffn_stream_kernel<2, INT8, UP><<<grid, kThreads, 0, s>>>(p);
+    ffn_stream_kernel<2, INT8, UP, W><<<grid, 64 * W, 0, s>>>(p);
   else
-    ffn_stream_kernel<4, INT8, UP><<<grid, kThreads, 0, s>>>(p);
+    ffn_stream_kernel<4, INT8, UP, W><<<grid, 64 * W, 0, s>>>(p);
   return hipGetLastError();
 }
 

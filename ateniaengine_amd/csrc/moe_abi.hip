@@ -251,12 +251,6 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   // f32-valued operands almost never satisfy the exactness test of the per-token kernel, so
   // f32 layers always take the sequential-order kernel.
   ra.token_kernel_max_tokens = f32w ? 0 : kRouterTokenKernelMaxTokens;
-  HIP_TRY(launch_router(ra, s));
-  L->launches[0] = 1;
-  tm.mark();  // ev[1]: router done
-  L->last_T = T;
-  if (stop_after == 1) return ATENIA_MOE_OK;
-
   PermuteArgs pa{};
   pa.idx = L->idx.as<int32_t>();
   pa.T = T;
@@ -274,8 +268,16 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   pa.tile_m0 = L->tile_m0.as<int32_t>();
   pa.n_tiles = L->shared_desc.as<int32_t>() + 4;
   pa.shared_n_tiles = L->shared_desc.as<int32_t>() + 5;
+  ra.fuse_permute = stop_after == 1 ? nullptr : &pa;
+  int fused = 0;
+  HIP_TRY(launch_router(ra, s, &fused));
+  L->launches[0] = 1;
+  tm.mark();  // ev[1]: router done
+  L->last_T = T;
+  if (stop_after == 1) return ATENIA_MOE_OK;
+
   int nl = 0;
-  HIP_TRY(launch_permute(pa, s, &nl));
+  if (!fused) HIP_TRY(launch_permute(pa, s, &nl));
   L->launches[1] = nl;
   tm.mark();  // ev[2]: permute done
 

@@ -47,6 +47,7 @@ struct WeightSet {
 };
 
 // ---- stage launchers (each returns a hipError_t from the launch) --------------------------
+struct PermuteArgs;
 struct RouterArgs {
   const void* x;        // [T, d] f32 or bf16
   int x_is_bf16;
@@ -61,8 +62,12 @@ struct RouterArgs {
   int d_pad;
   int32_t* status;           // [2]: code, (token << 10 | expert)
   int token_kernel_max_tokens;  // batches up to this size use the one-workgroup-per-token kernel
+  // When T == 1 and the per-token kernel runs, it also writes the expert grouping (the
+  // result of kernel 2 for a single token is known as soon as the top-k is), saving a launch.
+  const struct PermuteArgs* fuse_permute;  // null = do not fuse
 };
-hipError_t launch_router(const RouterArgs& a, hipStream_t s);
+// *fused_permute is set to 1 when the launch also produced the expert grouping.
+hipError_t launch_router(const RouterArgs& a, hipStream_t s, int* fused_permute);
 
 struct PermuteArgs {
   const int32_t* idx;  // [P] expert of each pair, P = T*k

@@ -194,13 +194,19 @@ __global__ __launch_bounds__(kRouterThreads) void router_tile_kernel(
                sWt + tls * E, sSel + tls * E, idx_out, w_out, status);
 }
 
+// Outputs of the expert grouping for the single-token case (see permute.hip for the contract).
+struct FusedGrouping {
+  int32_t *counts, *offsets, *perm, *inv, *active, *n_active, *shared_offsets;
+  int32_t *tile_group, *tile_m0, *n_tiles, *shared_n_tiles;
+};
+
 template <typename XT>
 __global__ __launch_bounds__(kTokenThreads) void router_token_kernel(
     const XT* __restrict__ x, int T, int d, int E, int k, int renorm,
     const float* __restrict__ w_router, const float* __restrict__ bias,
     const float* __restrict__ gate_vec, int32_t* __restrict__ idx_out,
     float* __restrict__ w_out, float* __restrict__ sgate_out, uint16_t* __restrict__ xb,
-    int d_pad, int32_t* __restrict__ status) {
+    int d_pad, int32_t* __restrict__ status, FusedGrouping fg) {
   const int R = E + (gate_vec ? 1 : 0);
   const int t = blockIdx.x;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -209,12 +215,15 @@ __global__ __launch_bounds__(kTokenThreads) void router_token_kernel(
   extern __shared__ double smem_d[];
   double* sAcc = smem_d;                       // [R]
   double* sExp = sAcc + R;                     // [E]
-  float* sX = (float*)(sExp + E);              // [d]
+  double* sPart = sExp + E;                    // [max(R, NW)]
+  double* sPartA = sPart + (R > NW ? R : NW);  // [max(R, NW)]
+  float* sX = (float*)(sPartA + (R > NW ? R : NW));  // [d]
   float* sLogit = sX + d;                      // [E]
   float* sWt = sLogit + E;                     // [E]
   int32_t* sSel = (int32_t*)(sWt + E);         // [E]
   int32_t* sBad = sSel + E;                    // [1]
-  int16_t* sLx = (int16_t*)(sBad + 1);         // [d]
+  int32_t* sPartQ = sBad + 1;                  // [max(R, NW)]
+  int16_t* sLx = (int16_t*)(sPartQ + (R > NW ? R : NW));  // [d]
 
   if (tid == 0) *sBad = 0;
   const int c_end = xb ? (d_pad > d ? d_pad : d) : d;
@@ -228,18 +237,38 @@ __global__ __launch_bounds__(kTokenThreads) void router_token_kernel(
   }
   __syncthreads();
 
-  for (int r = wave; r < R; r += NW) {
+  // Work items: (row, k slice).  With few rows each row is split over several waves so that
+  // all 16 waves stream the router matrix.  Partial results meet in LDS; under the exactness
+  // certificate their order of addition cannot change the sum.
+  const int KS = R >= NW ? 1 : NW / R;              // k slices per row
+  const int slice = ((d + KS - 1) / KS + 3) & ~3;   // multiple of 4 for float4 loads
+  const bool vec_ok = (d & 3) == 0;
+  for (int item = wave; item < R * KS; item += NW) {
+    const int r = item / KS, ksl = item - r * KS;
     const float* wr = r < E ? w_router + (size_t)r * d : gate_vec;
+    const int c_lo = ksl * slice, c_hi = min(d, c_lo + slice);
     double acc = 0.0, asum = 0.0;
     int qmin = kNoLsb;
-    for (int c = lane; c < d; c += 64) {
-      float wv = wr[c], xv = sX[c];
+    auto one = [&](float wv, int c) {
+      float xv = sX[c];
       double wd = (double)wv, xd = (double)xv;
       acc = fma(wd, xd, acc);
       asum = fma(fabs(wd), fabs(xd), asum);
       int lx = sLx[c];
       int lw = lsb_exponent(wv);
       if (lx != kNoLsb && lw != kNoLsb) qmin = min(qmin, lx + lw);
+    };
+    if (vec_ok) {
+#pragma unroll 4
+      for (int c = c_lo + lane * 4; c < c_hi; c += 256) {
+        float4 w4 = *(const float4*)(wr + c);
+        one(w4.x, c);
+        one(w4.y, c + 1);
+        one(w4.z, c + 2);
+        one(w4.w, c + 3);
+      }
+    } else {
+      for (int c = c_lo + lane; c < c_hi; c += 64) one(wr[c], c);
     }
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) {
@@ -248,12 +277,25 @@ __global__ __launch_bounds__(kTokenThreads) void router_token_kernel(
       qmin = min(qmin, __shfl_xor(qmin, off));
     }
     if (lane == 0) {
-      // Exact in every order iff sum|p| < 2^(q+53); asum itself carries a relative error of
-      // at most d * 2^-53, covered by the margin.
-      bool exact = qmin == kNoLsb || (qmin > -2000 && asum * 1.000001 < ldexp(1.0, qmin + 53));
-      sAcc[r] = acc;
-      if (!exact) *sBad = 1;
+      sPart[item] = acc;
+      sPartA[item] = asum;
+      sPartQ[item] = qmin;
     }
+  }
+  __syncthreads();
+  if (tid < R) {
+    double acc = 0.0, asum = 0.0;
+    int qmin = kNoLsb;
+    for (int ksl = 0; ksl < KS; ++ksl) {
+      acc += sPart[tid * KS + ksl];
+      asum += sPartA[tid * KS + ksl];
+      qmin = min(qmin, sPartQ[tid * KS + ksl]);
+    }
+    // Exact in every order iff sum|p| < 2^(q+53); asum itself carries a relative error of
+    // at most d * 2^-53, covered by the margin.
+    bool exact = qmin == kNoLsb || (qmin > -2000 && asum * 1.000001 < ldexp(1.0, qmin + 53));
+    sAcc[tid] = acc;
+    if (!exact) *sBad = 1;
   }
   __syncthreads();
   if (*sBad) {
@@ -278,25 +320,60 @@ __global__ __launch_bounds__(kTokenThreads) void router_token_kernel(
   }
   __syncthreads();
   softmax_topk(tid < E, tid, E, k, renorm, t, sLogit, sExp, sWt, sSel, idx_out, w_out, status);
+  if (fg.counts) {  // T == 1: the grouping of a single token follows from its top-k
+    __syncthreads();
+    if (tid == 0) {
+      int run = 0;
+      for (int e = 0; e < E; ++e) {
+        const int c = sSel[e] ? 1 : 0;
+        fg.counts[e] = c;
+        fg.offsets[e] = run;
+        if (c && run < k) {
+          fg.active[run] = e;
+          fg.perm[run] = run;
+          fg.inv[run] = run;
+          fg.tile_group[run] = e;
+          fg.tile_m0[run] = 0;
+          ++run;
+        }
+      }
+      fg.offsets[E] = run;
+      *fg.n_active = run;
+      *fg.n_tiles = run;
+      *fg.shared_n_tiles = 1;
+      fg.shared_offsets[0] = 0;
+      fg.shared_offsets[1] = 1;
+    }
+  }
 }
 
 }  // namespace
 
-hipError_t launch_router(const RouterArgs& a, hipStream_t s) {
+hipError_t launch_router(const RouterArgs& a, hipStream_t s, int* fused_permute) {
   const int R = a.E + (a.shared_gate ? 1 : 0);
+  if (fused_permute) *fused_permute = 0;
   if (R > kMaxRouterRows || a.T <= 0) return hipErrorInvalidValue;
   if (a.T <= a.token_kernel_max_tokens) {
-    size_t smem = ((size_t)R + a.E) * 8 + (size_t)a.d * 4 + (size_t)a.E * 12 + 4 +
-                  (size_t)a.d * 2 + 16;
+    const size_t np = R > kTokenThreads / 64 ? R : kTokenThreads / 64;
+    size_t smem = ((size_t)R + a.E + 2 * np) * 8 + (size_t)a.d * 4 + (size_t)a.E * 12 + 4 +
+                  np * 4 + (size_t)a.d * 2 + 16;
     if (smem <= 64 * 1024) {
+      FusedGrouping fg{};
+      if (a.T == 1 && a.fuse_permute) {
+        const PermuteArgs& pa = *a.fuse_permute;
+        fg = FusedGrouping{pa.counts, pa.offsets, pa.perm, pa.inv, pa.active, pa.n_active,
+                           pa.shared_offsets, pa.tile_group, pa.tile_m0, pa.n_tiles,
+                           pa.shared_n_tiles};
+        if (fused_permute) *fused_permute = 1;
+      }
       if (a.x_is_bf16)
         router_token_kernel<uint16_t><<<a.T, kTokenThreads, smem, s>>>(
             (const uint16_t*)a.x, a.T, a.d, a.E, a.k, a.renorm, a.w_router, a.router_bias,
-            a.shared_gate, a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status);
+            a.shared_gate, a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status, fg);
       else
         router_token_kernel<float><<<a.T, kTokenThreads, smem, s>>>(
             (const float*)a.x, a.T, a.d, a.E, a.k, a.renorm, a.w_router, a.router_bias,
-            a.shared_gate, a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status);
+            a.shared_gate, a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status, fg);
       return hipGetLastError();
     }
   }
