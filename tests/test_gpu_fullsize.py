@@ -1,0 +1,165 @@
+"""GPU parity at the full BASELINE shapes (configs 1-5), through the C ABI.
+
+Per config and batch size: routing indices, per-expert counts, offsets and permutation are
+compared bit for bit with the CPU oracle for EVERY token; layer outputs are compared with the
+all-f64 oracle (stored weight values, routing from the bit-exact path) on all tokens when
+T <= 16 and on >= 64 stratified tokens (every expert hit) otherwise, bar 1e-2 (bf16 / int8) or
+1e-5 (f32) of max|ref|.  Size-independent properties are checked on the whole batch:
+determinism, perm is a permutation consistent with counts/offsets, a batch equals its rows
+forwarded one at a time.
+"""
+import numpy as np
+import pytest
+
+from ateniaengine_amd import capi
+from tests import synth as S
+
+pytestmark = pytest.mark.gpu
+
+SAMPLE = 64
+
+
+def _normal(rng, shape, std):
+    a = rng.standard_normal(shape, dtype=np.float32)
+    a *= np.float32(std)
+    return a
+
+
+def _stratified(idx, E, n):
+    """>= n token ids such that every expert that received tokens is hit at least once."""
+    T = idx.shape[0]
+    chosen = set(np.linspace(0, T - 1, num=min(n, T), dtype=np.int64).tolist())
+    for e in range(E):
+        hit = np.nonzero((idx == e).any(axis=1))[0]
+        if hit.size and not chosen.intersection(hit.tolist()):
+            chosen.add(int(hit[0]))
+    return sorted(chosen)
+
+
+def _check(ora, oL, gL, x, tol, label):
+    T = x.shape[0]
+    out = gL.forward(x)
+    idx, w, counts, offsets, perm = gL.last_routing(T)
+    o_idx, o_w = oL.route_tokens(x)
+    bad = int((idx != o_idx).any(axis=1).sum())
+    assert bad == 0, f"{label}: {bad} of {T} tokens routed differently from the CPU path"
+    ul = np.abs(w.view(np.int32).astype(np.int64) - o_w.view(np.int32).astype(np.int64))
+    assert ul.max() <= 1, f"{label}: routing weights differ by {ul.max()} ulp"
+    oc, oo, op = ora.permute(o_idx, oL.E)
+    assert (counts == oc).all() and (offsets == oo).all() and (perm == op).all(), label
+    assert int(counts.sum()) == T * oL.top_k and offsets[-1] == T * oL.top_k
+    assert np.array_equal(np.sort(perm), np.arange(T * oL.top_k))
+    assert np.isfinite(out).all()
+    rows = range(T) if T <= 16 else _stratified(o_idx, oL.E, SAMPLE)
+    worst = 0.0
+    for t in rows:
+        ref = oL.forward_f64(x[t], fixed_idx=o_idx[t])
+        worst = max(worst, S.rel_err(out[t], ref))
+    assert worst <= tol, f"{label}: layer output off by {worst:.3e} (bar {tol})"
+    # determinism: same bits on a second call
+    assert gL.forward(x).tobytes() == out.tobytes(), f"{label}: not deterministic"
+    # position-wise op: a few rows forwarded alone agree with the batch.  A single row takes
+    # the decode kernels, so agreement is to the bf16 rounding of h, not bitwise.
+    for t in list(rows)[:3]:
+        alone = gL.forward(x[t:t + 1])[0]
+        assert S.rel_err(alone, out[t]) <= (2 * tol if tol > 1e-4 else 1e-6), label
+    print(f"{label}: T={T} routing exact, max rel err {worst:.2e} over {len(list(rows))} tokens, "
+          f"experts used {int((counts > 0).sum())}/{oL.E}, max load {int(counts.max())}")
+    return worst, counts
+
+
+@pytest.fixture(scope="module")
+def threads(ora):
+    ora.set_threads(ora.hw_threads())
+    yield
+    ora.set_threads(1)
+
+
+# ---- config 1: tiny f32 layer -----------------------------------------------------------------
+def test_config1_tiny_f32(ora, threads):
+    rng = np.random.default_rng(101)
+    E, k, d, f = 8, 2, 1024, 2048
+    W = dict(w_router=_normal(rng, (E, d), 0.02), w_gate=_normal(rng, (E, f, d), 0.02),
+             w_up=_normal(rng, (E, f, d), 0.02), w_down=_normal(rng, (E, d, f), 0.02))
+    oL, gL = S.build_pair(ora, W, k, capi.CONVENTION_ATENIA, capi.WEIGHT_F32)
+    with gL:
+        x = _normal(rng, (64, d), 1.0)
+        _check(ora, oL, gL, x, 1e-5, "config1 f32")
+        # the certified CPU path itself (f32 storage, f64 accumulation) is matched closely
+        cpu, _, _ = oL.execute(x[:8])
+        assert S.rel_err(gL.forward(x[:8]), cpu) <= 1e-6
+
+
+# ---- configs 2 and 3: Mixtral-8x7B shape, bf16 and INT8 W8A16 ----------------------------------
+@pytest.fixture(scope="module")
+def mixtral_weights():
+    rng = np.random.default_rng(202)
+    E, d, f = 8, 4096, 14336
+    return dict(w_router=_normal(rng, (E, d), 0.02), w_gate=_normal(rng, (E, f, d), 0.02),
+                w_up=_normal(rng, (E, f, d), 0.02), w_down=_normal(rng, (E, d, f), 0.02))
+
+
+def test_config2_mixtral_bf16(ora, threads, mixtral_weights):
+    oL, gL = S.build_pair(ora, mixtral_weights, 2, capi.CONVENTION_ATENIA, capi.WEIGHT_BF16,
+                          max_tokens_hint=4096)
+    with gL:
+        for T in (1, 16, 128, 512, 4096):
+            x = S.make_tokens(1000 + T, T, 4096)
+            _check(ora, oL, gL, x, 1e-2, "config2 mixtral bf16")
+    del oL
+
+
+def test_config3_mixtral_int8(ora, threads, mixtral_weights):
+    W = dict(mixtral_weights)
+    rng = np.random.default_rng(303)
+    for name in ("w_gate", "w_up", "w_down"):  # 0.1 % of output channels carry x8 magnitude
+        a = W[name] = W[name].copy()
+        rows = a.reshape(-1, a.shape[-1])
+        sel = rng.choice(rows.shape[0], size=rows.shape[0] // 1000, replace=False)
+        rows[sel] *= 8.0
+    oL, gL = S.build_pair(ora, W, 2, capi.CONVENTION_ATENIA, capi.WEIGHT_INT8_W8A16,
+                          max_tokens_hint=4096)
+    del W
+    with gL:
+        assert gL.info()["bytes_per_expert"] == 3 * 4096 * 14336 + (2 * 14336 + 4096) * 4
+        for T in (1, 16, 4096):
+            x = S.make_tokens(2000 + T, T, 4096)
+            _check(ora, oL, gL, x, 1e-2, "config3 mixtral int8")
+    del oL
+
+
+# ---- config 4: Qwen1.5-MoE-A2.7B shape -----------------------------------------------------------
+def test_config4_qwen_bf16(ora, threads):
+    rng = np.random.default_rng(404)
+    E, k, d, f, fs = 60, 4, 2048, 1408, 5632
+    W = dict(w_router=_normal(rng, (E, d), 1.0 / np.sqrt(d)), w_gate=_normal(rng, (E, f, d), 0.02),
+             w_up=_normal(rng, (E, f, d), 0.02), w_down=_normal(rng, (E, d, f), 0.02),
+             s_gate=_normal(rng, (fs, d), 0.02), s_up=_normal(rng, (fs, d), 0.02),
+             s_down=_normal(rng, (d, fs), 0.02), shared_gate=_normal(rng, (d,), 0.02))
+    oL, gL = S.build_pair(ora, W, k, capi.CONVENTION_HUGGINGFACE_QWEN, capi.WEIGHT_BF16,
+                          max_tokens_hint=8192)
+    del W
+    with gL:
+        for T in (1, 256, 8192):
+            x = S.make_tokens(3000 + T, T, d)
+            _check(ora, oL, gL, x, 1e-2, "config4 qwen bf16")
+
+
+# ---- config 5: DeepSeek-V2-Lite shape, skewed load ---------------------------------------------
+def test_config5_deepseek_bf16(ora, threads):
+    rng = np.random.default_rng(505)
+    E, k, d, f, fs = 64, 6, 2048, 1408, 2816
+    bias = (-1.2 * np.log(rng.permutation(E) + 1.0)).astype(np.float32)  # log-Zipf(1.2)
+    W = dict(w_router=_normal(rng, (E, d), 1.0 / np.sqrt(d)), w_gate=_normal(rng, (E, f, d), 0.02),
+             w_up=_normal(rng, (E, f, d), 0.02), w_down=_normal(rng, (E, d, f), 0.02),
+             s_gate=_normal(rng, (fs, d), 0.02), s_up=_normal(rng, (fs, d), 0.02),
+             s_down=_normal(rng, (d, fs), 0.02), router_bias=bias)
+    oL, gL = S.build_pair(ora, W, k, capi.CONVENTION_HUGGINGFACE_QWEN, capi.WEIGHT_BF16,
+                          max_tokens_hint=16384)
+    del W
+    with gL:
+        for T in (1, 1024, 16384):
+            x = S.make_tokens(4000 + T, T, d)
+            _, counts = _check(ora, oL, gL, x, 1e-2, "config5 deepseek bf16")
+            if T == 16384:
+                assert counts.max() > 4 * counts.min() + 1  # the bias really skews the load
