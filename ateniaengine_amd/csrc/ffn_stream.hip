@@ -80,7 +80,7 @@ __device__ inline f32x4 mfma(bf16x8 a, bf16x8 b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
 
-// MT  : 16-row tiles of tokens held per workgroup
+// MT  : 16-row tiles of tokens held per workgroup (1 or 2)
 // INT8: weights are int8 blocks (64 k per block) instead of bf16 blocks (32 k per block)
 // UP  : gate/up phase with SwiGLU epilogue, else down phase
 // WAVES: waves per workgroup = K slices of the strip
@@ -100,22 +100,6 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p) 
   constexpr int KB = INT8 ? kKbInt8 : kKbBf16;  // k per block
   constexpr int NACC = UP ? 2 : 1;
 
-  const uint16_t* arow[MT];
-#pragma unroll
-  for (int i = 0; i < MT; ++i) {
-    int pos = m0 + 16 * i + mm;
-    if (pos < cnt) {
-      if (UP) {
-        int pair = p.g.perm[base + pos];
-        arow[i] = p.a + (size_t)(pair / p.g.pair_div) * p.a_stride + (KB / 4) * kq;
-      } else {
-        arow[i] = p.a + (size_t)(base + pos) * p.a_stride + (KB / 4) * kq;
-      }
-    } else {
-      arow[i] = nullptr;
-    }
-  }
-
   const int kb_per = (p.nkb + kWavesPerWg - 1) / kWavesPerWg;
   const int kb0 = wave * kb_per;
   const int kb1 = min(p.nkb, kb0 + kb_per);
@@ -123,85 +107,99 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p) 
   const uint4* pb = UP ? p.wb + (size_t)e * p.w_stride_u4 + (size_t)nb * p.nkb * 64 + lane
                        : nullptr;
 
+  // Software pipeline over batches of U weight blocks with two register buffers: the loads
+  // of batch i+1 are in flight while batch i is multiplied.  The first batch is requested
+  // before the dependent look-ups (perm -> token row) below, so the weight stream starts one
+  // memory latency after the workgroup does.
+  constexpr int U = INT8 ? 2 : 4;        // blocks per batch
+  constexpr int AV = INT8 ? 2 : 1;       // 16-byte activation pieces per block and row tile
+  uint4 wA0[U], wB0[UP ? U : 1], wA1[U], wB1[UP ? U : 1];
+  uint4 xa0[U][MT][AV], xa1[U][MT][AV];
+  auto load_w = [&](uint4 (&wa)[U], uint4 (&wb)[UP ? U : 1], int kb) {
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      const int kk = min(kb + j, kb1 - 1);  // clamped: a batch past the end is loaded, not used
+      wa[j] = load_stream(pa + (size_t)kk * 64);
+      if (UP) wb[j] = load_stream(pb + (size_t)kk * 64);
+    }
+  };
+  if (kb0 < kb1) load_w(wA0, wB0, kb0);
+
+  // Token rows of the A operand.  Lanes whose row lies past the end of the group read the
+  // group's first row instead: an MFMA output row depends on its own input row only, and
+  // rows past the end are never stored.
+  const uint16_t* arow[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) {
+    int pos = m0 + 16 * i + mm;
+    if (pos >= cnt) pos = m0;
+    if (UP) {
+      int pair = p.g.perm[base + pos];
+      arow[i] = p.a + (size_t)(pair / p.g.pair_div) * p.a_stride + (KB / 4) * kq;
+    } else {
+      arow[i] = p.a + (size_t)(base + pos) * p.a_stride + (KB / 4) * kq;
+    }
+  }
+  auto load_x = [&](uint4 (&xa)[U][MT][AV], int kb) {
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      const int kk = min(kb + j, kb1 - 1);
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int v = 0; v < AV; ++v)
+          xa[j][i][v] = *((const uint4*)(arow[i] + (size_t)kk * KB) + v);
+    }
+  };
+
   f32x4 acc[NACC][MT];
 #pragma unroll
   for (int n = 0; n < NACC; ++n)
 #pragma unroll
     for (int i = 0; i < MT; ++i) acc[n][i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  constexpr int U = INT8 ? 4 : 8;  // blocks in flight per projection per wave
-  const uint4 zero4 = make_uint4(0, 0, 0, 0);
-  int kb = kb0;
-  for (; kb + U <= kb1; kb += U) {
-    uint4 ba[U], bb[U];
+  auto multiply = [&](const uint4 (&wa)[U], const uint4 (&wb)[UP ? U : 1],
+                      const uint4 (&xa)[U][MT][AV], int kb) {
 #pragma unroll
     for (int j = 0; j < U; ++j) {
-      ba[j] = load_stream(pa + (size_t)(kb + j) * 64);
-      if (UP) bb[j] = load_stream(pb + (size_t)(kb + j) * 64);
-    }
+      if (kb + j < kb1) {
+        if (INT8) {
+          bf16x8 al, ah, bl, bh;
+          widen_i8x16(wa[j], al, ah);
+          if (UP) widen_i8x16(wb[j], bl, bh);
 #pragma unroll
-    for (int j = 0; j < U; ++j) {
-      if (INT8) {
-        bf16x8 al, ah, bl, bh;
-        widen_i8x16(ba[j], al, ah);
-        if (UP) widen_i8x16(bb[j], bl, bh);
-#pragma unroll
-        for (int i = 0; i < MT; ++i) {
-          uint4 x0 = zero4, x1 = zero4;
-          if (arow[i]) {
-            const uint4* ap = (const uint4*)(arow[i] + (size_t)(kb + j) * KB);
-            x0 = ap[0];
-            x1 = ap[1];
+          for (int i = 0; i < MT; ++i) {
+            uint4 x0 = xa[j][i][0], x1 = xa[j][i][AV - 1];
+            acc[0][i] = mfma(*(bf16x8*)&x0, al, acc[0][i]);
+            acc[0][i] = mfma(*(bf16x8*)&x1, ah, acc[0][i]);
+            if (UP) {
+              acc[NACC - 1][i] = mfma(*(bf16x8*)&x0, bl, acc[NACC - 1][i]);
+              acc[NACC - 1][i] = mfma(*(bf16x8*)&x1, bh, acc[NACC - 1][i]);
+            }
           }
-          acc[0][i] = mfma(*(bf16x8*)&x0, al, acc[0][i]);
-          acc[0][i] = mfma(*(bf16x8*)&x1, ah, acc[0][i]);
-          if (UP) {
-            acc[NACC - 1][i] = mfma(*(bf16x8*)&x0, bl, acc[NACC - 1][i]);
-            acc[NACC - 1][i] = mfma(*(bf16x8*)&x1, bh, acc[NACC - 1][i]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < MT; ++i) {
+            acc[0][i] = mfma(xa[j][i][0], wa[j], acc[0][i]);
+            if (UP) acc[NACC - 1][i] = mfma(xa[j][i][0], wb[j], acc[NACC - 1][i]);
           }
         }
-      } else {
-#pragma unroll
-        for (int i = 0; i < MT; ++i) {
-          uint4 x0 = zero4;
-          if (arow[i]) x0 = *(const uint4*)(arow[i] + (size_t)(kb + j) * KB);
-          acc[0][i] = mfma(x0, ba[j], acc[0][i]);
-          if (UP) acc[NACC - 1][i] = mfma(x0, bb[j], acc[NACC - 1][i]);
-        }
       }
     }
-  }
-  for (; kb < kb1; ++kb) {
-    uint4 ba = pa[(size_t)kb * 64];
-    uint4 bb = UP ? pb[(size_t)kb * 64] : zero4;
-    if (INT8) {
-      bf16x8 al, ah, bl, bh;
-      widen_i8x16(ba, al, ah);
-      if (UP) widen_i8x16(bb, bl, bh);
-#pragma unroll
-      for (int i = 0; i < MT; ++i) {
-        uint4 x0 = zero4, x1 = zero4;
-        if (arow[i]) {
-          const uint4* ap = (const uint4*)(arow[i] + (size_t)kb * KB);
-          x0 = ap[0];
-          x1 = ap[1];
-        }
-        acc[0][i] = mfma(*(bf16x8*)&x0, al, acc[0][i]);
-        acc[0][i] = mfma(*(bf16x8*)&x1, ah, acc[0][i]);
-        if (UP) {
-          acc[NACC - 1][i] = mfma(*(bf16x8*)&x0, bl, acc[NACC - 1][i]);
-          acc[NACC - 1][i] = mfma(*(bf16x8*)&x1, bh, acc[NACC - 1][i]);
-        }
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < MT; ++i) {
-        uint4 x0 = zero4;
-        if (arow[i]) x0 = *(const uint4*)(arow[i] + (size_t)kb * KB);
-        acc[0][i] = mfma(x0, ba, acc[0][i]);
-        if (UP) acc[NACC - 1][i] = mfma(x0, bb, acc[NACC - 1][i]);
-      }
+  };
+
+  if (kb0 < kb1) load_x(xa0, kb0);
+  for (int kb = kb0; kb < kb1; kb += 2 * U) {
+    if (kb + U < kb1) {
+      load_w(wA1, wB1, kb + U);
+      load_x(xa1, kb + U);
     }
+    multiply(wA0, wB0, xa0, kb);
+    if (kb + 2 * U < kb1) {
+      load_w(wA0, wB0, kb + 2 * U);
+      load_x(xa0, kb + 2 * U);
+    }
+    if (kb + U < kb1) multiply(wA1, wB1, xa1, kb + U);
   }
 
   // Reduce the four K-slices through LDS; wave 0 finishes.
@@ -250,17 +248,16 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p) 
 template <bool INT8, bool UP>
 hipError_t launch_stream(const StreamParams& p, int n_pad, int n_groups, int rows_max,
                          hipStream_t s) {
-  int mt = rows_max <= 16 ? 1 : rows_max <= 32 ? 2 : 4;
+  // Up to 32 rows per expert per workgroup; larger groups take more workgroups along z.
+  int mt = rows_max <= 16 ? 1 : 2;
   dim3 grid(n_pad / 16, n_groups, (rows_max + 16 * mt - 1) / (16 * mt));
   // The down projection has few strips (d / 16) and a long K (f): eight K slices per strip
   // keep enough loads in flight; gate/up has 2f / 16 strips and uses four.
   constexpr int W = UP ? 4 : 8;
   if (mt == 1)
     ffn_stream_kernel<1, INT8, UP, W><<<grid, 64 * W, 0, s>>>(p);
-  else if (mt == 2)
-    ffn_stream_kernel<2, INT8, UP, W><<<grid, 64 * W, 0, s>>>(p);
   else
-    ffn_stream_kernel<4, INT8, UP, W><<<grid, 64 * W, 0, s>>>(p);
+    ffn_stream_kernel<2, INT8, UP, W><<<grid, 64 * W, 0, s>>>(p);
   return hipGetLastError();
 }
 

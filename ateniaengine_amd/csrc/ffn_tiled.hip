@@ -483,18 +483,32 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_dma_kernel(TiledParams p) 
     if (decltype(issue_b_c)::value) issue_b(Brefill, ks + 3);
     // Rows past the end of a partial tile were clamped to a real row when loading; their
     // products are computed and dropped, which keeps this loop free of per-row branches.
-    if (decltype(mul_c)::value) {
+    if (decltype(mul_c)::value == 2) {
 #pragma unroll
       for (int h = 0; h < 2; ++h)
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
           for (int j = 0; j < 4; ++j) acc[i][j] = mfma32(fa[h][i], fb[h][j], acc[i][j]);
+    } else if (decltype(mul_c)::value == 1) {
+      // partial tile: only the 32-row groups that hold rows (wave-uniform branches)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (i * 32 < my_rows) {
+#pragma unroll
+          for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[i][j] = mfma32(fa[h][i], fb[h][j], acc[i][j]);
+        }
+      }
     }
   };
   using std::integral_constant;
   typedef integral_constant<bool, true> yes;
   typedef integral_constant<bool, false> no;
+  typedef integral_constant<int, 2> mul_all;
+  typedef integral_constant<int, 1> mul_some;
+  typedef integral_constant<int, 0> mul_none;
   typedef integral_constant<int, 16> w16;
   typedef integral_constant<int, 8> w8;
   typedef integral_constant<int, 4> w4;
@@ -517,9 +531,11 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_dma_kernel(TiledParams p) 
     step(yes{}, w0{}, no{}, no{}, mul_c, A1, A0, B3, B2, ks + 3);
   };
   // nks is a multiple of 4 and at least 8 (checked by the launcher).  A wave whose half of
-  // a partial tile holds no rows still feeds LDS and meets the barriers, without MFMAs.
-  if (my_rows > 0) run(yes{});
-  else run(no{});
+  // a partial tile holds no rows still feeds LDS and meets the barriers, without MFMAs; one
+  // with fewer than four 32-row groups multiplies only those.
+  if (my_rows >= 97) run(mul_all{});
+  else if (my_rows > 0) run(mul_some{});
+  else run(mul_none{});
 
   if (UP) {
     uint16_t* h = (uint16_t*)p.out;

@@ -10,6 +10,7 @@
 #include <cstdarg>
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <new>
@@ -106,10 +107,26 @@ struct AteniaMoeLayer {
 
 namespace {
 
-// Largest batch served by the weight-streaming expert kernels.
-constexpr int kStreamMaxTokens = 128;
-// Largest batch routed by the one-workgroup-per-token router kernel.
-constexpr int kRouterTokenKernelMaxTokens = 512;
+// Largest batch served by the weight-streaming expert kernels (tuning knob:
+// ATENIA_MOE_STREAM_MAX_TOKENS, read once per process).
+int stream_max_tokens() {
+  static const int v = [] {
+    const char* e = getenv("ATENIA_MOE_STREAM_MAX_TOKENS");
+    int n = e ? atoi(e) : 0;
+    return n > 0 ? n : 32;
+  }();
+  return v;
+}
+// Largest batch routed by the one-workgroup-per-token router kernel (tuning knob:
+// ATENIA_MOE_ROUTER_TOKEN_MAX, read once per process).
+int router_token_max() {
+  static const int v = [] {
+    const char* e = getenv("ATENIA_MOE_ROUTER_TOKEN_MAX");
+    int n = e ? atoi(e) : -1;
+    return n >= 0 ? n : 512;
+  }();
+  return v;
+}
 
 bool valid_handle(const AteniaMoeLayer* L) { return L && L->magic == 0x4d6f4541u; }
 
@@ -250,7 +267,7 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   ra.status = L->status.as<int32_t>();
   // f32-valued operands almost never satisfy the exactness test of the per-token kernel, so
   // f32 layers always take the sequential-order kernel.
-  ra.token_kernel_max_tokens = f32w ? 0 : kRouterTokenKernelMaxTokens;
+  ra.token_kernel_max_tokens = f32w ? 0 : router_token_max();
   PermuteArgs pa{};
   pa.idx = L->idx.as<int32_t>();
   pa.T = T;
@@ -304,7 +321,7 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   fa.y_stride = L->d;
   // Tiled (MFMA-bound) kernels once an expert can see more rows than the streaming kernel
   // keeps in registers; below that the weights are streamed once (HBM-bound).
-  const bool tiled = T > kStreamMaxTokens && tiled_supported(L->gate, L->wdtype) &&
+  const bool tiled = T > stream_max_tokens() && tiled_supported(L->gate, L->wdtype) &&
                      tiled_supported(L->down, L->wdtype);
   fa.use_tiled = tiled;
   fa.tile_group = L->tile_group.as<int32_t>();
@@ -330,7 +347,7 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
     fsd.h = L->hs.p;
     fsd.h_stride = L->fs_kpad;
     fsd.y = L->ys.as<float>();
-    fsd.use_tiled = T > kStreamMaxTokens && tiled_supported(L->s_gate, L->wdtype) &&
+    fsd.use_tiled = T > stream_max_tokens() && tiled_supported(L->s_gate, L->wdtype) &&
                     tiled_supported(L->s_down, L->wdtype);
     fsd.tile_group = L->s_tile_group.as<int32_t>();
     fsd.tile_m0 = L->s_tile_m0.as<int32_t>();
