@@ -22,7 +22,21 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+# BASELINE configs.  The headline metric is quoted on mixtral_bf16; the others are reported
+# with --config for the tables in DESIGN.md.
+CONFIGS = {
+    "mixtral_bf16": dict(d=4096, E=8, k=2, f=14336, fs=0, gated=False, conv=0, wd="bf16",
+                         zipf=False, sweep=(1, 16, 128, 512, 4096)),
+    "mixtral_int8": dict(d=4096, E=8, k=2, f=14336, fs=0, gated=False, conv=0, wd="int8",
+                         zipf=False, sweep=(1, 16, 4096)),
+    "qwen_bf16": dict(d=2048, E=60, k=4, f=1408, fs=5632, gated=True, conv=1, wd="bf16",
+                      zipf=False, sweep=(1, 256, 8192)),
+    "deepseek_bf16": dict(d=2048, E=64, k=6, f=1408, fs=2816, gated=False, conv=1, wd="bf16",
+                          zipf=True, sweep=(1, 1024, 16384)),
+}
 D_MODEL, N_EXPERTS, TOP_K, D_FF = 4096, 8, 2, 14336
+D_FF_SHARED = 0
+W_BYTES = 2
 W_STD = 0.02
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, GB/s
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, TFLOP/s
@@ -43,7 +57,11 @@ def make_weights(torch, np, seed):
     up = np.stack([bf16_bits((D_FF, D_MODEL)) for _ in range(N_EXPERTS)])
     down = np.stack([bf16_bits((D_MODEL, D_FF)) for _ in range(N_EXPERTS)])
     router = bf16_bits((N_EXPERTS, D_MODEL))
-    return router, gate, up, down
+    shared = None
+    if D_FF_SHARED:
+        shared = (bf16_bits((D_FF_SHARED, D_MODEL)), bf16_bits((D_FF_SHARED, D_MODEL)),
+                  bf16_bits((D_MODEL, D_FF_SHARED)), upcast(np, bf16_bits((D_MODEL,))))
+    return router, gate, up, down, shared
 
 
 def upcast(np, bits):
@@ -89,15 +107,18 @@ def measure(torch, np, capi, layer, T, steps, warmup, seed):
         raise RuntimeError(f"device status {rc} at token {tok}, expert {ex}")
     U = active / steps  # experts with at least one token (mean over steps)
 
-    eb = 2  # bytes per bf16 weight
-    bytes_up = U * 2 * D_FF * D_MODEL * eb
-    bytes_down = U * D_MODEL * D_FF * eb
-    bytes_fwd = (U * 3 * D_FF * D_MODEL * eb + N_EXPERTS * D_MODEL * 4
-                 + T * D_MODEL * (2 + 4))
+    eb = W_BYTES  # bytes per stored weight
+    sc = 4 if W_BYTES == 1 else 0  # int8: one f32 scale per output row
+    fs = D_FF_SHARED
+    # the shared expert (if any) runs as a second launch of the same kernels; both launches
+    # of a stage are timed together, so their bytes / flops are added together too
+    bytes_up = U * (2 * D_FF * D_MODEL * eb + 2 * D_FF * sc) + 2 * fs * D_MODEL * eb + 2 * fs * sc
+    bytes_down = U * (D_MODEL * D_FF * eb + D_MODEL * sc) + fs * D_MODEL * eb + (D_MODEL * sc if fs else 0)
+    bytes_fwd = bytes_up + bytes_down + N_EXPERTS * D_MODEL * 4 + T * D_MODEL * (2 + 4)
     P = T * TOP_K
-    flops_up = 4.0 * P * D_MODEL * D_FF
-    flops_down = 2.0 * P * D_MODEL * D_FF
-    flops_fwd = T * (2.0 * D_MODEL * N_EXPERTS + 6.0 * TOP_K * D_MODEL * D_FF)
+    flops_up = 4.0 * P * D_MODEL * D_FF + 4.0 * T * D_MODEL * fs
+    flops_down = 2.0 * P * D_MODEL * D_FF + 2.0 * T * D_MODEL * fs
+    flops_fwd = T * (2.0 * D_MODEL * N_EXPERTS + 6.0 * TOP_K * D_MODEL * D_FF + 6.0 * D_MODEL * fs)
     r = dict(
         tokens=T, ms_per_step=wall_ms, tokens_per_s=T / (wall_ms * 1e-3),
         active_experts=U,
@@ -133,7 +154,10 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--tokens", type=int, default=4096, help="headline batch size T")
+    ap.add_argument("--config", default="mixtral_bf16", choices=sorted(CONFIGS),
+                    help="layer shape (the headline metric is quoted on mixtral_bf16)")
+    ap.add_argument("--tokens", type=int, default=0,
+                    help="headline batch size T (default: the config's largest)")
     ap.add_argument("--decode-tokens", type=int, default=1, help="decode batch (0 = skip)")
     ap.add_argument("--sweep", type=str, default="", help="extra batch sizes, comma separated")
     ap.add_argument("--cpu-tokens", type=int, default=16,
@@ -156,12 +180,47 @@ def main():
         print("bench.py: no gfx950 device; the HIP path has no fallback", file=sys.stderr)
         sys.exit(3)
     torch.cuda.set_device(0)
-    router, gate, up, down = make_weights(torch, np, a.seed)
+    global D_MODEL, N_EXPERTS, TOP_K, D_FF, D_FF_SHARED, W_BYTES
+    cfg = CONFIGS[a.config]
+    D_MODEL, N_EXPERTS, TOP_K, D_FF, D_FF_SHARED = cfg["d"], cfg["E"], cfg["k"], cfg["f"], cfg["fs"]
+    W_BYTES = 1 if cfg["wd"] == "int8" else 2
+    if a.tokens <= 0:
+        a.tokens = max(cfg["sweep"])
+    if a.sweep == "all":
+        a.sweep = ",".join(str(t) for t in cfg["sweep"] if t not in (a.tokens, a.decode_tokens))
+    router, gate, up, down, shared = make_weights(torch, np, a.seed)
     router_f32 = upcast(np, router)
+    if cfg["zipf"]:  # logits ~ N(0,1) plus a log-Zipf(1.2) bias: skewed expert load
+        router_f32 = router_f32 * np.float32(1.0 / (W_STD * np.sqrt(D_MODEL)))
+        router_f32 = upcast(np, capi.f32_to_bf16_trunc(router_f32))
     tmax = max([a.tokens, a.decode_tokens] + [int(t) for t in a.sweep.split(",") if t])
-    layer = capi.Layer(w_router=router_f32, w_gate=gate, w_up=up, w_down=down, top_k=TOP_K,
-                       convention=capi.CONVENTION_ATENIA, weight_dtype=capi.WEIGHT_BF16,
-                       max_tokens_hint=tmax)
+    kw = dict(w_router=router_f32, top_k=TOP_K, convention=cfg["conv"], max_tokens_hint=tmax)
+    if cfg["zipf"]:
+        rank = np.random.default_rng(a.seed).permutation(N_EXPERTS) + 1.0
+        kw["router_bias"] = (-1.2 * np.log(rank)).astype(np.float32)
+    if shared is not None and cfg["gated"]:
+        kw["shared_gate"] = shared[3]
+    if cfg["wd"] == "int8":
+        # per-output-row int8 of the bf16-valued weights, 0.1 % of rows scaled x8 first
+        rng = np.random.default_rng(a.seed + 1)
+
+        def q8(bits):
+            w = upcast(np, bits)
+            rows = w.reshape(-1, w.shape[-1])
+            rows[rng.choice(rows.shape[0], size=rows.shape[0] // 1000, replace=False)] *= 8.0
+            return capi.quantize_per_row_i8(w)
+        (gate, sg), (up, su), (down, sd) = q8(gate), q8(up), q8(down)
+        kw.update(scale_gate=sg, scale_up=su, scale_down=sd)
+        if shared is not None:
+            (g_, a1), (u_, a2), (d_, a3) = q8(shared[0]), q8(shared[1]), q8(shared[2])
+            shared = (g_, u_, d_, shared[3])
+            kw.update(s_scale_gate=a1, s_scale_up=a2, s_scale_down=a3)
+        wdt = capi.WEIGHT_INT8_W8A16
+    else:
+        wdt = capi.WEIGHT_BF16
+    if shared is not None:
+        kw.update(s_gate=shared[0], s_up=shared[1], s_down=shared[2])
+    layer = capi.Layer(w_gate=gate, w_up=up, w_down=down, weight_dtype=wdt, **kw)
 
     if a.calibrate_copy:
         src = torch.empty(1 << 28, device="cuda", dtype=torch.float32)  # 1 GiB
@@ -185,7 +244,7 @@ def main():
 
     cpu = None
     parity = None
-    if a.cpu_tokens > 0:
+    if a.cpu_tokens > 0 and a.config == "mixtral_bf16":
         from oracle import moe_oracle as ora  # checker + reported CPU baseline only
         n = min(a.cpu_tokens, a.tokens)
         # the headline batch, recomputed once so `out_head` matches `x_head`
@@ -218,9 +277,10 @@ def main():
         "value": head["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": a.steps,
         "warmup": a.warmup, "ms_per_step": head["ms_per_step"], "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"mixtral-8x7b-shape MoE layer, d_model={D_MODEL}, "
-                               f"experts={N_EXPERTS}, top_k={TOP_K}, d_ff={D_FF}, bf16 weights "
-                               f"resident in HBM, T={a.tokens} tokens per step",
+        "config": {"workload": f"{a.config}: MoE layer, d_model={D_MODEL}, experts={N_EXPERTS}, "
+                               f"top_k={TOP_K}, d_ff={D_FF}, shared d_ff={D_FF_SHARED}, "
+                               f"{cfg['wd']} weights resident in HBM, bf16 activations, "
+                               f"T={a.tokens} tokens per step",
                    "tokens_per_step": a.tokens},
         "roofline": head["roofline"],
         "cpu_baseline": cpu,
