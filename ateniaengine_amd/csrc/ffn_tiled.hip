@@ -312,32 +312,21 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_kernel(TiledParams p) {
   }
 }
 
-// ---- bf16 form with direct global->LDS loads and a four-stage ring -------------------------
-// Same tiling.  Each stage holds 32 k of both operands (16 KiB + 16 KiB); a wave fills a
-// 1 KiB chunk with one global_load_lds_dwordx4 (lane l's 16 bytes land at chunk + 16*l), so
-// no operand passes through registers on its way to LDS and three stages (about 3 * 64 MFMAs
-// of work) are always in flight behind the one being multiplied.  The four stage buffers are
-// separate arrays and the k loop is unrolled by four, so each fragment read names its buffer
-// statically.
-typedef __attribute__((address_space(1))) const void* gptr_t;
+// ---- bf16 form: direct global->LDS loads, multi-stage rings, software-pipelined k loop ------
+// Same 256 x 256 tiling on v_mfma_f32_32x32x16_bf16 (each wave 128 x 128 = 4 x 4 MFMA tiles).
+// LDS holds a ring of three 64-k A stages (32 KiB each) and a ring of four 32-k B stages
+// (16 KiB each).  A wave fills a 1 KiB chunk with one global_load_lds_dwordx4 (lane l's 16
+// bytes land at chunk + 16*l), so no operand passes through registers on its way to LDS.
+// The k loop works in k16 units of 16 MFMAs: while one unit multiplies, the 8 fragment reads
+// of the next unit and 4 loads of a stage several steps ahead are issued between its MFMAs
+// (pinned with sched_barrier), and the single barrier per 32-k step sits between the two
+// units of the step so that no wave waits for LDS right after it.
 typedef __attribute__((address_space(3))) void* lptr_t;
-constexpr int kDmaStageU4 = 2 * 16 * 64;  // uint4 per stage: 16 A chunks + 16 B chunks
-
-__device__ inline void wait_vmcnt(int n) {
-  // s_waitcnt vmcnt(n) lgkmcnt(0): vmcnt[3:0] in bits 3:0, vmcnt[5:4] in bits 15:14, expcnt
-  // (bits 6:4) left at "no wait", lgkmcnt (bits 11:8) = 0.  lgkmcnt(0) makes sure this wave's
-  // own LDS reads of the previous step have returned before it passes the barrier after
-  // which other waves refill that buffer.
-  if (n >= 16) __builtin_amdgcn_s_waitcnt(0x4070);
-  else if (n >= 8) __builtin_amdgcn_s_waitcnt(0x0078);
-  else if (n >= 4) __builtin_amdgcn_s_waitcnt(0x0074);
-  else __builtin_amdgcn_s_waitcnt(0x0070);
-}
 
 // One wave-wide 16-byte-per-lane load from global memory straight into LDS: lane l's bytes
 // land at lds_addr + 16*l.  Written as inline assembly so that the compiler's wait-count
 // insertion does not tie later LDS reads to these loads (it would drain all stages); the
-// kernel waits for exactly the stage it needs with wait_vmcnt() before its barrier.
+// kernel waits for exactly the stage it needs with an explicit s_waitcnt before its barrier.
 __device__ inline void dma16(const void* gaddr, uint32_t lds_addr) {
   asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off"
                :
@@ -356,16 +345,20 @@ __device__ inline f32x16 mfma32(uint4 a, uint4 b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8*)&a, *(bf16x8*)&b, c, 0, 0, 0);
 }
 
+// s_waitcnt vmcnt(N) lgkmcnt(0): vmcnt[3:0] in bits 3:0, vmcnt[5:4] in bits 15:14, expcnt
+// (bits 6:4) left at "no wait".  lgkmcnt(0) makes sure the wave's own LDS reads have returned
+// before it passes the barrier behind which other waves refill the buffers it read.
+template <int N>
+__device__ inline void wait_vm_lgkm0() {
+  __builtin_amdgcn_s_waitcnt(0x0070 | (N & 15) | ((N >> 4) << 14));
+}
+constexpr int kRingA = 3;  // A stages of 64 k (32 KiB each)
+constexpr int kRingB = 4;  // B stages of 32 k (16 KiB each)
+
 template <bool UP>
-__global__ __launch_bounds__(kThreads) void ffn_tiled_dma_kernel(TiledParams p) {
-  // B ring: four stages of 32 k, chunk c = (32-row group ng = c/2, k half c%2), 16 KiB each.
-  // A ring: two stages of 64 k (32 KiB each).  An A chunk is 8 rows x 64 k: one load
-  // instruction reads eight full 128-byte lines (a 32-row x 16-k fragment would touch 32
-  // lines for 32 bytes each and starve the load path).  Inside a chunk the 16-byte segment
-  // s of row r is stored at slot r*8 + (s ^ r ^ (chunk & 1)), which makes the 32-row
-  // fragment reads below free of LDS bank conflicts.
-  __shared__ uint4 A0[2048], A1[2048];
-  __shared__ uint4 B0[1024], B1[1024], B2[1024], B3[1024];
+__global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p) {
+  constexpr int NA = kRingA, NB = kRingB;
+  __shared__ uint4 S[NA * 2048 + NB * 1024];  // A ring, then B ring
   int rt, ct;
   if (!tile_of_workgroup(p, rt, ct)) return;
 
@@ -376,32 +369,29 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_dma_kernel(TiledParams p) 
   const int rows_here = min(TM, cnt - tm0);
 
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept scalar
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int kh = lane >> 5, l32 = lane & 31;
   const int wm = wave >> 1, wn = wave & 1;
   constexpr int BROWS = UP ? 128 : 256;
   const int nb0 = ct * (BROWS / 16);
 
-  // ---- loads issued by this thread --------------------------------------------------------
-  // A: per 64-k stage this wave fills chunks 8*wave .. 8*wave+7 (rows 64*wave .. +63); lane l
-  // fetches row l/8 of the chunk, segment (l%8) ^ (l/8) ^ (chunk&1).
+  // A stage: 256 rows x 64 k as 32 chunks of 8 rows x 128 bytes, so that one load instruction
+  // reads eight full 128-byte lines.  Row r, 16-byte segment s of chunk c is stored at slot
+  // 8r + (s ^ r ^ (c & 1)); lane l of the filling load fetches row l/8, segment
+  // (l%8) ^ (l/8) ^ (c&1).  Wave w fills chunks 8w .. 8w+7, four per step.
   const uint16_t* arow[8];
   {
     const int r8 = lane >> 3, pslot = lane & 7;
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
       int m = (wave * 8 + q) * 8 + r8;
-      if (m >= rows_here) m = 0;  // clamp: such rows are computed but never stored
+      if (m >= rows_here) m = 0;
       int src;
       if (UP) src = p.g.perm[base + tm0 + m] / p.g.pair_div;
       else src = base + tm0 + m;
-      const int seg = pslot ^ r8 ^ (q & 1);
-      arow[q] = p.a + (size_t)src * p.a_stride + seg * 8;
+      arow[q] = p.a + (size_t)src * p.a_stride + (pslot ^ r8 ^ (q & 1)) * 8;
     }
   }
-  // B: per 32-k stage this wave fills chunks 4*wave .. 4*wave+3 (row groups 2*wave, 2*wave+1,
-  // both k halves).  Inside a stored 16-row x 32-k block the lane slot is (k quarter)*16 +
-  // row%16 with k quarter = 2*half + kh.
   const uint4* bptr[2];
 #pragma unroll
   for (int q = 0; q < 2; ++q) {
@@ -416,12 +406,11 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_dma_kernel(TiledParams p) 
       brow = ng * 32 + l32;
     }
     int nb = nb0 + (brow >> 4);
-    if (nb >= p.n_blocks) nb = p.n_blocks - 1;  // clamp: columns past N are never stored
+    if (nb >= p.n_blocks) nb = p.n_blocks - 1;
     bptr[q] = wbase + (size_t)e * p.w_stride_u4 + (size_t)nb * p.nkb * 64 + kh * 16 + (brow & 15);
   }
-  // ---- fragment read offsets (uint4 units) ------------------------------------------------
-  // A fragment (row group mg = 4*wm + i, k16 index u of the stage): row m32 of the group is
-  // chunk mg*4 + m32/8, row m32%8; segment 2u + kh.
+  // fragment read offsets (uint4 units inside a stage): A row group i adds 256, k16 unit u of
+  // the 64-k stage selects the swizzled segment; B row group j of this wave, unit u adds 64.
   int aoff[4];
   {
     const int r8 = l32 & 7, cpar = (l32 >> 3) & 1;
@@ -429,6 +418,8 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_dma_kernel(TiledParams p) 
 #pragma unroll
     for (int u = 0; u < 4; ++u) aoff[u] = rowbase + ((2 * u + kh) ^ r8 ^ cpar);
   }
+  const int boff0 = NA * 2048 + (UP ? 2 * wn : 4 * wn) * 128 + lane;
+  constexpr int kBJ1 = 128, kBJ2 = UP ? 512 : 256, kBJ3 = UP ? 640 : 384;
 
   f32x16 acc[4][4];
 #pragma unroll
@@ -440,122 +431,162 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_dma_kernel(TiledParams p) 
   const int my_rows = rows_here - wm * 128;
   const int nks = p.k_pad / 32;
 
-  auto issue_a = [&](uint4* A, int t) {  // 64-k stage t
-    const uint32_t sbase = (uint32_t)(uintptr_t)(lptr_t)A + wave * 8 * kChunk;
-#pragma unroll
-    for (int q = 0; q < 8; ++q) dma16(arow[q] + (size_t)t * 64, sbase + q * kChunk);
+  const uint32_t sa_fill = (uint32_t)(uintptr_t)(lptr_t)S + wave * 8 * kChunk;
+  const uint32_t sb_fill = (uint32_t)(uintptr_t)(lptr_t)S + NA * 32768 + wave * 4 * kChunk;
+  auto dma_a = [&](int buf, int q, int t) {  // chunk q of this wave, 64-k stage t
+    dma16(arow[q] + (size_t)t * 64, sa_fill + buf * 32768 + q * kChunk);
   };
-  auto issue_b = [&](uint4* B, int ks) {  // 32-k stage ks
-    const uint32_t sbase = (uint32_t)(uintptr_t)(lptr_t)B + wave * 4 * kChunk;
-#pragma unroll
-    for (int q = 0; q < 2; ++q)
-#pragma unroll
-      for (int h = 0; h < 2; ++h)
-        dma16(bptr[q] + (size_t)ks * 64 + 32 * h, sbase + (q * 2 + h) * kChunk);
+  auto dma_b = [&](int buf, int q, int ks) {  // q = 2 * row group + k half
+    dma16(bptr[q >> 1] + (size_t)ks * 64 + 32 * (q & 1), sb_fill + buf * 16384 + q * kChunk);
   };
-  // One 32-k step.  Per wave the loads are issued in the order
-  //   A(0) B(0) B(1) B(2) | step 0: A(1) B(3) | step 1: B(4) | step 2: A(2) B(5) | ...
-  // (8 instructions per A stage, 4 per B stage) and complete in order, so before the
-  // barrier of an even step at most 8 younger loads may be pending and before an odd step
-  // 16; WAIT carries that count (smaller at the very end).  A bare s_barrier is used:
-  // __syncthreads() would also drain every outstanding load, and the later stages must stay
-  // in flight.  ODD / ISSUE_A / ISSUE_B / MUL are compile-time: a step is straight-line code.
-  auto step = [&](auto odd_c, auto wait_c, auto issue_a_c, auto issue_b_c, auto mul_c,
-                  const uint4* Acur, uint4* Anext, const uint4* Bcur, uint4* Brefill, int ks) {
-    wait_vmcnt(decltype(wait_c)::value);
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    uint4 fa[2][4], fb[2][4];
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        // gate/up: j < 2 gate groups 2*wn+j, j >= 2 the matching up groups
-        int ng = UP ? ((j < 2 ? 0 : 4) + 2 * wn + (j & 1)) : (4 * wn + j);
-        fb[h][j] = Bcur[(ng * 2 + h) * 64 + lane];
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        fa[h][i] = Acur[i * 256 + aoff[2 * decltype(odd_c)::value + h]];
+  // the 8 fragment reads of one k16 unit, in the order the MFMAs consume them
+  auto read_frag = [&](int n, uint4 (&FA)[4], uint4 (&FB)[4], int a0, int b0) {
+    switch (n) {
+      case 0: FA[0] = S[a0]; break;
+      case 1: FB[0] = S[b0]; break;
+      case 2: FB[1] = S[b0 + kBJ1]; break;
+      case 3: FB[2] = S[b0 + kBJ2]; break;
+      case 4: FB[3] = S[b0 + kBJ3]; break;
+      case 5: FA[1] = S[a0 + 256]; break;
+      case 6: FA[2] = S[a0 + 512]; break;
+      default: FA[3] = S[a0 + 768]; break;
     }
-    if (decltype(issue_a_c)::value) issue_a(Anext, ks / 2 + 1);
-    if (decltype(issue_b_c)::value) issue_b(Brefill, ks + 3);
-    // Rows past the end of a partial tile were clamped to a real row when loading; their
-    // products are computed and dropped, which keeps this loop free of per-row branches.
-    if (decltype(mul_c)::value == 2) {
+  };
+  // One k16 unit: 16 MFMAs on (FA, FB).  Behind MFMA m < 8 goes read m of the next unit;
+  // behind MFMAs 8, 10, 12, 14 one load each of the stage being refilled, so LDS and the load
+  // path see an even stream instead of bursts.
+  auto half = [&](auto mul_c, auto dma_c, auto dma_is_a_c, uint4 (&FA)[4], uint4 (&FB)[4],
+                  uint4 (&NA_)[4], uint4 (&NB_)[4], int a0, int b0, int dbuf, int dks, auto aq0_c) {
+    constexpr int MUL = decltype(mul_c)::value;
 #pragma unroll
-      for (int h = 0; h < 2; ++h)
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-          for (int j = 0; j < 4; ++j) acc[i][j] = mfma32(fa[h][i], fb[h][j], acc[i][j]);
-    } else if (decltype(mul_c)::value == 1) {
-      // partial tile: only the 32-row groups that hold rows (wave-uniform branches)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (i * 32 < my_rows) {
-#pragma unroll
-          for (int h = 0; h < 2; ++h)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) acc[i][j] = mfma32(fa[h][i], fb[h][j], acc[i][j]);
-        }
+    for (int m = 0; m < 16; ++m) {
+      const int i = m >> 2, j = m & 3;
+      if (MUL == 2 || (MUL == 1 && i * 32 < my_rows)) acc[i][j] = mfma32(FA[i], FB[j], acc[i][j]);
+      if (m < 8) read_frag(m, NA_, NB_, a0, b0);
+      if (decltype(dma_c)::value && m >= 8 && (m & 1) == 0) {
+        if (decltype(dma_is_a_c)::value) dma_a(dbuf, decltype(aq0_c)::value + ((m - 8) >> 1), dks);
+        else dma_b(dbuf, (m - 8) >> 1, dks);
       }
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
   using std::integral_constant;
   typedef integral_constant<bool, true> yes;
   typedef integral_constant<bool, false> no;
-  typedef integral_constant<int, 2> mul_all;
-  typedef integral_constant<int, 1> mul_some;
-  typedef integral_constant<int, 0> mul_none;
-  typedef integral_constant<int, 16> w16;
-  typedef integral_constant<int, 8> w8;
-  typedef integral_constant<int, 4> w4;
-  typedef integral_constant<int, 0> w0;
-  auto run = [&](auto mul_c) {
-    issue_a(A0, 0);
-    issue_b(B0, 0);
-    issue_b(B1, 1);
-    issue_b(B2, 2);
-    int ks = 0;
-    for (; ks + 4 < nks; ks += 4) {
-      step(no{}, w8{}, yes{}, yes{}, mul_c, A0, A1, B0, B3, ks);
-      step(yes{}, w16{}, no{}, yes{}, mul_c, A0, A1, B1, B0, ks + 1);
-      step(no{}, w8{}, yes{}, yes{}, mul_c, A1, A0, B2, B1, ks + 2);
-      step(yes{}, w16{}, no{}, yes{}, mul_c, A1, A0, B3, B2, ks + 3);
+
+  // Step s (32 k) = unit 0 on (fa0, fb0), then unit 1 on (fa1, fb1).
+  //   first half : reads unit 1 of stage s; issues A(s + NA - 1) into the A buffer freed by
+  //                the previous step's barrier
+  //   middle     : waits until this wave's loads of stage s + 1 have landed, barrier
+  //   second half: reads unit 0 of stage s + 1; issues B(s + NB) into the B buffer of stage s
+  // Loads complete in issue order ... A(s+1) | B(s+NB-2) A(s+2) B(s+NB-1) A(s+3) at the middle
+  // of step s, so 4 * (NA - 2) groups of 4 loads may stay in flight behind the wait (half of
+  // that in a wave that loads no A rows).  Stages past the end of k are clamped to the last
+  // one: they land in buffers nobody reads and keep the wait counts uniform.
+  auto run = [&](auto mul_c, auto la_c) {
+    constexpr bool LA = decltype(la_c)::value;
+    typedef integral_constant<int, 0> q0;
+    typedef integral_constant<int, 4> q4;
+    uint4 fa0[4], fb0[4], fa1[4], fb1[4];
+    const int nst = nks / 2;  // 64-k stages
+    auto fill_a = [&](int t) {
+      if (LA) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) dma_a(t, q, t);
+      }
+    };
+    auto fill_b = [&](int t) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) dma_b(t, q, t);
+    };
+    // issue order A0 B0 B1 A1 B2 B3, then per step: half of A(s/2 + 2), B(s + 4)
+    fill_a(0); fill_b(0); fill_b(1); fill_a(1); fill_b(2); fill_b(3);
+    wait_vm_lgkm0<LA ? 20 : 12>();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int n = 0; n < 8; ++n) read_frag(n, fa0, fb0, aoff[0], boff0);
+    int abuf = 0, bbuf = 0;  // buffers of the stages step s reads
+    for (int s = 0; s < nks; s += 2) {
+      const int abuf_n = abuf + 1 == NA ? 0 : abuf + 1;
+      const int abuf_i = abuf == 0 ? NA - 1 : abuf - 1;  // freed by the previous stage
+      const int ta = min(s / 2 + NA - 1, nst - 1);
+      // even step: k16 units 0, 1 of the A stage
+      {
+        const int bbuf_n = bbuf + 1 == NB ? 0 : bbuf + 1;
+        half(mul_c, la_c, yes{}, fa0, fb0, fa1, fb1, aoff[1] + abuf * 2048, boff0 + bbuf * 1024 + 64,
+             abuf_i, ta, q0{});
+        wait_vm_lgkm0<LA ? 16 : 8>();
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        half(mul_c, yes{}, no{}, fa1, fb1, fa0, fb0, aoff[2] + abuf * 2048, boff0 + bbuf_n * 1024,
+             bbuf, min(s + NB, nks - 1), q0{});
+        bbuf = bbuf_n;
+      }
+      // odd step: units 2, 3; its second half reads unit 0 of the next A stage
+      {
+        const int bbuf_n = bbuf + 1 == NB ? 0 : bbuf + 1;
+        half(mul_c, la_c, yes{}, fa0, fb0, fa1, fb1, aoff[3] + abuf * 2048, boff0 + bbuf * 1024 + 64,
+             abuf_i, ta, q4{});
+        wait_vm_lgkm0<LA ? 16 : 8>();
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        half(mul_c, yes{}, no{}, fa1, fb1, fa0, fb0, aoff[0] + abuf_n * 2048, boff0 + bbuf_n * 1024,
+             bbuf, min(s + 1 + NB, nks - 1), q0{});
+        bbuf = bbuf_n;
+      }
+      abuf = abuf_n;
     }
-    step(no{}, w8{}, yes{}, yes{}, mul_c, A0, A1, B0, B3, ks);
-    step(yes{}, w16{}, no{}, no{}, mul_c, A0, A1, B1, B0, ks + 1);
-    step(no{}, w4{}, no{}, no{}, mul_c, A1, A0, B2, B1, ks + 2);
-    step(yes{}, w0{}, no{}, no{}, mul_c, A1, A0, B3, B2, ks + 3);
+    wait_vm_lgkm0<0>();
   };
-  // nks is a multiple of 4 and at least 8 (checked by the launcher).  A wave whose half of
-  // a partial tile holds no rows still feeds LDS and meets the barriers, without MFMAs; one
-  // with fewer than four 32-row groups multiplies only those.
-  if (my_rows >= 97) run(mul_all{});
-  else if (my_rows > 0) run(mul_some{});
-  else run(mul_none{});
+  const bool loads_a = wave * 64 < rows_here;
+  if (my_rows >= 97) run(integral_constant<int, 2>{}, yes{});
+  else if (my_rows > 0) {
+    if (loads_a) run(integral_constant<int, 1>{}, yes{});
+    else run(integral_constant<int, 1>{}, no{});
+  } else {
+    if (loads_a) run(integral_constant<int, 0>{}, yes{});
+    else run(integral_constant<int, 0>{}, no{});
+  }
 
   if (UP) {
-    uint16_t* h = (uint16_t*)p.out;
+    // silu(g) * u, rounded to bf16, staged through LDS so that every global store is a full
+    // 128-byte line: the wave's 128 x 64 block goes to its own region with a row pitch of
+    // 144 bytes and is read back 16 bytes per lane, 8 lanes per row.
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();  // every wave's loads have landed and its reads are done
+    asm volatile("" ::: "memory");
+    constexpr int kPitch = 144;
+    char* stage = (char*)S + wave * (128 * kPitch);
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const int n = nb0 * 16 + (2 * wn + j) * 32 + l32;
-      const bool n_ok = n < p.n_blocks * 16;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int m = wm * 128 + i * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
-          if (m < rows_here && n_ok) {
-            float g = acc[i][j][r];
-            float u = acc[i][j + 2][r];
-            float hv = (g / (1.f + __expf(-g))) * u;
-            h[(size_t)(base + tm0 + m) * p.out_stride + n] = bf16_rne(hv);
-          }
+          const int m = i * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
+          const float g = acc[i][j][r];
+          const float u = acc[i][j + 2][r];
+          const float hv = g * __builtin_amdgcn_rcpf(1.f + __expf(-g)) * u;
+          *(uint16_t*)(stage + m * kPitch + (j * 32 + l32) * 2) = bf16_rne(hv);
         }
       }
+    }
+    // the region is private to the wave: no barrier, the compiler orders the LDS accesses
+    uint16_t* h = (uint16_t*)p.out;
+    const int n0 = nb0 * 16 + wn * 64;  // first column of the wave's block
+    const int c8 = lane & 7, r8 = lane >> 3;
+#pragma unroll
+    for (int it = 0; it < 16; ++it) {
+      const int m = it * 8 + r8;
+      const uint4 v = *(const uint4*)(stage + m * kPitch + c8 * 16);
+      const int mrow = wm * 128 + m;
+      const int n = n0 + c8 * 8;
+      if (mrow < rows_here && n < p.n_blocks * 16)
+        *(uint4*)(h + (size_t)(base + tm0 + mrow) * p.out_stride + n) = v;
     }
   } else {
     float* y = (float*)p.out;
@@ -581,7 +612,7 @@ template <bool UP>
 hipError_t launch_tiled_dma(const TiledParams& p, int max_row_tiles, hipStream_t s) {
   int n_wg = max_row_tiles * p.n_col_tiles;
   n_wg = (n_wg + 7) / 8 * 8;
-  ffn_tiled_dma_kernel<UP><<<n_wg, kThreads, 0, s>>>(p);
+  ffn_tiled_pipe_kernel<UP><<<n_wg, kThreads, 0, s>>>(p);
   return hipGetLastError();
 }
 
@@ -629,7 +660,7 @@ hipError_t launch_ffn_up_tiled(const FfnArgs& a, hipStream_t s) {
   p.tile_m0 = a.tile_m0;
   p.n_tiles = a.n_tiles;
   p.n_col_tiles = (a.gate.n_pad + 127) / 128;
-  if (!int8 && p.k_pad % 128 == 0 && p.k_pad >= 256) return launch_tiled_dma<true>(p, a.max_row_tiles, s);
+  if (!int8 && p.k_pad % 64 == 0 && p.k_pad >= 128) return launch_tiled_dma<true>(p, a.max_row_tiles, s);
   return int8 ? launch_tiled<true, true>(p, a.max_row_tiles, s)
               : launch_tiled<false, true>(p, a.max_row_tiles, s);
 }
@@ -655,7 +686,7 @@ hipError_t launch_ffn_down_tiled(const FfnArgs& a, hipStream_t s) {
   p.tile_m0 = a.tile_m0;
   p.n_tiles = a.n_tiles;
   p.n_col_tiles = (a.down.n_pad + 255) / 256;
-  if (!int8 && p.k_pad % 128 == 0 && p.k_pad >= 256) return launch_tiled_dma<false>(p, a.max_row_tiles, s);
+  if (!int8 && p.k_pad % 64 == 0 && p.k_pad >= 128) return launch_tiled_dma<false>(p, a.max_row_tiles, s);
   return int8 ? launch_tiled<true, false>(p, a.max_row_tiles, s)
               : launch_tiled<false, false>(p, a.max_row_tiles, s);
 }
