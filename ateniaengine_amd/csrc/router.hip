@@ -194,6 +194,184 @@ __global__ __launch_bounds__(kRouterThreads) void router_tile_kernel(
                sWt + tls * E, sSel + tls * E, idx_out, w_out, status);
 }
 
+// Batched form of the sequential kernel for up to 64 rows.  Same arithmetic and order as
+// router_tile_kernel (one c-ascending f64 fma chain per (token, row)); what changes is how the
+// chains are fed:
+//   * a thread owns one token and RPT rows (rows rg, rg + RG, ...), so an x value read from
+//     LDS serves RPT chains and the chains of one thread hide each other's fma latency;
+//   * tiles of KC columns are converted to f64 once while they are stored to LDS, so the
+//     inner loop is ds_read_b128 (two consecutive columns) + fma only;
+//   * the global loads of tile s+1 are issued into registers before tile s is multiplied.
+template <typename XT> struct XVec;
+template <> struct XVec<float> {
+  typedef float4 type;
+  static __device__ inline float4 load(const float* p) { return *(const float4*)p; }
+  static __device__ inline void unpack(float4 v, float (&f)[4]) { f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w; }
+  static __device__ inline float4 zero() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+};
+template <> struct XVec<uint16_t> {
+  typedef uint2 type;
+  static __device__ inline uint2 load(const uint16_t* p) { return *(const uint2*)p; }
+  static __device__ inline void unpack(uint2 v, float (&f)[4]) {
+    f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+    f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+  }
+  static __device__ inline uint2 zero() { return make_uint2(0u, 0u); }
+};
+
+template <typename XT, int RPT, int KC>
+__global__ __launch_bounds__(kRouterThreads) void router_batch_kernel(
+    const XT* __restrict__ x, int T, int d, int E, int k, int renorm,
+    const float* __restrict__ w_router, const float* __restrict__ bias,
+    const float* __restrict__ gate_vec, int32_t* __restrict__ idx_out,
+    float* __restrict__ w_out, float* __restrict__ sgate_out, uint16_t* __restrict__ xb,
+    int d_pad, int32_t* __restrict__ status) {
+  constexpr int RG = 16;                   // row groups = threads per token
+  constexpr int TT = kRouterThreads / RG;  // 16 tokens per block
+  constexpr int RW = RG * RPT;             // rows of the staged weight tile (>= R)
+  constexpr int LD = KC + 2;               // f64 row stride: rows 4 banks apart, 16-byte aligned
+  constexpr int KV = KC / 4;               // 4-column vectors per tile row
+  constexpr int NX = (TT * KV + kRouterThreads - 1) / kRouterThreads;
+  constexpr int NW = (RW * KV + kRouterThreads - 1) / kRouterThreads;
+  typedef XVec<XT> XV;
+  const int R = E + (gate_vec ? 1 : 0);
+  const int t0 = blockIdx.x * TT;
+  const int tid = threadIdx.x;
+  const int tl = tid / RG, rg = tid - tl * RG;
+
+  extern __shared__ double smem_b[];
+  double* sX = smem_b;            // [TT][LD]
+  double* sW = sX + TT * LD;      // [RW][LD]
+
+  typename XV::type xr[NX];
+  float4 wr[NW];
+  auto load_tile = [&](int c0) {
+#pragma unroll
+    for (int i = 0; i < NX; ++i) {
+      const int j = tid + i * kRouterThreads;
+      const int row = j / KV, c = c0 + (j - row * KV) * 4;
+      xr[i] = XV::zero();
+      if (j < TT * KV && t0 + row < T && c < d) xr[i] = XV::load(x + (size_t)(t0 + row) * d + c);
+    }
+#pragma unroll
+    for (int i = 0; i < NW; ++i) {
+      const int j = tid + i * kRouterThreads;
+      const int row = j / KV, c = c0 + (j - row * KV) * 4;
+      wr[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (j < RW * KV && row < R && c < d)
+        wr[i] = *(const float4*)((row < E ? w_router + (size_t)row * d : gate_vec) + c);
+    }
+  };
+  auto store_tile = [&](int c0) {
+#pragma unroll
+    for (int i = 0; i < NX; ++i) {
+      const int j = tid + i * kRouterThreads;
+      if (j < TT * KV) {
+        const int row = j / KV, cl = (j - row * KV) * 4;
+        float f[4];
+        XV::unpack(xr[i], f);
+        double* dst = sX + row * LD + cl;
+        *(double2*)dst = make_double2((double)f[0], (double)f[1]);
+        *(double2*)(dst + 2) = make_double2((double)f[2], (double)f[3]);
+        const int c = c0 + cl;
+        if (xb && t0 + row < T && c < d_pad) {
+          uint2 b;
+          b.x = f32_to_bf16_rne(f[0]) | ((uint32_t)f32_to_bf16_rne(f[1]) << 16);
+          b.y = f32_to_bf16_rne(f[2]) | ((uint32_t)f32_to_bf16_rne(f[3]) << 16);
+          *(uint2*)(xb + (size_t)(t0 + row) * d_pad + c) = b;
+        }
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < NW; ++i) {
+      const int j = tid + i * kRouterThreads;
+      if (j < RW * KV) {
+        const int row = j / KV, cl = (j - row * KV) * 4;
+        double* dst = sW + row * LD + cl;
+        *(double2*)dst = make_double2((double)wr[i].x, (double)wr[i].y);
+        *(double2*)(dst + 2) = make_double2((double)wr[i].z, (double)wr[i].w);
+      }
+    }
+  };
+
+  double acc[RPT];
+#pragma unroll
+  for (int i = 0; i < RPT; ++i) acc[i] = 0.0;
+  // Columns from d up to c_end exist only to zero-fill the padding of xb; both staged tiles
+  // hold +0.0 there, which leaves every sum unchanged.
+  const int c_end = xb ? (d_pad > d ? d_pad : d) : d;
+  load_tile(0);
+  for (int c0 = 0; c0 < c_end; c0 += KC) {
+    __syncthreads();  // everyone is done reading the previous tile
+    store_tile(c0);
+    __syncthreads();
+    if (c0 + KC < c_end) load_tile(c0 + KC);
+    const double* xs = sX + tl * LD;
+    const double* ws = sW + rg * LD;
+#pragma unroll 8
+    for (int c = 0; c < KC; c += 2) {
+      const double2 xv = *(const double2*)(xs + c);
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) {
+        const double2 wv = *(const double2*)(ws + i * RG * LD + c);
+        acc[i] = fma(wv.x, xv.x, acc[i]);
+        acc[i] = fma(wv.y, xv.y, acc[i]);
+      }
+    }
+  }
+  __syncthreads();
+
+  float* sLogit = (float*)smem_b;                          // [TT][R]
+  double* sExp = smem_b + ((TT * R + 1) / 2);              // [TT][E]
+  float* sWt = (float*)(sExp + TT * E);                    // [TT][E]
+  int32_t* sSel = (int32_t*)(sWt + TT * E);                // [TT][E]
+  if (t0 + tl < T) {
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+      const int r = rg + i * RG;
+      if (r < E) {
+        float logit = (float)acc[i];
+        if (bias) logit = logit + bias[r];
+        sLogit[tl * R + r] = logit;
+      } else if (r < R) {
+        sgate_out[t0 + tl] = (float)(1.0 / (1.0 + exp(-acc[i])));
+      }
+    }
+  }
+  __syncthreads();
+  // softmax_topk shares per-token arrays between its phases, so a pass takes whole tokens:
+  // kRouterThreads / E of them (E <= 64 here); every thread makes the same number of passes.
+  const int tpp = kRouterThreads / E;
+  for (int tk0 = 0; tk0 < TT; tk0 += tpp) {
+    const int ptl = tk0 + tid / E, r = tid % E;
+    const bool on = tid < tpp * E && ptl < TT && t0 + ptl < T;
+    const int q = on ? ptl : 0;
+    softmax_topk(on, r, E, k, renorm, t0 + q, sLogit + q * R, sExp + q * E, sWt + q * E,
+                 sSel + q * E, idx_out, w_out, status);
+  }
+}
+
+template <typename XT, int RPT, int KC>
+hipError_t launch_router_batch(const RouterArgs& a, hipStream_t s) {
+  constexpr int TT = kRouterThreads / 16, RW = 16 * RPT, LD = KC + 2;
+  const int R = a.E + (a.shared_gate ? 1 : 0);
+  size_t dot_bytes = (size_t)(TT + RW) * LD * 8;
+  size_t post_bytes = (((size_t)TT * R + 1) / 2) * 8 + (size_t)TT * a.E * (8 + 4 + 4);
+  size_t smem = dot_bytes > post_bytes ? dot_bytes : post_bytes;
+  const int blocks = (a.T + TT - 1) / TT;
+  router_batch_kernel<XT, RPT, KC><<<blocks, kRouterThreads, smem, s>>>(
+      (const XT*)a.x, a.T, a.d, a.E, a.k, a.renorm, a.w_router, a.router_bias, a.shared_gate,
+      a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status);
+  return hipGetLastError();
+}
+
+template <typename XT>
+hipError_t dispatch_router_batch(const RouterArgs& a, int R, hipStream_t s) {
+  if (R <= 16) return launch_router_batch<XT, 1, 128>(a, s);
+  if (R <= 32) return launch_router_batch<XT, 2, 64>(a, s);
+  return launch_router_batch<XT, 4, 32>(a, s);
+}
+
 // Outputs of the expert grouping for the single-token case (see permute.hip for the contract).
 struct FusedGrouping {
   int32_t *counts, *offsets, *perm, *inv, *active, *n_active, *shared_offsets;
@@ -376,6 +554,10 @@ hipError_t launch_router(const RouterArgs& a, hipStream_t s, int* fused_permute)
             a.shared_gate, a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status, fg);
       return hipGetLastError();
     }
+  }
+  if (R <= 64 && a.d % 4 == 0 && (!a.xb || a.d_pad % 4 == 0)) {
+    return a.x_is_bf16 ? dispatch_router_batch<uint16_t>(a, R, s)
+                       : dispatch_router_batch<float>(a, R, s);
   }
   int TT = kRouterThreads / R;
   if (TT < 1) TT = 1;

@@ -97,6 +97,12 @@ ROUTER_CASES = [
     (5, 1, 17, 3, 0, False, False, False),
     (128, 8, 96, 50, 1, False, False, False),
     (255, 3, 40, 7, 0, False, False, False),
+    # batched sequential kernel: 2 and 4 rows per thread, row-count boundaries, ragged last block
+    (24, 3, 256, 700, 1, True, False, True),
+    (24, 3, 260, 70, 0, False, True, False),
+    (16, 2, 64, 600, 0, True, True, False),
+    (63, 5, 128, 531, 1, True, False, True),
+    (33, 2, 36, 19, 0, False, False, False),
 ]
 
 
