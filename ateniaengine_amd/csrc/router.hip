@@ -25,6 +25,8 @@
 //    exact value.  The kernel checks this per row (true for bf16-valued operands in
 //    practice); when it fails for any row of the token, the token's rows are recomputed in
 //    the reference's order.
+#include <cstdlib>
+
 #include "moe_internal.h"
 
 namespace atenia_moe {
@@ -194,14 +196,91 @@ __global__ __launch_bounds__(kRouterThreads) void router_tile_kernel(
                sWt + tls * E, sSel + tls * E, idx_out, w_out, status);
 }
 
+// Softmax + top-k + renormalisation of a block of TT tokens at once, same arithmetic and order
+// as softmax_topk.  The steps that the reference does as sequential folds over the experts
+// (f64 sum of the exponentials, f64 sum of the selected weights) are dependent chains, so one
+// thread per token runs them for all tokens of the block side by side; the element-wise steps
+// (exp, weight, rank) are spread over all threads.  lg: [TT][R] f32 logits in LDS; scratch:
+// ex [TT][E] f64, wt [TT][E] f32, sel [TT][E] u8, tok [TT] f64 (max, then 1/sum).
+__device__ inline void softmax_topk_block(int TT, int R, int E, int k, int renorm, int t0, int T,
+                                          const float* lg, double* ex, float* wt, uint8_t* sel,
+                                          double* tok, int32_t* __restrict__ idx_out,
+                                          float* __restrict__ w_out,
+                                          int32_t* __restrict__ status) {
+  const int tid = threadIdx.x, nthr = blockDim.x;
+  const int pairs = TT * E;
+  if (tid < TT) {
+    const float* l = lg + tid * R;
+    float mx = -INFINITY;
+#pragma unroll 8
+    for (int e = 0; e < E; ++e) mx = fmaxf(mx, l[e]);  // skips NaN like f32::max
+    tok[tid] = (double)mx;
+  }
+  __syncthreads();
+  for (int pr = tid; pr < pairs; pr += nthr) {
+    const int t = pr / E, e = pr - t * E;
+    ex[pr] = exp((double)(lg[t * R + e] - (float)tok[t]));  // f32 subtraction, then f64 exp
+  }
+  __syncthreads();
+  if (tid < TT) {
+    const double* x = ex + tid * E;
+    double sum = 0.0;
+#pragma unroll 8
+    for (int e = 0; e < E; ++e) sum += x[e];  // sequential fold, e ascending
+    tok[tid] = sum > 0.0 ? 1.0 / sum : 0.0;
+  }
+  __syncthreads();
+  for (int pr = tid; pr < pairs; pr += nthr) {
+    const int t = pr / E, e = pr - t * E;
+    const float w = (float)(ex[pr] * tok[t]);
+    wt[pr] = w;
+    if ((!isfinite(w) || w < 0.f) && t0 + t < T) {
+      atomicMin(&status[0], -3);
+      atomicMin(&status[1], ((t0 + t) << 10) | e);
+    }
+  }
+  __syncthreads();
+  for (int pr = tid; pr < pairs; pr += nthr) {
+    const int t = pr / E, e = pr - t * E;
+    const float* w = wt + t * E;
+    const float my_w = w[e];
+    int rank = 0;  // experts that sort before me under (weight desc, index asc)
+#pragma unroll 8
+    for (int o = 0; o < E; ++o) {
+      const float wo = w[o];
+      rank += (wo > my_w) || (wo == my_w && o < e);
+    }
+    sel[pr] = rank < k ? 1 : 0;
+  }
+  __syncthreads();
+  if (tid < TT && t0 + tid < T) {
+    const float* w = wt + tid * E;
+    const uint8_t* sl = sel + tid * E;
+    double sum = 0.0;
+#pragma unroll 8
+    for (int e = 0; e < E; ++e)
+      if (sl[e]) sum += (double)w[e];  // ascending e, as the reference sums the sorted selection
+    const double scale = renorm ? 1.0 / sum : 1.0;
+    size_t o = (size_t)(t0 + tid) * k;
+    int slot = 0;
+    for (int e = 0; e < E && slot < k; ++e) {
+      if (sl[e]) {
+        idx_out[o + slot] = e;
+        w_out[o + slot] = (float)((double)w[e] * scale);
+        ++slot;
+      }
+    }
+  }
+}
+
 // Batched form of the sequential kernel for up to 64 rows.  Same arithmetic and order as
 // router_tile_kernel (one c-ascending f64 fma chain per (token, row)); what changes is how the
 // chains are fed:
-//   * a thread owns one token and RPT rows (rows rg, rg + RG, ...), so an x value read from
-//     LDS serves RPT chains and the chains of one thread hide each other's fma latency;
+//   * a thread owns TPT tokens and RPT rows (rows rg, rg + RG, ...), so a value read from
+//     LDS serves several chains and the chains of one thread hide each other's fma latency;
 //   * tiles of KC columns are converted to f64 once while they are stored to LDS, so the
 //     inner loop is ds_read_b128 (two consecutive columns) + fma only;
-//   * the global loads of tile s+1 are issued into registers before tile s is multiplied.
+//   * the global loads of tile s+2 are issued into registers before tile s is multiplied.
 template <typename XT> struct XVec;
 template <> struct XVec<float> {
   typedef float4 type;
@@ -219,7 +298,7 @@ template <> struct XVec<uint16_t> {
   static __device__ inline uint2 zero() { return make_uint2(0u, 0u); }
 };
 
-template <typename XT, int RPT, int KC>
+template <typename XT, int RPT, int TPT, int KC>
 __global__ __launch_bounds__(kRouterThreads) void router_batch_kernel(
     const XT* __restrict__ x, int T, int d, int E, int k, int renorm,
     const float* __restrict__ w_router, const float* __restrict__ bias,
@@ -227,7 +306,8 @@ __global__ __launch_bounds__(kRouterThreads) void router_batch_kernel(
     float* __restrict__ w_out, float* __restrict__ sgate_out, uint16_t* __restrict__ xb,
     int d_pad, int32_t* __restrict__ status) {
   constexpr int RG = 16;                   // row groups = threads per token
-  constexpr int TT = kRouterThreads / RG;  // 16 tokens per block
+  constexpr int TG = kRouterThreads / RG;  // 16 token groups = threads per row group
+  constexpr int TT = TG * TPT;             // tokens per block: a thread owns tokens tg, tg + TG, ...
   constexpr int RW = RG * RPT;             // rows of the staged weight tile (>= R)
   constexpr int LD = KC + 2;               // f64 row stride: rows 4 banks apart, 16-byte aligned
   constexpr int KV = KC / 4;               // 4-column vectors per tile row
@@ -237,15 +317,14 @@ __global__ __launch_bounds__(kRouterThreads) void router_batch_kernel(
   const int R = E + (gate_vec ? 1 : 0);
   const int t0 = blockIdx.x * TT;
   const int tid = threadIdx.x;
-  const int tl = tid / RG, rg = tid - tl * RG;
+  const int tg = tid / RG, rg = tid - tg * RG;
 
   extern __shared__ double smem_b[];
   double* sX = smem_b;            // [TT][LD]
   double* sW = sX + TT * LD;      // [RW][LD]
 
-  typename XV::type xr[NX];
-  float4 wr[NW];
-  auto load_tile = [&](int c0) {
+  typedef typename XV::type xvec_t;
+  auto load_tile = [&](xvec_t (&xr)[NX], float4 (&wr)[NW], int c0) {
 #pragma unroll
     for (int i = 0; i < NX; ++i) {
       const int j = tid + i * kRouterThreads;
@@ -262,7 +341,7 @@ __global__ __launch_bounds__(kRouterThreads) void router_batch_kernel(
         wr[i] = *(const float4*)((row < E ? w_router + (size_t)row * d : gate_vec) + c);
     }
   };
-  auto store_tile = [&](int c0) {
+  auto store_tile = [&](const xvec_t (&xr)[NX], const float4 (&wr)[NW], int c0) {
 #pragma unroll
     for (int i = 0; i < NX; ++i) {
       const int j = tid + i * kRouterThreads;
@@ -294,72 +373,118 @@ __global__ __launch_bounds__(kRouterThreads) void router_batch_kernel(
     }
   };
 
-  double acc[RPT];
+  double acc[TPT][RPT];
 #pragma unroll
-  for (int i = 0; i < RPT; ++i) acc[i] = 0.0;
+  for (int j = 0; j < TPT; ++j)
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) acc[j][i] = 0.0;
   // Columns from d up to c_end exist only to zero-fill the padding of xb; both staged tiles
   // hold +0.0 there, which leaves every sum unchanged.
   const int c_end = xb ? (d_pad > d ? d_pad : d) : d;
-  load_tile(0);
-  for (int c0 = 0; c0 < c_end; c0 += KC) {
-    __syncthreads();  // everyone is done reading the previous tile
-    store_tile(c0);
-    __syncthreads();
-    if (c0 + KC < c_end) load_tile(c0 + KC);
-    const double* xs = sX + tl * LD;
+  // Two register sets: the loads of tile s+2 are issued while tile s is multiplied, so a
+  // load has two multiply phases to land before its tile is stored to LDS.
+  xvec_t xr0[NX], xr1[NX];
+  float4 wr0[NW], wr1[NW];
+  // Workgroup barrier that orders LDS traffic only.  __syncthreads() would also wait for
+  // every outstanding global load, which is exactly the latency the prefetch is there to hide.
+  auto lds_barrier = [] {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  };
+  auto step = [&](xvec_t (&xr)[NX], float4 (&wr)[NW], int c0) {
+    lds_barrier();  // everyone is done reading the previous tile
+    store_tile(xr, wr, c0);
+    lds_barrier();
+    if (c0 + 2 * KC < c_end) load_tile(xr, wr, c0 + 2 * KC);
+    // Columns are taken in groups of CG: the LDS reads of group g+1 are issued before the
+    // fma chain steps of group g (two register sets), so no read latency sits between them.
+    const double* xs = sX + tg * LD;
     const double* ws = sW + rg * LD;
-#pragma unroll 8
-    for (int c = 0; c < KC; c += 2) {
-      const double2 xv = *(const double2*)(xs + c);
+    constexpr int CG = TPT * RPT <= 4 ? 8 : 4, NV = CG / 2;
+    double2 xa[TPT][NV], wa[RPT][NV], xb2[TPT][NV], wb2[RPT][NV];
+    auto rd = [&](double2 (&xv)[TPT][NV], double2 (&wv)[RPT][NV], int c) {
 #pragma unroll
-      for (int i = 0; i < RPT; ++i) {
-        const double2 wv = *(const double2*)(ws + i * RG * LD + c);
-        acc[i] = fma(wv.x, xv.x, acc[i]);
-        acc[i] = fma(wv.y, xv.y, acc[i]);
+      for (int u = 0; u < NV; ++u) {
+#pragma unroll
+        for (int j = 0; j < TPT; ++j) xv[j][u] = *(const double2*)(xs + j * TG * LD + c + 2 * u);
+#pragma unroll
+        for (int i = 0; i < RPT; ++i) wv[i][u] = *(const double2*)(ws + i * RG * LD + c + 2 * u);
       }
+    };
+    auto mul = [&](const double2 (&xv)[TPT][NV], const double2 (&wv)[RPT][NV]) {
+#pragma unroll
+      for (int u = 0; u < NV; ++u)
+#pragma unroll
+        for (int i = 0; i < RPT; ++i)
+#pragma unroll
+          for (int j = 0; j < TPT; ++j) {
+            acc[j][i] = fma(wv[i][u].x, xv[j][u].x, acc[j][i]);
+            acc[j][i] = fma(wv[i][u].y, xv[j][u].y, acc[j][i]);
+          }
+    };
+    static_assert(KC % (2 * CG) == 0, "tile width must hold whole pairs of column groups");
+    rd(xa, wa, 0);
+    for (int c = 0; c < KC; c += 2 * CG) {
+      rd(xb2, wb2, c + CG);
+      __builtin_amdgcn_sched_barrier(0);
+      mul(xa, wa);
+      __builtin_amdgcn_sched_barrier(0);
+      if (c + 2 * CG < KC) rd(xa, wa, c + 2 * CG);
+      __builtin_amdgcn_sched_barrier(0);
+      mul(xb2, wb2);
+      __builtin_amdgcn_sched_barrier(0);
     }
+  };
+  load_tile(xr0, wr0, 0);
+  if (KC < c_end) load_tile(xr1, wr1, KC);
+  for (int c0 = 0; c0 < c_end; c0 += 2 * KC) {
+    step(xr0, wr0, c0);
+    if (c0 + KC < c_end) step(xr1, wr1, c0 + KC);
   }
   __syncthreads();
 
+  // reuse of the tile memory: logits of the block, then the softmax scratch
   float* sLogit = (float*)smem_b;                          // [TT][R]
   double* sExp = smem_b + ((TT * R + 1) / 2);              // [TT][E]
-  float* sWt = (float*)(sExp + TT * E);                    // [TT][E]
-  int32_t* sSel = (int32_t*)(sWt + TT * E);                // [TT][E]
-  if (t0 + tl < T) {
+  double* sTok = sExp + TT * E;                            // [TT]
+  float* sWt = (float*)(sTok + TT);                        // [TT][E]
+  uint8_t* sSel = (uint8_t*)(sWt + TT * E);                // [TT][E]
+#pragma unroll
+  for (int j = 0; j < TPT; ++j) {
+    const int tl = tg + j * TG;
+    if (t0 + tl >= T) continue;
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
       const int r = rg + i * RG;
       if (r < E) {
-        float logit = (float)acc[i];
+        float logit = (float)acc[j][i];
         if (bias) logit = logit + bias[r];
         sLogit[tl * R + r] = logit;
       } else if (r < R) {
-        sgate_out[t0 + tl] = (float)(1.0 / (1.0 + exp(-acc[i])));
+        sgate_out[t0 + tl] = (float)(1.0 / (1.0 + exp(-acc[j][i])));
       }
     }
   }
   __syncthreads();
-  // softmax_topk shares per-token arrays between its phases, so a pass takes whole tokens:
-  // kRouterThreads / E of them (E <= 64 here); every thread makes the same number of passes.
-  const int tpp = kRouterThreads / E;
-  for (int tk0 = 0; tk0 < TT; tk0 += tpp) {
-    const int ptl = tk0 + tid / E, r = tid % E;
-    const bool on = tid < tpp * E && ptl < TT && t0 + ptl < T;
-    const int q = on ? ptl : 0;
-    softmax_topk(on, r, E, k, renorm, t0 + q, sLogit + q * R, sExp + q * E, sWt + q * E,
-                 sSel + q * E, idx_out, w_out, status);
-  }
+  softmax_topk_block(TT, R, E, k, renorm, t0, T, sLogit, sExp, sWt, sSel, sTok, idx_out, w_out,
+                     status);
 }
 
-template <typename XT, int RPT, int KC>
+template <typename XT, int RPT, int TPT, int KC>
 hipError_t launch_router_batch(const RouterArgs& a, hipStream_t s) {
-  constexpr int TT = kRouterThreads / 16, RW = 16 * RPT, LD = KC + 2;
+  constexpr int TT = kRouterThreads / 16 * TPT, RW = 16 * RPT, LD = KC + 2;
   const int R = a.E + (a.shared_gate ? 1 : 0);
   size_t dot_bytes = (size_t)(TT + RW) * LD * 8;
-  size_t post_bytes = (((size_t)TT * R + 1) / 2) * 8 + (size_t)TT * a.E * (8 + 4 + 4);
+  size_t post_bytes = (((size_t)TT * R + 1) / 2) * 8 + (size_t)TT * a.E * (8 + 4 + 1) + TT * 8 + 16;
   size_t smem = dot_bytes > post_bytes ? dot_bytes : post_bytes;
+  static size_t attr_bytes = 0;  // per instantiation: largest size the attribute was set for
+  if (smem > 64 * 1024 && smem > attr_bytes) {
+    hipError_t e = hipFuncSetAttribute((const void*)router_batch_kernel<XT, RPT, TPT, KC>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return e;
+    attr_bytes = smem;
+  }
   const int blocks = (a.T + TT - 1) / TT;
-  router_batch_kernel<XT, RPT, KC><<<blocks, kRouterThreads, smem, s>>>(
+  router_batch_kernel<XT, RPT, TPT, KC><<<blocks, kRouterThreads, smem, s>>>(
       (const XT*)a.x, a.T, a.d, a.E, a.k, a.renorm, a.w_router, a.router_bias, a.shared_gate,
       a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status);
   return hipGetLastError();
@@ -367,9 +492,19 @@ hipError_t launch_router_batch(const RouterArgs& a, hipStream_t s) {
 
 template <typename XT>
 hipError_t dispatch_router_batch(const RouterArgs& a, int R, hipStream_t s) {
-  if (R <= 16) return launch_router_batch<XT, 1, 128>(a, s);
-  if (R <= 32) return launch_router_batch<XT, 2, 64>(a, s);
-  return launch_router_batch<XT, 4, 32>(a, s);
+  if (R <= 16) return launch_router_batch<XT, 1, 1, 128>(a, s);
+  if (R <= 32) return launch_router_batch<XT, 2, 1, 64>(a, s);
+  // Many rows and many tokens: a thread takes two tokens as well (each w value read from LDS
+  // serves two chains, eight independent f64 chains per thread) while the grid still covers
+  // the chip.
+  static const int forced = [] {
+    const char* e = getenv("ATENIA_MOE_ROUTER_TPT");  // tuning knob: tokens per thread (1, 2)
+    return e ? atoi(e) : 0;
+  }();
+  // measured on MI355X at 64 rows, d = 2048: two tokens per thread pay from 8192 tokens on
+  const int tpt = forced ? forced : (a.T >= 8192 ? 2 : 1);
+  if (tpt >= 2) return launch_router_batch<XT, 4, 2, 64>(a, s);
+  return launch_router_batch<XT, 4, 1, 64>(a, s);
 }
 
 // Outputs of the expert grouping for the single-token case (see permute.hip for the contract).
