@@ -40,6 +40,16 @@ W_BYTES = 2
 W_STD = 0.02
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, GB/s
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, TFLOP/s
+CONFIG_NAME = "mixtral_bf16"
+# HBM bytes per launch (read + written) of the expert kernels, measured with rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE and scaled by what the same counters read for a 1 GiB device copy
+# (FETCH_SIZE counts 2 KiB units, WRITE_SIZE KiB): profiles/
+# ffn_kernels_mixtral_bf16_T4096_T1_hbm_counters.txt.  Keyed by (config, tokens per step).
+MEASURED_HBM_TRAFFIC = {
+    ("mixtral_bf16", 4096): {"expert_gate_up": 2509370.3 * 2048 + 233344.0 * 1024,
+                             "expert_down": 1262427.5 * 2048 + 131072.0 * 1024},
+    ("mixtral_bf16", 1): {"expert_gate_up": 229446.8 * 2048, "expert_down": 114935.2 * 2048},
+}
 
 
 def make_weights(torch, np, seed):
@@ -131,6 +141,7 @@ def measure(torch, np, capi, layer, T, steps, warmup, seed):
         algorithmic_bytes=bytes_fwd, algorithmic_flops=flops_fwd,
     )
     up_ms, down_ms = stage_ms[2], stage_ms[3]
+    traffic = MEASURED_HBM_TRAFFIC.get((CONFIG_NAME, T))
     dom, dom_ms, dom_bytes, dom_flops = (
         ("expert_gate_up", up_ms, bytes_up, flops_up) if up_ms >= down_ms
         else ("expert_down", down_ms, bytes_down, flops_down))
@@ -139,12 +150,14 @@ def measure(torch, np, capi, layer, T, steps, warmup, seed):
     if hbm_bound:
         ach = dom_bytes / (dom_ms * 1e-3) / 1e9
         r["roofline"] = dict(bound="hbm", kernel=dom, achieved=ach, peak=PEAK_HBM_GBS,
-                             unit="GB/s", frac=ach / PEAK_HBM_GBS, traffic=None,
+                             unit="GB/s", frac=ach / PEAK_HBM_GBS,
+                             traffic=traffic.get(dom) if traffic else None,
                              kernel_ms=float(dom_ms), algorithmic_bytes=dom_bytes)
     else:
         ach = dom_flops / (dom_ms * 1e-3) / 1e12
         r["roofline"] = dict(bound="mfma", kernel=dom, achieved=ach, peak=PEAK_BF16_TFLOPS,
-                             unit="TFLOP/s", frac=ach / PEAK_BF16_TFLOPS, traffic=None,
+                             unit="TFLOP/s", frac=ach / PEAK_BF16_TFLOPS,
+                             traffic=traffic.get(dom) if traffic else None,
                              kernel_ms=float(dom_ms), algorithmic_flops=dom_flops)
     return r, xs[0], out
 
@@ -180,8 +193,9 @@ def main():
         print("bench.py: no gfx950 device; the HIP path has no fallback", file=sys.stderr)
         sys.exit(3)
     torch.cuda.set_device(0)
-    global D_MODEL, N_EXPERTS, TOP_K, D_FF, D_FF_SHARED, W_BYTES
+    global D_MODEL, N_EXPERTS, TOP_K, D_FF, D_FF_SHARED, W_BYTES, CONFIG_NAME
     cfg = CONFIGS[a.config]
+    CONFIG_NAME = a.config
     D_MODEL, N_EXPERTS, TOP_K, D_FF, D_FF_SHARED = cfg["d"], cfg["E"], cfg["k"], cfg["f"], cfg["fs"]
     W_BYTES = 1 if cfg["wd"] == "int8" else 2
     if a.tokens <= 0:
