@@ -608,6 +608,266 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p)
   }
 }
 
+// ---- INT8 W8A16 form of the pipelined kernel -----------------------------------------------
+// Same tiling, A ring and k16-unit pipeline.  Weights stay int8 all the way into LDS: a B stage
+// is 64 k = 16 stored blocks (16 KiB, one load instruction per block), so there is one barrier
+// per 64 k.  A lane reads its 8 int8 of a fragment with one ds_read_b64 and widens them to
+// bf16 in registers (exact: |q| <= 127) between the MFMAs of the unit before; the per-row scale
+// multiplies the f32 accumulator in the epilogue.
+__device__ inline void widen_i8x4(uint32_t w, uint32_t& lo, uint32_t& hi) {
+  const float f0 = (float)(int8_t)(w & 0xff), f1 = (float)(int8_t)((w >> 8) & 0xff);
+  const float f2 = (float)(int8_t)((w >> 16) & 0xff), f3 = (float)(int8_t)(w >> 24);
+  // bf16 pair = high halves of two f32
+  lo = __builtin_amdgcn_perm(__float_as_uint(f1), __float_as_uint(f0), 0x07060302u);
+  hi = __builtin_amdgcn_perm(__float_as_uint(f3), __float_as_uint(f2), 0x07060302u);
+}
+
+template <bool UP>
+__global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_i8_kernel(TiledParams p) {
+  constexpr int NA = kRingA, NB = 4;          // 64-k stages: A 32 KiB, B 16 KiB
+  __shared__ uint4 S[NA * 2048 + NB * 1024];  // A ring, then B ring
+  int rt, ct;
+  if (!tile_of_workgroup(p, rt, ct)) return;
+
+  const int e = p.tile_group[rt];
+  const int tm0 = p.tile_m0[rt];
+  const int base = p.g.offsets[e];
+  const int cnt = p.g.offsets[e + 1] - base;
+  const int rows_here = min(TM, cnt - tm0);
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int kh = lane >> 5, l32 = lane & 31;
+  const int wm = wave >> 1, wn = wave & 1;
+  constexpr int BROWS = UP ? 128 : 256;
+  const int nb0 = ct * (BROWS / 16);
+
+  const uint16_t* arow[8];  // as in the bf16 kernel
+  {
+    const int r8 = lane >> 3, pslot = lane & 7;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      int m = (wave * 8 + q) * 8 + r8;
+      if (m >= rows_here) m = 0;
+      int src;
+      if (UP) src = p.g.perm[base + tm0 + m] / p.g.pair_div;
+      else src = base + tm0 + m;
+      arow[q] = p.a + (size_t)src * p.a_stride + (pslot ^ r8 ^ (q & 1)) * 8;
+    }
+  }
+  // B: LDS chunk c of a stage holds the stored block of strip c (gate/up: chunks 0-7 gate
+  // strips, 8-15 the matching up strips); wave w fills chunks 4w .. 4w+3.
+  const uint4* bptr[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int c = wave * 4 + q;
+    const uint4* wbase = (UP && c >= 8) ? p.wb : p.wa;
+    int nb = nb0 + (UP ? (c & 7) : c);
+    if (nb >= p.n_blocks) nb = p.n_blocks - 1;  // clamp: columns past N are never stored
+    bptr[q] = wbase + (size_t)e * p.w_stride_u4 + (size_t)nb * p.nkb * 64 + lane;
+  }
+  int aoff[4];
+  {
+    const int r8 = l32 & 7, cpar = (l32 >> 3) & 1;
+    const int rowbase = (wm * 16 + (l32 >> 3)) * 64 + r8 * 8;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) aoff[u] = rowbase + ((2 * u + kh) ^ r8 ^ cpar);
+  }
+  // B fragment j, k16 unit u, in 8-byte units: strip (2 * group + l32/16), slot 16u + l32%16 of
+  // the block, half kh of the slot.
+  const uint2* S2 = (const uint2*)S;
+  const int boff0 = NA * 4096 + ((UP ? 2 * wn : 4 * wn) * 2 + (l32 >> 4)) * 128 + (l32 & 15) * 2 + kh;
+  constexpr int kBJ1 = 256, kBJ2 = UP ? 1024 : 512, kBJ3 = UP ? 1280 : 768;
+
+  f32x16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  const int my_rows = rows_here - wm * 128;
+  const int nst = p.k_pad / 64;
+
+  const uint32_t sa_fill = (uint32_t)(uintptr_t)(lptr_t)S + wave * 8 * kChunk;
+  const uint32_t sb_fill = (uint32_t)(uintptr_t)(lptr_t)S + NA * 32768 + wave * 4 * kChunk;
+  auto dma_a = [&](int buf, int q, int t) {
+    dma16(arow[q] + (size_t)t * 64, sa_fill + buf * 32768 + q * kChunk);
+  };
+  auto dma_b = [&](int buf, int q, int t) {
+    dma16(bptr[q] + (size_t)t * 64, sb_fill + buf * 16384 + q * kChunk);
+  };
+  auto read_frag = [&](int n, uint4 (&FA)[4], uint2 (&RB)[4], int a0, int b0) {
+    switch (n) {
+      case 0: FA[0] = S[a0]; break;
+      case 1: RB[0] = S2[b0]; break;
+      case 2: RB[1] = S2[b0 + kBJ1]; break;
+      case 3: RB[2] = S2[b0 + kBJ2]; break;
+      case 4: RB[3] = S2[b0 + kBJ3]; break;
+      case 5: FA[1] = S[a0 + 256]; break;
+      case 6: FA[2] = S[a0 + 512]; break;
+      default: FA[3] = S[a0 + 768]; break;
+    }
+  };
+  auto widen_half = [&](int n, const uint2 (&RB)[4], uint4 (&FB)[4]) {  // n = 2 * fragment + half
+    if (n & 1) widen_i8x4(RB[n >> 1].y, FB[n >> 1].z, FB[n >> 1].w);
+    else widen_i8x4(RB[n >> 1].x, FB[n >> 1].x, FB[n >> 1].y);
+  };
+  // One k16 unit: 16 MFMAs on (FA, FB).  Behind MFMA m < 8: read m of the next unit (B raw);
+  // behind MFMA m >= 8: half a B fragment of the next unit is widened, and on even m a load
+  // of the stage being refilled is issued (A: four per unit, B: two per unit).
+  auto half = [&](auto mul_c, auto dma_c, auto dma_is_a_c, uint4 (&FA)[4], uint4 (&FB)[4],
+                  uint4 (&NA_)[4], uint4 (&NB_)[4], int a0, int b0, int dbuf, int dt, auto q0_c) {
+    constexpr int MUL = decltype(mul_c)::value;
+    uint2 raw[4];
+#pragma unroll
+    for (int m = 0; m < 16; ++m) {
+      const int i = m >> 2, j = m & 3;
+      if (MUL == 2 || (MUL == 1 && i * 32 < my_rows)) acc[i][j] = mfma32(FA[i], FB[j], acc[i][j]);
+      if (m < 8) read_frag(m, NA_, raw, a0, b0);
+      else widen_half(m - 8, raw, NB_);
+      if (decltype(dma_c)::value && m >= 8 && (m & 1) == 0) {
+        if (decltype(dma_is_a_c)::value) dma_a(dbuf, decltype(q0_c)::value + ((m - 8) >> 1), dt);
+        else if (m < 12) dma_b(dbuf, decltype(q0_c)::value + ((m - 8) >> 1), dt);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  using std::integral_constant;
+  typedef integral_constant<bool, true> yes;
+  typedef integral_constant<bool, false> no;
+
+  // Iteration t (64 k) = units 0..3 of stage t.  Loads issued: unit 0: first half of A(t+2),
+  // unit 1: first half of B(t+3), unit 2: second half of A(t+2), unit 3 (behind the barrier):
+  // second half of B(t+3).  The barrier sits between units 2 and 3: by then this wave has
+  // read all of stage t except unit 3 (already in registers), and waits for its loads of
+  // stage t+1; younger loads then in flight: A(t+2) (8) and half of B(t+2), B(t+3) (2 + 2).
+  auto run = [&](auto mul_c, auto la_c) {
+    constexpr bool LA = decltype(la_c)::value;
+    typedef integral_constant<int, 0> q0;
+    typedef integral_constant<int, 2> q2;
+    typedef integral_constant<int, 4> q4;
+    uint4 fa0[4], fb0[4], fa1[4], fb1[4];
+    auto fill_a = [&](int t) {
+      if (LA) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) dma_a(t, q, min(t, nst - 1));
+      }
+    };
+    auto fill_b = [&](int t) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) dma_b(t, q, min(t, nst - 1));
+    };
+    fill_a(0); fill_b(0); fill_b(1); fill_a(1); fill_b(2);
+    wait_vm_lgkm0<LA ? 16 : 8>();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    {
+      uint2 raw[4];
+#pragma unroll
+      for (int n = 0; n < 8; ++n) read_frag(n, fa0, raw, aoff[0], boff0);
+#pragma unroll
+      for (int n = 0; n < 8; ++n) widen_half(n, raw, fb0);
+    }
+    int abuf = 0, bbuf = 0;
+    for (int t = 0; t < nst; ++t) {
+      const int abuf_n = abuf + 1 == NA ? 0 : abuf + 1;
+      const int abuf_i = abuf == 0 ? NA - 1 : abuf - 1;
+      const int bbuf_n = bbuf + 1 == NB ? 0 : bbuf + 1;
+      const int bbuf_i = bbuf == 0 ? NB - 1 : bbuf - 1;
+      const int ta = min(t + NA - 1, nst - 1), tb = min(t + NB - 1, nst - 1);
+      const int a_cur = abuf * 2048, b_cur = boff0 + bbuf * 2048;
+      half(mul_c, la_c, yes{}, fa0, fb0, fa1, fb1, aoff[1] + a_cur, b_cur + 32, abuf_i, ta, q0{});
+      half(mul_c, yes{}, no{}, fa1, fb1, fa0, fb0, aoff[2] + a_cur, b_cur + 64, bbuf_i, tb, q0{});
+      half(mul_c, la_c, yes{}, fa0, fb0, fa1, fb1, aoff[3] + a_cur, b_cur + 96, abuf_i, ta, q4{});
+      wait_vm_lgkm0<LA ? 12 : 6>();
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      half(mul_c, yes{}, no{}, fa1, fb1, fa0, fb0, aoff[0] + abuf_n * 2048, boff0 + bbuf_n * 2048,
+           bbuf_i, tb, q2{});
+      abuf = abuf_n;
+      bbuf = bbuf_n;
+    }
+    wait_vm_lgkm0<0>();
+  };
+  const bool loads_a = wave * 64 < rows_here;
+  if (my_rows >= 97) run(integral_constant<int, 2>{}, yes{});
+  else if (my_rows > 0) {
+    if (loads_a) run(integral_constant<int, 1>{}, yes{});
+    else run(integral_constant<int, 1>{}, no{});
+  } else {
+    if (loads_a) run(integral_constant<int, 0>{}, yes{});
+    else run(integral_constant<int, 0>{}, no{});
+  }
+
+  if (UP) {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();  // every wave's loads have landed and its reads are done
+    asm volatile("" ::: "memory");
+    constexpr int kPitch = 144;
+    char* stage = (char*)S + wave * (128 * kPitch);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int n = min(nb0 * 16 + (2 * wn + j) * 32 + l32, p.n_rows - 1);
+      const float sg = p.sa[(size_t)e * p.n_rows + n], su = p.sb[(size_t)e * p.n_rows + n];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = i * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
+          const float g = acc[i][j][r] * sg;
+          const float u = acc[i][j + 2][r] * su;
+          const float hv = g * __builtin_amdgcn_rcpf(1.f + __expf(-g)) * u;
+          *(uint16_t*)(stage + m * kPitch + (j * 32 + l32) * 2) = bf16_rne(hv);
+        }
+      }
+    }
+    uint16_t* h = (uint16_t*)p.out;
+    const int n0 = nb0 * 16 + wn * 64;
+    const int c8 = lane & 7, r8 = lane >> 3;
+#pragma unroll
+    for (int it = 0; it < 16; ++it) {
+      const int m = it * 8 + r8;
+      const uint4 v = *(const uint4*)(stage + m * kPitch + c8 * 16);
+      const int mrow = wm * 128 + m;
+      const int n = n0 + c8 * 8;
+      if (mrow < rows_here && n < p.n_blocks * 16)
+        *(uint4*)(h + (size_t)(base + tm0 + mrow) * p.out_stride + n) = v;
+    }
+  } else {
+    float* y = (float*)p.out;
+    float sd[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      sd[j] = p.sa[(size_t)e * p.n_rows + min(nb0 * 16 + (4 * wn + j) * 32 + l32, p.n_rows - 1)];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = wm * 128 + i * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
+        if (m >= rows_here) continue;
+        const int pair = p.g.perm[base + tm0 + m];
+        float* yr = y + (size_t)pair * p.out_stride;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int n = nb0 * 16 + (4 * wn + j) * 32 + l32;
+          if (n < p.n_rows) yr[n] = acc[i][j][r] * sd[j];
+        }
+      }
+    }
+  }
+}
+
+template <bool UP>
+hipError_t launch_tiled_pipe_i8(const TiledParams& p, int max_row_tiles, hipStream_t s) {
+  int n_wg = max_row_tiles * p.n_col_tiles;
+  n_wg = (n_wg + 7) / 8 * 8;
+  ffn_tiled_pipe_i8_kernel<UP><<<n_wg, kThreads, 0, s>>>(p);
+  return hipGetLastError();
+}
+
 template <bool UP>
 hipError_t launch_tiled_dma(const TiledParams& p, int max_row_tiles, hipStream_t s) {
   int n_wg = max_row_tiles * p.n_col_tiles;
@@ -661,6 +921,7 @@ hipError_t launch_ffn_up_tiled(const FfnArgs& a, hipStream_t s) {
   p.n_tiles = a.n_tiles;
   p.n_col_tiles = (a.gate.n_pad + 127) / 128;
   if (!int8 && p.k_pad % 64 == 0 && p.k_pad >= 128) return launch_tiled_dma<true>(p, a.max_row_tiles, s);
+  if (int8 && p.k_pad >= 128) return launch_tiled_pipe_i8<true>(p, a.max_row_tiles, s);
   return int8 ? launch_tiled<true, true>(p, a.max_row_tiles, s)
               : launch_tiled<false, true>(p, a.max_row_tiles, s);
 }
@@ -687,6 +948,7 @@ hipError_t launch_ffn_down_tiled(const FfnArgs& a, hipStream_t s) {
   p.n_tiles = a.n_tiles;
   p.n_col_tiles = (a.down.n_pad + 255) / 256;
   if (!int8 && p.k_pad % 64 == 0 && p.k_pad >= 128) return launch_tiled_dma<false>(p, a.max_row_tiles, s);
+  if (int8 && p.k_pad >= 128) return launch_tiled_pipe_i8<false>(p, a.max_row_tiles, s);
   return int8 ? launch_tiled<true, false>(p, a.max_row_tiles, s)
               : launch_tiled<false, false>(p, a.max_row_tiles, s);
 }
