@@ -5,7 +5,9 @@
 // The reference multiplies and adds in f32 with two roundings and a fixed order; the same
 // sequence is kept here (no fused multiply-add, no atomics), so given equal expert outputs
 // the combine is bit-identical.  Expert outputs are stored by pair id t*k+slot, so a token's
-// k rows are adjacent and every read and write is a coalesced float4.
+// k rows are adjacent and every read and write is a coalesced float4.  When the down phase
+// split the k range of some tiles, an expert output there is the f32 sum of its partial
+// buffers, added in buffer order.
 #include "moe_internal.h"
 
 namespace atenia_moe {
@@ -15,6 +17,8 @@ namespace {
 __global__ __launch_bounds__(256) void combine_kernel(int T, int k, int d,
                                                       const float* __restrict__ w,
                                                       const float* __restrict__ y, int y_stride,
+                                                      const uint8_t* __restrict__ part_flags,
+                                                      int flag_cols, size_t y_part_stride,
                                                       const float* __restrict__ y_shared,
                                                       const float* __restrict__ sgate,
                                                       float* __restrict__ out) {
@@ -27,12 +31,21 @@ __global__ __launch_bounds__(256) void combine_kernel(int T, int k, int d,
   for (int slot = 0; slot < k; ++slot) {
     const float ws = w[(size_t)t * k + slot];
     const float* yr = y + ((size_t)t * k + slot) * y_stride + c;
+    const int y_parts = part_flags ? part_flags[((size_t)t * k + slot) * flag_cols + c / 256] : 1;
     float v[4] = {0.f, 0.f, 0.f, 0.f};
     if (vec) {
       float4 q = *(const float4*)yr;
       v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+      for (int part = 1; part < y_parts; ++part) {
+        q = *(const float4*)(yr + part * y_part_stride);
+        v[0] = __fadd_rn(v[0], q.x); v[1] = __fadd_rn(v[1], q.y);
+        v[2] = __fadd_rn(v[2], q.z); v[3] = __fadd_rn(v[3], q.w);
+      }
     } else {
-      for (int j = 0; j < 4 && c + j < d; ++j) v[j] = yr[j];
+      for (int j = 0; j < 4 && c + j < d; ++j) {
+        v[j] = yr[j];
+        for (int part = 1; part < y_parts; ++part) v[j] = __fadd_rn(v[j], yr[part * y_part_stride + j]);
+      }
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) o[j] = __fadd_rn(o[j], __fmul_rn(ws, v[j]));
@@ -62,8 +75,8 @@ __global__ __launch_bounds__(256) void combine_kernel(int T, int k, int d,
 
 hipError_t launch_combine(const CombineArgs& a, hipStream_t s) {
   const unsigned grid = (unsigned)((a.d + 1023) / 1024) * (unsigned)a.T;
-  combine_kernel<<<grid, 256, 0, s>>>(a.T, a.k, a.d, a.w, a.y, a.y_stride, a.y_shared, a.sgate,
-                                      a.out);
+  combine_kernel<<<grid, 256, 0, s>>>(a.T, a.k, a.d, a.w, a.y, a.y_stride, a.part_flags, a.flag_cols,
+                                      a.y_part_stride, a.y_shared, a.sgate, a.out);
   return hipGetLastError();
 }
 

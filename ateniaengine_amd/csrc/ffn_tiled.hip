@@ -61,6 +61,14 @@ struct TiledParams {
   const int32_t* tile_m0;     // [n_tiles] first row (relative to the group) of each row tile
   const int32_t* n_tiles;     // [1]
   int n_col_tiles;
+  // k split of the tail tiles (pipelined down kernels; max_parts <= 1: off).  Workgroup ids
+  // below wg_upper are the tiles themselves, ids from wg_upper on the extra k ranges of the
+  // tiles in the last, partly filled round over the n_cus compute units.
+  int max_parts;
+  int wg_upper;
+  int n_cus;
+  size_t out_part_stride;     // elements between the partial output buffers
+  uint8_t* part_flags;        // [pairs, n_col_tiles] partial buffers written per (row, column tile)
 };
 
 __device__ inline uint16_t bf16_rne(float f) {
@@ -98,13 +106,13 @@ __device__ inline f32x4 mfma(uint4 a, uint4 b, f32x4 c) {
 // (all row tiles of the expert) x (8 column tiles): the ~32 workgroups an XCD runs at a time
 // share ~4 activation tiles and 8 weight tiles instead of streaming 64 different ones.
 constexpr int kColGroup = 8;
-__device__ inline bool tile_of_workgroup(const TiledParams& p, int& rt, int& ct) {
+__device__ inline bool tile_of_workgroup(const TiledParams& p, int wid, int& rt, int& ct) {
   const int n_row_tiles = *p.n_tiles;
   const int nct = p.n_col_tiles;
   const int total = n_row_tiles * nct;
   const int per_xcd = (total + 7) / 8;
-  const int slot = blockIdx.x / 8;
-  const int logical = (blockIdx.x % 8) * per_xcd + slot;
+  const int slot = wid / 8;
+  const int logical = (wid % 8) * per_xcd + slot;
   if (slot >= per_xcd || logical >= total) return false;
   // Row tiles are sorted by expert, so the expert owning this logical id is the expert of
   // row tile logical / nct; that tile's m0 tells where the expert's tiles start.
@@ -132,11 +140,44 @@ __device__ inline bool tile_of_workgroup(const TiledParams& p, int& rt, int& ct)
   return true;
 }
 
+// Tail split of the down phase.  With one workgroup per CU at a time, tiles run in rounds of
+// n_cus; when the last round is at most half full, each of its tiles is cut into S k ranges
+// (S <= max_parts) so that the round fills the chip and lasts 1/S as long.  Range 0 is
+// computed by the tile's own workgroup, ranges 1..S-1 by workgroups with ids from wg_upper on;
+// range i writes its partial sums to buffer i, and range 0 records S per (row, column tile) so
+// that the combine adds up exactly the buffers that were written.  Sets wid (the tile's
+// workgroup id for tile_of_workgroup), S and part; false = nothing to do.
+__device__ inline bool split_of_workgroup(const TiledParams& p, int n_stages, int& wid, int& S,
+                                          int& part) {
+  wid = blockIdx.x;
+  S = 1;
+  part = 0;
+  if (p.max_parts <= 1) return true;
+  const int total = *p.n_tiles * p.n_col_tiles;
+  const int per_xcd = (total + 7) / 8;
+  const int full_slots = (total / p.n_cus) * (p.n_cus / 8);  // slots per XCD in the full rounds
+  const int tail = 8 * (per_xcd - full_slots);               // tile slots of the last round
+  int s_tail = 1;
+  if (tail > 0 && 2 * tail <= p.n_cus) s_tail = min(min(p.max_parts, p.n_cus / tail), n_stages / 2);
+  if (s_tail < 1) s_tail = 1;
+  if ((int)blockIdx.x >= p.wg_upper) {
+    const int x = blockIdx.x - p.wg_upper;
+    if (s_tail == 1 || x >= tail * (s_tail - 1)) return false;
+    part = 1 + x / tail;
+    const int j = x - (part - 1) * tail;
+    wid = (full_slots + j / 8) * 8 + (j & 7);
+    S = s_tail;
+    return true;
+  }
+  if (wid / 8 >= full_slots) S = s_tail;
+  return true;
+}
+
 template <bool INT8, bool UP>
 __global__ __launch_bounds__(kThreads) void ffn_tiled_kernel(TiledParams p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   int rt, ct;
-  if (!tile_of_workgroup(p, rt, ct)) return;
+  if (!tile_of_workgroup(p, blockIdx.x, rt, ct)) return;
 
   const int e = p.tile_group[rt];
   const int tm0 = p.tile_m0[rt];
@@ -359,8 +400,10 @@ template <bool UP>
 __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p) {
   constexpr int NA = kRingA, NB = kRingB;
   __shared__ uint4 S[NA * 2048 + NB * 1024];  // A ring, then B ring
+  int wid, n_parts, part;  // k range `part` of `n_parts` (1 unless this is a split tail tile)
+  if (!split_of_workgroup(p, p.k_pad / 64, wid, n_parts, part)) return;
   int rt, ct;
-  if (!tile_of_workgroup(p, rt, ct)) return;
+  if (!tile_of_workgroup(p, wid, rt, ct)) return;
 
   const int e = p.tile_group[rt];
   const int tm0 = p.tile_m0[rt];
@@ -429,15 +472,17 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
   const int my_rows = rows_here - wm * 128;
-  const int nks = p.k_pad / 32;
+  const int st_lo = (p.k_pad / 64) * part / n_parts, st_hi = (p.k_pad / 64) * (part + 1) / n_parts;
+  const int nks = 2 * (st_hi - st_lo);  // 32-k steps of this workgroup's k range
+  const int ks0 = 2 * st_lo;
 
   const uint32_t sa_fill = (uint32_t)(uintptr_t)(lptr_t)S + wave * 8 * kChunk;
   const uint32_t sb_fill = (uint32_t)(uintptr_t)(lptr_t)S + NA * 32768 + wave * 4 * kChunk;
   auto dma_a = [&](int buf, int q, int t) {  // chunk q of this wave, 64-k stage t
-    dma16(arow[q] + (size_t)t * 64, sa_fill + buf * 32768 + q * kChunk);
+    dma16(arow[q] + (size_t)(ks0 / 2 + t) * 64, sa_fill + buf * 32768 + q * kChunk);
   };
   auto dma_b = [&](int buf, int q, int ks) {  // q = 2 * row group + k half
-    dma16(bptr[q >> 1] + (size_t)ks * 64 + 32 * (q & 1), sb_fill + buf * 16384 + q * kChunk);
+    dma16(bptr[q >> 1] + (size_t)(ks0 + ks) * 64 + 32 * (q & 1), sb_fill + buf * 16384 + q * kChunk);
   };
   // the 8 fragment reads of one k16 unit, in the order the MFMAs consume them
   auto read_frag = [&](int n, uint4 (&FA)[4], uint4 (&FB)[4], int a0, int b0) {
@@ -492,12 +537,12 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p)
     auto fill_a = [&](int t) {
       if (LA) {
 #pragma unroll
-        for (int q = 0; q < 8; ++q) dma_a(t, q, t);
+        for (int q = 0; q < 8; ++q) dma_a(t, q, min(t, nst - 1));
       }
     };
     auto fill_b = [&](int t) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) dma_b(t, q, t);
+      for (int q = 0; q < 4; ++q) dma_b(t, q, min(t, nks - 1));
     };
     // issue order A0 B0 B1 A1 B2 B3, then per step: half of A(s/2 + 2), B(s + 4)
     fill_a(0); fill_b(0); fill_b(1); fill_a(1); fill_b(2); fill_b(3);
@@ -589,7 +634,7 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p)
         *(uint4*)(h + (size_t)(base + tm0 + mrow) * p.out_stride + n) = v;
     }
   } else {
-    float* y = (float*)p.out;
+    float* y = (float*)p.out + (size_t)part * p.out_part_stride;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
 #pragma unroll
@@ -597,6 +642,8 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p)
         const int m = wm * 128 + i * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
         if (m >= rows_here) continue;
         const int pair = p.g.perm[base + tm0 + m];
+        if (p.part_flags && part == 0 && wn == 0 && l32 == 0)
+          p.part_flags[(size_t)pair * p.n_col_tiles + ct] = (uint8_t)n_parts;
         float* yr = y + (size_t)pair * p.out_stride;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -626,8 +673,10 @@ template <bool UP>
 __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_i8_kernel(TiledParams p) {
   constexpr int NA = kRingA, NB = 4;          // 64-k stages: A 32 KiB, B 16 KiB
   __shared__ uint4 S[NA * 2048 + NB * 1024];  // A ring, then B ring
+  int wid, n_parts, part;  // k range `part` of `n_parts` (1 unless this is a split tail tile)
+  if (!split_of_workgroup(p, p.k_pad / 64, wid, n_parts, part)) return;
   int rt, ct;
-  if (!tile_of_workgroup(p, rt, ct)) return;
+  if (!tile_of_workgroup(p, wid, rt, ct)) return;
 
   const int e = p.tile_group[rt];
   const int tm0 = p.tile_m0[rt];
@@ -687,15 +736,16 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_i8_kernel(TiledParams
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
   const int my_rows = rows_here - wm * 128;
-  const int nst = p.k_pad / 64;
+  const int st0 = (p.k_pad / 64) * part / n_parts;
+  const int nst = (p.k_pad / 64) * (part + 1) / n_parts - st0;  // 64-k stages of this k range
 
   const uint32_t sa_fill = (uint32_t)(uintptr_t)(lptr_t)S + wave * 8 * kChunk;
   const uint32_t sb_fill = (uint32_t)(uintptr_t)(lptr_t)S + NA * 32768 + wave * 4 * kChunk;
   auto dma_a = [&](int buf, int q, int t) {
-    dma16(arow[q] + (size_t)t * 64, sa_fill + buf * 32768 + q * kChunk);
+    dma16(arow[q] + (size_t)(st0 + t) * 64, sa_fill + buf * 32768 + q * kChunk);
   };
   auto dma_b = [&](int buf, int q, int t) {
-    dma16(bptr[q] + (size_t)t * 64, sb_fill + buf * 16384 + q * kChunk);
+    dma16(bptr[q] + (size_t)(st0 + t) * 64, sb_fill + buf * 16384 + q * kChunk);
   };
   auto read_frag = [&](int n, uint4 (&FA)[4], uint2 (&RB)[4], int a0, int b0) {
     switch (n) {
@@ -837,7 +887,7 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_i8_kernel(TiledParams
         *(uint4*)(h + (size_t)(base + tm0 + mrow) * p.out_stride + n) = v;
     }
   } else {
-    float* y = (float*)p.out;
+    float* y = (float*)p.out + (size_t)part * p.out_part_stride;
     float sd[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
@@ -849,6 +899,8 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_i8_kernel(TiledParams
         const int m = wm * 128 + i * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
         if (m >= rows_here) continue;
         const int pair = p.g.perm[base + tm0 + m];
+        if (p.part_flags && part == 0 && wn == 0 && l32 == 0)
+          p.part_flags[(size_t)pair * p.n_col_tiles + ct] = (uint8_t)n_parts;
         float* yr = y + (size_t)pair * p.out_stride;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -861,18 +913,22 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_i8_kernel(TiledParams
 }
 
 template <bool UP>
-hipError_t launch_tiled_pipe_i8(const TiledParams& p, int max_row_tiles, hipStream_t s) {
+hipError_t launch_tiled_pipe_i8(TiledParams p, int max_row_tiles, hipStream_t s) {
   int n_wg = max_row_tiles * p.n_col_tiles;
   n_wg = (n_wg + 7) / 8 * 8;
-  ffn_tiled_pipe_i8_kernel<UP><<<n_wg, kThreads, 0, s>>>(p);
+  p.wg_upper = n_wg;
+  const int extra = p.max_parts > 1 ? p.n_cus : 0;  // room for the extra k ranges of a tail round
+  ffn_tiled_pipe_i8_kernel<UP><<<n_wg + extra, kThreads, 0, s>>>(p);
   return hipGetLastError();
 }
 
 template <bool UP>
-hipError_t launch_tiled_dma(const TiledParams& p, int max_row_tiles, hipStream_t s) {
+hipError_t launch_tiled_dma(TiledParams p, int max_row_tiles, hipStream_t s) {
   int n_wg = max_row_tiles * p.n_col_tiles;
   n_wg = (n_wg + 7) / 8 * 8;
-  ffn_tiled_pipe_kernel<UP><<<n_wg, kThreads, 0, s>>>(p);
+  p.wg_upper = n_wg;
+  const int extra = p.max_parts > 1 ? p.n_cus : 0;  // room for the extra k ranges of a tail round
+  ffn_tiled_pipe_kernel<UP><<<n_wg + extra, kThreads, 0, s>>>(p);
   return hipGetLastError();
 }
 
@@ -893,6 +949,12 @@ hipError_t launch_tiled(const TiledParams& p, int max_row_tiles, hipStream_t s) 
 }
 
 }  // namespace
+
+bool tiled_down_splits_tail(const WeightSet& down, int wdtype) {
+  if (wdtype == ATENIA_MOE_WEIGHT_F32) return false;
+  const bool int8 = wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
+  return int8 ? down.k_pad >= 128 : (down.k_pad % 64 == 0 && down.k_pad >= 128);
+}
 
 bool tiled_supported(const WeightSet& w, int wdtype) {
   if (wdtype == ATENIA_MOE_WEIGHT_F32) return false;
@@ -920,6 +982,7 @@ hipError_t launch_ffn_up_tiled(const FfnArgs& a, hipStream_t s) {
   p.tile_m0 = a.tile_m0;
   p.n_tiles = a.n_tiles;
   p.n_col_tiles = (a.gate.n_pad + 127) / 128;
+  p.max_parts = 1;
   if (!int8 && p.k_pad % 64 == 0 && p.k_pad >= 128) return launch_tiled_dma<true>(p, a.max_row_tiles, s);
   if (int8 && p.k_pad >= 128) return launch_tiled_pipe_i8<true>(p, a.max_row_tiles, s);
   return int8 ? launch_tiled<true, true>(p, a.max_row_tiles, s)
@@ -947,6 +1010,14 @@ hipError_t launch_ffn_down_tiled(const FfnArgs& a, hipStream_t s) {
   p.tile_m0 = a.tile_m0;
   p.n_tiles = a.n_tiles;
   p.n_col_tiles = (a.down.n_pad + 255) / 256;
+  p.max_parts = 1;
+  const bool pipelined = int8 ? p.k_pad >= 128 : (p.k_pad % 64 == 0 && p.k_pad >= 128);
+  if (pipelined && a.y_parts > 1 && a.part_flags && a.n_cus >= 8) {
+    p.max_parts = a.y_parts;
+    p.n_cus = a.n_cus / 8 * 8;
+    p.out_part_stride = a.y_part_stride;
+    p.part_flags = a.part_flags;
+  }
   if (!int8 && p.k_pad % 64 == 0 && p.k_pad >= 128) return launch_tiled_dma<false>(p, a.max_row_tiles, s);
   if (int8 && p.k_pad >= 128) return launch_tiled_pipe_i8<false>(p, a.max_row_tiles, s);
   return int8 ? launch_tiled<true, false>(p, a.max_row_tiles, s)

@@ -93,8 +93,10 @@ struct AteniaMoeLayer {
   // workspace (grow-only in tokens)
   int cap_tokens = 0;
   DevBuf x_in, out, xb, idx, w, sgate, counts, offsets, active, n_active, perm, inv, blk_counts,
-      shared_desc, ident, h, hs, y, ys, status, tile_group, tile_m0, s_tile_group, s_tile_m0;
+      shared_desc, ident, h, hs, y, ys, status, tile_group, tile_m0, s_tile_group, s_tile_m0,
+      part_flags;
   int last_T = 0;
+  bool last_split = false;  // the last forward's down phase may have split tail tiles
 
   hipStream_t stream = nullptr;
   std::mutex mu;
@@ -106,6 +108,20 @@ struct AteniaMoeLayer {
 };
 
 namespace {
+
+// Compute units of the current device (read once per process).
+constexpr int kMaxYParts = 4;  // partial output buffers of the tiled down phase
+
+int device_cu_count() {
+  static const int v = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      return 256;
+    return n;
+  }();
+  return v;
+}
 
 // Largest batch served by the weight-streaming expert kernels (tuning knob:
 // ATENIA_MOE_STREAM_MAX_TOKENS, read once per process).
@@ -206,7 +222,8 @@ int ensure_workspace(AteniaMoeLayer* L, int T) {
   ENS(s_tile_m0, ((size_t)T / kTileM + 1) * 4)
   ENS(ident, (size_t)T * 4)
   ENS(h, P * (size_t)L->f_kpad * act)
-  ENS(y, P * (size_t)L->d * 4)
+  ENS(y, kMaxYParts * P * (size_t)L->d * 4)  // partial buffers for k ranges of tail tiles
+  ENS(part_flags, P * (size_t)((L->d + 255) / 256))
   if (L->fs > 0) {
     ENS(hs, (size_t)T * L->fs_kpad * act)
     ENS(ys, (size_t)T * L->d * 4)
@@ -329,6 +346,12 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   fa.n_tiles = L->shared_desc.as<int32_t>() + 4;
   fa.max_row_tiles = (int)(((size_t)T * L->k + kTileM - 1) / kTileM +
                            std::min<long long>(L->E, (long long)T * L->k));
+  const bool split_tail = tiled && tiled_down_splits_tail(L->down, L->wdtype);
+  fa.y_parts = split_tail ? kMaxYParts : 1;
+  fa.y_part_stride = (size_t)T * L->k * L->d;
+  fa.part_flags = split_tail ? L->part_flags.as<uint8_t>() : nullptr;
+  fa.n_cus = device_cu_count();
+  L->last_split = split_tail;
 
   FfnArgs fsd{};
   if (L->fs > 0) {
@@ -347,6 +370,8 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
     fsd.h = L->hs.p;
     fsd.h_stride = L->fs_kpad;
     fsd.y = L->ys.as<float>();
+    fsd.y_parts = 1;
+    fsd.part_flags = nullptr;
     fsd.use_tiled = T > stream_max_tokens() && tiled_supported(L->s_gate, L->wdtype) &&
                     tiled_supported(L->s_down, L->wdtype);
     fsd.tile_group = L->s_tile_group.as<int32_t>();
@@ -377,6 +402,9 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   ca.w = L->w.as<float>();
   ca.y = L->y.as<float>();
   ca.y_stride = L->d;
+  ca.part_flags = fa.part_flags;
+  ca.flag_cols = (L->d + 255) / 256;
+  ca.y_part_stride = fa.y_part_stride;
   ca.y_shared = L->fs > 0 ? L->ys.as<float>() : nullptr;
   ca.sgate = gated ? L->sgate.as<float>() : nullptr;
   ca.out = d_out;
@@ -674,7 +702,25 @@ int atenia_moe_hip_layer_last_expert_outputs(AteniaMoeLayer* L, float* y_host,
   if (hipDeviceSynchronize() != hipSuccess)
     return fail(ATENIA_MOE_ERR_SYNC, "device synchronisation failed");
   const size_t P = (size_t)L->last_T * L->k;
-  if (y_host) HIP_TRY(hipMemcpy(y_host, L->y.p, P * L->d * 4, hipMemcpyDeviceToHost));
+  if (y_host) {
+    HIP_TRY(hipMemcpy(y_host, L->y.p, P * L->d * 4, hipMemcpyDeviceToHost));
+    if (L->last_split) {  // add the partial buffers the down phase wrote for split tail tiles
+      const int fc = (L->d + 255) / 256;
+      std::vector<uint8_t> flags(P * fc);
+      HIP_TRY(hipMemcpy(flags.data(), L->part_flags.p, flags.size(), hipMemcpyDeviceToHost));
+      std::vector<float> part(P * L->d);
+      for (int i = 1; i < kMaxYParts; ++i) {
+        bool any = false;
+        for (uint8_t f : flags) any = any || f > i;
+        if (!any) break;
+        HIP_TRY(hipMemcpy(part.data(), (const float*)L->y.p + (size_t)i * P * L->d, P * L->d * 4,
+                          hipMemcpyDeviceToHost));
+        for (size_t pr = 0; pr < P; ++pr)
+          for (int c = 0; c < L->d; ++c)
+            if (flags[pr * fc + c / 256] > i) y_host[pr * L->d + c] += part[pr * L->d + c];
+      }
+    }
+  }
   if (y_shared_host && L->fs > 0)
     HIP_TRY(hipMemcpy(y_shared_host, L->ys.p, (size_t)L->last_T * L->d * 4,
                       hipMemcpyDeviceToHost));

@@ -104,6 +104,14 @@ struct FfnArgs {
   WeightSet down;
   float* y;            // f32 [rows, y_stride] indexed by PAIR id (token*pair_div+slot)
   int y_stride;
+  // Tiled down phase only: the tiles of a partly filled last round may be cut into up to
+  // y_parts k ranges, range i writing its partial sums to y + i * y_part_stride; part_flags
+  // [pairs, ceil(d / 256)] receives the number of buffers written per (pair, column tile) and
+  // the combine adds those up in order.  y_parts <= 1 or part_flags == null: never split.
+  int y_parts;
+  size_t y_part_stride;  // elements
+  uint8_t* part_flags;
+  int n_cus;             // compute units of the device
   // tiled kernels only
   int use_tiled;
   const int32_t* tile_group;
@@ -112,6 +120,8 @@ struct FfnArgs {
   int max_row_tiles;   // upper bound of *n_tiles (grid sizing)
 };
 bool tiled_supported(const WeightSet& w, int wdtype);
+// True when the tiled down launch for these weights can split the k range of tail tiles.
+bool tiled_down_splits_tail(const WeightSet& down, int wdtype);
 hipError_t launch_ffn_up_tiled(const FfnArgs& a, hipStream_t s);
 hipError_t launch_ffn_down_tiled(const FfnArgs& a, hipStream_t s);
 hipError_t launch_ffn_up(const FfnArgs& a, hipStream_t s);
@@ -122,6 +132,11 @@ struct CombineArgs {
   const float* w;        // [T, k]
   const float* y;        // [T*k, y_stride] pair order
   int y_stride;
+  // partial buffers (see FfnArgs): part_flags[pair * flag_cols + c / 256] of them are added up
+  // in order before weighting; null = one buffer everywhere
+  const uint8_t* part_flags;
+  int flag_cols;
+  size_t y_part_stride;  // elements
   const float* y_shared; // [T, y_stride] or null
   const float* sgate;    // [T] or null (scale 1)
   float* out;            // [T, d]
