@@ -35,6 +35,8 @@ EXPORTS = (
     "atenia_moe_hip_layer_stage_ms", "atenia_moe_hip_layer_stage_launches",
     "atenia_moe_hip_layer_info", "atenia_moe_quantize_per_row_i8",
     "atenia_moe_f32_to_bf16_trunc",
+    "atenia_moe_router_launch_device", "atenia_moe_permute_launch_device",
+    "atenia_moe_expert_ffn_launch_device", "atenia_moe_combine_launch_device",
 )
 
 
@@ -94,6 +96,10 @@ def lib():
         L.atenia_moe_hip_layer_info.argtypes = [P, P]
         L.atenia_moe_quantize_per_row_i8.argtypes = [P, C.c_size_t, C.c_size_t, P, P]
         L.atenia_moe_f32_to_bf16_trunc.argtypes = [P, C.c_size_t, P]
+        L.atenia_moe_router_launch_device.argtypes = [P, P, C.c_int, C.c_int, P, P, P]
+        L.atenia_moe_permute_launch_device.argtypes = [P, C.c_int, P, P, P, P]
+        L.atenia_moe_expert_ffn_launch_device.argtypes = [P, P, C.c_int, C.c_int, P]
+        L.atenia_moe_combine_launch_device.argtypes = [P, C.c_int, P, P]
         _lib = L
     return _lib
 
@@ -202,6 +208,23 @@ class Layer:
         """Raw device pointers (ints); asynchronous on `stream`."""
         _check(lib().atenia_moe_hip_layer_forward_device(self._h, d_x, x_dtype, n_tokens, d_out,
                                                          stream))
+
+    # Stage launchers: the pipeline one kernel at a time (raw device pointers as ints, 0 = NULL).
+    def router_device(self, d_x: int, x_dtype: int, n_tokens: int, d_idx: int = 0, d_w: int = 0,
+                      stream: int = 0):
+        _check(lib().atenia_moe_router_launch_device(self._h, d_x, x_dtype, n_tokens, d_idx or None,
+                                                     d_w or None, stream))
+
+    def permute_device(self, n_tokens: int, d_counts: int = 0, d_offsets: int = 0, d_perm: int = 0,
+                       stream: int = 0):
+        _check(lib().atenia_moe_permute_launch_device(self._h, n_tokens, d_counts or None,
+                                                      d_offsets or None, d_perm or None, stream))
+
+    def expert_ffn_device(self, d_x: int, x_dtype: int, n_tokens: int, stream: int = 0):
+        _check(lib().atenia_moe_expert_ffn_launch_device(self._h, d_x, x_dtype, n_tokens, stream))
+
+    def combine_device(self, n_tokens: int, d_out: int, stream: int = 0):
+        _check(lib().atenia_moe_combine_launch_device(self._h, n_tokens, d_out, stream))
 
     def status(self, stream: int = 0):
         tok, ex = C.c_int32(-1), C.c_int32(-1)

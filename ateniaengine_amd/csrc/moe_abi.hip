@@ -96,6 +96,7 @@ struct AteniaMoeLayer {
       shared_desc, ident, h, hs, y, ys, status, tile_group, tile_m0, s_tile_group, s_tile_m0,
       part_flags;
   int last_T = 0;
+  int stage_T[4] = {-1, -1, -1, -1};  // token count each pipeline stage last completed for
   bool last_split = false;  // the last forward's down phase may have split tail tiles
 
   hipStream_t stream = nullptr;
@@ -251,9 +252,18 @@ struct StageTimer {
   }
 };
 
-// Runs the pipeline on `s`.  stop_after: 0 = all, 1 = router only.
+// Pipeline stages for run_forward's [first, last] range.
+enum { kStageRouter = 0, kStagePermute = 1, kStageFfn = 2, kStageCombine = 3 };
+
+// Runs stages first..last of the pipeline on `s`.  A stage reads what the stages before it
+// left in the handle's workspace, so a range that does not start at the router is only valid
+// after the earlier stages ran for the same n_tokens (checked) on the same activations.
 int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d_out,
-                hipStream_t s, int stop_after) {
+                hipStream_t s, int first, int last) {
+  for (int st = 0; st < first; ++st)
+    if (L->stage_T[st] != T)
+      return fail(ATENIA_MOE_ERR_DIM, "stage %d has not run for %d tokens on this handle", st, T);
+  for (int st = first; st < 4; ++st) L->stage_T[st] = -1;
   const bool f32w = L->wdtype == ATENIA_MOE_WEIGHT_F32;
   if (f32w && x_dtype != ATENIA_MOE_ACT_F32)
     return fail(ATENIA_MOE_ERR_UNSUPPORTED, "f32 weights need f32 activations");
@@ -302,18 +312,25 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   pa.tile_m0 = L->tile_m0.as<int32_t>();
   pa.n_tiles = L->shared_desc.as<int32_t>() + 4;
   pa.shared_n_tiles = L->shared_desc.as<int32_t>() + 5;
-  ra.fuse_permute = stop_after == 1 ? nullptr : &pa;
+  ra.fuse_permute = last >= kStagePermute ? &pa : nullptr;
   int fused = 0;
-  HIP_TRY(launch_router(ra, s, &fused));
-  L->launches[0] = 1;
+  if (first <= kStageRouter) {
+    HIP_TRY(launch_router(ra, s, &fused));
+    L->launches[0] = 1;
+    L->stage_T[kStageRouter] = T;
+  }
   tm.mark();  // ev[1]: router done
   L->last_T = T;
-  if (stop_after == 1) return ATENIA_MOE_OK;
+  if (last < kStagePermute) return ATENIA_MOE_OK;
 
-  int nl = 0;
-  if (!fused) HIP_TRY(launch_permute(pa, s, &nl));
-  L->launches[1] = nl;
+  if (first <= kStagePermute) {
+    int nl = 0;
+    if (!fused) HIP_TRY(launch_permute(pa, s, &nl));
+    L->launches[1] = nl;
+    L->stage_T[kStagePermute] = T;
+  }
   tm.mark();  // ev[2]: permute done
+  if (last < kStageFfn) return ATENIA_MOE_OK;
 
   const void* a_x = f32w ? d_x : (need_xb ? (const void*)L->xb.p : d_x);
   const int a_stride = f32w ? L->d : L->d_kpad;
@@ -380,20 +397,26 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
     fsd.max_row_tiles = (T + kTileM - 1) / kTileM;
   }
 
-  HIP_TRY(launch_ffn_up(fa, s));
-  L->launches[2] = 1;
-  if (L->fs > 0) {
-    HIP_TRY(launch_ffn_up(fsd, s));
-    L->launches[2] = 2;
+  if (first <= kStageFfn) {
+    HIP_TRY(launch_ffn_up(fa, s));
+    L->launches[2] = 1;
+    if (L->fs > 0) {
+      HIP_TRY(launch_ffn_up(fsd, s));
+      L->launches[2] = 2;
+    }
   }
   tm.mark();  // ev[3]: gate/up done
-  HIP_TRY(launch_ffn_down(fa, s));
-  L->launches[3] = 1;
-  if (L->fs > 0) {
-    HIP_TRY(launch_ffn_down(fsd, s));
-    L->launches[3] = 2;
+  if (first <= kStageFfn) {
+    HIP_TRY(launch_ffn_down(fa, s));
+    L->launches[3] = 1;
+    if (L->fs > 0) {
+      HIP_TRY(launch_ffn_down(fsd, s));
+      L->launches[3] = 2;
+    }
+    L->stage_T[kStageFfn] = T;
   }
   tm.mark();  // ev[4]: down done
+  if (last < kStageCombine) return ATENIA_MOE_OK;
 
   CombineArgs ca{};
   ca.T = T;
@@ -410,6 +433,7 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   ca.out = d_out;
   HIP_TRY(launch_combine(ca, s));
   L->launches[4] = 1;
+  L->stage_T[kStageCombine] = T;
   tm.mark();  // ev[5]: combine done
   L->launches[5] = L->launches[0] + L->launches[1] + L->launches[2] + L->launches[3] + 1;
   return ATENIA_MOE_OK;
@@ -580,7 +604,8 @@ int atenia_moe_hip_layer_forward_device(AteniaMoeLayer* L, const void* d_x, int 
   std::lock_guard<std::mutex> lock(L->mu);
   int rc = ensure_workspace(L, n_tokens);
   if (rc) return rc;
-  return run_forward(L, d_x, x_dtype, n_tokens, d_out, (hipStream_t)stream, 0);
+  return run_forward(L, d_x, x_dtype, n_tokens, d_out, (hipStream_t)stream, kStageRouter,
+                     kStageCombine);
 }
 
 int atenia_moe_hip_layer_forward(AteniaMoeLayer* L, const float* x_host, int n_tokens,
@@ -594,10 +619,81 @@ int atenia_moe_hip_layer_forward(AteniaMoeLayer* L, const float* x_host, int n_t
   if (rc) return rc;
   const size_t bytes = (size_t)n_tokens * L->d * 4;
   HIP_TRY(hipMemcpyAsync(L->x_in.p, x_host, bytes, hipMemcpyHostToDevice, L->stream));
-  rc = run_forward(L, L->x_in.p, ATENIA_MOE_ACT_F32, n_tokens, L->out.as<float>(), L->stream, 0);
+  rc = run_forward(L, L->x_in.p, ATENIA_MOE_ACT_F32, n_tokens, L->out.as<float>(), L->stream,
+                   kStageRouter, kStageCombine);
   if (rc) return rc;
   HIP_TRY(hipMemcpyAsync(out_host, L->out.p, bytes, hipMemcpyDeviceToHost, L->stream));
   return read_status(L, L->stream, nullptr, nullptr);
+}
+
+namespace {
+int stage_prologue(AteniaMoeLayer* L, int n_tokens) {
+  if (!valid_handle(L)) return fail(ATENIA_MOE_ERR_HANDLE, "invalid layer handle");
+  if (n_tokens <= 0) return fail(ATENIA_MOE_ERR_DIM, "token count must be positive");
+  if ((long long)n_tokens * L->k > (long long)INT_MAX / 4)
+    return fail(ATENIA_MOE_ERR_DIM, "too many tokens");
+  return ATENIA_MOE_OK;
+}
+}  // namespace
+
+int atenia_moe_router_launch_device(AteniaMoeLayer* L, const void* d_x, int x_dtype,
+                                    int n_tokens, int32_t* d_idx, float* d_w, void* stream) {
+  int rc = stage_prologue(L, n_tokens);
+  if (rc) return rc;
+  if (!d_x) return fail(ATENIA_MOE_ERR_DIM, "null activation pointer");
+  if (x_dtype != ATENIA_MOE_ACT_F32 && x_dtype != ATENIA_MOE_ACT_BF16)
+    return fail(ATENIA_MOE_ERR_DIM, "unknown activation dtype %d", x_dtype);
+  std::lock_guard<std::mutex> lock(L->mu);
+  rc = ensure_workspace(L, n_tokens);
+  if (rc) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  rc = run_forward(L, d_x, x_dtype, n_tokens, nullptr, s, kStageRouter, kStageRouter);
+  if (rc) return rc;
+  const size_t n = (size_t)n_tokens * L->k;
+  if (d_idx) HIP_TRY(hipMemcpyAsync(d_idx, L->idx.p, n * 4, hipMemcpyDeviceToDevice, s));
+  if (d_w) HIP_TRY(hipMemcpyAsync(d_w, L->w.p, n * 4, hipMemcpyDeviceToDevice, s));
+  return ATENIA_MOE_OK;
+}
+
+int atenia_moe_permute_launch_device(AteniaMoeLayer* L, int n_tokens, int32_t* d_counts,
+                                     int32_t* d_offsets, int32_t* d_perm, void* stream) {
+  int rc = stage_prologue(L, n_tokens);
+  if (rc) return rc;
+  std::lock_guard<std::mutex> lock(L->mu);
+  hipStream_t s = (hipStream_t)stream;
+  rc = run_forward(L, nullptr, L->wdtype == ATENIA_MOE_WEIGHT_F32 ? ATENIA_MOE_ACT_F32 : ATENIA_MOE_ACT_BF16,
+                   n_tokens, nullptr, s, kStagePermute, kStagePermute);
+  if (rc) return rc;
+  if (d_counts)
+    HIP_TRY(hipMemcpyAsync(d_counts, L->counts.p, (size_t)L->E * 4, hipMemcpyDeviceToDevice, s));
+  if (d_offsets)
+    HIP_TRY(hipMemcpyAsync(d_offsets, L->offsets.p, ((size_t)L->E + 1) * 4,
+                           hipMemcpyDeviceToDevice, s));
+  if (d_perm)
+    HIP_TRY(hipMemcpyAsync(d_perm, L->perm.p, (size_t)n_tokens * L->k * 4,
+                           hipMemcpyDeviceToDevice, s));
+  return ATENIA_MOE_OK;
+}
+
+int atenia_moe_expert_ffn_launch_device(AteniaMoeLayer* L, const void* d_x, int x_dtype,
+                                        int n_tokens, void* stream) {
+  int rc = stage_prologue(L, n_tokens);
+  if (rc) return rc;
+  if (!d_x) return fail(ATENIA_MOE_ERR_DIM, "null activation pointer");
+  if (x_dtype != ATENIA_MOE_ACT_F32 && x_dtype != ATENIA_MOE_ACT_BF16)
+    return fail(ATENIA_MOE_ERR_DIM, "unknown activation dtype %d", x_dtype);
+  std::lock_guard<std::mutex> lock(L->mu);
+  return run_forward(L, d_x, x_dtype, n_tokens, nullptr, (hipStream_t)stream, kStageFfn, kStageFfn);
+}
+
+int atenia_moe_combine_launch_device(AteniaMoeLayer* L, int n_tokens, float* d_out,
+                                     void* stream) {
+  int rc = stage_prologue(L, n_tokens);
+  if (rc) return rc;
+  if (!d_out) return fail(ATENIA_MOE_ERR_DIM, "null output pointer");
+  std::lock_guard<std::mutex> lock(L->mu);
+  return run_forward(L, nullptr, L->wdtype == ATENIA_MOE_WEIGHT_F32 ? ATENIA_MOE_ACT_F32 : ATENIA_MOE_ACT_BF16,
+                     n_tokens, d_out, (hipStream_t)stream, kStageCombine, kStageCombine);
 }
 
 int atenia_moe_hip_layer_status(AteniaMoeLayer* L, void* stream, int32_t* token,
@@ -618,7 +714,8 @@ int atenia_moe_hip_layer_route(AteniaMoeLayer* L, const float* x_host, int n_tok
   if (rc) return rc;
   HIP_TRY(hipMemcpyAsync(L->x_in.p, x_host, (size_t)n_tokens * L->d * 4, hipMemcpyHostToDevice,
                          L->stream));
-  rc = run_forward(L, L->x_in.p, ATENIA_MOE_ACT_F32, n_tokens, nullptr, L->stream, 1);
+  rc = run_forward(L, L->x_in.p, ATENIA_MOE_ACT_F32, n_tokens, nullptr, L->stream, kStageRouter,
+                   kStageRouter);
   if (rc) return rc;
   rc = read_status(L, L->stream, nullptr, nullptr);
   if (rc) return rc;

@@ -156,6 +156,35 @@ int atenia_moe_hip_layer_permute(AteniaMoeLayer* layer, const int32_t* idx_host,
                                  int32_t* counts_host, int32_t* offsets_host,
                                  int32_t* perm_host);
 
+/* ---- stage launchers: the four kernels of the pipeline, one call each, device pointers ----
+ * Same convention as the reference's device launchers (matmul_f32_launch_device,
+ * src/cuda/matmul.rs:37-47: raw device pointers and int dimensions in, int code out) applied to
+ * the stages of src/moe/layer.rs:405-431.  Each stage reads what the stages before it left in
+ * the handle's workspace, so they are called in order router -> permute -> expert_ffn ->
+ * combine for the same n_tokens and the same activations; calling a stage whose predecessors
+ * have not run for that n_tokens returns ATENIA_MOE_ERR_DIM.  All four are asynchronous on
+ * `stream`; the four calls together are exactly atenia_moe_hip_layer_forward_device. */
+
+/* Kernel 1 (src/moe/dense.rs:325-337, 172-187; src/moe/sparse.rs:142-191).  d_idx / d_w
+ * (device, [n_tokens * top_k], either may be NULL) receive copies of the routing. */
+int atenia_moe_router_launch_device(AteniaMoeLayer* layer, const void* d_x, int x_dtype,
+                                    int n_tokens, int32_t* d_idx, float* d_w, void* stream);
+
+/* Kernel 2 (expert grouping; contract of atenia_moe_hip_layer_permute).  d_counts [E],
+ * d_offsets [E+1], d_perm [n_tokens * top_k]: device, any may be NULL. */
+int atenia_moe_permute_launch_device(AteniaMoeLayer* layer, int n_tokens, int32_t* d_counts,
+                                     int32_t* d_offsets, int32_t* d_perm, void* stream);
+
+/* Kernel 3, both phases (src/moe/dense.rs:253-270), routed and shared experts.  d_x must be
+ * the activations the router stage was given. */
+int atenia_moe_expert_ffn_launch_device(AteniaMoeLayer* layer, const void* d_x, int x_dtype,
+                                        int n_tokens, void* stream);
+
+/* Kernel 4 (src/moe/sparse.rs:226-233, src/moe/layer.rs:415-429).  d_out: [n_tokens, d_model]
+ * f32 on the device. */
+int atenia_moe_combine_launch_device(AteniaMoeLayer* layer, int n_tokens, float* d_out,
+                                     void* stream);
+
 /* Routing/grouping of the handle's most recent forward, copied to host buffers (any pointer
  * may be NULL): idx[T*k], w[T*k], counts[E], offsets[E+1], perm[T*k]. */
 int atenia_moe_hip_layer_last_routing(AteniaMoeLayer* layer, int32_t* idx_host, float* w_host,
