@@ -35,7 +35,7 @@ EXPORTS = (
     "atenia_moe_hip_layer_stage_ms", "atenia_moe_hip_layer_stage_launches",
     "atenia_moe_hip_layer_info", "atenia_moe_quantize_per_row_i8",
     "atenia_moe_f32_to_bf16_trunc",
-    "atenia_moe_router_launch_device", "atenia_moe_permute_launch_device",
+    "atenia_moe_hip_layer_last_non_finite", "atenia_moe_router_launch_device", "atenia_moe_permute_launch_device",
     "atenia_moe_expert_ffn_launch_device", "atenia_moe_combine_launch_device",
 )
 
@@ -96,6 +96,7 @@ def lib():
         L.atenia_moe_hip_layer_info.argtypes = [P, P]
         L.atenia_moe_quantize_per_row_i8.argtypes = [P, C.c_size_t, C.c_size_t, P, P]
         L.atenia_moe_f32_to_bf16_trunc.argtypes = [P, C.c_size_t, P]
+        L.atenia_moe_hip_layer_last_non_finite.argtypes = [P, P, P]
         L.atenia_moe_router_launch_device.argtypes = [P, P, C.c_int, C.c_int, P, P, P]
         L.atenia_moe_permute_launch_device.argtypes = [P, C.c_int, P, P, P, P]
         L.atenia_moe_expert_ffn_launch_device.argtypes = [P, P, C.c_int, C.c_int, P]
@@ -230,6 +231,12 @@ class Layer:
         tok, ex = C.c_int32(-1), C.c_int32(-1)
         rc = lib().atenia_moe_hip_layer_status(self._h, stream, C.addressof(tok), C.addressof(ex))
         return rc, tok.value, ex.value
+
+    def last_non_finite(self):
+        """(token, expert) of the most recent non-finite routing weight, (-1, -1) if none."""
+        tok, ex = C.c_int32(-1), C.c_int32(-1)
+        _check(lib().atenia_moe_hip_layer_last_non_finite(self._h, C.addressof(tok), C.addressof(ex)))
+        return tok.value, ex.value
 
     # -- parity taps ----------------------------------------------------------------------
     def route(self, x):

@@ -97,6 +97,7 @@ struct AteniaMoeLayer {
       part_flags;
   int last_T = 0;
   int stage_T[4] = {-1, -1, -1, -1};  // token count each pipeline stage last completed for
+  int nf_token = -1, nf_expert = -1;  // location of the last non-finite routing weight reported
   bool last_split = false;  // the last forward's down phase may have split tail tiles
 
   hipStream_t stream = nullptr;
@@ -449,6 +450,8 @@ int read_status(AteniaMoeLayer* L, hipStream_t s, int32_t* token, int32_t* exper
   int tk = st[1] >> 10, ex = st[1] & 1023;
   if (token) *token = tk;
   if (expert) *expert = ex;
+  L->nf_token = tk;
+  L->nf_expert = ex;
   int32_t reset[2] = {0, INT_MAX};
   HIP_TRY(hipMemcpy(L->status.p, reset, 8, hipMemcpyHostToDevice));
   return fail(ATENIA_MOE_ERR_NON_FINITE, "non-finite routing weight at token %d, expert %d", tk,
@@ -701,6 +704,14 @@ int atenia_moe_hip_layer_status(AteniaMoeLayer* L, void* stream, int32_t* token,
   if (!valid_handle(L)) return fail(ATENIA_MOE_ERR_HANDLE, "invalid layer handle");
   std::lock_guard<std::mutex> lock(L->mu);
   return read_status(L, (hipStream_t)stream, token, expert);
+}
+
+int atenia_moe_hip_layer_last_non_finite(AteniaMoeLayer* L, int32_t* token, int32_t* expert) {
+  if (!valid_handle(L)) return fail(ATENIA_MOE_ERR_HANDLE, "invalid layer handle");
+  std::lock_guard<std::mutex> lock(L->mu);
+  if (token) *token = L->nf_token;
+  if (expert) *expert = L->nf_expert;
+  return ATENIA_MOE_OK;
 }
 
 int atenia_moe_hip_layer_route(AteniaMoeLayer* L, const float* x_host, int n_tokens,

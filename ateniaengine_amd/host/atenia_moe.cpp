@@ -1,0 +1,470 @@
+// Implementation of the host mirror over the C ABI (see atenia_moe.hpp for the reference
+// interface each part follows).
+#include "atenia_moe.hpp"
+
+#include <cstring>
+#include <map>
+#include <utility>
+
+#include "../../include/atenia_moe_hip.h"
+
+namespace atenia {
+namespace moe {
+
+// ---- error text: the reference's Display implementations -------------------------------------
+std::string MoeConfigError::to_string() const {
+  switch (kind) {  // src/moe/layer.rs:56-75
+    case ZeroExperts: return "moe-config: num_experts is 0";
+    case ZeroExpertsPerToken: return "moe-config: experts_per_token is 0";
+    case ExpertsPerTokenExceedsCount:
+      return "moe-config: experts_per_token (" + std::to_string(per_token) + ") > num_experts (" +
+             std::to_string(total) + ")";
+    case ZeroDModel: return "moe-config: d_model is 0";
+    case ZeroDFf: return "moe-config: d_ff is 0";
+  }
+  return "moe-config";
+}
+
+std::string MoeDenseError::to_string() const {
+  switch (kind) {  // src/moe/dense.rs:51-69
+    case DimMismatch:
+      return std::string("moe-dense: ") + what + " dim mismatch: expected " +
+             std::to_string(expected) + ", got " + std::to_string(actual);
+    case WeightShapeMismatch:
+      return std::string("moe-dense: ") + what + " weight shape mismatch: expected " +
+             std::to_string(expected) + " elems, got " + std::to_string(actual);
+    case NoExperts: return "moe-dense: layer has no experts";
+    case RouterExpertCountMismatch:
+      return "moe-dense: router expert count (" + std::to_string(expected) + ") != experts (" +
+             std::to_string(actual) + ")";
+  }
+  return "moe-dense";
+}
+
+std::string MoeSparseError::to_string() const {
+  switch (kind) {  // src/moe/sparse.rs:52-72
+    case ZeroK: return "moe-sparse: k must be > 0";
+    case KExceedsExperts:
+      return "moe-sparse: k (" + std::to_string(k) + ") exceeds num_experts (" +
+             std::to_string(num_experts) + ")";
+    case NonFiniteWeight:
+      return "moe-sparse: routing weight at " + std::to_string(index) + " is non-finite";
+    case NegativeWeight:
+      return "moe-sparse: routing weight at " + std::to_string(index) + " is negative";
+    case SelectedSumNonPositive: return "moe-sparse: selected top-k weights sum to <= 0";
+    case Dense: return "moe-sparse: " + dense.to_string();
+  }
+  return "moe-sparse";
+}
+
+std::string MoeBindingError::to_string() const {
+  switch (kind) {  // src/moe/binding.rs:72-76
+    case LayerNotFound:
+      return "moe-binding: layer " + std::to_string(layer_id) + " has no MoE weights";
+    case Dense: return "moe-binding: " + dense.to_string();
+  }
+  return "moe-binding";
+}
+
+std::string MoeLayerError::to_string() const {
+  switch (kind) {
+    case Config: return "moe-layer: " + config.to_string();
+    case Binding: return "moe-layer: " + binding.to_string();
+    case Sparse: return "moe-layer: " + sparse.to_string();
+    case ConfigMismatch: return "moe-layer: config mismatch: " + detail;
+    case Device: return "moe-layer: device path failed (rc " + std::to_string(rc) + "): " + detail;
+  }
+  return "moe-layer";
+}
+
+namespace {
+MoeLayerError dense_dim_error(const char* what, size_t expected, size_t actual) {
+  MoeLayerError e{MoeLayerError::Sparse};
+  e.sparse.kind = MoeSparseError::Dense;
+  e.sparse.dense = MoeDenseError{MoeDenseError::DimMismatch, what, expected, actual};
+  return e;
+}
+MoeLayerError device_error(int rc) {
+  MoeLayerError e{MoeLayerError::Device};
+  e.rc = rc;
+  e.detail = atenia_moe_hip_last_error_string();
+  return e;
+}
+}  // namespace
+
+// ---- config / parts -----------------------------------------------------------------------
+std::optional<MoeConfigError> MoeLayerConfig::validate() const {
+  if (num_experts == 0) return MoeConfigError{MoeConfigError::ZeroExperts};
+  if (experts_per_token == 0) return MoeConfigError{MoeConfigError::ZeroExpertsPerToken};
+  if (experts_per_token > num_experts)
+    return MoeConfigError{MoeConfigError::ExpertsPerTokenExceedsCount, experts_per_token, num_experts};
+  if (d_model == 0) return MoeConfigError{MoeConfigError::ZeroDModel};
+  if (d_ff == 0) return MoeConfigError{MoeConfigError::ZeroDFf};
+  return std::nullopt;
+}
+
+Result<MoeLayerConfig, MoeConfigError> MoeLayerConfig::make(size_t num_experts,
+                                                            size_t experts_per_token,
+                                                            bool has_shared_expert, size_t d_model,
+                                                            size_t d_ff) {
+  MoeLayerConfig c{num_experts, experts_per_token, has_shared_expert, d_model, d_ff};
+  if (auto e = c.validate()) return Result<MoeLayerConfig, MoeConfigError>::Err(*e);
+  return Result<MoeLayerConfig, MoeConfigError>::Ok(c);
+}
+
+Result<MoeDenseExpert, MoeDenseError> MoeDenseExpert::make(size_t d_model, size_t d_ff,
+                                                           std::vector<float> w_gate,
+                                                           std::vector<float> w_up,
+                                                           std::vector<float> w_down) {
+  typedef Result<MoeDenseExpert, MoeDenseError> R;
+  if (w_gate.size() != d_ff * d_model)
+    return R::Err({MoeDenseError::WeightShapeMismatch, "w_gate", d_ff * d_model, w_gate.size()});
+  if (w_up.size() != d_ff * d_model)
+    return R::Err({MoeDenseError::WeightShapeMismatch, "w_up", d_ff * d_model, w_up.size()});
+  if (w_down.size() != d_model * d_ff)
+    return R::Err({MoeDenseError::WeightShapeMismatch, "w_down", d_model * d_ff, w_down.size()});
+  MoeDenseExpert e;
+  e.d_model = d_model;
+  e.d_ff = d_ff;
+  e.w_gate = std::move(w_gate);
+  e.w_up = std::move(w_up);
+  e.w_down = std::move(w_down);
+  return R::Ok(std::move(e));
+}
+
+Result<MoeDenseLayer, MoeDenseError> MoeDenseLayer::make(size_t d_model, size_t d_ff,
+                                                         std::vector<float> w_router,
+                                                         std::vector<MoeDenseExpert> experts,
+                                                         size_t conceptual_top_k) {
+  typedef Result<MoeDenseLayer, MoeDenseError> R;  // src/moe/dense.rs:289-322
+  if (experts.empty()) return R::Err({MoeDenseError::NoExperts});
+  const size_t n = experts.size();
+  if (w_router.size() != n * d_model)
+    return R::Err({MoeDenseError::RouterExpertCountMismatch, "", d_model ? w_router.size() / d_model : 0, n});
+  for (const auto& e : experts) {
+    if (e.d_model != d_model)
+      return R::Err({MoeDenseError::DimMismatch, "expert d_model", d_model, e.d_model});
+    if (e.d_ff != d_ff) return R::Err({MoeDenseError::DimMismatch, "expert d_ff", d_ff, e.d_ff});
+  }
+  MoeDenseLayer l;
+  l.d_model = d_model;
+  l.d_ff = d_ff;
+  l.w_router = std::move(w_router);
+  l.experts = std::move(experts);
+  l.conceptual_top_k = conceptual_top_k;
+  return R::Ok(std::move(l));
+}
+
+// ---- RealMoeLayer ---------------------------------------------------------------------------
+struct RealMoeLayer::Device {
+  std::mutex mu;
+  // key: convention * 2 + with_shared
+  std::map<int, AteniaMoeLayer*> handles;
+  ~Device() {
+    for (auto& kv : handles) atenia_moe_hip_layer_destroy(kv.second);
+  }
+};
+
+RealMoeLayer::RealMoeLayer() : dev_(new Device()) {}
+RealMoeLayer::RealMoeLayer(const RealMoeLayer& o)
+    : config(o.config), routed(o.routed), shared(o.shared), shared_gate(o.shared_gate),
+      storage(o.storage), dev_(new Device()) {}
+RealMoeLayer& RealMoeLayer::operator=(const RealMoeLayer& o) {
+  if (this != &o) {
+    config = o.config;
+    routed = o.routed;
+    shared = o.shared;
+    shared_gate = o.shared_gate;
+    storage = o.storage;
+    dev_.reset(new Device());
+  }
+  return *this;
+}
+RealMoeLayer::RealMoeLayer(RealMoeLayer&& o) noexcept
+    : config(o.config), routed(std::move(o.routed)), shared(std::move(o.shared)),
+      shared_gate(std::move(o.shared_gate)), storage(o.storage), dev_(std::move(o.dev_)) {
+  o.dev_.reset(new Device());
+}
+RealMoeLayer& RealMoeLayer::operator=(RealMoeLayer&& o) noexcept {
+  if (this != &o) {
+    config = o.config;
+    routed = std::move(o.routed);
+    shared = std::move(o.shared);
+    shared_gate = std::move(o.shared_gate);
+    storage = o.storage;
+    dev_ = std::move(o.dev_);
+    o.dev_.reset(new Device());
+  }
+  return *this;
+}
+RealMoeLayer::~RealMoeLayer() = default;
+
+Result<RealMoeLayer, MoeLayerError> RealMoeLayer::assemble(
+    MoeLayerConfig config, MoeDenseLayer routed, std::optional<MoeDenseExpert> shared,
+    std::optional<std::vector<float>> shared_gate, MoeWeightStorage storage) {
+  typedef Result<RealMoeLayer, MoeLayerError> R;
+  if (auto e = config.validate()) {
+    MoeLayerError le{MoeLayerError::Config};
+    le.config = *e;
+    return R::Err(le);
+  }
+  auto mismatch = [](std::string d) {
+    MoeLayerError le{MoeLayerError::ConfigMismatch};
+    le.detail = std::move(d);
+    return le;
+  };
+  if (routed.num_experts() != config.num_experts)
+    return R::Err(mismatch("resolved " + std::to_string(routed.num_experts()) +
+                           " experts but config.num_experts = " + std::to_string(config.num_experts)));
+  if (routed.d_model != config.d_model || routed.d_ff != config.d_ff)
+    return R::Err(mismatch("resolved (d_model=" + std::to_string(routed.d_model) + ", d_ff=" +
+                           std::to_string(routed.d_ff) + ") but config (d_model=" +
+                           std::to_string(config.d_model) + ", d_ff=" + std::to_string(config.d_ff) + ")"));
+  if (config.has_shared_expert != shared.has_value())
+    return R::Err(mismatch(config.has_shared_expert ? "config asks for a shared expert, none given"
+                                                    : "shared expert given but config has none"));
+  if (shared && shared->d_model != config.d_model)
+    return R::Err(mismatch("shared expert d_model=" + std::to_string(shared->d_model) +
+                           " != config d_model=" + std::to_string(config.d_model)));
+  if (shared_gate && !shared) shared_gate.reset();  // captured only next to a shared expert
+  RealMoeLayer l;
+  l.config = config;
+  l.routed = std::move(routed);
+  l.routed.conceptual_top_k = config.experts_per_token;
+  l.shared = std::move(shared);
+  l.shared_gate = std::move(shared_gate);
+  l.storage = storage;
+  return R::Ok(std::move(l));
+}
+
+namespace {
+// Expert weights in the storage form the descriptor asks for.
+struct Packed {
+  std::vector<float> f32;
+  std::vector<uint16_t> b16;
+  std::vector<int8_t> i8;
+  std::vector<float> scale;
+  const void* data(MoeWeightStorage s) const {
+    return s == MoeWeightStorage::F32 ? (const void*)f32.data()
+           : s == MoeWeightStorage::Bf16 ? (const void*)b16.data() : (const void*)i8.data();
+  }
+};
+
+int pack(const std::vector<const std::vector<float>*>& mats, size_t rows, size_t cols,
+         MoeWeightStorage s, Packed& out) {
+  const size_t per = rows * cols, n = mats.size();
+  if (s == MoeWeightStorage::F32) {
+    out.f32.resize(n * per);
+    for (size_t i = 0; i < n; ++i) std::memcpy(&out.f32[i * per], mats[i]->data(), per * 4);
+    return 0;
+  }
+  if (s == MoeWeightStorage::Bf16) {  // truncation, as the reference stores bf16 (tensor.rs:306-308)
+    out.b16.resize(n * per);
+    for (size_t i = 0; i < n; ++i) {
+      int rc = atenia_moe_f32_to_bf16_trunc(mats[i]->data(), per, &out.b16[i * per]);
+      if (rc) return rc;
+    }
+    return 0;
+  }
+  out.i8.resize(n * per);  // per output row (disk_tier.rs:231-248)
+  out.scale.resize(n * rows);
+  for (size_t i = 0; i < n; ++i) {
+    int rc = atenia_moe_quantize_per_row_i8(mats[i]->data(), rows, cols, &out.i8[i * per],
+                                            &out.scale[i * rows]);
+    if (rc) return rc;
+  }
+  return 0;
+}
+}  // namespace
+
+// The C-ABI handle for (convention, with shared expert), created and uploaded on first use.
+// Caller holds dev_->mu.
+Result<void*, MoeLayerError> RealMoeLayer::handle_for(MoeExecutionConvention convention,
+                                                      bool with_shared) const {
+  typedef Result<void*, MoeLayerError> R;
+  const size_t d = config.d_model;
+  const bool use_shared = with_shared && shared.has_value();
+  const int key = (int)convention * 2 + (use_shared ? 1 : 0);
+  auto it = dev_->handles.find(key);
+  if (it != dev_->handles.end()) return R::Ok(it->second);
+  const size_t E = routed.num_experts(), f = config.d_ff;
+  std::vector<const std::vector<float>*> g, u, dn;
+  for (const auto& e : routed.experts) {
+    g.push_back(&e.w_gate);
+    u.push_back(&e.w_up);
+    dn.push_back(&e.w_down);
+  }
+  Packed pg, pu, pd, sg, su, sd;
+  int rc = pack(g, f, d, storage, pg);
+  if (!rc) rc = pack(u, f, d, storage, pu);
+  if (!rc) rc = pack(dn, d, f, storage, pd);
+  AteniaMoeLayerDesc desc;
+  std::memset(&desc, 0, sizeof(desc));
+  desc.num_experts = (int32_t)E;
+  desc.top_k = (int32_t)config.experts_per_token;
+  desc.d_model = (int32_t)d;
+  desc.d_ff = (int32_t)f;
+  desc.convention = (int32_t)convention;
+  desc.weight_dtype = (int32_t)storage;
+  desc.w_router = routed.w_router.data();
+  desc.w_gate = pg.data(storage);
+  desc.w_up = pu.data(storage);
+  desc.w_down = pd.data(storage);
+  if (storage == MoeWeightStorage::Int8W8A16) {
+    desc.scale_gate = pg.scale.data();
+    desc.scale_up = pu.scale.data();
+    desc.scale_down = pd.scale.data();
+  }
+  if (use_shared) {
+    const size_t fs = shared->d_ff;
+    desc.d_ff_shared = (int32_t)fs;
+    if (!rc) rc = pack({&shared->w_gate}, fs, d, storage, sg);
+    if (!rc) rc = pack({&shared->w_up}, fs, d, storage, su);
+    if (!rc) rc = pack({&shared->w_down}, d, fs, storage, sd);
+    desc.s_gate = sg.data(storage);
+    desc.s_up = su.data(storage);
+    desc.s_down = sd.data(storage);
+    if (storage == MoeWeightStorage::Int8W8A16) {
+      desc.s_scale_gate = sg.scale.data();
+      desc.s_scale_up = su.scale.data();
+      desc.s_scale_down = sd.scale.data();
+    }
+    if (shared_gate) desc.shared_gate = shared_gate->data();
+  }
+  if (rc) return R::Err(device_error(rc));
+  AteniaMoeLayer* h = nullptr;
+  rc = atenia_moe_hip_layer_create(&desc, &h);
+  if (rc == ATENIA_MOE_ERR_K) {
+    MoeLayerError e{MoeLayerError::Sparse};
+    if (config.experts_per_token == 0) {
+      e.sparse.kind = MoeSparseError::ZeroK;
+    } else {
+      e.sparse.kind = MoeSparseError::KExceedsExperts;
+      e.sparse.k = config.experts_per_token;
+      e.sparse.num_experts = E;
+    }
+    return R::Err(e);
+  }
+  if (rc) return R::Err(device_error(rc));
+  dev_->handles[key] = h;
+  return R::Ok(h);
+}
+
+namespace {
+MoeLayerError non_finite_error(AteniaMoeLayer* h) {
+  int32_t token = 0, expert = 0;
+  atenia_moe_hip_layer_last_non_finite(h, &token, &expert);
+  MoeLayerError e{MoeLayerError::Sparse};
+  e.sparse.kind = MoeSparseError::NonFiniteWeight;
+  e.sparse.index = (size_t)expert;
+  e.sparse.token = (size_t)token;
+  return e;
+}
+}  // namespace
+
+Result<std::vector<float>, MoeLayerError> RealMoeLayer::run(const std::vector<float>& x,
+                                                            MoeExecutionConvention convention,
+                                                            bool with_shared) const {
+  typedef Result<std::vector<float>, MoeLayerError> R;
+  const size_t d = config.d_model;
+  // One token or a flat batch; anything else is the dimension error the row forward raises
+  // (src/moe/dense.rs:325-331 via graph_op.rs:340-343).
+  if (d == 0 || x.empty() || x.size() % d != 0) return R::Err(dense_dim_error("x", d, x.size()));
+  std::lock_guard<std::mutex> lock(dev_->mu);
+  auto hr = handle_for(convention, with_shared);
+  if (hr.is_err()) return R::Err(hr.error());
+  AteniaMoeLayer* h = (AteniaMoeLayer*)hr.value();
+  std::vector<float> out(x.size());
+  const int rc = atenia_moe_hip_layer_forward(h, x.data(), (int)(x.size() / d), out.data());
+  if (rc == ATENIA_MOE_ERR_NON_FINITE) return R::Err(non_finite_error(h));
+  if (rc == ATENIA_MOE_ERR_DIM) return R::Err(dense_dim_error("x", d, x.size()));
+  if (rc) return R::Err(device_error(rc));
+  return R::Ok(std::move(out));
+}
+
+Result<std::vector<float>, MoeLayerError> RealMoeLayer::forward(const std::vector<float>& x) const {
+  return forward_with(x, MoeExecutionConvention::Atenia);
+}
+Result<std::vector<float>, MoeLayerError> RealMoeLayer::forward_auto(const std::vector<float>& x) const {
+  return forward_with(x, resolve_convention());
+}
+Result<std::vector<float>, MoeLayerError> RealMoeLayer::forward_with(
+    const std::vector<float>& x, MoeExecutionConvention convention) const {
+  return run(x, convention, true);
+}
+Result<std::vector<float>, MoeLayerError> RealMoeLayer::forward_routed(const std::vector<float>& x) const {
+  return run(x, MoeExecutionConvention::Atenia, false);
+}
+
+Result<std::vector<float>, MoeLayerError> RealMoeLayer::route(const std::vector<float>& x,
+                                                              MoeExecutionConvention convention,
+                                                              std::vector<int32_t>* indices) const {
+  typedef Result<std::vector<float>, MoeLayerError> R;
+  const size_t d = config.d_model;
+  if (d == 0 || x.empty() || x.size() % d != 0) return R::Err(dense_dim_error("x", d, x.size()));
+  std::lock_guard<std::mutex> lock(dev_->mu);
+  auto hr = handle_for(convention, true);
+  if (hr.is_err()) return R::Err(hr.error());
+  AteniaMoeLayer* h = (AteniaMoeLayer*)hr.value();
+  const int T = (int)(x.size() / d);
+  const size_t k = config.experts_per_token;
+  std::vector<int32_t> idx((size_t)T * k);
+  std::vector<float> w((size_t)T * k);
+  const int rc = atenia_moe_hip_layer_route(h, x.data(), T, idx.data(), w.data());
+  if (rc == ATENIA_MOE_ERR_NON_FINITE) return R::Err(non_finite_error(h));
+  if (rc) return R::Err(device_error(rc));
+  if (indices) *indices = std::move(idx);
+  return R::Ok(std::move(w));
+}
+
+// ---- registry -------------------------------------------------------------------------------
+namespace {
+std::mutex& registry_mutex() {
+  static std::mutex m;
+  return m;
+}
+std::vector<std::shared_ptr<RealMoeLayer>>& registry() {
+  static std::vector<std::shared_ptr<RealMoeLayer>> r;
+  return r;
+}
+MoeLayerError layer_not_found(uint32_t id) {
+  MoeLayerError e{MoeLayerError::Binding};
+  e.binding.kind = MoeBindingError::LayerNotFound;
+  e.binding.layer_id = id;
+  return e;
+}
+}  // namespace
+
+uint32_t register_real_moe_layer(RealMoeLayer layer) {
+  std::lock_guard<std::mutex> lock(registry_mutex());
+  registry().push_back(std::make_shared<RealMoeLayer>(std::move(layer)));
+  return (uint32_t)(registry().size() - 1);
+}
+
+std::shared_ptr<const RealMoeLayer> get_real_moe_layer(uint32_t layer_id) {
+  std::lock_guard<std::mutex> lock(registry_mutex());
+  if (layer_id >= registry().size()) return nullptr;
+  return registry()[layer_id];
+}
+
+Result<std::vector<float>, MoeLayerError> execute_real_moe_layer(uint32_t layer_id,
+                                                                 const std::vector<float>& input) {
+  auto layer = get_real_moe_layer(layer_id);
+  if (!layer) return Result<std::vector<float>, MoeLayerError>::Err(layer_not_found(layer_id));
+  return layer->forward_auto(input);  // whole batch, one call into the device library
+}
+
+Result<std::vector<float>, MoeLayerError> execute_real_moe_layer_with(
+    uint32_t layer_id, const std::vector<float>& input, MoeExecutionConvention convention) {
+  auto layer = get_real_moe_layer(layer_id);
+  if (!layer) return Result<std::vector<float>, MoeLayerError>::Err(layer_not_found(layer_id));
+  return layer->forward_with(input, convention);
+}
+
+std::vector<float> moe_real_layer_reference_node(uint32_t layer_id, const std::vector<float>& input) {
+  return execute_real_moe_layer(layer_id, input)
+      .expect("MoeRealLayerReference: forward failed (unknown layer_id or bad input dim)");
+}
+
+}  // namespace moe
+}  // namespace atenia

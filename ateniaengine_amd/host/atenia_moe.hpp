@@ -1,0 +1,224 @@
+// Host-side mirror of the reference's MoE operator interface, over the C ABI of
+// libatenia_moe_hip.so.  The reference is Rust; these are the same types, names, argument
+// meanings and error behaviour in C++, so a test written against the reference reads the same
+// here:
+//
+//   MoeLayerConfig, MoeConfigError            src/moe/layer.rs:37-117
+//   MoeExecutionConvention                    src/moe/layer.rs:185-195
+//   MoeDenseExpert, MoeDenseLayer             src/moe/dense.rs:203-250, 276-322
+//   RealMoeLayer::{forward, forward_auto, forward_with, forward_routed, resolve_convention}
+//                                             src/moe/layer.rs:200-431
+//   MoeDenseError / MoeSparseError / MoeBindingError / MoeLayerError
+//                                             dense.rs:31-49, sparse.rs:35-50, binding.rs:41-70,
+//                                             layer.rs:119-136
+//   register_real_moe_layer, get_real_moe_layer, execute_real_moe_layer[_with]
+//                                             src/moe/graph_op.rs:228-232, 294-299, 327-364
+//   moe_real_layer_reference_node             the executor arm, src/amg/graph.rs:5572-5589
+//
+// What differs on purpose: a forward runs on the GPU through one C-ABI call for the whole
+// [T * d_model] batch (the reference loops over rows on the CPU), and a layer carries the
+// storage type its weights are uploaded as (f32 keeps the reference's certified arithmetic;
+// bf16 and int8 are the throughput forms).  There is no CPU fallback: without the device
+// every forward returns MoeLayerError::Device.
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+#include <memory>
+#include <mutex>
+#include <optional>
+#include <string>
+#include <vector>
+
+namespace atenia {
+namespace moe {
+
+// ---- errors ---------------------------------------------------------------------------------
+struct MoeConfigError {
+  enum Kind { ZeroExperts, ZeroExpertsPerToken, ExpertsPerTokenExceedsCount, ZeroDModel, ZeroDFf };
+  Kind kind;
+  size_t per_token = 0, total = 0;
+  std::string to_string() const;
+  bool operator==(const MoeConfigError& o) const {
+    return kind == o.kind && per_token == o.per_token && total == o.total;
+  }
+};
+
+struct MoeDenseError {
+  enum Kind { DimMismatch, WeightShapeMismatch, NoExperts, RouterExpertCountMismatch };
+  Kind kind;
+  const char* what = "";
+  size_t expected = 0, actual = 0;  // RouterExpertCountMismatch: router, experts
+  std::string to_string() const;
+};
+
+struct MoeSparseError {
+  enum Kind { ZeroK, KExceedsExperts, NonFiniteWeight, NegativeWeight, SelectedSumNonPositive, Dense };
+  Kind kind;
+  size_t k = 0, num_experts = 0;  // KExceedsExperts
+  size_t index = 0;               // NonFiniteWeight / NegativeWeight: expert index
+  size_t token = 0;               // row of the batch the weight belongs to (extension)
+  MoeDenseError dense{MoeDenseError::NoExperts};
+  std::string to_string() const;
+};
+
+struct MoeBindingError {
+  enum Kind { LayerNotFound, Dense };
+  Kind kind;
+  size_t layer_id = 0;
+  MoeDenseError dense{MoeDenseError::NoExperts};
+  std::string to_string() const;
+};
+
+struct MoeLayerError {
+  // Config / Binding / Sparse / ConfigMismatch as in the reference; Device = the HIP library
+  // reported a failure that has no counterpart there (no device, out of memory, launch failed).
+  enum Kind { Config, Binding, Sparse, ConfigMismatch, Device };
+  Kind kind;
+  MoeConfigError config{MoeConfigError::ZeroExperts};
+  MoeBindingError binding{MoeBindingError::LayerNotFound};
+  MoeSparseError sparse{MoeSparseError::ZeroK};
+  std::string detail;  // ConfigMismatch / Device
+  int rc = 0;          // Device: return code of the C ABI
+  std::string to_string() const;
+};
+
+// Result<T, E> of the reference, reduced to what the mirror needs.
+template <typename T, typename E>
+class Result {
+ public:
+  static Result Ok(T v) { Result r; r.v_ = std::move(v); return r; }
+  static Result Err(E e) { Result r; r.e_ = std::move(e); return r; }
+  bool is_ok() const { return v_.has_value(); }
+  bool is_err() const { return !is_ok(); }
+  const T& value() const { return *v_; }
+  T& value() { return *v_; }
+  const E& error() const { return *e_; }
+  // `.unwrap()` / `.expect(msg)`: the value, or std::runtime_error carrying the error text.
+  T unwrap() const;
+  T expect(const char* msg) const;
+
+ private:
+  std::optional<T> v_;
+  std::optional<E> e_;
+};
+
+// ---- types ----------------------------------------------------------------------------------
+struct MoeLayerConfig {
+  size_t num_experts = 0, experts_per_token = 0;
+  bool has_shared_expert = false;
+  size_t d_model = 0, d_ff = 0;
+  // src/moe/layer.rs:86-116 (new + validate)
+  static Result<MoeLayerConfig, MoeConfigError> make(size_t num_experts, size_t experts_per_token,
+                                                     bool has_shared_expert, size_t d_model,
+                                                     size_t d_ff);
+  std::optional<MoeConfigError> validate() const;
+};
+
+enum class MoeExecutionConvention { Atenia = 0, HuggingFaceQwen = 1 };
+
+// How the layer's expert weights are stored in HBM.
+enum class MoeWeightStorage { F32 = 0, Bf16 = 1, Int8W8A16 = 2 };
+
+struct MoeDenseExpert {
+  size_t d_model = 0, d_ff = 0;
+  std::vector<float> w_gate, w_up, w_down;  // [d_ff,d_model], [d_ff,d_model], [d_model,d_ff]
+  static Result<MoeDenseExpert, MoeDenseError> make(size_t d_model, size_t d_ff,
+                                                    std::vector<float> w_gate,
+                                                    std::vector<float> w_up,
+                                                    std::vector<float> w_down);
+};
+
+struct MoeDenseLayer {
+  size_t d_model = 0, d_ff = 0;
+  std::vector<float> w_router;  // [num_experts, d_model]
+  std::vector<MoeDenseExpert> experts;
+  size_t conceptual_top_k = 0;
+  static Result<MoeDenseLayer, MoeDenseError> make(size_t d_model, size_t d_ff,
+                                                   std::vector<float> w_router,
+                                                   std::vector<MoeDenseExpert> experts,
+                                                   size_t conceptual_top_k);
+  size_t num_experts() const { return experts.size(); }
+};
+
+class RealMoeLayer {
+ public:
+  MoeLayerConfig config;
+  MoeDenseLayer routed;
+  std::optional<MoeDenseExpert> shared;
+  std::optional<std::vector<float>> shared_gate;
+  MoeWeightStorage storage = MoeWeightStorage::F32;
+
+  // Cross-checks the parts against the config the way RealMoeLayer::assemble does
+  // (src/moe/layer.rs:282-343): expert count, dimensions, shared expert present iff asked for.
+  static Result<RealMoeLayer, MoeLayerError> assemble(MoeLayerConfig config, MoeDenseLayer routed,
+                                                      std::optional<MoeDenseExpert> shared,
+                                                      std::optional<std::vector<float>> shared_gate,
+                                                      MoeWeightStorage storage = MoeWeightStorage::F32);
+
+  size_t num_experts() const { return routed.num_experts(); }
+  bool has_shared_expert() const { return shared.has_value(); }
+  MoeExecutionConvention resolve_convention() const {
+    return shared_gate ? MoeExecutionConvention::HuggingFaceQwen : MoeExecutionConvention::Atenia;
+  }
+
+  // x: one token [d_model] or a flat batch [n * d_model]; the layer is position-wise.
+  Result<std::vector<float>, MoeLayerError> forward(const std::vector<float>& x) const;
+  Result<std::vector<float>, MoeLayerError> forward_auto(const std::vector<float>& x) const;
+  Result<std::vector<float>, MoeLayerError> forward_with(const std::vector<float>& x,
+                                                         MoeExecutionConvention convention) const;
+  // Routed experts only, renormalised combine (src/moe/layer.rs:366-369).
+  Result<std::vector<float>, MoeLayerError> forward_routed(const std::vector<float>& x) const;
+  // Routing of each row: indices [n * k] (ascending per row) and weights, under `convention`.
+  Result<std::vector<float>, MoeLayerError> route(const std::vector<float>& x,
+                                                  MoeExecutionConvention convention,
+                                                  std::vector<int32_t>* indices) const;
+
+  RealMoeLayer();
+  RealMoeLayer(const RealMoeLayer& o);             // copies the host weights, not device state
+  RealMoeLayer& operator=(const RealMoeLayer& o);
+  RealMoeLayer(RealMoeLayer&&) noexcept;
+  RealMoeLayer& operator=(RealMoeLayer&&) noexcept;
+  ~RealMoeLayer();
+
+ private:
+  struct Device;  // lazily created C-ABI handles, one per (convention, with shared)
+  mutable std::unique_ptr<Device> dev_;
+  Result<std::vector<float>, MoeLayerError> run(const std::vector<float>& x,
+                                                MoeExecutionConvention convention,
+                                                bool with_shared) const;
+  Result<void*, MoeLayerError> handle_for(MoeExecutionConvention convention, bool with_shared) const;
+};
+
+// ---- registry and graph op --------------------------------------------------------------------
+// Process-global, grow-only, ids stable per process (src/moe/graph_op.rs:221-232).
+uint32_t register_real_moe_layer(RealMoeLayer layer);
+std::shared_ptr<const RealMoeLayer> get_real_moe_layer(uint32_t layer_id);
+Result<std::vector<float>, MoeLayerError> execute_real_moe_layer(uint32_t layer_id,
+                                                                 const std::vector<float>& input);
+Result<std::vector<float>, MoeLayerError> execute_real_moe_layer_with(
+    uint32_t layer_id, const std::vector<float>& input, MoeExecutionConvention convention);
+// The executor arm of NodeType::MoeRealLayerReference{layer_id}: returns the output tensor's data
+// or throws std::runtime_error("MoeRealLayerReference: forward failed (unknown layer_id or bad
+// input dim)") as the reference panics.
+std::vector<float> moe_real_layer_reference_node(uint32_t layer_id, const std::vector<float>& input);
+
+// ---- template members -------------------------------------------------------------------------
+}  // namespace moe
+}  // namespace atenia
+
+#include <stdexcept>
+namespace atenia {
+namespace moe {
+template <typename T, typename E>
+T Result<T, E>::unwrap() const {
+  if (!is_ok()) throw std::runtime_error("called `Result::unwrap()` on an `Err` value: " + e_->to_string());
+  return *v_;
+}
+template <typename T, typename E>
+T Result<T, E>::expect(const char* msg) const {
+  if (!is_ok()) throw std::runtime_error(std::string(msg) + ": " + e_->to_string());
+  return *v_;
+}
+}  // namespace moe
+}  // namespace atenia

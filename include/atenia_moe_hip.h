@@ -19,7 +19,8 @@
  *                                                        KExceedsExperts, src/moe/sparse.rs:35-50)
  *   -3  a routing weight is not finite                  (MoeSparseError::NonFiniteWeight{index},
  *                                                        src/moe/sparse.rs:156-160); token and
- *                                                        expert via atenia_moe_hip_layer_status
+ *                                                        expert via ..._layer_status (device
+ *                                                        entry points) or ..._last_non_finite
  *   -4  out of device memory
  *   -5  invalid handle / unknown layer                  (MoeBindingError::LayerNotFound)
  *   -6  configuration not supported by this build
@@ -140,6 +141,12 @@ int atenia_moe_hip_layer_forward_device(AteniaMoeLayer* layer, const void* d_x, 
  * first offending token / expert (either pointer may be NULL). */
 int atenia_moe_hip_layer_status(AteniaMoeLayer* layer, void* stream, int32_t* token,
                                 int32_t* expert);
+
+/* Where the most recent ATENIA_MOE_ERR_NON_FINITE of this handle was found: token (row of the
+ * batch) and expert index, -1 / -1 if none was ever reported.  The index is the `index` of the
+ * reference's MoeSparseError::NonFiniteWeight (src/moe/sparse.rs:41-42, 150-158); the host
+ * entry points consume the device status themselves, so this is how their caller learns it. */
+int atenia_moe_hip_layer_last_non_finite(AteniaMoeLayer* layer, int32_t* token, int32_t* expert);
 
 /* Parity taps -------------------------------------------------------------------------- */
 

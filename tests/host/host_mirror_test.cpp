@@ -1,0 +1,343 @@
+// Tests of the C++ host mirror, written after the reference's own tests of the same interface:
+//   tests/moe_real_layer_graph_op_test.rs  (graph op == forward_auto, determinism, unknown id,
+//                                            bad input dim, explicit convention)
+//   src/moe/layer.rs tests                 (config validation, convention resolution)
+//   src/moe/binding.rs:611-640             (identical experts reproduce a single expert)
+// The expected values come from the committed golden fixtures (written to a flat file by the
+// pytest wrapper) and from the CPU oracle, which this test links as the checker.
+//
+// usage: host_mirror_test <fixtures.bin> [--no-gpu]
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <functional>
+#include <string>
+#include <vector>
+
+#include "../../ateniaengine_amd/host/atenia_moe.hpp"
+
+using namespace atenia::moe;
+
+// ---- the oracle's C interface (oracle/moe_oracle.c) -------------------------------------------
+extern "C" {
+typedef struct {
+  int32_t num_experts, top_k, d_model, d_ff, d_ff_shared, convention;
+  const float *w_router, *router_bias, *w_gate, *w_up, *w_down, *s_gate, *s_up, *s_down, *shared_gate;
+} OraLayer;
+int ora_layer_forward_with(const OraLayer* L, const float* x, int convention, int policy, float* out,
+                           int32_t* idx_out, float* w_out, int32_t* err_index);
+void ora_expert_forward(const float* w_gate, const float* w_up, const float* w_down, size_t d, size_t f,
+                        const float* x, float* out, int policy);
+void ora_seeded(uint64_t seed, size_t n, float* out);
+}
+
+static int g_failed = 0, g_run = 0;
+#define CHECK(cond, ...)                                         \
+  do {                                                           \
+    if (!(cond)) {                                               \
+      printf("    CHECK FAILED %s:%d: %s -- ", __FILE__, __LINE__, #cond); \
+      printf(__VA_ARGS__);                                       \
+      printf("\n");                                              \
+      throw std::runtime_error("check failed");                  \
+    }                                                            \
+  } while (0)
+
+static void run_test(const char* name, const std::function<void()>& fn) {
+  ++g_run;
+  try {
+    fn();
+    printf("ok   %s\n", name);
+  } catch (const std::exception& e) {
+    ++g_failed;
+    printf("FAIL %s: %s\n", name, e.what());
+  }
+  fflush(stdout);
+}
+
+struct Metrics {  // src/moe/numerical.rs:58-88
+  double max_abs_diff = 0, mean_abs_diff = 0, rmse = 0;
+  bool argmax_match = false;
+};
+static Metrics metrics(const std::vector<float>& a, const std::vector<float>& r) {
+  Metrics m;
+  size_t ia = 0, ir = 0;
+  double sum = 0, sq = 0;
+  for (size_t i = 0; i < a.size(); ++i) {
+    double d = std::fabs((double)a[i] - (double)r[i]);
+    m.max_abs_diff = std::max(m.max_abs_diff, d);
+    sum += d;
+    sq += d * d;
+    if ((double)a[i] > (double)a[ia]) ia = i;
+    if ((double)r[i] > (double)r[ir]) ir = i;
+  }
+  m.mean_abs_diff = sum / a.size();
+  m.rmse = std::sqrt(sq / a.size());
+  m.argmax_match = ia == ir;
+  return m;
+}
+
+// ---- fixtures ---------------------------------------------------------------------------------
+struct Fixture {
+  std::string name;
+  int E, k, d, f, fs, gated;
+  std::vector<float> w_router, gate, up, down, s_gate, s_up, s_down, shared_gate, input, atenia_ref, hf_ref;
+};
+
+static std::vector<Fixture> load_fixtures(const char* path) {
+  std::vector<Fixture> out;
+  FILE* fp = fopen(path, "rb");
+  if (!fp) return out;
+  int32_t n = 0;
+  if (fread(&n, 4, 1, fp) != 1) n = 0;
+  for (int i = 0; i < n; ++i) {
+    Fixture fx;
+    char nm[32];
+    int32_t h[6];
+    if (fread(nm, 1, 32, fp) != 32 || fread(h, 4, 6, fp) != 6) break;
+    fx.name = nm;
+    fx.E = h[0]; fx.k = h[1]; fx.d = h[2]; fx.f = h[3]; fx.fs = h[4]; fx.gated = h[5];
+    auto rd = [&](std::vector<float>& v, size_t cnt) {
+      v.resize(cnt);
+      if (cnt && fread(v.data(), 4, cnt, fp) != cnt) v.clear();
+    };
+    const size_t E = fx.E, d = fx.d, f = fx.f, fs = fx.fs;
+    rd(fx.w_router, E * d); rd(fx.gate, E * f * d); rd(fx.up, E * f * d); rd(fx.down, E * d * f);
+    rd(fx.s_gate, fs * d); rd(fx.s_up, fs * d); rd(fx.s_down, d * fs);
+    rd(fx.shared_gate, fx.gated ? d : 0);
+    rd(fx.input, d); rd(fx.atenia_ref, d); rd(fx.hf_ref, d);
+    out.push_back(std::move(fx));
+  }
+  fclose(fp);
+  return out;
+}
+
+static RealMoeLayer layer_from(const Fixture& fx, MoeWeightStorage st = MoeWeightStorage::F32) {
+  const size_t E = fx.E, d = fx.d, f = fx.f, fs = fx.fs;
+  auto cfg = MoeLayerConfig::make(E, fx.k, fs > 0, d, f).unwrap();
+  std::vector<MoeDenseExpert> ex;
+  for (size_t e = 0; e < E; ++e) {
+    auto sl = [&](const std::vector<float>& v, size_t per) {
+      return std::vector<float>(v.begin() + e * per, v.begin() + (e + 1) * per);
+    };
+    ex.push_back(MoeDenseExpert::make(d, f, sl(fx.gate, f * d), sl(fx.up, f * d), sl(fx.down, d * f)).unwrap());
+  }
+  auto routed = MoeDenseLayer::make(d, f, fx.w_router, std::move(ex), fx.k).unwrap();
+  std::optional<MoeDenseExpert> shared;
+  if (fs) shared = MoeDenseExpert::make(d, fs, fx.s_gate, fx.s_up, fx.s_down).unwrap();
+  std::optional<std::vector<float>> sg;
+  if (fx.gated) sg = fx.shared_gate;
+  return RealMoeLayer::assemble(cfg, std::move(routed), std::move(shared), std::move(sg), st).unwrap();
+}
+
+// The reference's synthetic fixture generator (dense.rs:368-379) through the oracle's restatement.
+static std::vector<float> seeded(uint64_t seed, size_t n) {
+  std::vector<float> v(n);
+  ora_seeded(seed, n, v.data());
+  return v;
+}
+static Fixture synthetic(int E, int k, int d, int f, bool identical = false) {
+  Fixture fx;
+  fx.name = "synthetic";
+  fx.E = E; fx.k = k; fx.d = d; fx.f = f; fx.fs = 0; fx.gated = 0;
+  fx.w_router = seeded(1, (size_t)E * d);
+  for (int e = 0; e < E; ++e) {
+    const uint64_t s = identical ? 100 : 100 + 10 * e;
+    auto g = seeded(s, (size_t)f * d), u = seeded(s + 1, (size_t)f * d), dn = seeded(s + 2, (size_t)d * f);
+    fx.gate.insert(fx.gate.end(), g.begin(), g.end());
+    fx.up.insert(fx.up.end(), u.begin(), u.end());
+    fx.down.insert(fx.down.end(), dn.begin(), dn.end());
+  }
+  fx.input = seeded(7, d);
+  return fx;
+}
+static OraLayer ora_of(const Fixture& fx, int conv) {
+  OraLayer L;
+  memset(&L, 0, sizeof(L));
+  L.num_experts = fx.E; L.top_k = fx.k; L.d_model = fx.d; L.d_ff = fx.f; L.d_ff_shared = fx.fs;
+  L.convention = conv;
+  L.w_router = fx.w_router.data(); L.w_gate = fx.gate.data(); L.w_up = fx.up.data(); L.w_down = fx.down.data();
+  if (fx.fs) { L.s_gate = fx.s_gate.data(); L.s_up = fx.s_up.data(); L.s_down = fx.s_down.data(); }
+  if (fx.gated) L.shared_gate = fx.shared_gate.data();
+  return L;
+}
+
+int main(int argc, char** argv) {
+  const bool no_gpu = argc > 2 && !strcmp(argv[2], "--no-gpu");
+  std::vector<Fixture> fixtures = argc > 1 ? load_fixtures(argv[1]) : std::vector<Fixture>();
+  auto find = [&](const char* n) -> const Fixture* {
+    for (auto& f : fixtures) if (f.name == n) return &f;
+    return nullptr;
+  };
+
+  // ---- host logic (no device needed) --------------------------------------------------------
+  run_test("config_validation_errors", [] {
+    CHECK(MoeLayerConfig::make(0, 1, false, 4, 4).error().kind == MoeConfigError::ZeroExperts, "kind");
+    CHECK(MoeLayerConfig::make(4, 0, false, 4, 4).error().kind == MoeConfigError::ZeroExpertsPerToken, "kind");
+    auto e = MoeLayerConfig::make(2, 3, false, 4, 4).error();
+    CHECK(e.kind == MoeConfigError::ExpertsPerTokenExceedsCount && e.per_token == 3 && e.total == 2, "payload");
+    CHECK(MoeLayerConfig::make(2, 1, false, 0, 4).error().kind == MoeConfigError::ZeroDModel, "kind");
+    CHECK(MoeLayerConfig::make(2, 1, false, 4, 0).error().kind == MoeConfigError::ZeroDFf, "kind");
+    CHECK(MoeLayerConfig::make(8, 2, true, 64, 128).is_ok(), "valid config rejected");
+  });
+  run_test("expert_and_layer_shape_errors", [] {
+    auto e = MoeDenseExpert::make(4, 8, std::vector<float>(31), std::vector<float>(32), std::vector<float>(32));
+    CHECK(e.is_err() && e.error().kind == MoeDenseError::WeightShapeMismatch, "kind");
+    CHECK(e.error().to_string() == "moe-dense: w_gate weight shape mismatch: expected 32 elems, got 31", "%s",
+          e.error().to_string().c_str());
+    auto l = MoeDenseLayer::make(4, 8, std::vector<float>(8), {}, 1);
+    CHECK(l.is_err() && l.error().kind == MoeDenseError::NoExperts, "kind");
+    auto ex = MoeDenseExpert::make(4, 8, std::vector<float>(32), std::vector<float>(32), std::vector<float>(32)).unwrap();
+    auto l2 = MoeDenseLayer::make(4, 8, std::vector<float>(12), {ex, ex}, 1);
+    CHECK(l2.is_err() && l2.error().kind == MoeDenseError::RouterExpertCountMismatch, "kind");
+  });
+  run_test("assemble_cross_checks_config", [] {
+    Fixture fx = synthetic(4, 2, 8, 16);
+    RealMoeLayer ok = layer_from(fx);
+    CHECK(ok.num_experts() == 4 && !ok.has_shared_expert(), "topology");
+    CHECK(ok.resolve_convention() == MoeExecutionConvention::Atenia, "no gate => Atenia");
+    auto cfg = MoeLayerConfig::make(5, 2, false, 8, 16).unwrap();
+    auto bad = RealMoeLayer::assemble(cfg, ok.routed, std::nullopt, std::nullopt);
+    CHECK(bad.is_err() && bad.error().kind == MoeLayerError::ConfigMismatch, "kind");
+    CHECK(bad.error().detail == "resolved 4 experts but config.num_experts = 5", "%s", bad.error().detail.c_str());
+    auto cfg2 = MoeLayerConfig::make(4, 2, true, 8, 16).unwrap();
+    CHECK(RealMoeLayer::assemble(cfg2, ok.routed, std::nullopt, std::nullopt).is_err(), "missing shared accepted");
+  });
+  run_test("graph_real_moe_layer_rejects_unknown_layer", [] {
+    auto r = execute_real_moe_layer(0xffffffffu, std::vector<float>(64, 0.f));
+    CHECK(r.is_err() && r.error().kind == MoeLayerError::Binding &&
+              r.error().binding.kind == MoeBindingError::LayerNotFound, "kind");
+    CHECK(r.error().binding.layer_id == 0xffffffffu, "layer id");
+    bool thrown = false;
+    try {
+      moe_real_layer_reference_node(0xffffffffu, std::vector<float>(64, 0.f));
+    } catch (const std::runtime_error& e) {
+      thrown = strstr(e.what(), "unknown layer_id") != nullptr;
+    }
+    CHECK(thrown, "node did not fail loudly with the reference's message");
+  });
+  run_test("graph_real_moe_layer_rejects_bad_input_dim", [] {
+    uint32_t id = register_real_moe_layer(layer_from(synthetic(4, 2, 8, 16)));
+    auto r = execute_real_moe_layer(id, std::vector<float>(5, 0.f));
+    CHECK(r.is_err() && r.error().kind == MoeLayerError::Sparse &&
+              r.error().sparse.kind == MoeSparseError::Dense &&
+              r.error().sparse.dense.kind == MoeDenseError::DimMismatch, "kind");
+    CHECK(r.error().sparse.dense.expected == 8 && r.error().sparse.dense.actual == 5, "payload");
+    bool thrown = false;
+    try { moe_real_layer_reference_node(id, std::vector<float>(5, 0.f)); } catch (const std::runtime_error&) { thrown = true; }
+    CHECK(thrown, "node accepted a bad input dim");
+    CHECK(get_real_moe_layer(id) != nullptr && get_real_moe_layer(id + 1000) == nullptr, "registry lookup");
+  });
+  if (no_gpu) {
+    run_test("forward_without_device_fails_loudly", [] {
+      RealMoeLayer l = layer_from(synthetic(4, 2, 8, 16));
+      auto r = l.forward_auto(seeded(3, 8));
+      CHECK(r.is_err() && r.error().kind == MoeLayerError::Device, "a forward without a GPU must be a Device error");
+    });
+    printf("%d tests, %d failed\n", g_run, g_failed);
+    return g_failed ? 1 : 0;
+  }
+
+  // ---- device path ----------------------------------------------------------------------------
+  const Fixture* mix = find("mixtral_layer0");
+  const Fixture* q15 = find("qwen15_moe_layer0");
+  run_test("fixtures_present", [&] { CHECK(mix && q15, "fixture file missing or truncated"); });
+  if (!mix || !q15) return 1;
+
+  run_test("graph_real_moe_layer_matches_reference", [&] {
+    RealMoeLayer layer = layer_from(*mix);
+    auto reference = layer.forward_auto(mix->input).unwrap();
+    uint32_t id = register_real_moe_layer(layer);
+    auto got = moe_real_layer_reference_node(id, mix->input);
+    Metrics m = metrics(got, reference);
+    CHECK(m.max_abs_diff < 1e-5, "graph vs forward_auto: %g", m.max_abs_diff);
+    Metrics mhf = metrics(got, mix->hf_ref);
+    CHECK(mhf.argmax_match && mhf.max_abs_diff < 0.5, "graph vs HF: %g", mhf.max_abs_diff);
+    Metrics ma = metrics(got, mix->atenia_ref);  // the fixture's f64 reference, much tighter
+    CHECK(ma.max_abs_diff < 1e-5, "graph vs f64 reference: %g", ma.max_abs_diff);
+  });
+  run_test("graph_real_moe_layer_is_deterministic", [&] {
+    uint32_t id = register_real_moe_layer(layer_from(*mix));
+    auto a = moe_real_layer_reference_node(id, mix->input), b = moe_real_layer_reference_node(id, mix->input);
+    CHECK(a == b, "two runs differ");
+    for (float v : a) CHECK(std::isfinite(v), "non-finite output");
+  });
+  run_test("graph_real_moe_layer_with_explicit_convention", [&] {
+    RealMoeLayer layer = layer_from(*mix);
+    auto direct = layer.forward_auto(mix->input).unwrap();
+    uint32_t id = register_real_moe_layer(layer);
+    auto via = execute_real_moe_layer_with(id, mix->input, MoeExecutionConvention::Atenia).unwrap();
+    CHECK(via == direct, "explicit Atenia convention differs from forward_auto on a layer without gate");
+  });
+  run_test("qwen_convention_auto_resolved", [&] {
+    RealMoeLayer layer = layer_from(*q15);
+    CHECK(layer.has_shared_expert() && layer.resolve_convention() == MoeExecutionConvention::HuggingFaceQwen,
+          "gate present => HuggingFaceQwen");
+    auto hf = layer.forward_auto(q15->input).unwrap();
+    CHECK(metrics(hf, q15->hf_ref).max_abs_diff < 1e-5, "HuggingFaceQwen vs hf_ref: %g",
+          metrics(hf, q15->hf_ref).max_abs_diff);
+    auto at = layer.forward(q15->input).unwrap();
+    CHECK(metrics(at, q15->atenia_ref).max_abs_diff < 1e-5, "Atenia vs atenia_ref: %g",
+          metrics(at, q15->atenia_ref).max_abs_diff);
+    CHECK(metrics(at, hf).max_abs_diff > 1e-7, "the two conventions must differ on this layer");
+  });
+  run_test("batch_equals_rows_and_oracle", [&] {
+    Fixture fx = synthetic(4, 2, 8, 16);
+    RealMoeLayer layer = layer_from(fx);
+    uint32_t id = register_real_moe_layer(layer);
+    const int T = 5, d = fx.d;
+    std::vector<float> x = seeded(11, (size_t)T * d);
+    auto batch = execute_real_moe_layer(id, x).unwrap();
+    std::vector<int32_t> idx;
+    auto w = layer.route(x, MoeExecutionConvention::Atenia, &idx).unwrap();
+    OraLayer ol = ora_of(fx, 0);
+    for (int t = 0; t < T; ++t) {
+      std::vector<float> row(x.begin() + t * d, x.begin() + (t + 1) * d), want(d), ow(fx.k);
+      std::vector<int32_t> oi(fx.k);
+      int32_t err = 0;
+      CHECK(ora_layer_forward_with(&ol, row.data(), 0, 0, want.data(), oi.data(), ow.data(), &err) == 0, "oracle");
+      auto one = execute_real_moe_layer(id, row).unwrap();
+      std::vector<float> brow(batch.begin() + t * d, batch.begin() + (t + 1) * d);
+      CHECK(metrics(one, want).max_abs_diff < 1e-5, "row %d vs oracle: %g", t, metrics(one, want).max_abs_diff);
+      CHECK(metrics(brow, one).max_abs_diff < 1e-6, "row %d of the batch vs the row alone", t);
+      for (int s = 0; s < fx.k; ++s) {
+        CHECK(idx[t * fx.k + s] == oi[s], "row %d slot %d routed to %d, oracle %d", t, s, idx[t * fx.k + s], oi[s]);
+        CHECK(std::fabs(w[t * fx.k + s] - ow[s]) <= 1.2e-7f * std::fabs(ow[s]), "routing weight");
+      }
+    }
+  });
+  run_test("identical_experts_reproduce_single_expert", [&] {
+    Fixture fx = synthetic(4, 2, 8, 16, true);
+    RealMoeLayer layer = layer_from(fx);
+    auto out = layer.forward_routed(fx.input).unwrap();
+    std::vector<float> want(fx.d);
+    ora_expert_forward(fx.gate.data(), fx.up.data(), fx.down.data(), fx.d, fx.f, fx.input.data(), want.data(), 0);
+    CHECK(metrics(out, want).max_abs_diff < 1e-5, "renormalised combine of identical experts: %g",
+          metrics(out, want).max_abs_diff);
+  });
+  run_test("non_finite_input_surfaces_as_sparse_error", [&] {
+    Fixture fx = synthetic(4, 2, 8, 16);
+    RealMoeLayer layer = layer_from(fx);
+    std::vector<float> x = seeded(5, 3 * 8);
+    x[8 + 2] = NAN;  // token 1
+    auto r = layer.forward_auto(x);
+    CHECK(r.is_err() && r.error().kind == MoeLayerError::Sparse &&
+              r.error().sparse.kind == MoeSparseError::NonFiniteWeight, "kind");
+    CHECK(r.error().sparse.token == 1 && r.error().sparse.index == 0, "token %zu index %zu", r.error().sparse.token,
+          r.error().sparse.index);
+    CHECK(r.error().to_string() == "moe-layer: moe-sparse: routing weight at 0 is non-finite", "%s",
+          r.error().to_string().c_str());
+    CHECK(layer.forward_auto(seeded(5, 8)).is_ok(), "the handle must stay usable after an error");
+  });
+  run_test("bf16_and_int8_storage_track_f32", [&] {
+    auto f32 = layer_from(*mix).forward_auto(mix->input).unwrap();
+    double scale = 0;
+    for (float v : mix->atenia_ref) scale = std::max(scale, (double)std::fabs(v));
+    auto b16 = layer_from(*mix, MoeWeightStorage::Bf16).forward_auto(mix->input).unwrap();
+    auto i8 = layer_from(*mix, MoeWeightStorage::Int8W8A16).forward_auto(mix->input).unwrap();
+    CHECK(metrics(b16, f32).max_abs_diff <= 3e-2 * scale, "bf16 storage: %g of %g", metrics(b16, f32).max_abs_diff, scale);
+    CHECK(metrics(i8, f32).max_abs_diff <= 3e-2 * scale, "int8 storage: %g of %g", metrics(i8, f32).max_abs_diff, scale);
+  });
+  printf("%d tests, %d failed\n", g_run, g_failed);
+  return g_failed ? 1 : 0;
+}
