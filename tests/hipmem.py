@@ -1,0 +1,61 @@
+"""Device buffers for tests through the HIP runtime itself (ctypes on libamdhip64), so that tests
+of the device-pointer entry points need nothing but the library under test and the runtime."""
+import ctypes as C
+
+import numpy as np
+
+_hip = None
+
+
+def hip():
+    global _hip
+    if _hip is None:
+        _hip = C.CDLL("libamdhip64.so")
+        _hip.hipMalloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
+        _hip.hipFree.argtypes = [C.c_void_p]
+        _hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+        _hip.hipMemset.argtypes = [C.c_void_p, C.c_int, C.c_size_t]
+    return _hip
+
+
+class DeviceArray:
+    """A device allocation with a NumPy dtype/shape; `.ptr` is the raw device pointer."""
+
+    def __init__(self, shape, dtype, fill=None):
+        self.shape, self.dtype = tuple(shape), np.dtype(dtype)
+        self.nbytes = int(np.prod(self.shape)) * self.dtype.itemsize
+        p = C.c_void_p()
+        rc = hip().hipMalloc(C.byref(p), max(self.nbytes, 4))
+        if rc:
+            raise RuntimeError(f"hipMalloc failed: {rc}")
+        self.ptr = p.value
+        if fill is not None:
+            hip().hipMemset(self.ptr, fill, self.nbytes)
+
+    @classmethod
+    def from_host(cls, a):
+        a = np.ascontiguousarray(a)
+        d = cls(a.shape, a.dtype)
+        rc = hip().hipMemcpy(d.ptr, a.ctypes.data, a.nbytes, 1)  # hipMemcpyHostToDevice
+        if rc:
+            raise RuntimeError(f"hipMemcpy H2D failed: {rc}")
+        return d
+
+    def to_host(self):
+        out = np.empty(self.shape, self.dtype)
+        rc = hip().hipDeviceSynchronize()
+        rc = rc or hip().hipMemcpy(out.ctypes.data, self.ptr, self.nbytes, 2)  # DeviceToHost
+        if rc:
+            raise RuntimeError(f"hipMemcpy D2H failed: {rc}")
+        return out
+
+    def free(self):
+        if self.ptr:
+            hip().hipFree(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass

@@ -8,6 +8,7 @@ import pytest
 
 from ateniaengine_amd import capi
 from tests import synth as S
+from tests.hipmem import DeviceArray
 
 pytestmark = pytest.mark.gpu
 
@@ -23,58 +24,55 @@ def _layer(ora, wd, gated):
                                       (capi.WEIGHT_INT8_W8A16, False), (capi.WEIGHT_F32, True)])
 @pytest.mark.parametrize("T", [1, 19, 300])
 def test_stages_equal_pipeline(ora, wd, gated, T):
-    import torch
-
     oL, gL = _layer(ora, wd, gated)
     with gL:
         E, k, d = oL.E, oL.top_k, oL.d
         x = S.make_tokens(500 + T, T, d, bf16=wd != capi.WEIGHT_F32)
-        dx = torch.from_numpy(x).cuda()
-        whole = torch.empty((T, d), dtype=torch.float32, device="cuda")
-        gL.forward_device(dx.data_ptr(), capi.ACT_F32, T, whole.data_ptr())
-        torch.cuda.synchronize()
+        dx = DeviceArray.from_host(x)
+        whole = DeviceArray((T, d), np.float32, fill=0)
+        gL.forward_device(dx.ptr, capi.ACT_F32, T, whole.ptr)
         assert gL.status()[0] == 0
+        want = whole.to_host()
 
-        idx = torch.empty((T, k), dtype=torch.int32, device="cuda")
-        w = torch.empty((T, k), dtype=torch.float32, device="cuda")
-        counts = torch.empty((E,), dtype=torch.int32, device="cuda")
-        offsets = torch.empty((E + 1,), dtype=torch.int32, device="cuda")
-        perm = torch.empty((T * k,), dtype=torch.int32, device="cuda")
-        staged = torch.zeros((T, d), dtype=torch.float32, device="cuda")
-        gL.router_device(dx.data_ptr(), capi.ACT_F32, T, idx.data_ptr(), w.data_ptr())
-        gL.permute_device(T, counts.data_ptr(), offsets.data_ptr(), perm.data_ptr())
-        gL.expert_ffn_device(dx.data_ptr(), capi.ACT_F32, T)
-        gL.combine_device(T, staged.data_ptr())
-        torch.cuda.synchronize()
-        assert torch.equal(staged, whole), "stages composed differ from the pipeline"
+        idx = DeviceArray((T, k), np.int32)
+        w = DeviceArray((T, k), np.float32)
+        counts = DeviceArray((E,), np.int32)
+        offsets = DeviceArray((E + 1,), np.int32)
+        perm = DeviceArray((T * k,), np.int32)
+        staged = DeviceArray((T, d), np.float32, fill=0)
+        gL.router_device(dx.ptr, capi.ACT_F32, T, idx.ptr, w.ptr)
+        gL.permute_device(T, counts.ptr, offsets.ptr, perm.ptr)
+        gL.expert_ffn_device(dx.ptr, capi.ACT_F32, T)
+        gL.combine_device(T, staged.ptr)
+        assert staged.to_host().tobytes() == want.tobytes(), "stages composed differ from the pipeline"
+        ref = oL.execute(x)[0] if wd == capi.WEIGHT_F32 else None
+        if ref is not None:  # f32 layers: also against the certified CPU path itself
+            assert S.rel_err(want, ref) <= 1e-5
 
         h_idx, h_w = gL.route(x)
-        assert np.array_equal(idx.cpu().numpy(), h_idx)
-        assert np.array_equal(w.cpu().numpy().view(np.int32), h_w.view(np.int32))
+        assert np.array_equal(idx.to_host(), h_idx)
+        assert np.array_equal(w.to_host().view(np.int32), h_w.view(np.int32))
         oc, oo, op = ora.permute(h_idx, E)
-        assert np.array_equal(counts.cpu().numpy(), oc)
-        assert np.array_equal(offsets.cpu().numpy(), oo)
-        assert np.array_equal(perm.cpu().numpy(), op)
+        assert np.array_equal(counts.to_host(), oc)
+        assert np.array_equal(offsets.to_host(), oo)
+        assert np.array_equal(perm.to_host(), op)
 
 
 def test_stage_order_is_enforced(ora):
-    import torch
-
     oL, gL = _layer(ora, capi.WEIGHT_BF16, False)
     with gL:
         T, d = 5, oL.d
-        x = torch.from_numpy(S.make_tokens(9, T, d, bf16=True)).cuda()
-        out = torch.empty((T, d), dtype=torch.float32, device="cuda")
+        x = DeviceArray.from_host(S.make_tokens(9, T, d, bf16=True))
+        out = DeviceArray((T + 1, d), np.float32, fill=0)
         with pytest.raises(capi.MoeHipError) as e:
-            gL.combine_device(T, out.data_ptr())
+            gL.combine_device(T, out.ptr)
         assert e.value.rc == -1
-        gL.router_device(x.data_ptr(), capi.ACT_F32, T)
+        gL.router_device(x.ptr, capi.ACT_F32, T)
         with pytest.raises(capi.MoeHipError):
-            gL.expert_ffn_device(x.data_ptr(), capi.ACT_F32, T)  # permute has not run
+            gL.expert_ffn_device(x.ptr, capi.ACT_F32, T)  # permute has not run
         gL.permute_device(T)
         with pytest.raises(capi.MoeHipError):
-            gL.combine_device(T + 1, out.data_ptr())  # other token count
-        gL.expert_ffn_device(x.data_ptr(), capi.ACT_F32, T)
-        gL.combine_device(T, out.data_ptr())
-        torch.cuda.synchronize()
-        assert torch.isfinite(out).all()
+            gL.combine_device(T + 1, out.ptr)  # other token count
+        gL.expert_ffn_device(x.ptr, capi.ACT_F32, T)
+        gL.combine_device(T, out.ptr)
+        assert np.isfinite(out.to_host()).all()
