@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MoE layer hot path on one MI355X.
 
-Workload (BASELINE config 2): Mixtral-8x7B-shape layer, d_model 4096, 8 experts, top-2 with
+Workload (the headline configuration): Mixtral-8x7B-shape layer, d_model 4096, 8 experts, top-2 with
 renormalisation, expert d_ff 14336, bf16 weights resident in HBM (2.8 GB), bf16 activations
 already on the device.  A step is one layer forward over one batch of T tokens through the
 C ABI (`atenia_moe_hip_layer_forward_device`).  The default run times the prefill point
@@ -22,8 +22,8 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-# BASELINE configs.  The headline metric is quoted on mixtral_bf16; the others are reported
-# with --config for the tables in DESIGN.md.
+# Benchmark configurations.  The headline metric is quoted on mixtral_bf16; the others are
+# reported with --config.
 CONFIGS = {
     "mixtral_bf16": dict(d=4096, E=8, k=2, f=14336, fs=0, gated=False, conv=0, wd="bf16",
                          zipf=False, sweep=(1, 16, 128, 512, 4096)),

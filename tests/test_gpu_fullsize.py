@@ -1,4 +1,4 @@
-"""GPU parity at the full BASELINE shapes (configs 1-5), through the C ABI.
+"""GPU parity at the full benchmark shapes (configurations 1-5), through the C ABI.
 
 Per config and batch size: routing indices, per-expert counts, offsets and permutation are
 compared bit for bit with the CPU oracle for EVERY token; layer outputs are compared with the
