@@ -78,6 +78,21 @@ __device__ inline uint16_t bf16_rne(float f) {
   return (uint16_t)(u >> 16);
 }
 
+// Two f32 -> two bf16 (round to nearest even) in one v_cvt_pk_bf16_f32; low half = a.
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+__device__ inline uint32_t bf16_rne_pair(float a, float b) {
+  f32x2_t v = {a, b};
+  bf16x2_t h = __builtin_convertvector(v, bf16x2_t);
+  return *(uint32_t*)&h;
+}
+
+// silu(g) * u with the hardware exp2 / rcp (1 ulp each; the result is rounded to bf16 next).
+__device__ inline float swiglu_fast(float g, float u) {
+  const float t = __builtin_amdgcn_exp2f(g * -1.4426950408889634f);
+  return g * __builtin_amdgcn_rcpf(1.f + t) * u;
+}
+
 __device__ inline uint32_t pack_i8_pair(uint32_t w, int sh) {
   float f0 = (float)(int8_t)((w >> sh) & 0xff);
   float f1 = (float)(int8_t)((w >> (sh + 8)) & 0xff);
@@ -611,12 +626,13 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
+        for (int r = 0; r < 16; r += 2) {  // rows m and m + 1
           const int m = i * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
-          const float g = acc[i][j][r];
-          const float u = acc[i][j + 2][r];
-          const float hv = g * __builtin_amdgcn_rcpf(1.f + __expf(-g)) * u;
-          *(uint16_t*)(stage + m * kPitch + (j * 32 + l32) * 2) = bf16_rne(hv);
+          const uint32_t hh = bf16_rne_pair(swiglu_fast(acc[i][j][r], acc[i][j + 2][r]),
+                                            swiglu_fast(acc[i][j][r + 1], acc[i][j + 2][r + 1]));
+          char* dst = stage + m * kPitch + (j * 32 + l32) * 2;
+          *(uint16_t*)dst = (uint16_t)hh;
+          *(uint16_t*)(dst + kPitch) = (uint16_t)(hh >> 16);
         }
       }
     }
@@ -635,13 +651,24 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p)
     }
   } else {
     float* y = (float*)p.out + (size_t)part * p.out_part_stride;
+    // The pair id of every row first, in one batch of loads: fetched next to the stores they
+    // address, each would wait out its own L2 round trip (the compiler cannot move a load of
+    // perm above a store to y).
+    int pair_of[4][16];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = wm * 128 + i * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
+        pair_of[i][r] = p.g.perm[base + tm0 + min(m, rows_here - 1)];
+      }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int m = wm * 128 + i * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
         if (m >= rows_here) continue;
-        const int pair = p.g.perm[base + tm0 + m];
+        const int pair = pair_of[i][r];
         if (p.part_flags && part == 0 && wn == 0 && l32 == 0)
           p.part_flags[(size_t)pair * p.n_col_tiles + ct] = (uint8_t)n_parts;
         float* yr = y + (size_t)pair * p.out_stride;
@@ -865,12 +892,14 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_i8_kernel(TiledParams
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
+        for (int r = 0; r < 16; r += 2) {  // rows m and m + 1
           const int m = i * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
-          const float g = acc[i][j][r] * sg;
-          const float u = acc[i][j + 2][r] * su;
-          const float hv = g * __builtin_amdgcn_rcpf(1.f + __expf(-g)) * u;
-          *(uint16_t*)(stage + m * kPitch + (j * 32 + l32) * 2) = bf16_rne(hv);
+          const uint32_t hh =
+              bf16_rne_pair(swiglu_fast(acc[i][j][r] * sg, acc[i][j + 2][r] * su),
+                            swiglu_fast(acc[i][j][r + 1] * sg, acc[i][j + 2][r + 1] * su));
+          char* dst = stage + m * kPitch + (j * 32 + l32) * 2;
+          *(uint16_t*)dst = (uint16_t)hh;
+          *(uint16_t*)(dst + kPitch) = (uint16_t)(hh >> 16);
         }
       }
     }
@@ -892,13 +921,21 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_i8_kernel(TiledParams
 #pragma unroll
     for (int j = 0; j < 4; ++j)
       sd[j] = p.sa[(size_t)e * p.n_rows + min(nb0 * 16 + (4 * wn + j) * 32 + l32, p.n_rows - 1)];
+    int pair_of[4][16];  // all pair ids first, in one batch of loads (see the bf16 kernel)
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = wm * 128 + i * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
+        pair_of[i][r] = p.g.perm[base + tm0 + min(m, rows_here - 1)];
+      }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int m = wm * 128 + i * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
         if (m >= rows_here) continue;
-        const int pair = p.g.perm[base + tm0 + m];
+        const int pair = pair_of[i][r];
         if (p.part_flags && part == 0 && wn == 0 && l32 == 0)
           p.part_flags[(size_t)pair * p.n_col_tiles + ct] = (uint8_t)n_parts;
         float* yr = y + (size_t)pair * p.out_stride;
