@@ -433,23 +433,6 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p)
   constexpr int BROWS = UP ? 128 : 256;
   const int nb0 = ct * (BROWS / 16);
 
-  // A stage: 256 rows x 64 k as 32 chunks of 8 rows x 128 bytes, so that one load instruction
-  // reads eight full 128-byte lines.  Row r, 16-byte segment s of chunk c is stored at slot
-  // 8r + (s ^ r ^ (c & 1)); lane l of the filling load fetches row l/8, segment
-  // (l%8) ^ (l/8) ^ (c&1).  Wave w fills chunks 8w .. 8w+7, four per step.
-  const uint16_t* arow[8];
-  {
-    const int r8 = lane >> 3, pslot = lane & 7;
-#pragma unroll
-    for (int q = 0; q < 8; ++q) {
-      int m = (wave * 8 + q) * 8 + r8;
-      if (m >= rows_here) m = 0;
-      int src;
-      if (UP) src = p.g.perm[base + tm0 + m] / p.g.pair_div;
-      else src = base + tm0 + m;
-      arow[q] = p.a + (size_t)src * p.a_stride + (pslot ^ r8 ^ (q & 1)) * 8;
-    }
-  }
   const uint4* bptr[2];
 #pragma unroll
   for (int q = 0; q < 2; ++q) {
@@ -466,6 +449,38 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p)
     int nb = nb0 + (brow >> 4);
     if (nb >= p.n_blocks) nb = p.n_blocks - 1;
     bptr[q] = wbase + (size_t)e * p.w_stride_u4 + (size_t)nb * p.nkb * 64 + kh * 16 + (brow & 15);
+  }
+  // The first four B stages are requested before anything that depends on the row list:
+  // weight tiles come from HBM (the longest latency of the prologue) and need nothing but
+  // the tile coordinates, so they fly while the pair ids of the A rows are looked up.
+  const int st_lo = (p.k_pad / 64) * part / n_parts, st_hi = (p.k_pad / 64) * (part + 1) / n_parts;
+  const int nks = 2 * (st_hi - st_lo);  // 32-k steps of this workgroup's k range
+  const int ks0 = 2 * st_lo;
+  const uint32_t sb_fill = (uint32_t)(uintptr_t)(lptr_t)S + NA * 32768 + wave * 4 * kChunk;
+  auto dma_b = [&](int buf, int q, int ks) {  // q = 2 * row group + k half
+    dma16(bptr[q >> 1] + (size_t)(ks0 + ks) * 64 + 32 * (q & 1), sb_fill + buf * 16384 + q * kChunk);
+  };
+#pragma unroll
+  for (int t = 0; t < NB; ++t)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) dma_b(t, q, min(t, nks - 1));
+
+  // A stage: 256 rows x 64 k as 32 chunks of 8 rows x 128 bytes, so that one load instruction
+  // reads eight full 128-byte lines.  Row r, 16-byte segment s of chunk c is stored at slot
+  // 8r + (s ^ r ^ (c & 1)); lane l of the filling load fetches row l/8, segment
+  // (l%8) ^ (l/8) ^ (c&1).  Wave w fills chunks 8w .. 8w+7, four per step.
+  const uint16_t* arow[8];
+  {
+    const int r8 = lane >> 3, pslot = lane & 7;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      int m = (wave * 8 + q) * 8 + r8;
+      if (m >= rows_here) m = 0;
+      int src;
+      if (UP) src = p.g.perm[base + tm0 + m] / p.g.pair_div;
+      else src = base + tm0 + m;
+      arow[q] = p.a + (size_t)src * p.a_stride + (pslot ^ r8 ^ (q & 1)) * 8;
+    }
   }
   // fragment read offsets (uint4 units inside a stage): A row group i adds 256, k16 unit u of
   // the 64-k stage selects the swizzled segment; B row group j of this wave, unit u adds 64.
@@ -487,17 +502,10 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
   const int my_rows = rows_here - wm * 128;
-  const int st_lo = (p.k_pad / 64) * part / n_parts, st_hi = (p.k_pad / 64) * (part + 1) / n_parts;
-  const int nks = 2 * (st_hi - st_lo);  // 32-k steps of this workgroup's k range
-  const int ks0 = 2 * st_lo;
 
   const uint32_t sa_fill = (uint32_t)(uintptr_t)(lptr_t)S + wave * 8 * kChunk;
-  const uint32_t sb_fill = (uint32_t)(uintptr_t)(lptr_t)S + NA * 32768 + wave * 4 * kChunk;
   auto dma_a = [&](int buf, int q, int t) {  // chunk q of this wave, 64-k stage t
     dma16(arow[q] + (size_t)(ks0 / 2 + t) * 64, sa_fill + buf * 32768 + q * kChunk);
-  };
-  auto dma_b = [&](int buf, int q, int ks) {  // q = 2 * row group + k half
-    dma16(bptr[q >> 1] + (size_t)(ks0 + ks) * 64 + 32 * (q & 1), sb_fill + buf * 16384 + q * kChunk);
   };
   // the 8 fragment reads of one k16 unit, in the order the MFMAs consume them
   auto read_frag = [&](int n, uint4 (&FA)[4], uint4 (&FB)[4], int a0, int b0) {
@@ -555,13 +563,11 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p)
         for (int q = 0; q < 8; ++q) dma_a(t, q, min(t, nst - 1));
       }
     };
-    auto fill_b = [&](int t) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) dma_b(t, q, min(t, nks - 1));
-    };
-    // issue order A0 B0 B1 A1 B2 B3, then per step: half of A(s/2 + 2), B(s + 4)
-    fill_a(0); fill_b(0); fill_b(1); fill_a(1); fill_b(2); fill_b(3);
-    wait_vm_lgkm0<LA ? 20 : 12>();
+    // issued so far: B0 B1 B2 B3; now A0 A1, then per step: half of A(s/2 + 2), B(s + 4).
+    // A wave that loads A rows waits for everything (A1 lands right behind A0), one that
+    // does not only for B0.
+    fill_a(0); fill_a(1);
+    wait_vm_lgkm0<LA ? 0 : 12>();
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
@@ -718,6 +724,30 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_i8_kernel(TiledParams
   constexpr int BROWS = UP ? 128 : 256;
   const int nb0 = ct * (BROWS / 16);
 
+  // B: LDS chunk c of a stage holds the stored block of strip c (gate/up: chunks 0-7 gate
+  // strips, 8-15 the matching up strips); wave w fills chunks 4w .. 4w+3.
+  const uint4* bptr[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int c = wave * 4 + q;
+    const uint4* wbase = (UP && c >= 8) ? p.wb : p.wa;
+    int nb = nb0 + (UP ? (c & 7) : c);
+    if (nb >= p.n_blocks) nb = p.n_blocks - 1;  // clamp: columns past N are never stored
+    bptr[q] = wbase + (size_t)e * p.w_stride_u4 + (size_t)nb * p.nkb * 64 + lane;
+  }
+  // The first three B stages are requested before the row list is looked up (see the bf16
+  // kernel).
+  const int st0 = (p.k_pad / 64) * part / n_parts;
+  const int nst = (p.k_pad / 64) * (part + 1) / n_parts - st0;  // 64-k stages of this k range
+  const uint32_t sb_fill = (uint32_t)(uintptr_t)(lptr_t)S + NA * 32768 + wave * 4 * kChunk;
+  auto dma_b = [&](int buf, int q, int t) {
+    dma16(bptr[q] + (size_t)(st0 + t) * 64, sb_fill + buf * 16384 + q * kChunk);
+  };
+#pragma unroll
+  for (int t = 0; t < 3; ++t)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) dma_b(t, q, min(t, nst - 1));
+
   const uint16_t* arow[8];  // as in the bf16 kernel
   {
     const int r8 = lane >> 3, pslot = lane & 7;
@@ -730,17 +760,6 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_i8_kernel(TiledParams
       else src = base + tm0 + m;
       arow[q] = p.a + (size_t)src * p.a_stride + (pslot ^ r8 ^ (q & 1)) * 8;
     }
-  }
-  // B: LDS chunk c of a stage holds the stored block of strip c (gate/up: chunks 0-7 gate
-  // strips, 8-15 the matching up strips); wave w fills chunks 4w .. 4w+3.
-  const uint4* bptr[4];
-#pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    const int c = wave * 4 + q;
-    const uint4* wbase = (UP && c >= 8) ? p.wb : p.wa;
-    int nb = nb0 + (UP ? (c & 7) : c);
-    if (nb >= p.n_blocks) nb = p.n_blocks - 1;  // clamp: columns past N are never stored
-    bptr[q] = wbase + (size_t)e * p.w_stride_u4 + (size_t)nb * p.nkb * 64 + lane;
   }
   int aoff[4];
   {
@@ -763,16 +782,10 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_i8_kernel(TiledParams
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
   const int my_rows = rows_here - wm * 128;
-  const int st0 = (p.k_pad / 64) * part / n_parts;
-  const int nst = (p.k_pad / 64) * (part + 1) / n_parts - st0;  // 64-k stages of this k range
 
   const uint32_t sa_fill = (uint32_t)(uintptr_t)(lptr_t)S + wave * 8 * kChunk;
-  const uint32_t sb_fill = (uint32_t)(uintptr_t)(lptr_t)S + NA * 32768 + wave * 4 * kChunk;
   auto dma_a = [&](int buf, int q, int t) {
     dma16(arow[q] + (size_t)(st0 + t) * 64, sa_fill + buf * 32768 + q * kChunk);
-  };
-  auto dma_b = [&](int buf, int q, int t) {
-    dma16(bptr[q] + (size_t)(st0 + t) * 64, sb_fill + buf * 16384 + q * kChunk);
   };
   auto read_frag = [&](int n, uint4 (&FA)[4], uint2 (&RB)[4], int a0, int b0) {
     switch (n) {
@@ -831,12 +844,9 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_i8_kernel(TiledParams
         for (int q = 0; q < 8; ++q) dma_a(t, q, min(t, nst - 1));
       }
     };
-    auto fill_b = [&](int t) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) dma_b(t, q, min(t, nst - 1));
-    };
-    fill_a(0); fill_b(0); fill_b(1); fill_a(1); fill_b(2);
-    wait_vm_lgkm0<LA ? 16 : 8>();
+    // issued so far: B0 B1 B2; now A0 A1 (a wave that loads A rows then waits for all of it)
+    fill_a(0); fill_a(1);
+    wait_vm_lgkm0<LA ? 0 : 8>();
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
