@@ -58,9 +58,26 @@ std::string MoeSparseError::to_string() const {
 }
 
 std::string MoeBindingError::to_string() const {
-  switch (kind) {  // src/moe/binding.rs:72-76
-    case LayerNotFound:
-      return "moe-binding: layer " + std::to_string(layer_id) + " has no MoE weights";
+  const std::string L = std::to_string(layer_id);
+  switch (kind) {  // src/moe/binding.rs:72-113
+    case LayerNotFound: return "moe-binding: layer " + L + " has no MoE weights";
+    case NoExperts: return "moe-binding: layer " + L + " has no experts";
+    case IncompleteExpert:
+      return "moe-binding: layer " + L + " expert " + std::to_string(expert_id) +
+             " is missing a gate/up/down projection";
+    case MissingRouter: return "moe-binding: layer " + L + " has no router tensor";
+    case UnresolvedTensor: return "moe-binding: byte resolver returned no data for '" + name + "'";
+    case BadRank:
+      return "moe-binding: tensor '" + name + "' has rank " + std::to_string(rank) +
+             ", expected 2-D [rows, cols]";
+    case ShapeInconsistency: return "moe-binding: shape inconsistency: " + detail;
+    case DataLengthMismatch:
+      return "moe-binding: tensor '" + name + "' data length " + std::to_string(actual) +
+             " != shape product " + std::to_string(expected);
+    case MissingPackedTensor:
+      return "moe-binding: layer " + L + " missing packed expert tensor '" + which + "'";
+    case PackedBadRank:
+      return "moe-binding: packed tensor '" + name + "' has rank " + std::to_string(rank) + ", expected 3-D";
     case Dense: return "moe-binding: " + dense.to_string();
   }
   return "moe-binding";
@@ -72,6 +89,13 @@ std::string MoeLayerError::to_string() const {
     case Binding: return "moe-layer: " + binding.to_string();
     case Sparse: return "moe-layer: " + sparse.to_string();
     case ConfigMismatch: return "moe-layer: config mismatch: " + detail;
+    case SharedExpertMissing:
+      return "moe-layer: layer " + std::to_string(layer_id) + " has no shared-expert tensors";
+    case SharedExpertIncomplete:
+      return "moe-layer: layer " + std::to_string(layer_id) + " shared expert is missing gate/up/down";
+    case MixedExpertFormat:
+      return "moe-layer: layer " + std::to_string(layer_id) +
+             " has both classic and packed expert tensors";
     case Device: return "moe-layer: device path failed (rc " + std::to_string(rc) + "): " + detail;
   }
   return "moe-layer";

@@ -62,10 +62,18 @@ struct MoeSparseError {
   std::string to_string() const;
 };
 
-struct MoeBindingError {
-  enum Kind { LayerNotFound, Dense };
+struct MoeBindingError {  // src/moe/binding.rs:41-70
+  enum Kind {
+    LayerNotFound, NoExperts, IncompleteExpert, MissingRouter, UnresolvedTensor, BadRank,
+    ShapeInconsistency, DataLengthMismatch, MissingPackedTensor, PackedBadRank, Dense
+  };
   Kind kind;
-  size_t layer_id = 0;
+  size_t layer_id = 0, expert_id = 0;
+  std::string name;               // UnresolvedTensor / BadRank / DataLengthMismatch / PackedBadRank
+  size_t rank = 0;                // BadRank / PackedBadRank
+  size_t expected = 0, actual = 0;  // DataLengthMismatch
+  std::string detail;             // ShapeInconsistency
+  const char* which = "";         // MissingPackedTensor: "gate_up_proj" or "down_proj"
   MoeDenseError dense{MoeDenseError::NoExperts};
   std::string to_string() const;
 };
@@ -73,8 +81,12 @@ struct MoeBindingError {
 struct MoeLayerError {
   // Config / Binding / Sparse / ConfigMismatch as in the reference; Device = the HIP library
   // reported a failure that has no counterpart there (no device, out of memory, launch failed).
-  enum Kind { Config, Binding, Sparse, ConfigMismatch, Device };
+  enum Kind {
+    Config, Binding, Sparse, ConfigMismatch, SharedExpertMissing, SharedExpertIncomplete,
+    MixedExpertFormat, Device
+  };
   Kind kind;
+  size_t layer_id = 0;  // SharedExpertMissing / SharedExpertIncomplete / MixedExpertFormat
   MoeConfigError config{MoeConfigError::ZeroExperts};
   MoeBindingError binding{MoeBindingError::LayerNotFound};
   MoeSparseError sparse{MoeSparseError::ZeroK};
@@ -210,14 +222,17 @@ std::vector<float> moe_real_layer_reference_node(uint32_t layer_id, const std::v
 #include <stdexcept>
 namespace atenia {
 namespace moe {
+inline std::string error_text(const std::string& e) { return e; }
+template <typename E>
+std::string error_text(const E& e) { return e.to_string(); }
 template <typename T, typename E>
 T Result<T, E>::unwrap() const {
-  if (!is_ok()) throw std::runtime_error("called `Result::unwrap()` on an `Err` value: " + e_->to_string());
+  if (!is_ok()) throw std::runtime_error("called `Result::unwrap()` on an `Err` value: " + error_text(*e_));
   return *v_;
 }
 template <typename T, typename E>
 T Result<T, E>::expect(const char* msg) const {
-  if (!is_ok()) throw std::runtime_error(std::string(msg) + ": " + e_->to_string());
+  if (!is_ok()) throw std::runtime_error(std::string(msg) + ": " + error_text(*e_));
   return *v_;
 }
 }  // namespace moe
