@@ -19,6 +19,7 @@ CONVENTION_ATENIA = 0
 CONVENTION_HUGGINGFACE_QWEN = 1
 WEIGHT_F32, WEIGHT_BF16, WEIGHT_INT8_W8A16 = 0, 1, 2
 ACT_F32, ACT_BF16 = 0, 1
+NORM_GRAPH_F32, NORM_F64 = 0, 1
 OK, ERR_SYNC, ERR_LAUNCH = 0, 1, 2
 ERR_DIM, ERR_K, ERR_NON_FINITE, ERR_OOM, ERR_HANDLE, ERR_UNSUPPORTED = -1, -2, -3, -4, -5, -6
 N_STAGES = 6
@@ -37,6 +38,8 @@ EXPORTS = (
     "atenia_moe_f32_to_bf16_trunc",
     "atenia_moe_hip_layer_last_non_finite", "atenia_moe_router_launch_device", "atenia_moe_permute_launch_device",
     "atenia_moe_expert_ffn_launch_device", "atenia_moe_combine_launch_device",
+    "atenia_moe_hip_layer_block_forward", "atenia_moe_hip_layer_block_forward_device",
+    "atenia_moe_hip_layer_last_normed",
 )
 
 
@@ -97,6 +100,10 @@ def lib():
         L.atenia_moe_quantize_per_row_i8.argtypes = [P, C.c_size_t, C.c_size_t, P, P]
         L.atenia_moe_f32_to_bf16_trunc.argtypes = [P, C.c_size_t, P]
         L.atenia_moe_hip_layer_last_non_finite.argtypes = [P, P, P]
+        L.atenia_moe_hip_layer_block_forward.argtypes = [P, P, C.c_int, P, C.c_float, C.c_int, P]
+        L.atenia_moe_hip_layer_block_forward_device.argtypes = [P, P, C.c_int, P, C.c_float,
+                                                                C.c_int, P, P]
+        L.atenia_moe_hip_layer_last_normed.argtypes = [P, P]
         L.atenia_moe_router_launch_device.argtypes = [P, P, C.c_int, C.c_int, P, P, P]
         L.atenia_moe_permute_launch_device.argtypes = [P, C.c_int, P, P, P, P]
         L.atenia_moe_expert_ffn_launch_device.argtypes = [P, P, C.c_int, C.c_int, P]
@@ -209,6 +216,26 @@ class Layer:
         """Raw device pointers (ints); asynchronous on `stream`."""
         _check(lib().atenia_moe_hip_layer_forward_device(self._h, d_x, x_dtype, n_tokens, d_out,
                                                          stream))
+
+    # The decoder layer's FFN block around the op: out = x1 + MoE(RMSNorm(x1) * gamma).
+    def block_forward(self, x1, gamma, eps: float, norm_policy: int = NORM_GRAPH_F32) -> np.ndarray:
+        x1 = np.ascontiguousarray(x1, dtype=np.float32)
+        gamma = np.ascontiguousarray(gamma, dtype=np.float32)
+        assert x1.size % self.d == 0 and gamma.size == self.d
+        out = np.empty_like(x1)
+        _check(lib().atenia_moe_hip_layer_block_forward(self._h, _ptr(x1), x1.size // self.d,
+                                                        _ptr(gamma), eps, norm_policy, _ptr(out)))
+        return out
+
+    def block_forward_device(self, d_x1: int, n_tokens: int, d_gamma: int, eps: float,
+                             norm_policy: int, d_out: int, stream: int = 0):
+        _check(lib().atenia_moe_hip_layer_block_forward_device(self._h, d_x1, n_tokens, d_gamma, eps,
+                                                               norm_policy, d_out, stream))
+
+    def last_normed(self, T: int) -> np.ndarray:
+        h2 = np.empty((T, self.d), dtype=np.float32)
+        _check(lib().atenia_moe_hip_layer_last_normed(self._h, _ptr(h2)))
+        return h2
 
     # Stage launchers: the pipeline one kernel at a time (raw device pointers as ints, 0 = NULL).
     def router_device(self, d_x: int, x_dtype: int, n_tokens: int, d_idx: int = 0, d_w: int = 0,

@@ -1,7 +1,8 @@
 // Kernel 4: weighted combine back to token order.
 //
 // out[t] = sum over the token's slots (ascending expert id) of w[t,slot] * y[t,slot], then
-// += scale[t] * y_shared[t]      (src/moe/sparse.rs:226-233, src/moe/layer.rs:415-429).
+// += scale[t] * y_shared[t]      (src/moe/sparse.rs:226-233, src/moe/layer.rs:415-429), and,
+// for the decoder layer's FFN block, out[t] = residual[t] + that (src/moe/full_forward.rs:251).
 // The reference multiplies and adds in f32 with two roundings and a fixed order; the same
 // sequence is kept here (no fused multiply-add, no atomics), so given equal expert outputs
 // the combine is bit-identical.  Expert outputs are stored by pair id t*k+slot, so a token's
@@ -9,6 +10,11 @@
 // split the k range of some tiles, an expert output there is the f32 sum of its partial
 // buffers, added in buffer order.
 #include "moe_internal.h"
+
+// This file is compiled with -ffp-contract=off (see the Makefile): the reference rounds every
+// product and every sum on its own, and hipcc would otherwise fuse `a * b + c` into one FMA
+// (its default is -ffp-contract=fast, under which __fmul_rn / __fadd_rn are plain `*` and `+`
+// and the fp-contract pragma is ignored).
 
 namespace atenia_moe {
 
@@ -21,7 +27,7 @@ __global__ __launch_bounds__(256) void combine_kernel(int T, int k, int d,
                                                       int flag_cols, size_t y_part_stride,
                                                       const float* __restrict__ y_shared,
                                                       const float* __restrict__ sgate,
-                                                      float* __restrict__ out) {
+                                                      const float* residual, float* out) {
   const int chunks = (d + 1023) / 1024;
   const int t = blockIdx.x / chunks;
   const int c = ((blockIdx.x - t * chunks) * 256 + threadIdx.x) * 4;
@@ -63,6 +69,16 @@ __global__ __launch_bounds__(256) void combine_kernel(int T, int k, int d,
 #pragma unroll
     for (int j = 0; j < 4; ++j) o[j] = __fadd_rn(o[j], __fmul_rn(sc, v[j]));
   }
+  if (residual) {  // may alias `out`: each element is read and written by this thread only
+    const float* rr = residual + (size_t)t * d + c;
+    if (vec) {
+      const float4 q = *(const float4*)rr;
+      o[0] = __fadd_rn(q.x, o[0]); o[1] = __fadd_rn(q.y, o[1]);
+      o[2] = __fadd_rn(q.z, o[2]); o[3] = __fadd_rn(q.w, o[3]);
+    } else {
+      for (int j = 0; j < 4 && c + j < d; ++j) o[j] = __fadd_rn(rr[j], o[j]);
+    }
+  }
   float* orow = out + (size_t)t * d + c;
   if (vec) {
     *(float4*)orow = make_float4(o[0], o[1], o[2], o[3]);
@@ -76,7 +92,7 @@ __global__ __launch_bounds__(256) void combine_kernel(int T, int k, int d,
 hipError_t launch_combine(const CombineArgs& a, hipStream_t s) {
   const unsigned grid = (unsigned)((a.d + 1023) / 1024) * (unsigned)a.T;
   combine_kernel<<<grid, 256, 0, s>>>(a.T, a.k, a.d, a.w, a.y, a.y_stride, a.part_flags, a.flag_cols,
-                                      a.y_part_stride, a.y_shared, a.sgate, a.out);
+                                      a.y_part_stride, a.y_shared, a.sgate, a.residual, a.out);
   return hipGetLastError();
 }
 

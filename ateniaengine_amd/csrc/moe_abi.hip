@@ -95,6 +95,8 @@ struct AteniaMoeLayer {
   DevBuf x_in, out, xb, idx, w, sgate, counts, offsets, active, n_active, perm, inv, blk_counts,
       shared_desc, ident, h, hs, y, ys, status, tile_group, tile_m0, s_tile_group, s_tile_m0,
       part_flags;
+  DevBuf xn, gamma_in;  // block forward: normalised rows [T, d] f32; gamma of the host variant
+  int normed_T = 0;     // rows of xn the last block forward wrote
   int last_T = 0;
   int stage_T[4] = {-1, -1, -1, -1};  // token count each pipeline stage last completed for
   int nf_token = -1, nf_expert = -1;  // location of the last non-finite routing weight reported
@@ -260,7 +262,7 @@ enum { kStageRouter = 0, kStagePermute = 1, kStageFfn = 2, kStageCombine = 3 };
 // left in the handle's workspace, so a range that does not start at the router is only valid
 // after the earlier stages ran for the same n_tokens (checked) on the same activations.
 int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d_out,
-                hipStream_t s, int first, int last) {
+                hipStream_t s, int first, int last, const float* d_residual = nullptr) {
   for (int st = 0; st < first; ++st)
     if (L->stage_T[st] != T)
       return fail(ATENIA_MOE_ERR_DIM, "stage %d has not run for %d tokens on this handle", st, T);
@@ -431,6 +433,7 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   ca.y_part_stride = fa.y_part_stride;
   ca.y_shared = L->fs > 0 ? L->ys.as<float>() : nullptr;
   ca.sgate = gated ? L->sgate.as<float>() : nullptr;
+  ca.residual = d_residual;
   ca.out = d_out;
   HIP_TRY(launch_combine(ca, s));
   L->launches[4] = 1;
@@ -627,6 +630,80 @@ int atenia_moe_hip_layer_forward(AteniaMoeLayer* L, const float* x_host, int n_t
   if (rc) return rc;
   HIP_TRY(hipMemcpyAsync(out_host, L->out.p, bytes, hipMemcpyDeviceToHost, L->stream));
   return read_status(L, L->stream, nullptr, nullptr);
+}
+
+namespace {
+// RMSNorm * gamma into the handle's xn, then the whole pipeline on xn with x1 as the residual.
+int run_block(AteniaMoeLayer* L, const float* d_x1, int T, const float* d_gamma, float eps,
+              int norm_policy, float* d_out, hipStream_t s) {
+  int rc = ensure_workspace(L, T);
+  if (rc) return rc;
+  if ((rc = L->xn.ensure((size_t)L->cap_tokens * L->d * 4))) return rc;
+  NormArgs na{};
+  na.x = d_x1;
+  na.gamma = d_gamma;
+  na.eps = eps;
+  na.policy = norm_policy;
+  na.T = T;
+  na.d = L->d;
+  na.y = L->xn.as<float>();
+  HIP_TRY(launch_rmsnorm_gamma(na, s));
+  L->normed_T = T;
+  return run_forward(L, L->xn.p, ATENIA_MOE_ACT_F32, T, d_out, s, kStageRouter, kStageCombine,
+                     d_x1);
+}
+
+int block_prologue(AteniaMoeLayer* L, int n_tokens, const void* x1, const void* gamma,
+                   const void* out, float eps, int norm_policy) {
+  if (!valid_handle(L)) return fail(ATENIA_MOE_ERR_HANDLE, "invalid layer handle");
+  if (n_tokens < 0) return fail(ATENIA_MOE_ERR_DIM, "negative token count");
+  if (n_tokens > 0 && (!x1 || !gamma || !out))
+    return fail(ATENIA_MOE_ERR_DIM, "null activation or gamma pointer");
+  if (norm_policy != ATENIA_MOE_NORM_GRAPH_F32 && norm_policy != ATENIA_MOE_NORM_F64)
+    return fail(ATENIA_MOE_ERR_DIM, "unknown norm policy %d", norm_policy);
+  if (!(eps >= 0.0f)) return fail(ATENIA_MOE_ERR_DIM, "eps must be a non-negative number");
+  if ((long long)n_tokens * L->k > (long long)INT_MAX / 4)
+    return fail(ATENIA_MOE_ERR_DIM, "too many tokens");
+  return ATENIA_MOE_OK;
+}
+}  // namespace
+
+int atenia_moe_hip_layer_block_forward_device(AteniaMoeLayer* L, const float* d_x1, int n_tokens,
+                                              const float* d_gamma, float eps, int norm_policy,
+                                              float* d_out, void* stream) {
+  int rc = block_prologue(L, n_tokens, d_x1, d_gamma, d_out, eps, norm_policy);
+  if (rc || n_tokens == 0) return rc;
+  std::lock_guard<std::mutex> lock(L->mu);
+  return run_block(L, d_x1, n_tokens, d_gamma, eps, norm_policy, d_out, (hipStream_t)stream);
+}
+
+int atenia_moe_hip_layer_block_forward(AteniaMoeLayer* L, const float* x1_host, int n_tokens,
+                                       const float* gamma_host, float eps, int norm_policy,
+                                       float* out_host) {
+  int rc = block_prologue(L, n_tokens, x1_host, gamma_host, out_host, eps, norm_policy);
+  if (rc || n_tokens == 0) return rc;
+  std::lock_guard<std::mutex> lock(L->mu);
+  if ((rc = ensure_workspace(L, n_tokens))) return rc;
+  if ((rc = L->gamma_in.ensure((size_t)L->d * 4))) return rc;
+  const size_t bytes = (size_t)n_tokens * L->d * 4;
+  HIP_TRY(hipMemcpyAsync(L->x_in.p, x1_host, bytes, hipMemcpyHostToDevice, L->stream));
+  HIP_TRY(hipMemcpyAsync(L->gamma_in.p, gamma_host, (size_t)L->d * 4, hipMemcpyHostToDevice,
+                         L->stream));
+  rc = run_block(L, L->x_in.as<float>(), n_tokens, L->gamma_in.as<float>(), eps, norm_policy,
+                 L->out.as<float>(), L->stream);
+  if (rc) return rc;
+  HIP_TRY(hipMemcpyAsync(out_host, L->out.p, bytes, hipMemcpyDeviceToHost, L->stream));
+  return read_status(L, L->stream, nullptr, nullptr);
+}
+
+int atenia_moe_hip_layer_last_normed(AteniaMoeLayer* L, float* h2_host) {
+  if (!valid_handle(L)) return fail(ATENIA_MOE_ERR_HANDLE, "invalid layer handle");
+  if (!h2_host) return fail(ATENIA_MOE_ERR_DIM, "null output pointer");
+  std::lock_guard<std::mutex> lock(L->mu);
+  if (L->normed_T <= 0 || !L->xn.p) return fail(ATENIA_MOE_ERR_DIM, "no block forward has run on this handle");
+  HIP_TRY(hipDeviceSynchronize());
+  HIP_TRY(hipMemcpy(h2_host, L->xn.p, (size_t)L->normed_T * L->d * 4, hipMemcpyDeviceToHost));
+  return ATENIA_MOE_OK;
 }
 
 namespace {

@@ -139,9 +139,20 @@ struct CombineArgs {
   size_t y_part_stride;  // elements
   const float* y_shared; // [T, y_stride] or null
   const float* sgate;    // [T] or null (scale 1)
+  const float* residual; // [T, d] or null: out = residual + combine (one more f32 add); may be `out`
   float* out;            // [T, d]
 };
 hipError_t launch_combine(const CombineArgs& a, hipStream_t s);
+
+struct NormArgs {
+  const float* x;      // [T, d]
+  const float* gamma;  // [d]
+  float eps;
+  int policy;          // ATENIA_MOE_NORM_*
+  int T, d;
+  float* y;            // [T, d]
+};
+hipError_t launch_rmsnorm_gamma(const NormArgs& a, hipStream_t s);
 
 // Rewrites a row-major [n_rows, k_cols] matrix (bf16 bits or int8) into B blocks.
 hipError_t launch_repack_blocks(const void* src, void* dst, int n_rows, int k_cols, int n_pad,

@@ -420,6 +420,25 @@ Result<std::vector<float>, MoeLayerError> RealMoeLayer::forward_routed(const std
   return run(x, MoeExecutionConvention::Atenia, false);
 }
 
+Result<std::vector<float>, MoeLayerError> RealMoeLayer::ffn_block(
+    const std::vector<float>& x1, const std::vector<float>& gamma, float eps, NormPolicy norm_policy,
+    MoeExecutionConvention convention) const {
+  typedef Result<std::vector<float>, MoeLayerError> R;
+  const size_t d = config.d_model;
+  if (d == 0 || x1.empty() || x1.size() % d != 0) return R::Err(dense_dim_error("x", d, x1.size()));
+  if (gamma.size() != d) return R::Err(dense_dim_error("gamma", d, gamma.size()));
+  std::lock_guard<std::mutex> lock(dev_->mu);
+  auto hr = handle_for(convention, true);
+  if (hr.is_err()) return R::Err(hr.error());
+  AteniaMoeLayer* h = (AteniaMoeLayer*)hr.value();
+  std::vector<float> out(x1.size());
+  const int rc = atenia_moe_hip_layer_block_forward(h, x1.data(), (int)(x1.size() / d), gamma.data(),
+                                                    eps, (int)norm_policy, out.data());
+  if (rc == ATENIA_MOE_ERR_NON_FINITE) return R::Err(non_finite_error(h));
+  if (rc) return R::Err(device_error(rc));
+  return R::Ok(std::move(out));
+}
+
 Result<std::vector<float>, MoeLayerError> RealMoeLayer::route(const std::vector<float>& x,
                                                               MoeExecutionConvention convention,
                                                               std::vector<int32_t>* indices) const {

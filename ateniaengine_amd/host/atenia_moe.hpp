@@ -181,6 +181,16 @@ class RealMoeLayer {
                                                          MoeExecutionConvention convention) const;
   // Routed experts only, renormalised combine (src/moe/layer.rs:366-369).
   Result<std::vector<float>, MoeLayerError> forward_routed(const std::vector<float>& x) const;
+  // The FFN half of a decoder layer: x1 + MoE(RMSNorm(x1) * gamma) for each row of x1, the
+  // layer run under `convention`.  Steps 13-15 of the layer loop in
+  // src/moe/full_forward.rs:239-252 (norm_policy GraphF32: RmsNorm + BroadcastMul nodes in
+  // f32), and the second half of src/moe/mla.rs:442-453 / decoder_layer_reference
+  // (norm_policy F64: src/moe/decoder_layer.rs:97-107).  One C-ABI call for the whole batch.
+  enum class NormPolicy { GraphF32 = 0, F64 = 1 };
+  Result<std::vector<float>, MoeLayerError> ffn_block(const std::vector<float>& x1,
+                                                      const std::vector<float>& gamma, float eps,
+                                                      NormPolicy norm_policy,
+                                                      MoeExecutionConvention convention) const;
   // Routing of each row: indices [n * k] (ascending per row) and weights, under `convention`.
   Result<std::vector<float>, MoeLayerError> route(const std::vector<float>& x,
                                                   MoeExecutionConvention convention,

@@ -162,6 +162,41 @@ def measure(torch, np, capi, layer, T, steps, warmup, seed):
     return r, xs[0], out
 
 
+def measure_block(torch, np, capi, layer, T, steps, warmup, seed):
+    """The decoder layer's FFN block (RMSNorm * gamma -> layer -> residual add, f32 residual
+    stream on the device) next to the bare layer forward on f32 rows of the same batch."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed + 7 * T)
+    x1 = torch.randn((T, D_MODEL), generator=g, device="cuda", dtype=torch.float32)
+    gamma = 1.0 + 0.1 * torch.randn((D_MODEL,), generator=g, device="cuda", dtype=torch.float32)
+    out = torch.empty_like(x1)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps
+
+    fwd = timed(lambda: layer.forward_device(x1.data_ptr(), capi.ACT_F32, T, out.data_ptr(), stream))
+    res = {"tokens": T, "forward_f32_rows_ms": fwd}
+    for name, pol in (("graph_f32", capi.NORM_GRAPH_F32), ("f64", capi.NORM_F64)):
+        ms = timed(lambda: layer.block_forward_device(x1.data_ptr(), T, gamma.data_ptr(), 1e-5, pol,
+                                                      out.data_ptr(), stream))
+        res[f"block_{name}_ms"] = ms
+        res[f"block_{name}_over_forward_ms"] = ms - fwd
+    rc, tok, ex = layer.status(stream)
+    if rc != 0:
+        raise RuntimeError(f"device status {rc} at token {tok}, expert {ex}")
+    # the norm kernel reads x once from HBM (the second pass hits L2) and writes y once
+    res["norm_algorithmic_bytes"] = 8.0 * T * D_MODEL
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -177,6 +212,8 @@ def main():
                     help="tokens of the CPU-baseline sample (0 = skip)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (reference point for HBM counters)")
+    ap.add_argument("--block", action="store_true",
+                    help="also time the decoder-layer FFN block entry point (norm + layer + residual)")
     ap.add_argument("--seed", type=int, default=1234)
     a = ap.parse_args()
     if a.gpus != 1:
@@ -256,6 +293,13 @@ def main():
                           a.warmup, a.seed)
         sweep.append(r)
 
+    block = None
+    if a.block:
+        block = [measure_block(torch, np, capi, layer, t, a.steps if t >= 512 else max(a.steps, 50),
+                               a.warmup, a.seed)
+                 for t in sorted({a.tokens, a.decode_tokens} | {int(t) for t in a.sweep.split(",") if t})
+                 if t > 0]
+
     cpu = None
     parity = None
     if a.cpu_tokens > 0 and a.config == "mixtral_bf16":
@@ -303,6 +347,8 @@ def main():
         "sweep": sweep,
         "parity": parity,
     }
+    if block is not None:
+        line["block"] = block
     print(json.dumps(line))
 
 

@@ -56,6 +56,9 @@ extern "C" {
 /* Element type of device activations handed to `forward_device`. */
 #define ATENIA_MOE_ACT_F32 0
 #define ATENIA_MOE_ACT_BF16 1
+/* Arithmetic of the RMSNorm in front of the layer (atenia_moe_hip_layer_block_forward*). */
+#define ATENIA_MOE_NORM_GRAPH_F32 0 /* graph nodes: f32 left-to-right sum, (x*inv)*gamma in f32 */
+#define ATENIA_MOE_NORM_F64 1       /* imperative decoders: f64 sum and inverse root */
 
 #define ATENIA_MOE_OK 0
 #define ATENIA_MOE_ERR_SYNC 1
@@ -137,6 +140,26 @@ int atenia_moe_hip_layer_forward(AteniaMoeLayer* layer, const float* x_host, int
 int atenia_moe_hip_layer_forward_device(AteniaMoeLayer* layer, const void* d_x, int x_dtype,
                                         int n_tokens, float* d_out, void* stream);
 
+/* The FFN block of a decoder layer around the op, on device-resident rows, asynchronous on
+ * `stream`:  out[t] = x1[t] + MoE(RMSNorm(x1[t]) * gamma),  x1 / out: [T, d] f32, gamma: [d] f32.
+ * Replaces steps 13-15 of the reference's layer loop -- the RmsNorm, BroadcastMul,
+ * MoeRealLayerReference and Add nodes of src/moe/full_forward.rs:239-252 (also
+ * src/moe/generate.rs:161-170, src/moe/decoder_layer.rs:199-210), whose executor copies every
+ * node's tensor to the host (`ensure_cpu`, src/amg/graph.rs:5361, 5580) -- and the imperative
+ * form of src/moe/mla.rs:442-453.  `norm_policy` picks the reference arithmetic of the norm:
+ * ATENIA_MOE_NORM_GRAPH_F32 = src/nn/normalization.rs:8-37 + broadcast_mul
+ * (src/amg/graph.rs:6647-6673); ATENIA_MOE_NORM_F64 = src/moe/mla.rs:230-239.
+ * d_out may be d_x1 (the residual stream is updated in place).  Pointers are 16-byte aligned
+ * when d % 4 == 0.  The normalised rows stay in the handle (tap: ..._last_normed). */
+int atenia_moe_hip_layer_block_forward_device(AteniaMoeLayer* layer, const float* d_x1,
+                                              int n_tokens, const float* d_gamma, float eps,
+                                              int norm_policy, float* d_out, void* stream);
+
+/* Same block with host buffers (x1, out: [T*d]; gamma: [d]); synchronous. */
+int atenia_moe_hip_layer_block_forward(AteniaMoeLayer* layer, const float* x1_host, int n_tokens,
+                                       const float* gamma_host, float eps, int norm_policy,
+                                       float* out_host);
+
 /* Waits for the handle's last forward and returns its device-side status: 0, or -3 with the
  * first offending token / expert (either pointer may be NULL). */
 int atenia_moe_hip_layer_status(AteniaMoeLayer* layer, void* stream, int32_t* token,
@@ -205,6 +228,10 @@ int atenia_moe_hip_layer_last_routing(AteniaMoeLayer* layer, int32_t* idx_host, 
  * (docs/decisions/ADR-007-moe-certification-ladder.md:62-73). */
 int atenia_moe_hip_layer_last_expert_outputs(AteniaMoeLayer* layer, float* y_host,
                                              float* y_shared_host);
+
+/* The rows the MoE layer saw in the most recent block forward: RMSNorm(x1) * gamma, [T, d] f32,
+ * host buffer (the `h2` of src/moe/full_forward.rs:243). */
+int atenia_moe_hip_layer_last_normed(AteniaMoeLayer* layer, float* h2_host);
 
 /* Stage timing with HIP events recorded on the forward's own stream.  After
  * `set_profiling(layer, 1)` every forward records an event before/after each stage;

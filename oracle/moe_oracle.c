@@ -22,7 +22,8 @@
  *              ora_absmax_per_channel_symmetric, ora_int8_to_bf16_per_channel,
  *              ora_f32_to_bf16_bits / ora_bf16_bits_to_f32,
  *              ora_numerical_metrics, ora_layer_forward_f64, ora_permute
- *              (brute force), ora_matvec_f32acc.
+ *              (brute force), ora_matvec_f32acc, ora_rms_norm_gamma,
+ *              ora_block_forward.
  *   parity unpinned (no reference counterpart; defined by this build):
  *              the `router_bias` term of ora_route (the reference router has
  *              no bias, dense.rs:333).  With router_bias == NULL ora_route is
@@ -316,6 +317,64 @@ int ora_execute_layer(const OraLayer* L, const float* input, size_t n_tokens, in
     }
   }
   return ORA_OK;
+}
+
+/* ---- the FFN block of a decoder layer: out = x1 + MoE(RMSNorm(x1) * gamma) ---------
+ * Two arithmetic policies exist in the reference for the norm:
+ *   ORA_NORM_GRAPH_F32 (0): the graph path.  RmsNorm node = nn/normalization.rs:8-37
+ *     (f32 sum of squares folded left to right, mean = sum / cols, inv = 1 / sqrt(mean + eps),
+ *     y = v * inv, all f32), then a BroadcastMul node by gamma (amg/graph.rs:6647-6673, one
+ *     more f32 rounding).  Used by full_forward.rs:239-243, generate.rs:161, decoder_layer.rs:199.
+ *   ORA_NORM_F64 (1): the imperative path, moe/mla.rs:230-239 and decoder_layer.rs:97-107
+ *     (f64 sum of squares, mean and inverse root in f64, y = (f32)(x * inv) * gamma).
+ * Pinned by closed forms (3-4-0-0; a 2^24 head that swallows later ones in f32 but not in f64),
+ * and, through ora_block_forward, by the tiny-Mixtral whole-model fixture (HF f64 logits).    */
+#define ORA_NORM_GRAPH_F32 0
+#define ORA_NORM_F64 1
+void ora_rms_norm_gamma(const float* x, const float* gamma, size_t n, float eps, int norm_policy,
+                        float* y) {
+  if (norm_policy == ORA_NORM_F64) {
+    double ms = 0.0;
+    for (size_t i = 0; i < n; ++i) ms += (double)x[i] * (double)x[i];
+    ms /= (double)n;
+    double inv = 1.0 / sqrt(ms + (double)eps);
+    for (size_t i = 0; i < n; ++i) y[i] = (float)((double)x[i] * inv) * gamma[i];
+    return;
+  }
+  float sum_sq = 0.0f;
+  for (size_t i = 0; i < n; ++i) sum_sq += x[i] * x[i];
+  float cols = (float)n;
+  float mean_sq = sum_sq / (cols > 1.0f ? cols : 1.0f);
+  float inv_rms = 1.0f / sqrtf(mean_sq + eps);
+  for (size_t i = 0; i < n; ++i) {
+    float normed = x[i] * inv_rms;
+    y[i] = normed * gamma[i];
+  }
+}
+
+/* full_forward.rs:239-252 / mla.rs:442-453: h2 = norm(x1) * gamma; out = x1 + MoE(h2), row by
+ * row.  h2_out (optional) receives the normalised rows the MoE saw. */
+int ora_block_forward(const OraLayer* L, const float* x1, size_t n_tokens, const float* gamma,
+                      float eps, int norm_policy, int policy, float* out, float* h2_out,
+                      int32_t* idx_out, float* w_out, int32_t* err_token, int32_t* err_index) {
+  size_t d = (size_t)L->d_model, k = (size_t)L->top_k;
+  float* h2 = (float*)malloc(d * sizeof(float));
+  float* y = (float*)malloc(d * sizeof(float));
+  int rc = ORA_OK;
+  for (size_t t = 0; t < n_tokens && rc == ORA_OK; ++t) {
+    ora_rms_norm_gamma(x1 + t * d, gamma, d, eps, norm_policy, h2);
+    if (h2_out) memcpy(h2_out + t * d, h2, d * sizeof(float));
+    rc = ora_layer_forward_with(L, h2, L->convention, policy, y, idx_out ? idx_out + t * k : NULL,
+                                w_out ? w_out + t * k : NULL, err_index);
+    if (rc != ORA_OK) {
+      if (err_token) *err_token = (int32_t)t;
+      break;
+    }
+    for (size_t i = 0; i < d; ++i) out[t * d + i] = x1[t * d + i] + y[i];
+  }
+  free(h2);
+  free(y);
+  return rc;
 }
 
 /* Routing only (router -> softmax -> top-k) for n_tokens rows. */

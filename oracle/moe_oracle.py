@@ -28,6 +28,8 @@ ATENIA = 0
 HUGGINGFACE_QWEN = 1
 CERTIFIED = 0  # f64 accumulation (reference default)
 STRICT = 1  # f32 accumulation
+NORM_GRAPH_F32 = 0  # RmsNorm + BroadcastMul graph nodes, f32 throughout
+NORM_F64 = 1  # imperative decoder paths, f64 accumulation
 
 
 def build(force: bool = False) -> str:
@@ -90,6 +92,9 @@ def lib():
         L.ora_layer_forward_with.restype = C.c_int
         L.ora_execute_layer.argtypes = [P, P, Z, C.c_int, P, P, P, P, P]
         L.ora_execute_layer.restype = C.c_int
+        L.ora_rms_norm_gamma.argtypes = [P, P, Z, C.c_float, C.c_int, P]
+        L.ora_block_forward.argtypes = [P, P, Z, P, C.c_float, C.c_int, C.c_int, P, P, P, P, P, P]
+        L.ora_block_forward.restype = C.c_int
         L.ora_route_tokens.argtypes = [P, P, Z, P, P, P, P, P]
         L.ora_route_tokens.restype = C.c_int
         L.ora_permute.argtypes = [P, Z, Z, Z, P, P, P]
@@ -192,6 +197,16 @@ def expert_forward_f64(w_gate, w_up, w_down, x) -> np.ndarray:
     return y
 
 
+def rms_norm_gamma(x, gamma, eps: float, norm_policy: int = 0) -> np.ndarray:
+    """RMSNorm(x) * gamma over one row; norm_policy 0 = the graph's f32 arithmetic
+    (nn/normalization.rs:8-37 + BroadcastMul), 1 = f64 accumulation (mla.rs:230-239)."""
+    x, gamma = _f32(x), _f32(gamma)
+    assert x.size == gamma.size
+    y = np.empty(x.size, dtype=np.float32)
+    lib().ora_rms_norm_gamma(_p(x), _p(gamma), x.size, eps, norm_policy, _p(y))
+    return y
+
+
 def sigmoid_dot(g, x) -> float:
     g, x = _f32(g), _f32(x)
     return float(lib().ora_sigmoid_dot(_p(g), _p(x), min(g.size, x.size)))
@@ -281,6 +296,26 @@ class Layer:
         if rc != OK:
             raise OracleError(rc, et.value, ei.value)
         return out, idx, w
+
+    def block_forward(self, x1, gamma, eps: float, norm_policy: int = NORM_GRAPH_F32,
+                      policy: int = CERTIFIED):
+        """full_forward.rs:239-252: out = x1 + MoE(RMSNorm(x1) * gamma), row by row.
+        Returns (out, h2, idx, w)."""
+        x1 = _f32(x1).reshape(-1, self.d)
+        gamma = _f32(gamma)
+        assert gamma.size == self.d
+        T = x1.shape[0]
+        out = np.empty((T, self.d), dtype=np.float32)
+        h2 = np.empty((T, self.d), dtype=np.float32)
+        idx = np.empty((T, self.top_k), dtype=np.int32)
+        w = np.empty((T, self.top_k), dtype=np.float32)
+        et, ei = C.c_int32(-1), C.c_int32(-1)
+        c = self._c()
+        rc = lib().ora_block_forward(C.addressof(c), _p(x1), T, _p(gamma), eps, norm_policy, policy,
+                                     _p(out), _p(h2), _p(idx), _p(w), C.addressof(et), C.addressof(ei))
+        if rc != OK:
+            raise OracleError(rc, et.value, ei.value)
+        return out, h2, idx, w
 
     def route_tokens(self, x, want_logits: bool = False):
         x = _f32(x).reshape(-1, self.d)

@@ -27,6 +27,9 @@ typedef struct {
 } OraLayer;
 int ora_layer_forward_with(const OraLayer* L, const float* x, int convention, int policy, float* out,
                            int32_t* idx_out, float* w_out, int32_t* err_index);
+int ora_block_forward(const OraLayer* L, const float* x1, size_t n_tokens, const float* gamma, float eps,
+                      int norm_policy, int policy, float* out, float* h2_out, int32_t* idx_out, float* w_out,
+                      int32_t* err_token, int32_t* err_index);
 void ora_expert_forward(const float* w_gate, const float* w_up, const float* w_down, size_t d, size_t f,
                         const float* x, float* out, int policy);
 void ora_seeded(uint64_t seed, size_t n, float* out);
@@ -314,6 +317,29 @@ int main(int argc, char** argv) {
     ora_expert_forward(fx.gate.data(), fx.up.data(), fx.down.data(), fx.d, fx.f, fx.input.data(), want.data(), 0);
     CHECK(metrics(out, want).max_abs_diff < 1e-5, "renormalised combine of identical experts: %g",
           metrics(out, want).max_abs_diff);
+  });
+  run_test("ffn_block_is_residual_plus_layer_of_normed_rows", [&] {
+    // src/moe/full_forward.rs:239-252 on the Qwen fixture's weights (gated shared expert), three
+    // rows, both norm arithmetics; the oracle's block is the checker.
+    RealMoeLayer layer = layer_from(*q15);
+    const size_t d = q15->d;
+    std::vector<float> x1 = seeded(21, 3 * d), gamma = seeded(22, d);
+    for (auto& g : gamma) g = 1.0f + 0.25f * g;
+    const MoeExecutionConvention conv = layer.resolve_convention();
+    OraLayer L = ora_of(*q15, (int)conv);
+    for (int pol = 0; pol < 2; ++pol) {
+      auto got = layer.ffn_block(x1, gamma, 1e-6f, (RealMoeLayer::NormPolicy)pol, conv).unwrap();
+      std::vector<float> want(x1.size());
+      int32_t et = -1, ei = -1;
+      CHECK(ora_block_forward(&L, x1.data(), 3, gamma.data(), 1e-6f, pol, 0, want.data(), nullptr, nullptr,
+                              nullptr, &et, &ei) == 0, "oracle block");
+      double scale = 0;
+      for (float v : want) scale = std::max(scale, (double)std::fabs(v));
+      CHECK(metrics(got, want).max_abs_diff <= 1e-5 * scale, "policy %d: %g of %g", pol,
+            metrics(got, want).max_abs_diff, scale);
+    }
+    auto bad = layer.ffn_block(x1, std::vector<float>(d - 1, 1.0f), 1e-6f, RealMoeLayer::NormPolicy::GraphF32, conv);
+    CHECK(bad.is_err() && bad.error().kind == MoeLayerError::Sparse, "gamma of the wrong length");
   });
   run_test("non_finite_input_surfaces_as_sparse_error", [&] {
     Fixture fx = synthetic(4, 2, 8, 16);

@@ -355,3 +355,31 @@ def test_packed_gate_up_layout(ora):
     with capi.Layer(top_k=2, w_router=W["w_router"], w_gate=packed, w_down=W["w_down"]) as a, \
             capi.Layer(top_k=2, **W) as b:
         assert a.forward(x).tobytes() == b.forward(x).tobytes()
+
+
+@pytest.mark.parametrize("wd", [capi.WEIGHT_F32, capi.WEIGHT_BF16])
+@pytest.mark.parametrize("T,shared", [(1, False), (37, True), (700, False)])
+def test_combine_is_bit_exact_given_expert_outputs(ora, wd, T, shared):
+    """src/moe/sparse.rs:87-116, 226-233: out = sum over slots of w * y with the product and the
+    sum rounded separately in f32 (an FMA gives other bits), then += the shared expert's row.
+    Fed with the GPU's own expert outputs and routing weights (taps), the oracle's combine must
+    reproduce the layer output bit for bit."""
+    d, k = 256, 3
+    W = S.make_weights(88, 8, d, 128, f_s=64 if shared else 0)
+    oL, gL = S.build_pair(ora, W, k, capi.CONVENTION_ATENIA, wd)
+    with gL:
+        x = S.make_tokens(89 + T, T, d, bf16=wd != capi.WEIGHT_F32)
+        out = gL.forward(x).reshape(T, d)
+        _, w, *_ = gL.last_routing(T)
+        y, ys = gL.last_expert_outputs(T)
+        want = np.zeros((T, d), dtype=np.float32)
+        for s_ in range(k):
+            want = want + w[:, s_, None] * y[:, s_, :]  # f32 * f32 and f32 + f32, each rounded
+        if shared:
+            want = want + ys
+        assert want.dtype == np.float32 and out.tobytes() == want.tobytes()
+        for t in {0, T // 2, T - 1}:  # the same through the oracle's combine_selected
+            o = ora.combine_selected(np.arange(k), w[t], y[t], d)
+            if shared:
+                o = o + ys[t]
+            assert out[t].tobytes() == o.tobytes()
