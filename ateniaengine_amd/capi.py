@@ -39,7 +39,7 @@ EXPORTS = (
     "atenia_moe_hip_layer_last_non_finite", "atenia_moe_router_launch_device", "atenia_moe_permute_launch_device",
     "atenia_moe_expert_ffn_launch_device", "atenia_moe_combine_launch_device",
     "atenia_moe_hip_layer_block_forward", "atenia_moe_hip_layer_block_forward_device",
-    "atenia_moe_hip_layer_last_normed",
+    "atenia_moe_hip_layer_last_normed", "atenia_moe_hip_layer_set_v3_router",
 )
 
 
@@ -104,6 +104,7 @@ def lib():
         L.atenia_moe_hip_layer_block_forward_device.argtypes = [P, P, C.c_int, P, C.c_float,
                                                                 C.c_int, P, P]
         L.atenia_moe_hip_layer_last_normed.argtypes = [P, P]
+        L.atenia_moe_hip_layer_set_v3_router.argtypes = [P, C.c_int, C.c_int, C.c_double, C.c_int, P]
         L.atenia_moe_router_launch_device.argtypes = [P, P, C.c_int, C.c_int, P, P, P]
         L.atenia_moe_permute_launch_device.argtypes = [P, C.c_int, P, P, P, P]
         L.atenia_moe_expert_ffn_launch_device.argtypes = [P, P, C.c_int, C.c_int, P]
@@ -216,6 +217,15 @@ class Layer:
         """Raw device pointers (ints); asynchronous on `stream`."""
         _check(lib().atenia_moe_hip_layer_forward_device(self._h, d_x, x_dtype, n_tokens, d_out,
                                                          stream))
+
+    def set_v3_router(self, n_group: int, topk_group: int, routed_scaling_factor: float,
+                      norm_topk_prob: bool, e_score_correction_bias):
+        """DeepSeek-V3 routing for every later call on this layer (v3_router.rs:206-309)."""
+        b = np.ascontiguousarray(e_score_correction_bias, dtype=np.float32)
+        assert b.size == self.E
+        _check(lib().atenia_moe_hip_layer_set_v3_router(self._h, n_group, topk_group,
+                                                        routed_scaling_factor, int(norm_topk_prob),
+                                                        _ptr(b)))
 
     # The decoder layer's FFN block around the op: out = x1 + MoE(RMSNorm(x1) * gamma).
     def block_forward(self, x1, gamma, eps: float, norm_policy: int = NORM_GRAPH_F32) -> np.ndarray:

@@ -96,6 +96,11 @@ struct AteniaMoeLayer {
       shared_desc, ident, h, hs, y, ys, status, tile_group, tile_m0, s_tile_group, s_tile_m0,
       part_flags;
   DevBuf xn, gamma_in;  // block forward: normalised rows [T, d] f32; gamma of the host variant
+  // DeepSeek-V3 routing (off while v3_n_group == 0): the router kernels leave raw logits in
+  // `logits` and v3_route_kernel decides from them
+  int v3_n_group = 0, v3_topk_group = 0, v3_norm = 0;
+  double v3_scale = 1.0;
+  DevBuf v3_bias, logits;
   int normed_T = 0;     // rows of xn the last block forward wrote
   int last_T = 0;
   int stage_T[4] = {-1, -1, -1, -1};  // token count each pipeline stage last completed for
@@ -287,7 +292,7 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   ra.w_router = L->w_router.as<float>();
   ra.router_bias = L->router_bias.as<float>();
   const bool gated = L->fs > 0 && L->conv == ATENIA_MOE_CONVENTION_HUGGINGFACE_QWEN &&
-                     L->shared_gate.p != nullptr;
+                     L->shared_gate.p != nullptr && L->v3_n_group == 0;
   ra.shared_gate = gated ? L->shared_gate.as<float>() : nullptr;
   ra.idx = L->idx.as<int32_t>();
   ra.w = L->w.as<float>();
@@ -316,10 +321,34 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   pa.n_tiles = L->shared_desc.as<int32_t>() + 4;
   pa.shared_n_tiles = L->shared_desc.as<int32_t>() + 5;
   ra.fuse_permute = last >= kStagePermute ? &pa : nullptr;
+  const bool v3 = L->v3_n_group > 0;
+  if (v3) {
+    int rc = L->logits.ensure((size_t)L->cap_tokens * L->E * 4);
+    if (rc) return rc;
+    ra.logits_out = L->logits.as<float>();
+    ra.shared_gate = nullptr;  // the V3 block adds its shared experts ungated
+  }
   int fused = 0;
   if (first <= kStageRouter) {
     HIP_TRY(launch_router(ra, s, &fused));
     L->launches[0] = 1;
+    if (v3) {
+      V3RouteArgs va{};
+      va.logits = L->logits.as<float>();
+      va.bias = L->v3_bias.as<float>();
+      va.T = T;
+      va.E = L->E;
+      va.k = L->k;
+      va.n_group = L->v3_n_group;
+      va.topk_group = L->v3_topk_group;
+      va.norm_topk_prob = L->v3_norm;
+      va.routed_scaling_factor = L->v3_scale;
+      va.idx = L->idx.as<int32_t>();
+      va.w = L->w.as<float>();
+      va.status = L->status.as<int32_t>();
+      HIP_TRY(launch_v3_route(va, s));
+      L->launches[0] = 2;
+    }
     L->stage_T[kStageRouter] = T;
   }
   tm.mark();  // ev[1]: router done
@@ -502,8 +531,9 @@ int atenia_moe_hip_layer_create(const AteniaMoeLayerDesc* D, AteniaMoeLayer** ou
     if (int8 && (!D->s_scale_gate || !D->s_scale_up || !D->s_scale_down))
       return fail(ATENIA_MOE_ERR_DIM, "int8 shared expert needs per-row scales");
   }
-  if (D->num_experts + 1 > kMaxRouterRows)
-    return fail(ATENIA_MOE_ERR_UNSUPPORTED, "at most %d experts", kMaxRouterRows - 1);
+  if (D->num_experts + (D->shared_gate ? 1 : 0) > kMaxRouterRows)
+    return fail(ATENIA_MOE_ERR_UNSUPPORTED, "at most %d router rows (experts + shared-expert gate)",
+                kMaxRouterRows);
   if (!atenia_moe_hip_available())
     return fail(ATENIA_MOE_ERR_LAUNCH, "no gfx950 device available");
 
@@ -788,6 +818,47 @@ int atenia_moe_hip_layer_last_non_finite(AteniaMoeLayer* L, int32_t* token, int3
   std::lock_guard<std::mutex> lock(L->mu);
   if (token) *token = L->nf_token;
   if (expert) *expert = L->nf_expert;
+  return ATENIA_MOE_OK;
+}
+
+int atenia_moe_hip_layer_set_v3_router(AteniaMoeLayer* L, int n_group, int topk_group,
+                                       double routed_scaling_factor, int norm_topk_prob,
+                                       const float* e_score_correction_bias_host) {
+  if (!valid_handle(L)) return fail(ATENIA_MOE_ERR_HANDLE, "invalid layer handle");
+  // V3RouterConfig::validate (src/moe/v3_router.rs:148-181), same order, same texts.
+  if (n_group <= 0) return fail(ATENIA_MOE_ERR_K, "v3-router: n_group must be > 0");
+  if (topk_group <= 0) return fail(ATENIA_MOE_ERR_K, "v3-router: topk_group must be > 0");
+  if (L->E % n_group != 0)
+    return fail(ATENIA_MOE_ERR_K, "v3-router: n_routed_experts (%d) not divisible by n_group (%d)",
+                L->E, n_group);
+  const int epg = L->E / n_group;
+  if (epg < 2)
+    return fail(ATENIA_MOE_ERR_K, "v3-router: experts_per_group (%d) < 2 (HF takes top-2 per group)",
+                epg);
+  if (topk_group > n_group)
+    return fail(ATENIA_MOE_ERR_K, "v3-router: topk_group (%d) > n_group (%d)", topk_group, n_group);
+  if (L->k > topk_group * epg)
+    return fail(ATENIA_MOE_ERR_K, "v3-router: top_k (%d) exceeds experts in selected groups (%d)",
+                L->k, topk_group * epg);
+  if (!e_score_correction_bias_host)
+    return fail(ATENIA_MOE_ERR_DIM, "v3-router: e_score_correction_bias length 0 != n_routed_experts %d",
+                L->E);
+  for (int i = 0; i < L->E; ++i)
+    if (!std::isfinite(e_score_correction_bias_host[i]))
+      return fail(ATENIA_MOE_ERR_NON_FINITE, "v3-router: e_score_correction_bias at %d is non-finite", i);
+  if (!std::isfinite(routed_scaling_factor))
+    return fail(ATENIA_MOE_ERR_NON_FINITE, "v3-router: routed_scaling_factor is non-finite");
+  if (L->router_bias.p)
+    return fail(ATENIA_MOE_ERR_UNSUPPORTED, "v3-router: the layer was created with an additive router bias");
+  if (L->E > 256) return fail(ATENIA_MOE_ERR_UNSUPPORTED, "v3-router: at most 256 experts");
+  std::lock_guard<std::mutex> lock(L->mu);
+  int rc = upload_f32(e_score_correction_bias_host, (size_t)L->E, L->v3_bias);
+  if (rc) return rc;
+  L->v3_n_group = n_group;
+  L->v3_topk_group = topk_group;
+  L->v3_norm = norm_topk_prob ? 1 : 0;
+  L->v3_scale = routed_scaling_factor;
+  for (int st = 0; st < 4; ++st) L->stage_T[st] = -1;
   return ATENIA_MOE_OK;
 }
 

@@ -65,9 +65,23 @@ struct RouterArgs {
   // When T == 1 and the per-token kernel runs, it also writes the expert grouping (the
   // result of kernel 2 for a single token is known as soon as the top-k is), saving a launch.
   const struct PermuteArgs* fuse_permute;  // null = do not fuse
+  // non-null: write the raw logits [T, E] here and leave idx / w alone (another kernel routes)
+  float* logits_out;
 };
 // *fused_permute is set to 1 when the launch also produced the expert grouping.
 hipError_t launch_router(const RouterArgs& a, hipStream_t s, int* fused_permute);
+
+// DeepSeek-V3 routing from raw logits (src/moe/v3_router.rs:206-309).
+struct V3RouteArgs {
+  const float* logits;  // [T, E]
+  const float* bias;    // [E] e_score_correction_bias (selection only)
+  int T, E, k, n_group, topk_group, norm_topk_prob;
+  double routed_scaling_factor;
+  int32_t* idx;         // [T, k] ascending
+  float* w;             // [T, k]
+  int32_t* status;      // [2]: code, (token << 10 | expert)
+};
+hipError_t launch_v3_route(const V3RouteArgs& a, hipStream_t s);
 
 struct PermuteArgs {
   const int32_t* idx;  // [P] expert of each pair, P = T*k

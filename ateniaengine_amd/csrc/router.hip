@@ -130,7 +130,7 @@ __global__ __launch_bounds__(kRouterThreads) void router_tile_kernel(
     const float* __restrict__ w_router, const float* __restrict__ bias,
     const float* __restrict__ gate_vec, int32_t* __restrict__ idx_out,
     float* __restrict__ w_out, float* __restrict__ sgate_out, uint16_t* __restrict__ xb,
-    int d_pad, int32_t* __restrict__ status, int tokens_per_block) {
+    int d_pad, int32_t* __restrict__ status, float* __restrict__ logits_out, int tokens_per_block) {
   const int R = E + (gate_vec ? 1 : 0);  // rows of the stacked [W_r ; gate] matrix
   const int TT = tokens_per_block;
   const int t0 = blockIdx.x * TT;
@@ -186,11 +186,13 @@ __global__ __launch_bounds__(kRouterThreads) void router_tile_kernel(
     if (r < E) {
       if (bias) logit = logit + bias[r];
       sLogit[tl * R + r] = logit;
+      if (logits_out) logits_out[(size_t)(t0 + tl) * E + r] = logit;
     } else {
       sgate_out[t0 + tl] = (float)(1.0 / (1.0 + exp(-acc)));
     }
   }
   __syncthreads();
+  if (logits_out) return;  // routing is decided by another kernel from the raw logits
   const int tls = owner ? tl : 0;
   softmax_topk(owner && r < E, r, E, k, renorm, t0 + tls, sLogit + tls * R, sExp + tls * E,
                sWt + tls * E, sSel + tls * E, idx_out, w_out, status);
@@ -304,7 +306,7 @@ __global__ __launch_bounds__(kRouterThreads) void router_batch_kernel(
     const float* __restrict__ w_router, const float* __restrict__ bias,
     const float* __restrict__ gate_vec, int32_t* __restrict__ idx_out,
     float* __restrict__ w_out, float* __restrict__ sgate_out, uint16_t* __restrict__ xb,
-    int d_pad, int32_t* __restrict__ status) {
+    int d_pad, int32_t* __restrict__ status, float* __restrict__ logits_out) {
   constexpr int RG = 16;                   // row groups = threads per token
   constexpr int TG = kRouterThreads / RG;  // 16 token groups = threads per row group
   constexpr int TT = TG * TPT;             // tokens per block: a thread owns tokens tg, tg + TG, ...
@@ -316,6 +318,9 @@ __global__ __launch_bounds__(kRouterThreads) void router_batch_kernel(
   typedef XVec<XT> XV;
   const int R = E + (gate_vec ? 1 : 0);
   const int t0 = blockIdx.x * TT;
+  // More than RW rows: blockIdx.y picks the block of RW rows (only when the logits go to
+  // `logits_out`, since the softmax below needs all rows of a token in one workgroup).
+  const int r_lo = blockIdx.y * RW;
   const int tid = threadIdx.x;
   const int tg = tid / RG, rg = tid - tg * RG;
 
@@ -337,8 +342,8 @@ __global__ __launch_bounds__(kRouterThreads) void router_batch_kernel(
       const int j = tid + i * kRouterThreads;
       const int row = j / KV, c = c0 + (j - row * KV) * 4;
       wr[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (j < RW * KV && row < R && c < d)
-        wr[i] = *(const float4*)((row < E ? w_router + (size_t)row * d : gate_vec) + c);
+      if (j < RW * KV && r_lo + row < R && c < d)
+        wr[i] = *(const float4*)((r_lo + row < E ? w_router + (size_t)(r_lo + row) * d : gate_vec) + c);
     }
   };
   auto store_tile = [&](const xvec_t (&xr)[NX], const float4 (&wr)[NW], int c0) {
@@ -353,7 +358,7 @@ __global__ __launch_bounds__(kRouterThreads) void router_batch_kernel(
         *(double2*)dst = make_double2((double)f[0], (double)f[1]);
         *(double2*)(dst + 2) = make_double2((double)f[2], (double)f[3]);
         const int c = c0 + cl;
-        if (xb && t0 + row < T && c < d_pad) {
+        if (xb && blockIdx.y == 0 && t0 + row < T && c < d_pad) {
           uint2 b;
           b.x = f32_to_bf16_rne(f[0]) | ((uint32_t)f32_to_bf16_rne(f[1]) << 16);
           b.y = f32_to_bf16_rne(f[2]) | ((uint32_t)f32_to_bf16_rne(f[3]) << 16);
@@ -454,17 +459,19 @@ __global__ __launch_bounds__(kRouterThreads) void router_batch_kernel(
     if (t0 + tl >= T) continue;
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
-      const int r = rg + i * RG;
+      const int r = r_lo + rg + i * RG;
       if (r < E) {
         float logit = (float)acc[j][i];
         if (bias) logit = logit + bias[r];
         sLogit[tl * R + r] = logit;
+        if (logits_out) logits_out[(size_t)(t0 + tl) * E + r] = logit;
       } else if (r < R) {
         sgate_out[t0 + tl] = (float)(1.0 / (1.0 + exp(-acc[j][i])));
       }
     }
   }
   __syncthreads();
+  if (logits_out) return;  // routing is decided by another kernel from the raw logits
   softmax_topk_block(TT, R, E, k, renorm, t0, T, sLogit, sExp, sWt, sSel, sTok, idx_out, w_out,
                      status);
 }
@@ -484,9 +491,11 @@ hipError_t launch_router_batch(const RouterArgs& a, hipStream_t s) {
     attr_bytes = smem;
   }
   const int blocks = (a.T + TT - 1) / TT;
-  router_batch_kernel<XT, RPT, TPT, KC><<<blocks, kRouterThreads, smem, s>>>(
+  const int row_blocks = (R + RW - 1) / RW;
+  if (row_blocks > 1 && !a.logits_out) return hipErrorInvalidValue;
+  router_batch_kernel<XT, RPT, TPT, KC><<<dim3(blocks, row_blocks), kRouterThreads, smem, s>>>(
       (const XT*)a.x, a.T, a.d, a.E, a.k, a.renorm, a.w_router, a.router_bias, a.shared_gate,
-      a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status);
+      a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status, a.logits_out);
   return hipGetLastError();
 }
 
@@ -502,7 +511,8 @@ hipError_t dispatch_router_batch(const RouterArgs& a, int R, hipStream_t s) {
     return e ? atoi(e) : 0;
   }();
   // measured on MI355X at 64 rows, d = 2048: two tokens per thread pay from 8192 tokens on
-  const int tpt = forced ? forced : (a.T >= 8192 ? 2 : 1);
+  const long long work = (long long)a.T * ((R + 63) / 64);  // row blocks count like more tokens
+  const int tpt = forced ? forced : (work >= 8192 ? 2 : 1);
   if (tpt >= 2) return launch_router_batch<XT, 4, 2, 64>(a, s);
   return launch_router_batch<XT, 4, 1, 64>(a, s);
 }
@@ -519,8 +529,13 @@ __global__ __launch_bounds__(kTokenThreads) void router_token_kernel(
     const float* __restrict__ w_router, const float* __restrict__ bias,
     const float* __restrict__ gate_vec, int32_t* __restrict__ idx_out,
     float* __restrict__ w_out, float* __restrict__ sgate_out, uint16_t* __restrict__ xb,
-    int d_pad, int32_t* __restrict__ status, FusedGrouping fg) {
-  const int R = E + (gate_vec ? 1 : 0);
+    int d_pad, int32_t* __restrict__ status, float* __restrict__ logits_out, FusedGrouping fg) {
+  // gridDim.y > 1 (only when the logits go to `logits_out`): this workgroup computes rows
+  // row_lo .. row_lo + R - 1 of the stacked matrix; otherwise all of them.
+  const int R_all = E + (gate_vec ? 1 : 0);
+  const int rows_per_block = (R_all + gridDim.y - 1) / gridDim.y;
+  const int row_lo = blockIdx.y * rows_per_block;
+  const int R = min(rows_per_block, R_all - row_lo);
   const int t = blockIdx.x;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   constexpr int NW = kTokenThreads / 64;
@@ -546,7 +561,7 @@ __global__ __launch_bounds__(kTokenThreads) void router_token_kernel(
       sX[c] = v;
       sLx[c] = (int16_t)max(lsb_exponent(v), -32000);
     }
-    if (xb && c < d_pad) xb[(size_t)t * d_pad + c] = f32_to_bf16_rne(v);
+    if (xb && blockIdx.y == 0 && c < d_pad) xb[(size_t)t * d_pad + c] = f32_to_bf16_rne(v);
   }
   __syncthreads();
 
@@ -558,7 +573,7 @@ __global__ __launch_bounds__(kTokenThreads) void router_token_kernel(
   const bool vec_ok = (d & 3) == 0;
   for (int item = wave; item < R * KS; item += NW) {
     const int r = item / KS, ksl = item - r * KS;
-    const float* wr = r < E ? w_router + (size_t)r * d : gate_vec;
+    const float* wr = row_lo + r < E ? w_router + (size_t)(row_lo + r) * d : gate_vec;
     const int c_lo = ksl * slice, c_hi = min(d, c_lo + slice);
     double acc = 0.0, asum = 0.0;
     int qmin = kNoLsb;
@@ -614,7 +629,7 @@ __global__ __launch_bounds__(kTokenThreads) void router_token_kernel(
   if (*sBad) {
     // The reference's own order: one sequential c-ascending f64 sum per row.
     for (int r = tid; r < R; r += kTokenThreads) {
-      const float* wr = r < E ? w_router + (size_t)r * d : gate_vec;
+      const float* wr = row_lo + r < E ? w_router + (size_t)(row_lo + r) * d : gate_vec;
       double acc = 0.0;
       for (int c = 0; c < d; ++c) acc = fma((double)wr[c], (double)sX[c], acc);
       sAcc[r] = acc;
@@ -623,15 +638,18 @@ __global__ __launch_bounds__(kTokenThreads) void router_token_kernel(
   }
   if (tid < R) {
     double acc = sAcc[tid];
-    if (tid < E) {
+    const int gr = row_lo + tid;
+    if (gr < E) {
       float logit = (float)acc;
-      if (bias) logit = logit + bias[tid];
-      sLogit[tid] = logit;
+      if (bias) logit = logit + bias[gr];
+      sLogit[tid] = logit;  // indexed by expert when the workgroup holds all rows (row_lo == 0)
+      if (logits_out) logits_out[(size_t)t * E + gr] = logit;
     } else {
       sgate_out[t] = (float)(1.0 / (1.0 + exp(-acc)));
     }
   }
   __syncthreads();
+  if (logits_out) return;  // routing is decided by another kernel from the raw logits
   softmax_topk(tid < E, tid, E, k, renorm, t, sLogit, sExp, sWt, sSel, idx_out, w_out, status);
   if (fg.counts) {  // T == 1: the grouping of a single token follows from its top-k
     __syncthreads();
@@ -666,31 +684,41 @@ hipError_t launch_router(const RouterArgs& a, hipStream_t s, int* fused_permute)
   const int R = a.E + (a.shared_gate ? 1 : 0);
   if (fused_permute) *fused_permute = 0;
   if (R > kMaxRouterRows || a.T <= 0) return hipErrorInvalidValue;
-  if (a.T <= a.token_kernel_max_tokens) {
+  // The per-token kernel re-reads the whole stacked matrix for every token; with many rows
+  // (row blocks, logits mode) that only pays for a handful of tokens.
+  const bool token_ok = a.T <= a.token_kernel_max_tokens &&
+                        (R <= 64 || (long long)a.T * R * a.d <= (16ll << 20));
+  if (token_ok) {
     const size_t np = R > kTokenThreads / 64 ? R : kTokenThreads / 64;
     size_t smem = ((size_t)R + a.E + 2 * np) * 8 + (size_t)a.d * 4 + (size_t)a.E * 12 + 4 +
                   np * 4 + (size_t)a.d * 2 + 16;
     if (smem <= 64 * 1024) {
       FusedGrouping fg{};
-      if (a.T == 1 && a.fuse_permute) {
+      if (a.T == 1 && a.fuse_permute && !a.logits_out) {
         const PermuteArgs& pa = *a.fuse_permute;
         fg = FusedGrouping{pa.counts, pa.offsets, pa.perm, pa.inv, pa.active, pa.n_active,
                            pa.shared_offsets, pa.tile_group, pa.tile_m0, pa.n_tiles,
                            pa.shared_n_tiles};
         if (fused_permute) *fused_permute = 1;
       }
+      // Four rows per workgroup (a row split over four waves) once the rows can be spread over
+      // workgroups, i.e. when the logits leave the kernel: the few tokens this kernel serves
+      // then keep R / 4 workgroups streaming the router matrix instead of one.
+      const int row_blocks = a.logits_out && R > 32 ? (R + 3) / 4 : 1;
+      const dim3 grid(a.T, row_blocks);
       if (a.x_is_bf16)
-        router_token_kernel<uint16_t><<<a.T, kTokenThreads, smem, s>>>(
+        router_token_kernel<uint16_t><<<grid, kTokenThreads, smem, s>>>(
             (const uint16_t*)a.x, a.T, a.d, a.E, a.k, a.renorm, a.w_router, a.router_bias,
-            a.shared_gate, a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status, fg);
+            a.shared_gate, a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status, a.logits_out, fg);
       else
-        router_token_kernel<float><<<a.T, kTokenThreads, smem, s>>>(
+        router_token_kernel<float><<<grid, kTokenThreads, smem, s>>>(
             (const float*)a.x, a.T, a.d, a.E, a.k, a.renorm, a.w_router, a.router_bias,
-            a.shared_gate, a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status, fg);
+            a.shared_gate, a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status, a.logits_out, fg);
       return hipGetLastError();
     }
   }
-  if (R <= 64 && a.d % 4 == 0 && (!a.xb || a.d_pad % 4 == 0)) {
+  // Up to 64 rows per workgroup; more rows only when the logits leave the kernel (row blocks).
+  if ((R <= 64 || a.logits_out) && a.d % 4 == 0 && (!a.xb || a.d_pad % 4 == 0)) {
     return a.x_is_bf16 ? dispatch_router_batch<uint16_t>(a, R, s)
                        : dispatch_router_batch<float>(a, R, s);
   }
@@ -705,11 +733,11 @@ hipError_t launch_router(const RouterArgs& a, hipStream_t s, int* fused_permute)
   if (a.x_is_bf16) {
     router_tile_kernel<uint16_t><<<blocks, kRouterThreads, smem, s>>>(
         (const uint16_t*)a.x, a.T, a.d, a.E, a.k, a.renorm, a.w_router, a.router_bias,
-        a.shared_gate, a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status, TT);
+        a.shared_gate, a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status, a.logits_out, TT);
   } else {
     router_tile_kernel<float><<<blocks, kRouterThreads, smem, s>>>(
         (const float*)a.x, a.T, a.d, a.E, a.k, a.renorm, a.w_router, a.router_bias,
-        a.shared_gate, a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status, TT);
+        a.shared_gate, a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status, a.logits_out, TT);
   }
   return hipGetLastError();
 }

@@ -2,6 +2,7 @@
 // interface each part follows).
 #include "atenia_moe.hpp"
 
+#include <cmath>
 #include <cstring>
 #include <map>
 #include <utility>
@@ -81,6 +82,57 @@ std::string MoeBindingError::to_string() const {
     case Dense: return "moe-binding: " + dense.to_string();
   }
   return "moe-binding";
+}
+
+std::string V3RouterError::to_string() const {
+  const std::string A = std::to_string(a), B = std::to_string(b);
+  switch (kind) {  // src/moe/v3_router.rs:96-122
+    case UnsupportedScoringFunc:
+      return "v3-router: unsupported scoring_func '" + got + "' (only 'sigmoid')";
+    case ExpertsNotDivisibleByGroups:
+      return "v3-router: n_routed_experts (" + A + ") not divisible by n_group (" + B + ")";
+    case GroupTooSmall:
+      return "v3-router: experts_per_group (" + A + ") < 2 (HF takes top-2 per group)";
+    case TopkGroupExceedsGroups: return "v3-router: topk_group (" + A + ") > n_group (" + B + ")";
+    case TopKExceedsSelectable:
+      return "v3-router: top_k (" + A + ") exceeds experts in selected groups (" + B + ")";
+    case ZeroParameter: return std::string("v3-router: ") + what + " must be > 0";
+    case LengthMismatch:
+      return std::string("v3-router: ") + what + " length " + B + " != n_routed_experts " + A;
+    case NonFinite: return std::string("v3-router: ") + what + " at " + A + " is non-finite";
+    case TopKMismatch:
+      return "v3-router: top_k (" + A + ") differs from the layer's experts_per_token (" + B + ")";
+  }
+  return "v3-router";
+}
+
+Result<ScoringFunc, V3RouterError> parse_scoring_func(const std::string& s) {
+  typedef Result<ScoringFunc, V3RouterError> R;
+  if (s == "sigmoid") return R::Ok(ScoringFunc::Sigmoid);
+  V3RouterError e{V3RouterError::UnsupportedScoringFunc};
+  e.got = s;
+  return R::Err(e);
+}
+
+std::optional<V3RouterError> V3RouterConfig::validate() const {
+  auto err = [](V3RouterError::Kind k, size_t a = 0, size_t b = 0, const char* what = "") {
+    V3RouterError e{k};
+    e.a = a;
+    e.b = b;
+    e.what = what;
+    return e;
+  };
+  if (top_k == 0) return err(V3RouterError::ZeroParameter, 0, 0, "top_k");
+  if (n_group == 0) return err(V3RouterError::ZeroParameter, 0, 0, "n_group");
+  if (topk_group == 0) return err(V3RouterError::ZeroParameter, 0, 0, "topk_group");
+  if (n_routed_experts % n_group != 0)
+    return err(V3RouterError::ExpertsNotDivisibleByGroups, n_routed_experts, n_group);
+  const size_t per_group = n_routed_experts / n_group;
+  if (per_group < 2) return err(V3RouterError::GroupTooSmall, per_group);
+  if (topk_group > n_group) return err(V3RouterError::TopkGroupExceedsGroups, topk_group, n_group);
+  if (top_k > topk_group * per_group)
+    return err(V3RouterError::TopKExceedsSelectable, top_k, topk_group * per_group);
+  return std::nullopt;
 }
 
 std::string MoeLayerError::to_string() const {
@@ -192,7 +244,8 @@ struct RealMoeLayer::Device {
 RealMoeLayer::RealMoeLayer() : dev_(new Device()) {}
 RealMoeLayer::RealMoeLayer(const RealMoeLayer& o)
     : config(o.config), routed(o.routed), shared(o.shared), shared_gate(o.shared_gate),
-      storage(o.storage), dev_(new Device()) {}
+      storage(o.storage), v3_router(o.v3_router),
+      e_score_correction_bias(o.e_score_correction_bias), dev_(new Device()) {}
 RealMoeLayer& RealMoeLayer::operator=(const RealMoeLayer& o) {
   if (this != &o) {
     config = o.config;
@@ -200,13 +253,16 @@ RealMoeLayer& RealMoeLayer::operator=(const RealMoeLayer& o) {
     shared = o.shared;
     shared_gate = o.shared_gate;
     storage = o.storage;
+    v3_router = o.v3_router;
+    e_score_correction_bias = o.e_score_correction_bias;
     dev_.reset(new Device());
   }
   return *this;
 }
 RealMoeLayer::RealMoeLayer(RealMoeLayer&& o) noexcept
     : config(o.config), routed(std::move(o.routed)), shared(std::move(o.shared)),
-      shared_gate(std::move(o.shared_gate)), storage(o.storage), dev_(std::move(o.dev_)) {
+      shared_gate(std::move(o.shared_gate)), storage(o.storage), v3_router(o.v3_router),
+      e_score_correction_bias(std::move(o.e_score_correction_bias)), dev_(std::move(o.dev_)) {
   o.dev_.reset(new Device());
 }
 RealMoeLayer& RealMoeLayer::operator=(RealMoeLayer&& o) noexcept {
@@ -216,6 +272,8 @@ RealMoeLayer& RealMoeLayer::operator=(RealMoeLayer&& o) noexcept {
     shared = std::move(o.shared);
     shared_gate = std::move(o.shared_gate);
     storage = o.storage;
+    v3_router = o.v3_router;
+    e_score_correction_bias = std::move(o.e_score_correction_bias);
     dev_ = std::move(o.dev_);
     o.dev_.reset(new Device());
   }
@@ -370,8 +428,46 @@ Result<void*, MoeLayerError> RealMoeLayer::handle_for(MoeExecutionConvention con
     return R::Err(e);
   }
   if (rc) return R::Err(device_error(rc));
+  if (v3_router) {  // validated by set_v3_router; the device repeats the checks
+    rc = atenia_moe_hip_layer_set_v3_router(h, (int)v3_router->n_group, (int)v3_router->topk_group,
+                                            v3_router->routed_scaling_factor,
+                                            v3_router->norm_topk_prob ? 1 : 0,
+                                            e_score_correction_bias.data());
+    if (rc) {
+      MoeLayerError e = device_error(rc);
+      atenia_moe_hip_layer_destroy(h);
+      return R::Err(e);
+    }
+  }
   dev_->handles[key] = h;
   return R::Ok(h);
+}
+
+std::optional<V3RouterError> RealMoeLayer::set_v3_router(const V3RouterConfig& cfg,
+                                                         std::vector<float> bias) {
+  if (auto e = cfg.validate()) return e;
+  auto err = [](V3RouterError::Kind k, const char* what, size_t a, size_t b) {
+    V3RouterError e{k};
+    e.what = what;
+    e.a = a;
+    e.b = b;
+    return e;
+  };
+  if (cfg.n_routed_experts != num_experts())
+    return err(V3RouterError::LengthMismatch, "router_logits", cfg.n_routed_experts, num_experts());
+  if (bias.size() != cfg.n_routed_experts)
+    return err(V3RouterError::LengthMismatch, "e_score_correction_bias", cfg.n_routed_experts,
+               bias.size());
+  for (size_t i = 0; i < bias.size(); ++i)
+    if (!std::isfinite(bias[i])) return err(V3RouterError::NonFinite, "e_score_correction_bias", i, 0);
+  if (cfg.top_k != config.experts_per_token)
+    return err(V3RouterError::TopKMismatch, "", cfg.top_k, config.experts_per_token);
+  std::lock_guard<std::mutex> lock(dev_->mu);
+  for (auto& kv : dev_->handles) atenia_moe_hip_layer_destroy(kv.second);  // rebuilt on next use
+  dev_->handles.clear();
+  v3_router = cfg;
+  e_score_correction_bias = std::move(bias);
+  return std::nullopt;
 }
 
 namespace {

@@ -11,6 +11,8 @@
 //   MoeDenseError / MoeSparseError / MoeBindingError / MoeLayerError
 //                                             dense.rs:31-49, sparse.rs:35-50, binding.rs:41-70,
 //                                             layer.rs:119-136
+//   V3RouterConfig, ScoringFunc, V3RouterError (DeepSeek-V3 routing)
+//                                             src/moe/v3_router.rs:36-123, 148-181
 //   register_real_moe_layer, get_real_moe_layer, execute_real_moe_layer[_with]
 //                                             src/moe/graph_op.rs:228-232, 294-299, 327-364
 //   moe_real_layer_reference_node             the executor arm, src/amg/graph.rs:5572-5589
@@ -95,6 +97,22 @@ struct MoeLayerError {
   std::string to_string() const;
 };
 
+// DeepSeek-V3 routing (src/moe/v3_router.rs).  Display texts as in the reference.
+struct V3RouterError {
+  enum Kind {
+    UnsupportedScoringFunc, ExpertsNotDivisibleByGroups, GroupTooSmall, TopkGroupExceedsGroups,
+    TopKExceedsSelectable, ZeroParameter, LengthMismatch, NonFinite,
+    TopKMismatch  // extension: the configuration's top_k is not the layer's experts_per_token
+  };
+  Kind kind;
+  std::string got;          // UnsupportedScoringFunc
+  const char* what = "";    // ZeroParameter / LengthMismatch / NonFinite
+  size_t a = 0, b = 0;      // (n_routed, n_group) | experts_per_group | (topk_group, n_group) |
+                            // (top_k, selectable) | (expected, actual) | index
+  std::string to_string() const;
+};
+enum class ScoringFunc { Sigmoid };
+
 // Result<T, E> of the reference, reduced to what the mirror needs.
 template <typename T, typename E>
 class Result {
@@ -129,6 +147,18 @@ struct MoeLayerConfig {
 
 enum class MoeExecutionConvention { Atenia = 0, HuggingFaceQwen = 1 };
 
+// "sigmoid" only; anything else (also "softmax", which has its own path) is refused
+// (src/moe/v3_router.rs:44-57).
+Result<ScoringFunc, V3RouterError> parse_scoring_func(const std::string& s);
+
+struct V3RouterConfig {  // src/moe/v3_router.rs:59-72
+  size_t n_routed_experts = 0, top_k = 0, n_group = 0, topk_group = 0;
+  double routed_scaling_factor = 1.0;
+  bool norm_topk_prob = true;
+  ScoringFunc scoring_func = ScoringFunc::Sigmoid;
+  std::optional<V3RouterError> validate() const;  // src/moe/v3_router.rs:148-181
+};
+
 // How the layer's expert weights are stored in HBM.
 enum class MoeWeightStorage { F32 = 0, Bf16 = 1, Int8W8A16 = 2 };
 
@@ -160,6 +190,15 @@ class RealMoeLayer {
   std::optional<MoeDenseExpert> shared;
   std::optional<std::vector<float>> shared_gate;
   MoeWeightStorage storage = MoeWeightStorage::F32;
+  // DeepSeek-V3 routing in front of this layer's experts (unset = softmax routing).
+  std::optional<V3RouterConfig> v3_router;
+  std::vector<float> e_score_correction_bias;
+
+  // Routes every later forward the DeepSeek-V3 way (sigmoid scores, bias-corrected and
+  // group-limited selection, scaled weights; src/moe/v3_router.rs:206-309).  The shared expert,
+  // if any, is then added ungated.  Fails like v3_route does on a bad configuration or bias;
+  // cfg.n_routed_experts / cfg.top_k must be this layer's.
+  std::optional<V3RouterError> set_v3_router(const V3RouterConfig& cfg, std::vector<float> bias);
 
   // Cross-checks the parts against the config the way RealMoeLayer::assemble does
   // (src/moe/layer.rs:282-343): expert count, dimensions, shared expert present iff asked for.

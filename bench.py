@@ -33,6 +33,11 @@ CONFIGS = {
                       zipf=False, sweep=(1, 256, 8192)),
     "deepseek_bf16": dict(d=2048, E=64, k=6, f=1408, fs=2816, gated=False, conv=1, wd="bf16",
                           zipf=True, sweep=(1, 1024, 16384)),
+    # DeepSeek-V3 router shape (256 experts in 8 groups, top-8 of the 4 best groups) in front of
+    # narrow experts: times the sigmoid / group-limited routing path, not a checkpoint shape.
+    "v3route_bf16": dict(d=7168, E=256, k=8, f=256, fs=256, gated=False, conv=1, wd="bf16",
+                         zipf=False, sweep=(1, 256, 4096),
+                         v3=dict(n_group=8, topk_group=4, scale=2.5, norm=True)),
 }
 D_MODEL, N_EXPERTS, TOP_K, D_FF = 4096, 8, 2, 14336
 D_FF_SHARED = 0
@@ -272,6 +277,10 @@ def main():
     if shared is not None:
         kw.update(s_gate=shared[0], s_up=shared[1], s_down=shared[2])
     layer = capi.Layer(w_gate=gate, w_up=up, w_down=down, weight_dtype=wdt, **kw)
+    if cfg.get("v3"):
+        v3 = cfg["v3"]
+        e_bias = (0.05 * np.random.default_rng(a.seed + 2).standard_normal(N_EXPERTS)).astype(np.float32)
+        layer.set_v3_router(v3["n_group"], v3["topk_group"], v3["scale"], v3["norm"], e_bias)
 
     if a.calibrate_copy:
         src = torch.empty(1 << 28, device="cuda", dtype=torch.float32)  # 1 GiB

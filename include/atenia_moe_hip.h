@@ -140,6 +140,20 @@ int atenia_moe_hip_layer_forward(AteniaMoeLayer* layer, const float* x_host, int
 int atenia_moe_hip_layer_forward_device(AteniaMoeLayer* layer, const void* d_x, int x_dtype,
                                         int n_tokens, float* d_out, void* stream);
 
+/* Switches the handle's router to DeepSeek-V3 routing (src/moe/v3_router.rs:36-52, 206-309):
+ * scores = sigmoid(W_r x) instead of a softmax, selection on scores + e_score_correction_bias
+ * ([E] f32, host) limited to the `topk_group` best of `n_group` expert groups (group score = its
+ * two largest corrected scores), combine weights = the uncorrected scores of the top_k selected
+ * experts, normalised when `norm_topk_prob`, times `routed_scaling_factor`.  top_k is the
+ * layer's.  The shared expert, if any, is added ungated, as DeepSeek's shared experts are.
+ * Configuration errors are the reference's V3RouterError cases (rc ATENIA_MOE_ERR_K, or
+ * ATENIA_MOE_ERR_NON_FINITE for a non-finite bias, with its message text); a non-finite logit
+ * at run time is reported like a non-finite routing weight (rc -3, token and expert).  Every
+ * later forward / route / stage launch of the handle uses it. */
+int atenia_moe_hip_layer_set_v3_router(AteniaMoeLayer* layer, int n_group, int topk_group,
+                                       double routed_scaling_factor, int norm_topk_prob,
+                                       const float* e_score_correction_bias_host);
+
 /* The FFN block of a decoder layer around the op, on device-resident rows, asynchronous on
  * `stream`:  out[t] = x1[t] + MoE(RMSNorm(x1[t]) * gamma),  x1 / out: [T, d] f32, gamma: [d] f32.
  * Replaces steps 13-15 of the reference's layer loop -- the RmsNorm, BroadcastMul,

@@ -23,7 +23,10 @@
  *              ora_f32_to_bf16_bits / ora_bf16_bits_to_f32,
  *              ora_numerical_metrics, ora_layer_forward_f64, ora_permute
  *              (brute force), ora_matvec_f32acc, ora_rms_norm_gamma,
- *              ora_block_forward.
+ *              ora_block_forward, ora_v3_validate, ora_v3_route,
+ *              ora_v3_layer_forward (router and block output against the
+ *              HuggingFace f64 fixture; its f32 combine is this build's choice,
+ *              see the function).
  *   parity unpinned (no reference counterpart; defined by this build):
  *              the `router_bias` term of ora_route (the reference router has
  *              no bias, dense.rs:333).  With router_bias == NULL ora_route is
@@ -374,6 +377,151 @@ int ora_block_forward(const OraLayer* L, const float* x1, size_t n_tokens, const
   }
   free(h2);
   free(y);
+  return rc;
+}
+
+/* ---- v3_router.rs:148-309 : DeepSeek-V3 routing of one token ------------------------
+ * scores = sigmoid(logits) in f64; choice = scores + e_score_correction_bias; the score of a
+ * group is the sum of its two largest choices; the topk_group best groups stay, experts of the
+ * other groups are masked to -inf; the top_k best remaining experts are selected (ties go to
+ * the lower index, for groups and for experts), reported ascending; the combine weights are
+ * the ORIGINAL scores of the selected experts, divided by (their sum + 1e-20) when
+ * norm_topk_prob, then multiplied by routed_scaling_factor, then rounded to f32.
+ * Pinned by the known-answer cases of the reference's own unit tests (v3_router.rs:340-462)
+ * and by the HuggingFace f64 fixture v3_route_ref (selected sets, dense weights, block out). */
+typedef struct {
+  int32_t n_group, topk_group, norm_topk_prob;
+  double routed_scaling_factor;
+} OraV3Config;
+#define ORA_V3_ERR_ZERO_PARAMETER -10      /* err_index: 0 top_k, 1 n_group, 2 topk_group */
+#define ORA_V3_ERR_NOT_DIVISIBLE -11       /* ExpertsNotDivisibleByGroups */
+#define ORA_V3_ERR_GROUP_TOO_SMALL -12     /* err_index: experts per group */
+#define ORA_V3_ERR_TOPK_GROUP_EXCEEDS -13  /* TopkGroupExceedsGroups */
+#define ORA_V3_ERR_TOPK_EXCEEDS -14        /* TopKExceedsSelectable; err_index: selectable */
+#define ORA_V3_ERR_NON_FINITE_LOGIT -15    /* NonFinite{router_logits, index} */
+#define ORA_V3_ERR_NON_FINITE_BIAS -16     /* NonFinite{e_score_correction_bias, index} */
+
+/* v3_router.rs:148-181 (V3RouterConfig::validate), same order of checks. */
+int ora_v3_validate(size_t n, size_t top_k, const OraV3Config* c, int32_t* err_index) {
+  int32_t dummy;
+  if (!err_index) err_index = &dummy;
+  if (top_k == 0) { *err_index = 0; return ORA_V3_ERR_ZERO_PARAMETER; }
+  if (c->n_group <= 0) { *err_index = 1; return ORA_V3_ERR_ZERO_PARAMETER; }
+  if (c->topk_group <= 0) { *err_index = 2; return ORA_V3_ERR_ZERO_PARAMETER; }
+  if (n % (size_t)c->n_group != 0) return ORA_V3_ERR_NOT_DIVISIBLE;
+  size_t epg = n / (size_t)c->n_group;
+  if (epg < 2) { *err_index = (int32_t)epg; return ORA_V3_ERR_GROUP_TOO_SMALL; }
+  if (c->topk_group > c->n_group) return ORA_V3_ERR_TOPK_GROUP_EXCEEDS;
+  size_t selectable = (size_t)c->topk_group * epg;
+  if (top_k > selectable) { *err_index = (int32_t)selectable; return ORA_V3_ERR_TOPK_EXCEEDS; }
+  return ORA_OK;
+}
+
+/* v3_router.rs:188-199 (top_k_by_score): the k best of score[0..n), ties to the lower index;
+ * -inf entries come last.  taken[] marks the picks. */
+static void ora_pick_top(const double* score, size_t n, size_t k, uint8_t* taken) {
+  memset(taken, 0, n);
+  for (size_t pick = 0; pick < k && pick < n; ++pick) {
+    size_t best = n;
+    for (size_t i = 0; i < n; ++i) {
+      if (taken[i]) continue;
+      if (best == n || score[i] > score[best]) best = i;  /* strict: the lower index keeps a tie */
+    }
+    taken[best] = 1;
+  }
+}
+
+int ora_v3_route(const float* logits, const float* bias, size_t n, size_t top_k,
+                 const OraV3Config* c, int32_t* idx_out, float* w_out, float* dense_out,
+                 double* margin_out, int32_t* err_index) {
+  int rc = ora_v3_validate(n, top_k, c, err_index);
+  if (rc != ORA_OK) return rc;
+  for (size_t i = 0; i < n; ++i)
+    if (!isfinite(logits[i])) { if (err_index) *err_index = (int32_t)i; return ORA_V3_ERR_NON_FINITE_LOGIT; }
+  for (size_t i = 0; i < n; ++i)
+    if (!isfinite(bias[i])) { if (err_index) *err_index = (int32_t)i; return ORA_V3_ERR_NON_FINITE_BIAS; }
+  size_t ng = (size_t)c->n_group, epg = n / ng;
+  double* scores = (double*)malloc(n * sizeof(double));
+  double* choice = (double*)malloc(n * sizeof(double));
+  double* masked = (double*)malloc(n * sizeof(double));
+  double* gscore = (double*)malloc(ng * sizeof(double));
+  uint8_t* gsel = (uint8_t*)malloc(ng);
+  uint8_t* sel = (uint8_t*)malloc(n);
+  for (size_t i = 0; i < n; ++i) {
+    scores[i] = 1.0 / (1.0 + exp(-(double)logits[i]));
+    choice[i] = scores[i] + (double)bias[i];
+  }
+  for (size_t g = 0; g < ng; ++g) {  /* sum of the two largest choices of the group */
+    double m1 = -INFINITY, m2 = -INFINITY;
+    for (size_t j = 0; j < epg; ++j) {
+      double v = choice[g * epg + j];
+      if (v > m1) { m2 = m1; m1 = v; } else if (v > m2) { m2 = v; }
+    }
+    gscore[g] = m1 + m2;
+  }
+  ora_pick_top(gscore, ng, (size_t)c->topk_group, gsel);
+  for (size_t i = 0; i < n; ++i) masked[i] = gsel[i / epg] ? choice[i] : -INFINITY;
+  ora_pick_top(masked, n, top_k, sel);
+  /* diagnostic margin: lowest selected choice - highest unselected choice inside the groups */
+  double min_sel = INFINITY, max_unsel = -INFINITY;
+  for (size_t i = 0; i < n; ++i) {
+    if (sel[i]) { if (choice[i] < min_sel) min_sel = choice[i]; }
+    else if (gsel[i / epg] && choice[i] > max_unsel) max_unsel = choice[i];
+  }
+  if (margin_out) *margin_out = isfinite(max_unsel) ? min_sel - max_unsel : INFINITY;
+  double denom = 0.0;
+  for (size_t i = 0; i < n; ++i)
+    if (sel[i]) denom += scores[i];  /* ascending index, as the sorted selection is summed */
+  denom += 1e-20;
+  if (dense_out) for (size_t i = 0; i < n; ++i) dense_out[i] = 0.0f;
+  size_t slot = 0;
+  for (size_t i = 0; i < n; ++i) {
+    if (!sel[i]) continue;
+    double w = scores[i];
+    if (c->norm_topk_prob) w /= denom;
+    w *= c->routed_scaling_factor;
+    if (idx_out) idx_out[slot] = (int32_t)i;
+    if (w_out) w_out[slot] = (float)w;
+    if (dense_out) dense_out[i] = (float)w;
+    ++slot;
+  }
+  free(scores); free(choice); free(masked); free(gscore); free(gsel); free(sel);
+  return ORA_OK;
+}
+
+/* A whole layer with the V3 router in front: logits = (f32) W_r x (f64 accumulation, no bias),
+ * v3_route, then the layer's own combine (sparse.rs:226-233: f32 multiply and add per selected
+ * expert, ascending) plus the ungated shared expert (layer.rs:415-429 with scale 1).  The
+ * reference ships the router as a mechanism and combines in f64 inside its certification test
+ * (tests/moe_v3_route_scale_cert_test.rs:121-137); the f32 combine here is the reference's
+ * layer arithmetic applied to the V3 weights -- the fixture's block output pins both to 1e-6. */
+int ora_v3_layer_forward(const OraLayer* L, const OraV3Config* c, const float* bias,
+                         const float* x, int policy, float* out, int32_t* idx_out,
+                         float* w_out, int32_t* err_index) {
+  size_t E = (size_t)L->num_experts, k = (size_t)L->top_k, d = (size_t)L->d_model,
+         f = (size_t)L->d_ff, fs = (size_t)L->d_ff_shared;
+  float* logits = (float*)malloc(E * sizeof(float));
+  int32_t* idx = (int32_t*)malloc(k * sizeof(int32_t));
+  float* w = (float*)malloc(k * sizeof(float));
+  float* y = (float*)malloc(d * sizeof(float));
+  ora_matvec(L->w_router, E, d, x, logits);
+  int rc = ora_v3_route(logits, bias, E, k, c, idx, w, NULL, NULL, err_index);
+  if (rc == ORA_OK) {
+    for (size_t i = 0; i < d; ++i) out[i] = 0.0f;
+    for (size_t s = 0; s < k; ++s) {
+      size_t e = (size_t)idx[s];
+      ora_expert_forward(L->w_gate + e * f * d, L->w_up + e * f * d, L->w_down + e * d * f, d, f, x, y,
+                         policy);
+      for (size_t i = 0; i < d; ++i) out[i] += w[s] * y[i];
+    }
+    if (fs > 0) {
+      ora_expert_forward(L->s_gate, L->s_up, L->s_down, d, fs, x, y, policy);
+      for (size_t i = 0; i < d; ++i) out[i] += 1.0f * y[i];
+    }
+    if (idx_out) memcpy(idx_out, idx, k * sizeof(int32_t));
+    if (w_out) memcpy(w_out, w, k * sizeof(float));
+  }
+  free(logits); free(idx); free(w); free(y);
   return rc;
 }
 

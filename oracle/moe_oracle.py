@@ -52,6 +52,11 @@ class _OraLayer(C.Structure):
     ]
 
 
+class _OraV3Config(C.Structure):
+    _fields_ = [("n_group", C.c_int32), ("topk_group", C.c_int32), ("norm_topk_prob", C.c_int32),
+                ("routed_scaling_factor", C.c_double)]
+
+
 class _OraMetrics(C.Structure):
     _fields_ = [("max_abs_diff", C.c_double), ("mean_abs_diff", C.c_double),
                 ("rmse", C.c_double), ("argmax_match", C.c_int32)]
@@ -95,6 +100,12 @@ def lib():
         L.ora_rms_norm_gamma.argtypes = [P, P, Z, C.c_float, C.c_int, P]
         L.ora_block_forward.argtypes = [P, P, Z, P, C.c_float, C.c_int, C.c_int, P, P, P, P, P, P]
         L.ora_block_forward.restype = C.c_int
+        L.ora_v3_validate.argtypes = [Z, Z, P, P]
+        L.ora_v3_validate.restype = C.c_int
+        L.ora_v3_route.argtypes = [P, P, Z, Z, P, P, P, P, P, P]
+        L.ora_v3_route.restype = C.c_int
+        L.ora_v3_layer_forward.argtypes = [P, P, P, P, C.c_int, P, P, P, P]
+        L.ora_v3_layer_forward.restype = C.c_int
         L.ora_route_tokens.argtypes = [P, P, Z, P, P, P, P, P]
         L.ora_route_tokens.restype = C.c_int
         L.ora_permute.argtypes = [P, Z, Z, Z, P, P, P]
@@ -207,6 +218,31 @@ def rms_norm_gamma(x, gamma, eps: float, norm_policy: int = 0) -> np.ndarray:
     return y
 
 
+V3_ERR_ZERO_PARAMETER, V3_ERR_NOT_DIVISIBLE, V3_ERR_GROUP_TOO_SMALL = -10, -11, -12
+V3_ERR_TOPK_GROUP_EXCEEDS, V3_ERR_TOPK_EXCEEDS = -13, -14
+V3_ERR_NON_FINITE_LOGIT, V3_ERR_NON_FINITE_BIAS = -15, -16
+
+
+def v3_route(logits, bias, top_k: int, n_group: int, topk_group: int, scale: float = 1.0,
+             norm_topk_prob: bool = True):
+    """v3_router.rs:206-309 for one token.  Returns (indices ascending, weights, dense weights,
+    selection margin)."""
+    logits, bias = _f32(logits), _f32(bias)
+    if logits.size != bias.size:
+        raise OracleError(ERR_DIM)  # LengthMismatch
+    n = logits.size
+    cfg = _OraV3Config(n_group, topk_group, int(norm_topk_prob), scale)
+    idx = np.empty(max(top_k, 1), dtype=np.int32)
+    w = np.empty(max(top_k, 1), dtype=np.float32)
+    dense = np.empty(n, dtype=np.float32)
+    margin, err = C.c_double(0.0), C.c_int32(-1)
+    rc = lib().ora_v3_route(_p(logits), _p(bias), n, top_k, C.addressof(cfg), _p(idx), _p(w),
+                            _p(dense), C.addressof(margin), C.addressof(err))
+    if rc != OK:
+        raise OracleError(rc, index=err.value)
+    return idx[:top_k].copy(), w[:top_k].copy(), dense, margin.value
+
+
 def sigmoid_dot(g, x) -> float:
     g, x = _f32(g), _f32(x)
     return float(lib().ora_sigmoid_dot(_p(g), _p(x), min(g.size, x.size)))
@@ -316,6 +352,29 @@ class Layer:
         if rc != OK:
             raise OracleError(rc, et.value, ei.value)
         return out, h2, idx, w
+
+    def v3_forward(self, x, bias, n_group: int, topk_group: int, scale: float, norm_topk_prob: bool,
+                   policy: int = CERTIFIED):
+        """Rows through the layer with the DeepSeek-V3 router in front (sigmoid scores,
+        `bias` = e_score_correction_bias, group-limited top-k, scaled weights), ungated shared
+        expert.  Returns (out, idx, w)."""
+        x = _f32(x).reshape(-1, self.d)
+        bias = _f32(bias)
+        assert bias.size == self.E
+        T = x.shape[0]
+        out = np.empty((T, self.d), dtype=np.float32)
+        idx = np.empty((T, self.top_k), dtype=np.int32)
+        w = np.empty((T, self.top_k), dtype=np.float32)
+        cfg = _OraV3Config(n_group, topk_group, int(norm_topk_prob), scale)
+        c = self._c(HUGGINGFACE_QWEN)
+        c.shared_gate = None
+        for t in range(T):
+            err = C.c_int32(-1)
+            rc = lib().ora_v3_layer_forward(C.addressof(c), C.addressof(cfg), _p(bias), _p(x[t]),
+                                            policy, _p(out[t]), _p(idx[t]), _p(w[t]), C.addressof(err))
+            if rc != OK:
+                raise OracleError(rc, t, err.value)
+        return out, idx, w
 
     def route_tokens(self, x, want_logits: bool = False):
         x = _f32(x).reshape(-1, self.d)

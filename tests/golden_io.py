@@ -53,3 +53,17 @@ def layer_arrays(name):
 def oracle_layer(ora, name, top_k, convention):
     a = layer_arrays(name)
     return ora.Layer(top_k=top_k, convention=convention, **a)
+
+
+def v3_arrays():
+    """The DeepSeek-V3 routing fixture as layer arrays (8 experts, one shared expert)."""
+    t = tensors("v3_route_ref")
+    n = sidecar("v3_route_ref")["n_routed_experts"]
+    st = lambda part: np.stack([t[f"expert.{e}.{part}"] for e in range(n)])
+    return dict(w_router=t["router.weight"], w_gate=st("w_gate"), w_up=st("w_up"), w_down=st("w_down"),
+                s_gate=t["shared.w_gate"], s_up=t["shared.w_up"], s_down=t["shared.w_down"])
+
+
+def v3_oracle_layer(ora):
+    return ora.Layer(top_k=sidecar("v3_route_ref")["top_k"], convention=ora.HUGGINGFACE_QWEN,
+                     **v3_arrays())

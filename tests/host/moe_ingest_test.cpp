@@ -7,6 +7,8 @@
 //   src/moe/convention.rs tests          (convention from the weight map)
 //   src/nn/llama/moe_config.rs tests     (config.json keys of Mixtral / Qwen-MoE / DeepSeek-MoE)
 //   tests/moe_deepseek_block_test.rs:42-74  (DeepSeek block: packed experts + fused shared experts)
+//   tests/moe_v3_route_scale_cert_test.rs:56-175, src/moe/v3_router.rs:340-462
+//                                        (DeepSeek-V3 routing: configuration errors, HF f64 fixture)
 //   tests/moe_numerical_equivalence_test.rs:44-110, tests/moe_hf_convention_test.rs:123-146
 //                                        (golden layer files -> assemble -> forward vs the f64 refs)
 // The golden layer files are read directly (safetensors + JSON side file).  Without a device the
@@ -391,6 +393,43 @@ int main(int argc, char** argv) {
     CHECK(zero.experts_per_token_or(2) == 1, "top-k is at least one");
   });
 
+  run_test("v3_router_config_errors", [] {
+    auto cfg = [](size_t n, size_t k, size_t g, size_t tg) {
+      V3RouterConfig c;
+      c.n_routed_experts = n; c.top_k = k; c.n_group = g; c.topk_group = tg;
+      return c;
+    };
+    CHECK(!cfg(8, 2, 4, 2).validate(), "a valid configuration");
+    auto text = [](const std::optional<V3RouterError>& e) { return e ? e->to_string() : std::string("ok"); };
+    CHECK(text(cfg(7, 2, 4, 2).validate()) == "v3-router: n_routed_experts (7) not divisible by n_group (4)", "divisible");
+    CHECK(text(cfg(4, 1, 4, 2).validate()) == "v3-router: experts_per_group (1) < 2 (HF takes top-2 per group)", "group size");
+    CHECK(text(cfg(8, 2, 4, 5).validate()) == "v3-router: topk_group (5) > n_group (4)", "topk_group");
+    CHECK(text(cfg(8, 5, 4, 2).validate()) == "v3-router: top_k (5) exceeds experts in selected groups (4)", "selectable");
+    CHECK(text(cfg(8, 0, 4, 2).validate()) == "v3-router: top_k must be > 0", "zero top_k");
+    CHECK(text(cfg(8, 2, 0, 2).validate()) == "v3-router: n_group must be > 0", "zero n_group");
+    CHECK(text(cfg(8, 2, 4, 0).validate()) == "v3-router: topk_group must be > 0", "zero topk_group");
+    CHECK(parse_scoring_func("sigmoid").is_ok(), "sigmoid");
+    auto sm = parse_scoring_func("softmax");
+    CHECK(sm.is_err() && sm.error().to_string() == "v3-router: unsupported scoring_func 'softmax' (only 'sigmoid')", "softmax refused");
+    // on a layer: lengths, finiteness, and the layer's own top_k
+    Listing ls;
+    Store st;
+    mixtral_classic(ls, st, {0, 1, 2, 3, 4, 5, 6, 7}, 8, 12);
+    auto layer = assemble_real_moe_layer(MoeWeightMap::from_tensors(ls), 0, MoeLayerConfig::make(8, 2, false, 8, 12).unwrap(),
+                                         resolver_of(st)).unwrap();
+    CHECK(text(layer.set_v3_router(cfg(8, 2, 4, 2), std::vector<float>(7, 0.f))) ==
+              "v3-router: e_score_correction_bias length 7 != n_routed_experts 8", "bias length");
+    std::vector<float> bad(8, 0.f);
+    bad[5] = INFINITY;
+    CHECK(text(layer.set_v3_router(cfg(8, 2, 4, 2), bad)) == "v3-router: e_score_correction_bias at 5 is non-finite", "bias finite");
+    CHECK(text(layer.set_v3_router(cfg(16, 2, 4, 2), std::vector<float>(16, 0.f))) ==
+              "v3-router: router_logits length 8 != n_routed_experts 16", "expert count");
+    CHECK(text(layer.set_v3_router(cfg(8, 3, 4, 2), std::vector<float>(8, 0.f))) ==
+              "v3-router: top_k (3) differs from the layer's experts_per_token (2)", "top_k of the layer");
+    CHECK(!layer.v3_router, "failed calls leave the layer as it was");
+    CHECK(!layer.set_v3_router(cfg(8, 2, 4, 2), std::vector<float>(8, 0.f)) && layer.v3_router, "accepted");
+  });
+
   // ---- classic binding ------------------------------------------------------------------------
   run_test("classic_binding_is_byte_exact_and_id_ordered", [] {
     Listing ls;
@@ -772,6 +811,49 @@ int main(int argc, char** argv) {
     DeepSeekBlock b = load_deepseek();
     auto out = b.layer.forward_with(b.probe, b.convention).unwrap();
     CHECK(max_abs_diff(out, b.want) <= 1e-5 * max_abs(b.want), "%g", max_abs_diff(out, b.want));
+  });
+  run_test("deepseek_v3_routing_fixture_on_device", [&] {
+    // tests/moe_v3_route_scale_cert_test.rs: 8 experts in 4 groups, 2 groups kept, top-2, weights
+    // normalised and scaled by 2.5, one ungated shared expert; HuggingFace f64 block output.
+    atenia::json::Value side;
+    const std::string text = slurp(golden + "/v3_route_ref.json");
+    CHECK(!text.empty() && atenia::json::parse(text, side), "side file");
+    auto num = [&](const char* k) { return (size_t)side.get(k)->num; };
+    auto rd = SafetensorsReader::open(golden + "/v3_route_ref.safetensors");
+    CHECK(rd.is_ok(), "reader");
+    const SafetensorsReader& reader = rd.value();
+    const size_t n = num("n_routed_experts"), d = num("hidden_size"), f = num("moe_intermediate_size");
+    std::vector<MoeDenseExpert> experts;
+    for (size_t e = 0; e < n; ++e) {
+      const std::string p = "expert." + std::to_string(e) + ".";
+      experts.push_back(MoeDenseExpert::make(d, f, *reader.to_vec_f32(p + "w_gate"), *reader.to_vec_f32(p + "w_up"),
+                                             *reader.to_vec_f32(p + "w_down")).unwrap());
+    }
+    auto routed = MoeDenseLayer::make(d, f, *reader.to_vec_f32("router.weight"), std::move(experts), num("top_k")).unwrap();
+    auto shared = MoeDenseExpert::make(d, num("shared_intermediate_size"), *reader.to_vec_f32("shared.w_gate"),
+                                       *reader.to_vec_f32("shared.w_up"), *reader.to_vec_f32("shared.w_down")).unwrap();
+    auto layer = RealMoeLayer::assemble(MoeLayerConfig::make(n, num("top_k"), true, d, f).unwrap(), std::move(routed),
+                                        std::move(shared), std::nullopt).unwrap();
+    V3RouterConfig cfg;
+    cfg.n_routed_experts = n; cfg.top_k = num("top_k"); cfg.n_group = num("n_group"); cfg.topk_group = num("topk_group");
+    cfg.routed_scaling_factor = side.get("routed_scaling_factor")->num;
+    cfg.norm_topk_prob = side.get("norm_topk_prob")->b;
+    cfg.scoring_func = parse_scoring_func(side.get("scoring_func")->str).unwrap();
+    auto err = layer.set_v3_router(cfg, *reader.to_vec_f32("router.bias"));
+    CHECK(!err, "%s", err ? err->to_string().c_str() : "");
+    const std::vector<float> hidden = *reader.to_vec_f32("hidden");
+    std::vector<int32_t> idx;
+    auto w = layer.route(hidden, MoeExecutionConvention::HuggingFaceQwen, &idx).unwrap();
+    const auto& want_sets = side.get("selected_experts")->arr;
+    const std::vector<float> dense = floats(side.get("dense_combine_weights"));
+    for (size_t t = 0; t < num("tokens"); ++t)
+      for (size_t s_ = 0; s_ < cfg.top_k; ++s_) {
+        CHECK((size_t)idx[t * cfg.top_k + s_] == (size_t)want_sets[t].arr[s_].num, "token %zu slot %zu", t, s_);
+        CHECK(std::fabs(w[t * cfg.top_k + s_] - dense[t * n + idx[t * cfg.top_k + s_]]) < 1e-6, "weight of token %zu", t);
+      }
+    auto out = layer.forward_with(hidden, MoeExecutionConvention::HuggingFaceQwen).unwrap();
+    const std::vector<float> want = floats(side.get("block_out"));
+    CHECK(max_abs_diff(out, want) < 1e-6, "block output: %g", max_abs_diff(out, want));
   });
   run_test("ingested_layer_through_the_registry", [&] {
     Golden g = load_golden(golden, "qwen2_moe");
