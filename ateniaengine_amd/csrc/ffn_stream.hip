@@ -245,6 +245,106 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p) 
   }
 }
 
+// Down projection + combine for ONE token with k <= 2 experts, one launch.  A workgroup owns a
+// 16-row strip of W_d for every expert of the token: waves [8 j, 8 j + 8) stream the strip of
+// expert j, split over K exactly as the eight waves of ffn_stream_kernel<1, INT8, false, 8> do,
+// and the partial sums meet in LDS in the same order -- so y is bit-identical to the separate
+// down launch -- and lanes 0..15 then finish out[n] = sum_j w_j * y_j[n] (+ residual) with the
+// combine kernel's arithmetic (product and sum rounded separately; src/moe/sparse.rs:226-233).
+// Saves the combine launch and the bubble in front of it, about 4 % of a batch-1 forward.
+template <bool INT8>
+__global__ __launch_bounds__(1024) void ffn_down_decode1_kernel(StreamParams p, int k,
+                                                               const float* __restrict__ w,
+                                                               const float* residual, float* out) {
+  constexpr int KS = 8;  // K slices per expert, as in the separate down launch
+  const int nb = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int kq = lane >> 4, mm = lane & 15;
+  const int j = wave / KS, slice = wave - j * KS;
+  constexpr int KB = INT8 ? kKbInt8 : kKbBf16;
+  __shared__ float red[16][16];
+  float partial = 0.f;
+  if (j < k && j < *p.g.n_active) {  // uniform per wave
+    const int e = p.g.active[j];
+    const int base = p.g.offsets[e];
+    const int kb_per = (p.nkb + KS - 1) / KS;
+    const int kb0 = slice * kb_per;
+    const int kb1 = min(p.nkb, kb0 + kb_per);
+    const uint4* pa = p.wa + (size_t)e * p.w_stride_u4 + (size_t)nb * p.nkb * 64 + lane;
+    constexpr int U = INT8 ? 2 : 4;
+    constexpr int AV = INT8 ? 2 : 1;
+    uint4 wA0[U], wA1[U], xa0[U][AV], xa1[U][AV];
+    auto load_w = [&](uint4 (&wa)[U], int kb) {
+#pragma unroll
+      for (int q = 0; q < U; ++q) wa[q] = load_stream(pa + (size_t)min(kb + q, kb1 - 1) * 64);
+    };
+    if (kb0 < kb1) load_w(wA0, kb0);
+    // The expert's single row of h; all 16 MFMA rows read it, only row 0 is kept.
+    const uint16_t* arow = p.a + (size_t)base * p.a_stride + (KB / 4) * kq;
+    auto load_x = [&](uint4 (&xa)[U][AV], int kb) {
+#pragma unroll
+      for (int q = 0; q < U; ++q)
+#pragma unroll
+        for (int v = 0; v < AV; ++v)
+          xa[q][v] = *((const uint4*)(arow + (size_t)min(kb + q, kb1 - 1) * KB) + v);
+    };
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    auto multiply = [&](const uint4 (&wa)[U], const uint4 (&xa)[U][AV], int kb) {
+#pragma unroll
+      for (int q = 0; q < U; ++q) {
+        if (kb + q < kb1) {
+          if (INT8) {
+            bf16x8 al, ah;
+            widen_i8x16(wa[q], al, ah);
+            uint4 x0 = xa[q][0], x1 = xa[q][AV - 1];
+            acc = mfma(*(bf16x8*)&x0, al, acc);
+            acc = mfma(*(bf16x8*)&x1, ah, acc);
+          } else {
+            acc = mfma(xa[q][0], wa[q], acc);
+          }
+        }
+      }
+    };
+    if (kb0 < kb1) load_x(xa0, kb0);
+    for (int kb = kb0; kb < kb1; kb += 2 * U) {
+      if (kb + U < kb1) {
+        load_w(wA1, kb + U);
+        load_x(xa1, kb + U);
+      }
+      multiply(wA0, xa0, kb);
+      if (kb + 2 * U < kb1) {
+        load_w(wA0, kb + 2 * U);
+        load_x(xa0, kb + 2 * U);
+      }
+      if (kb + U < kb1) multiply(wA1, xa1, kb + U);
+    }
+    partial = acc[0];  // D layout: lanes 0..15 (kq == 0), element 0 = row 0, column mm
+  }
+  if (kq == 0) red[wave][mm] = partial;
+  __syncthreads();
+  if (threadIdx.x >= 16) return;
+  const int n = nb * 16 + mm;
+  if (n >= p.n_rows) return;
+  float o = 0.f;
+  const int n_active = *p.g.n_active;
+  for (int jj = 0; jj < k && jj < n_active; ++jj) {
+    float y = red[jj * KS][mm];
+#pragma unroll
+    for (int sl = 1; sl < KS; ++sl) y += red[jj * KS + sl][mm];
+    const int e = p.g.active[jj];
+    if (INT8) y = y * p.sa[(size_t)e * p.n_rows + n];
+    const int pair = p.g.perm[p.g.offsets[e]];
+    ((float*)p.out)[(size_t)pair * p.out_stride + n] = y;
+    // The product must be rounded before it is added: an opaque multiply keeps the compiler
+    // (-ffp-contract=fast in this file) from fusing it into an FMA.
+    float prod;
+    asm volatile("v_mul_f32 %0, %1, %2" : "=v"(prod) : "v"(w[pair]), "v"(y));
+    o = o + prod;
+  }
+  if (residual) o = residual[n] + o;
+  out[n] = o;
+}
+
 template <bool INT8, bool UP>
 hipError_t launch_stream(const StreamParams& p, int n_pad, int n_groups, int rows_max,
                          hipStream_t s) {
@@ -306,6 +406,36 @@ hipError_t launch_ffn_down(const FfnArgs& a, hipStream_t s) {
   p.g = a.g;
   return int8 ? launch_stream<true, false>(p, a.down.n_pad, a.n_groups_max, a.rows_max, s)
               : launch_stream<false, false>(p, a.down.n_pad, a.n_groups_max, a.rows_max, s);
+}
+
+bool ffn_down_decode1_supported(int T, int k, int wdtype, bool tiled, bool shared) {
+  return T == 1 && k >= 1 && k <= 2 && wdtype != ATENIA_MOE_WEIGHT_F32 && !tiled && !shared;
+}
+
+hipError_t launch_ffn_down_decode1(const FfnArgs& a, hipStream_t s) {
+  const bool int8 = a.wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
+  StreamParams p;
+  p.wa = (const uint4*)a.down.w;
+  p.wb = nullptr;
+  p.sa = a.down.scale;
+  p.sb = nullptr;
+  p.w_stride_u4 = a.down.expert_stride / 16;
+  p.n_rows = a.down.n_rows;
+  p.nkb = a.down.k_pad / (int8 ? kKbInt8 : kKbBf16);
+  p.a = (const uint16_t*)a.h;
+  p.a_stride = a.h_stride;
+  p.out = a.y;
+  p.out_stride = a.y_stride;
+  p.g = a.g;
+  const dim3 grid(a.down.n_pad / 16);
+  const int threads = 64 * 8 * a.fuse_k;
+  if (int8)
+    ffn_down_decode1_kernel<true><<<grid, threads, 0, s>>>(p, a.fuse_k, a.fuse_w, a.fuse_residual,
+                                                           a.fuse_out);
+  else
+    ffn_down_decode1_kernel<false><<<grid, threads, 0, s>>>(p, a.fuse_k, a.fuse_w, a.fuse_residual,
+                                                            a.fuse_out);
+  return hipGetLastError();
 }
 
 // ---- load-time repack of a row-major matrix into B blocks -------------------------------

@@ -438,8 +438,20 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
     }
   }
   tm.mark();  // ev[3]: gate/up done
+  // One token, up to two experts, no shared expert, whole pipeline requested: the down launch
+  // finishes the combine as well (same bits as the two launches, one launch less).
+  const bool fuse1 = first <= kStageFfn && last >= kStageCombine &&
+                     ffn_down_decode1_supported(T, L->k, L->wdtype, tiled, L->fs > 0);
   if (first <= kStageFfn) {
-    HIP_TRY(launch_ffn_down(fa, s));
+    if (fuse1) {
+      fa.fuse_w = L->w.as<float>();
+      fa.fuse_out = d_out;
+      fa.fuse_residual = d_residual;
+      fa.fuse_k = L->k;
+      HIP_TRY(launch_ffn_down_decode1(fa, s));
+    } else {
+      HIP_TRY(launch_ffn_down(fa, s));
+    }
     L->launches[3] = 1;
     if (L->fs > 0) {
       HIP_TRY(launch_ffn_down(fsd, s));
@@ -449,6 +461,13 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   }
   tm.mark();  // ev[4]: down done
   if (last < kStageCombine) return ATENIA_MOE_OK;
+  if (fuse1) {
+    L->launches[4] = 0;
+    L->stage_T[kStageCombine] = T;
+    tm.mark();  // ev[5]: nothing left to do
+    L->launches[5] = L->launches[0] + L->launches[1] + L->launches[2] + L->launches[3];
+    return ATENIA_MOE_OK;
+  }
 
   CombineArgs ca{};
   ca.T = T;

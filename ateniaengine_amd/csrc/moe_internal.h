@@ -132,6 +132,12 @@ struct FfnArgs {
   const int32_t* tile_m0;
   const int32_t* n_tiles;
   int max_row_tiles;   // upper bound of *n_tiles (grid sizing)
+  // Single-token decode (see launch_ffn_down_decode1): routing weights [k], layer output [d]
+  // and optional residual [d] of the one token; the down launch then also does the combine.
+  const float* fuse_w;
+  float* fuse_out;
+  const float* fuse_residual;
+  int fuse_k;
 };
 bool tiled_supported(const WeightSet& w, int wdtype);
 // True when the tiled down launch for these weights can split the k range of tail tiles.
@@ -140,6 +146,10 @@ hipError_t launch_ffn_up_tiled(const FfnArgs& a, hipStream_t s);
 hipError_t launch_ffn_down_tiled(const FfnArgs& a, hipStream_t s);
 hipError_t launch_ffn_up(const FfnArgs& a, hipStream_t s);
 hipError_t launch_ffn_down(const FfnArgs& a, hipStream_t s);
+// One token, at most two experts per token, blocked (bf16 / int8) weights: the down projection
+// of all the token's experts and the weighted combine in one launch.
+bool ffn_down_decode1_supported(int T, int k, int wdtype, bool tiled, bool shared);
+hipError_t launch_ffn_down_decode1(const FfnArgs& a, hipStream_t s);
 
 struct CombineArgs {
   int T, k, d;

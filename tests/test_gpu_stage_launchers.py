@@ -76,3 +76,38 @@ def test_stage_order_is_enforced(ora):
         gL.expert_ffn_device(x.ptr, capi.ACT_F32, T)
         gL.combine_device(T, out.ptr)
         assert np.isfinite(out.to_host()).all()
+
+
+@pytest.mark.parametrize("wd", [capi.WEIGHT_BF16, capi.WEIGHT_INT8_W8A16])
+@pytest.mark.parametrize("k", [1, 2])
+def test_single_token_fused_down_and_combine(ora, wd, k):
+    """One token with up to two experts per token: the pipeline's down launch also does the
+    combine.  It must give the bits of the stages called one by one (which use the separate
+    down and combine kernels), also with a residual (the block entry point), and leave the same
+    per-expert outputs in the tap."""
+    d = 512
+    W = S.make_weights(300 + k, 8, d, 1024, router_std=1.0 / 16.0)
+    oL, gL = S.build_pair(ora, W, k, capi.CONVENTION_ATENIA, wd)
+    with gL:
+        for seed in range(4):
+            x = S.make_tokens(900 + seed, 1, d)
+            dx = DeviceArray.from_host(x)
+            whole = DeviceArray((1, d), np.float32, fill=0)
+            gL.forward_device(dx.ptr, capi.ACT_F32, 1, whole.ptr)
+            assert gL.status()[0] == 0
+            y_fused = gL.last_expert_outputs(1)[0]
+            assert gL.stage_launches()[4] == 0, "the combine launch must be gone"
+            staged = DeviceArray((1, d), np.float32, fill=0)
+            gL.router_device(dx.ptr, capi.ACT_F32, 1)
+            gL.permute_device(1)
+            gL.expert_ffn_device(dx.ptr, capi.ACT_F32, 1)
+            gL.combine_device(1, staged.ptr)
+            assert gL.stage_launches()[4] == 1
+            assert whole.to_host().tobytes() == staged.to_host().tobytes()
+            assert y_fused.tobytes() == gL.last_expert_outputs(1)[0].tobytes()
+            assert S.rel_err(whole.to_host(), oL.execute(x)[0]) <= 2e-2
+        x1 = S.make_tokens(77, 1, d, bf16=False)
+        gamma = np.linspace(0.8, 1.2, d).astype(np.float32)
+        blk = gL.block_forward(x1, gamma, 1e-5, capi.NORM_GRAPH_F32)
+        h2 = gL.last_normed(1)
+        assert blk.tobytes() == (x1 + gL.forward(h2).reshape(1, d)).astype(np.float32).tobytes()
