@@ -208,6 +208,38 @@ Result<MoeDenseExpert, MoeDenseError> MoeDenseExpert::make(size_t d_model, size_
   return R::Ok(std::move(e));
 }
 
+std::vector<float> QInt8Tensor::dequantize() const {
+  std::vector<float> out(rows * cols);
+  for (size_t r = 0; r < rows; ++r) {
+    const float sc = scales[r];
+    for (size_t c = 0; c < cols; ++c) out[r * cols + c] = (float)q[r * cols + c] * sc;
+  }
+  return out;
+}
+
+Result<MoeDenseExpert, MoeDenseError> MoeDenseExpert::from_qint8(size_t d_model, size_t d_ff,
+                                                                 QInt8Tensor gate, QInt8Tensor up,
+                                                                 QInt8Tensor down) {
+  typedef Result<MoeDenseExpert, MoeDenseError> R;
+  auto bad = [&](const QInt8Tensor& t, size_t rows, size_t cols) {
+    return t.rows != rows || t.cols != cols || t.q.size() != rows * cols || t.scales.size() != rows;
+  };
+  if (bad(gate, d_ff, d_model))
+    return R::Err(MoeDenseError{MoeDenseError::WeightShapeMismatch, "w_gate", d_ff * d_model, gate.q.size()});
+  if (bad(up, d_ff, d_model))
+    return R::Err(MoeDenseError{MoeDenseError::WeightShapeMismatch, "w_up", d_ff * d_model, up.q.size()});
+  if (bad(down, d_model, d_ff))
+    return R::Err(MoeDenseError{MoeDenseError::WeightShapeMismatch, "w_down", d_model * d_ff, down.q.size()});
+  auto ex = make(d_model, d_ff, gate.dequantize(), up.dequantize(), down.dequantize());
+  if (ex.is_err()) return ex;
+  auto payload = std::make_shared<QInt8Projections>();
+  payload->gate = std::move(gate);
+  payload->up = std::move(up);
+  payload->down = std::move(down);
+  ex.value().q8 = std::move(payload);
+  return ex;
+}
+
 Result<MoeDenseLayer, MoeDenseError> MoeDenseLayer::make(size_t d_model, size_t d_ff,
                                                          std::vector<float> w_router,
                                                          std::vector<MoeDenseExpert> experts,
@@ -332,8 +364,9 @@ struct Packed {
   }
 };
 
+// `pre` (optional, one per matrix or empty): int8 tier data to upload as it is.
 int pack(const std::vector<const std::vector<float>*>& mats, size_t rows, size_t cols,
-         MoeWeightStorage s, Packed& out) {
+         MoeWeightStorage s, Packed& out, const std::vector<const QInt8Tensor*>& pre = {}) {
   const size_t per = rows * cols, n = mats.size();
   if (s == MoeWeightStorage::F32) {
     out.f32.resize(n * per);
@@ -350,7 +383,15 @@ int pack(const std::vector<const std::vector<float>*>& mats, size_t rows, size_t
   }
   out.i8.resize(n * per);  // per output row (disk_tier.rs:231-248)
   out.scale.resize(n * rows);
+  bool have_pre = pre.size() == n;
+  for (size_t i = 0; have_pre && i < n; ++i)
+    have_pre = pre[i] && pre[i]->rows == rows && pre[i]->cols == cols;
   for (size_t i = 0; i < n; ++i) {
+    if (have_pre) {
+      std::memcpy(&out.i8[i * per], pre[i]->q.data(), per);
+      std::memcpy(&out.scale[i * rows], pre[i]->scales.data(), rows * 4);
+      continue;
+    }
     int rc = atenia_moe_quantize_per_row_i8(mats[i]->data(), rows, cols, &out.i8[i * per],
                                             &out.scale[i * rows]);
     if (rc) return rc;
@@ -376,10 +417,17 @@ Result<void*, MoeLayerError> RealMoeLayer::handle_for(MoeExecutionConvention con
     u.push_back(&e.w_up);
     dn.push_back(&e.w_down);
   }
+  std::vector<const QInt8Tensor*> qg, qu, qd;  // tier data, when every expert carries it
+  for (const auto& e : routed.experts) {
+    if (!e.q8) break;
+    qg.push_back(&e.q8->gate);
+    qu.push_back(&e.q8->up);
+    qd.push_back(&e.q8->down);
+  }
   Packed pg, pu, pd, sg, su, sd;
-  int rc = pack(g, f, d, storage, pg);
-  if (!rc) rc = pack(u, f, d, storage, pu);
-  if (!rc) rc = pack(dn, d, f, storage, pd);
+  int rc = pack(g, f, d, storage, pg, qg);
+  if (!rc) rc = pack(u, f, d, storage, pu, qu);
+  if (!rc) rc = pack(dn, d, f, storage, pd, qd);
   AteniaMoeLayerDesc desc;
   std::memset(&desc, 0, sizeof(desc));
   desc.num_experts = (int32_t)E;
@@ -400,9 +448,10 @@ Result<void*, MoeLayerError> RealMoeLayer::handle_for(MoeExecutionConvention con
   if (use_shared) {
     const size_t fs = shared->d_ff;
     desc.d_ff_shared = (int32_t)fs;
-    if (!rc) rc = pack({&shared->w_gate}, fs, d, storage, sg);
-    if (!rc) rc = pack({&shared->w_up}, fs, d, storage, su);
-    if (!rc) rc = pack({&shared->w_down}, d, fs, storage, sd);
+    const QInt8Projections* sq = shared->q8.get();
+    if (!rc) rc = pack({&shared->w_gate}, fs, d, storage, sg, sq ? std::vector<const QInt8Tensor*>{&sq->gate} : std::vector<const QInt8Tensor*>{});
+    if (!rc) rc = pack({&shared->w_up}, fs, d, storage, su, sq ? std::vector<const QInt8Tensor*>{&sq->up} : std::vector<const QInt8Tensor*>{});
+    if (!rc) rc = pack({&shared->w_down}, d, fs, storage, sd, sq ? std::vector<const QInt8Tensor*>{&sq->down} : std::vector<const QInt8Tensor*>{});
     desc.s_gate = sg.data(storage);
     desc.s_up = su.data(storage);
     desc.s_down = sd.data(storage);

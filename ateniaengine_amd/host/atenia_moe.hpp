@@ -162,9 +162,28 @@ struct V3RouterConfig {  // src/moe/v3_router.rs:59-72
 // How the layer's expert weights are stored in HBM.
 enum class MoeWeightStorage { F32 = 0, Bf16 = 1, Int8W8A16 = 2 };
 
+// A per-output-row symmetric int8 weight [rows, cols]: w[r, c] = q[r, c] * scales[r]
+// (src/tensor/disk_tier.rs:225-262; the payload of the reference's qint8 tier files).
+struct QInt8Tensor {
+  size_t rows = 0, cols = 0;
+  std::vector<int8_t> q;      // [rows * cols]
+  std::vector<float> scales;  // [rows]
+  std::vector<float> dequantize() const;  // disk_tier.rs:251-262
+};
+struct QInt8Projections {
+  QInt8Tensor gate, up, down;
+};
+
 struct MoeDenseExpert {
   size_t d_model = 0, d_ff = 0;
   std::vector<float> w_gate, w_up, w_down;  // [d_ff,d_model], [d_ff,d_model], [d_model,d_ff]
+  // Set when the expert came from int8 tier data (from_qint8): w_* hold the dequantised values
+  // the reference computes with, and a layer stored as Int8W8A16 uploads q / scales as they
+  // are instead of quantising w_* again.
+  std::shared_ptr<const QInt8Projections> q8;
+  static Result<MoeDenseExpert, MoeDenseError> from_qint8(size_t d_model, size_t d_ff,
+                                                          QInt8Tensor gate, QInt8Tensor up,
+                                                          QInt8Tensor down);
   static Result<MoeDenseExpert, MoeDenseError> make(size_t d_model, size_t d_ff,
                                                     std::vector<float> w_gate,
                                                     std::vector<float> w_up,

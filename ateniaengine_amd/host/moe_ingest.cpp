@@ -5,6 +5,7 @@
 #include <cstring>
 #include <initializer_list>
 
+#include "../../include/atenia_moe_hip.h"
 #include "json_mini.hpp"
 
 namespace atenia {
@@ -367,6 +368,80 @@ bool MoeConfig::operator==(const MoeConfig& o) const {
          norm_topk_prob == o.norm_topk_prob && router_aux_loss_coef == o.router_aux_loss_coef &&
          expert_intermediate_size == o.expert_intermediate_size &&
          shared_expert_intermediate_size == o.shared_expert_intermediate_size;
+}
+
+// ---- qint8 tier files -------------------------------------------------------------------------
+QInt8Tensor quantize_per_row_i8(const std::vector<float>& data, size_t rows, size_t cols) {
+  QInt8Tensor t;
+  t.rows = rows;
+  t.cols = cols;
+  t.q.resize(rows * cols);
+  t.scales.resize(rows);
+  if (data.size() == rows * cols && rows * cols > 0)
+    atenia_moe_quantize_per_row_i8(data.data(), rows, cols, t.q.data(), t.scales.data());
+  return t;
+}
+
+std::optional<std::string> write_qint8_tensor_named(const std::string& path,
+                                                    const std::vector<float>& data, size_t rows,
+                                                    size_t cols) {
+  if (data.size() != rows * cols) return "qint8: data length does not match rows * cols";
+  const QInt8Tensor t = quantize_per_row_i8(data, rows, cols);
+  FILE* f = std::fopen(path.c_str(), "wb");
+  if (!f) return "qint8: cannot create '" + path + "'";
+  bool ok = true;
+  for (size_t r = 0; r < rows && ok; ++r) {  // little-endian f32, whatever the host order
+    uint32_t b;
+    std::memcpy(&b, &t.scales[r], 4);
+    const unsigned char le[4] = {(unsigned char)b, (unsigned char)(b >> 8), (unsigned char)(b >> 16),
+                                 (unsigned char)(b >> 24)};
+    ok = std::fwrite(le, 1, 4, f) == 4;
+  }
+  ok = ok && std::fwrite(t.q.data(), 1, t.q.size(), f) == t.q.size();
+  ok = (std::fclose(f) == 0) && ok;
+  if (!ok) return "qint8: short write to '" + path + "'";
+  return std::nullopt;
+}
+
+Result<QInt8Tensor, std::string> read_qint8_tensor(const std::string& path, size_t numel,
+                                                   size_t rows) {
+  typedef Result<QInt8Tensor, std::string> R;
+  if (rows == 0 || numel % rows != 0) return R::Err("qint8: bad rows for numel");
+  FILE* f = std::fopen(path.c_str(), "rb");
+  if (!f) return R::Err("qint8: cannot open '" + path + "'");
+  std::fseek(f, 0, SEEK_END);
+  const long sz = std::ftell(f);
+  std::fseek(f, 0, SEEK_SET);
+  const size_t expected = qint8_disk_bytes(numel, rows);
+  if (sz < 0 || (size_t)sz != expected) {
+    std::fclose(f);
+    return R::Err("qint8 file '" + path + "': " + std::to_string(sz < 0 ? 0 : sz) +
+                  " bytes, expected " + std::to_string(expected));
+  }
+  QInt8Tensor t;
+  t.rows = rows;
+  t.cols = numel / rows;
+  t.scales.resize(rows);
+  t.q.resize(numel);
+  std::vector<unsigned char> raw(rows * 4);
+  bool ok = std::fread(raw.data(), 1, raw.size(), f) == raw.size();
+  ok = ok && std::fread(t.q.data(), 1, numel, f) == numel;
+  std::fclose(f);
+  if (!ok) return R::Err("qint8: short read of '" + path + "'");
+  for (size_t r = 0; r < rows; ++r) {
+    const uint32_t b = (uint32_t)raw[4 * r] | (uint32_t)raw[4 * r + 1] << 8 |
+                       (uint32_t)raw[4 * r + 2] << 16 | (uint32_t)raw[4 * r + 3] << 24;
+    std::memcpy(&t.scales[r], &b, 4);
+  }
+  return R::Ok(std::move(t));
+}
+
+Result<std::vector<float>, std::string> read_qint8_to_f32(const std::string& path, size_t numel,
+                                                          size_t rows) {
+  typedef Result<std::vector<float>, std::string> R;
+  auto t = read_qint8_tensor(path, numel, rows);
+  if (t.is_err()) return R::Err(t.error());
+  return R::Ok(t.value().dequantize());
 }
 
 // ---- binding ----------------------------------------------------------------------------------

@@ -13,6 +13,8 @@
 //   assemble_real_moe_layer = RealMoeLayer::assemble    src/moe/layer.rs:212-343
 //   MoeConventionResolver                               src/moe/convention.rs
 //   MoeConfig (config.json keys of the MoE families)    src/nn/llama/moe_config.rs:52-150
+//   qint8 tier files: quantize_per_row_i8, qint8_disk_bytes, write_qint8_tensor_named,
+//   read_qint8_tensor / read_qint8_to_f32               src/tensor/disk_tier.rs:168-262
 #pragma once
 
 #include <functional>
@@ -147,6 +149,23 @@ struct MoeConfig {
   bool renormalize_topk_or(bool fallback) const { return norm_topk_prob.value_or(fallback); }
   bool operator==(const MoeConfig& o) const;
 };
+
+// ---- qint8 tier files -------------------------------------------------------------------------
+// One tensor per file: [rows x f32 scale, little endian][rows * cols x i8], the layout the
+// reference's residency tier writes for expert weights (src/moe/residency.rs:344-355).  Read
+// back, q and scales go to HBM as they are (MoeDenseExpert::from_qint8 + Int8W8A16 storage).
+QInt8Tensor quantize_per_row_i8(const std::vector<float>& data, size_t rows, size_t cols);
+inline size_t qint8_disk_bytes(size_t numel, size_t rows) { return rows * 4 + numel; }
+// nullopt on success, else what failed.
+std::optional<std::string> write_qint8_tensor_named(const std::string& path,
+                                                    const std::vector<float>& data, size_t rows,
+                                                    size_t cols);
+// `rows` is the quantisation axis (the tensor's first dimension), cols = numel / rows.  A file
+// whose size is not rows * 4 + numel is refused (the reference's InvalidData).
+Result<QInt8Tensor, std::string> read_qint8_tensor(const std::string& path, size_t numel,
+                                                   size_t rows);
+Result<std::vector<float>, std::string> read_qint8_to_f32(const std::string& path, size_t numel,
+                                                          size_t rows);
 
 // ---- binding ----------------------------------------------------------------------------------
 // name -> f32 data, or nullopt (the reference's `resolve: &Fn(&str) -> Option<Vec<f32>>`).

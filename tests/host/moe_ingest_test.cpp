@@ -7,6 +7,8 @@
 //   src/moe/convention.rs tests          (convention from the weight map)
 //   src/nn/llama/moe_config.rs tests     (config.json keys of Mixtral / Qwen-MoE / DeepSeek-MoE)
 //   tests/moe_deepseek_block_test.rs:42-74  (DeepSeek block: packed experts + fused shared experts)
+//   src/tensor/disk_tier.rs tests, tests/moe_qint8_tier_test.rs
+//                                        (qint8 tier files: size, round trip, refusal of a wrong size)
 //   tests/moe_v3_route_scale_cert_test.rs:56-175, src/moe/v3_router.rs:340-462
 //                                        (DeepSeek-V3 routing: configuration errors, HF f64 fixture)
 //   tests/moe_numerical_equivalence_test.rs:44-110, tests/moe_hf_convention_test.rs:123-146
@@ -708,6 +710,45 @@ int main(int argc, char** argv) {
     CHECK(e.is_ok() && e.value().entries().empty(), "empty checkpoint");
   });
 
+  // ---- qint8 tier files -----------------------------------------------------------------------
+  run_test("qint8_tier_file_round_trip", [&] {
+    const size_t rows = 6, cols = 40;
+    std::vector<float> w = seeded(31, rows * cols);
+    for (size_t c = 0; c < cols; ++c) w[2 * cols + c] = 0.f;  // an all-zero row: scale 1, q 0
+    w[4 * cols + 7] = 3.5f;                                   // an outlier sets its row's scale
+    const std::string path = work + "/gate.qint8";
+    auto werr = write_qint8_tensor_named(path, w, rows, cols);
+    CHECK(!werr, "%s", werr ? werr->c_str() : "");
+    CHECK(slurp(path).size() == qint8_disk_bytes(rows * cols, rows) && qint8_disk_bytes(rows * cols, rows) == 264,
+          "rows * 4 + numel bytes: about one byte per element");
+    auto t = read_qint8_tensor(path, rows * cols, rows).unwrap();
+    const QInt8Tensor direct = quantize_per_row_i8(w, rows, cols);
+    CHECK(t.q == direct.q && t.scales == direct.scales && t.rows == rows && t.cols == cols, "file == quantiser");
+    CHECK(t.scales[2] == 1.0f && t.scales[4] == 3.5f / 127.0f && t.q[4 * cols + 7] == 127, "scales");
+    const std::vector<float> back = read_qint8_to_f32(path, rows * cols, rows).unwrap();
+    CHECK(back == t.dequantize(), "read_qint8_to_f32 is q * scale");
+    for (size_t r = 0; r < rows; ++r)
+      for (size_t c = 0; c < cols; ++c)
+        CHECK(std::fabs(back[r * cols + c] - w[r * cols + c]) <= 0.5f * t.scales[r] * 1.0001f,
+              "round trip within half a step at (%zu, %zu)", r, c);
+    // the quantisation axis must divide the element count, and the size must match
+    CHECK(read_qint8_tensor(path, rows * cols, 7).is_err(), "rows that do not divide numel");
+    CHECK(read_qint8_tensor(path, rows * cols, 3).is_err(), "a file of another size");
+    CHECK(read_qint8_tensor(work + "/absent.qint8", 8, 2).is_err(), "missing file");
+    CHECK(write_qint8_tensor_named(path, w, rows, cols + 1).has_value(), "length mismatch on write");
+  });
+  run_test("expert_from_qint8_keeps_the_tier_data", [&] {
+    const size_t d = 16, f = 24;
+    auto g = quantize_per_row_i8(seeded(1, f * d), f, d), u = quantize_per_row_i8(seeded(2, f * d), f, d),
+         dn = quantize_per_row_i8(seeded(3, d * f), d, f);
+    auto ex = MoeDenseExpert::from_qint8(d, f, g, u, dn).unwrap();
+    CHECK(ex.q8 && ex.q8->gate.q == g.q && ex.q8->down.scales == dn.scales, "payload kept");
+    CHECK(ex.w_gate == g.dequantize() && ex.w_up == u.dequantize() && ex.w_down == dn.dequantize(),
+          "w_* are the dequantised values");
+    auto bad = MoeDenseExpert::from_qint8(d, f, g, u, g);
+    CHECK(bad.is_err() && bad.error().kind == MoeDenseError::WeightShapeMismatch, "down of the wrong shape");
+  });
+
   // ---- golden layer files ---------------------------------------------------------------------
   const char* models[] = {"mixtral", "qwen15_moe", "qwen2_moe", "qwen3_moe"};
   run_test("golden_layers_assemble_with_sidecar_config", [&] {
@@ -854,6 +895,33 @@ int main(int argc, char** argv) {
     auto out = layer.forward_with(hidden, MoeExecutionConvention::HuggingFaceQwen).unwrap();
     const std::vector<float> want = floats(side.get("block_out"));
     CHECK(max_abs_diff(out, want) < 1e-6, "block output: %g", max_abs_diff(out, want));
+  });
+  run_test("qint8_tier_files_to_device_without_requantising", [&] {
+    // The Mixtral golden layer written as qint8 tier files, read back, and run as an Int8W8A16
+    // layer: the tier data reaches the device as it is, so the result equals the layer that
+    // quantises the same f32 weights itself, bit for bit; and it stays within the int8 bar of
+    // the oracle run on the dequantised weights (the values the reference computes with).
+    Golden g = load_golden(golden, "mixtral", MoeWeightStorage::Int8W8A16);
+    const size_t E = g.layer.num_experts(), d = g.config.d_model, f = g.config.d_ff;
+    std::vector<MoeDenseExpert> experts;
+    for (size_t e = 0; e < E; ++e) {
+      const MoeDenseExpert& src = g.layer.routed.experts[e];
+      const std::string base = work + "/expert" + std::to_string(e);
+      CHECK(!write_qint8_tensor_named(base + ".gate", src.w_gate, f, d) &&
+                !write_qint8_tensor_named(base + ".up", src.w_up, f, d) &&
+                !write_qint8_tensor_named(base + ".down", src.w_down, d, f), "write tier files");
+      experts.push_back(MoeDenseExpert::from_qint8(d, f, read_qint8_tensor(base + ".gate", f * d, f).unwrap(),
+                                                   read_qint8_tensor(base + ".up", f * d, f).unwrap(),
+                                                   read_qint8_tensor(base + ".down", d * f, d).unwrap()).unwrap());
+    }
+    auto routed = MoeDenseLayer::make(d, f, g.layer.routed.w_router, std::move(experts), g.config.experts_per_token).unwrap();
+    auto tier = RealMoeLayer::assemble(g.config, std::move(routed), std::nullopt, std::nullopt,
+                                       MoeWeightStorage::Int8W8A16).unwrap();
+    const std::vector<float> from_tier = tier.forward_auto(g.input).unwrap();
+    const std::vector<float> from_f32 = g.layer.forward_auto(g.input).unwrap();
+    CHECK(from_tier == from_f32, "tier data must reach the device unchanged: %g", max_abs_diff(from_tier, from_f32));
+    const std::vector<float> want = oracle_forward(tier, g.input, 0);  // tier.routed holds the dequantised weights
+    CHECK(max_abs_diff(from_tier, want) <= 1e-2 * max_abs(want), "%g of %g", max_abs_diff(from_tier, want), max_abs(want));
   });
   run_test("ingested_layer_through_the_registry", [&] {
     Golden g = load_golden(golden, "qwen2_moe");
