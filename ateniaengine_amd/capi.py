@@ -17,7 +17,7 @@ LIB_PATH = os.path.join(_HERE, "libatenia_moe_hip.so")
 
 CONVENTION_ATENIA = 0
 CONVENTION_HUGGINGFACE_QWEN = 1
-WEIGHT_F32, WEIGHT_BF16, WEIGHT_INT8_W8A16 = 0, 1, 2
+WEIGHT_F32, WEIGHT_BF16, WEIGHT_INT8_W8A16, WEIGHT_INT8_PER_GROUP = 0, 1, 2, 3
 ACT_F32, ACT_BF16 = 0, 1
 NORM_GRAPH_F32, NORM_F64 = 0, 1
 OK, ERR_SYNC, ERR_LAUNCH = 0, 1, 2
@@ -40,6 +40,7 @@ EXPORTS = (
     "atenia_moe_expert_ffn_launch_device", "atenia_moe_combine_launch_device",
     "atenia_moe_hip_layer_block_forward", "atenia_moe_hip_layer_block_forward_device",
     "atenia_moe_hip_layer_last_normed", "atenia_moe_hip_layer_set_v3_router",
+    "atenia_moe_quantize_per_group_i8",
 )
 
 
@@ -59,7 +60,7 @@ class LayerDesc(C.Structure):
         ("scale_gate", C.c_void_p), ("scale_up", C.c_void_p), ("scale_down", C.c_void_p),
         ("s_gate", C.c_void_p), ("s_up", C.c_void_p), ("s_down", C.c_void_p),
         ("s_scale_gate", C.c_void_p), ("s_scale_up", C.c_void_p), ("s_scale_down", C.c_void_p),
-        ("shared_gate", C.c_void_p),
+        ("shared_gate", C.c_void_p), ("group_size", C.c_int32),
     ]
 
 
@@ -104,6 +105,7 @@ def lib():
         L.atenia_moe_hip_layer_block_forward_device.argtypes = [P, P, C.c_int, P, C.c_float,
                                                                 C.c_int, P, P]
         L.atenia_moe_hip_layer_last_normed.argtypes = [P, P]
+        L.atenia_moe_quantize_per_group_i8.argtypes = [P, C.c_size_t, C.c_size_t, C.c_size_t, P, P]
         L.atenia_moe_hip_layer_set_v3_router.argtypes = [P, C.c_int, C.c_int, C.c_double, C.c_int, P]
         L.atenia_moe_router_launch_device.argtypes = [P, P, C.c_int, C.c_int, P, P, P]
         L.atenia_moe_permute_launch_device.argtypes = [P, C.c_int, P, P, P, P]
@@ -140,6 +142,17 @@ def quantize_per_row_i8(w):
     return q, s
 
 
+def quantize_per_group_i8(w, group_size: int):
+    """Per-group symmetric int8 along the last axis: returns (q like w, scales [..., ceil(cols/gs)])."""
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    rows = int(np.prod(w.shape[:-1]))
+    cols = w.shape[-1]
+    q = np.empty(w.shape, dtype=np.int8)
+    s = np.empty(w.shape[:-1] + ((cols + group_size - 1) // group_size,), dtype=np.float32)
+    _check(lib().atenia_moe_quantize_per_group_i8(_ptr(w), rows, cols, group_size, _ptr(q), _ptr(s)))
+    return q, s
+
+
 def f32_to_bf16_trunc(a) -> np.ndarray:
     a = np.ascontiguousarray(a, dtype=np.float32)
     out = np.empty(a.shape, dtype=np.uint16)
@@ -147,7 +160,8 @@ def f32_to_bf16_trunc(a) -> np.ndarray:
     return out
 
 
-_WDTYPE_NP = {WEIGHT_F32: np.float32, WEIGHT_BF16: np.uint16, WEIGHT_INT8_W8A16: np.int8}
+_WDTYPE_NP = {WEIGHT_F32: np.float32, WEIGHT_BF16: np.uint16, WEIGHT_INT8_W8A16: np.int8,
+              WEIGHT_INT8_PER_GROUP: np.int8}
 
 
 class Layer:
@@ -156,7 +170,8 @@ class Layer:
     def __init__(self, *, w_router, w_gate, w_down, top_k, w_up=None, convention=CONVENTION_ATENIA,
                  weight_dtype=WEIGHT_F32, router_bias=None, scale_gate=None, scale_up=None,
                  scale_down=None, s_gate=None, s_up=None, s_down=None, s_scale_gate=None,
-                 s_scale_up=None, s_scale_down=None, shared_gate=None, max_tokens_hint=0):
+                 s_scale_up=None, s_scale_down=None, shared_gate=None, max_tokens_hint=0,
+                 group_size=0):
         wt = _WDTYPE_NP[weight_dtype]
         w_router = _arr(w_router, np.float32)
         E, d = w_router.shape
@@ -180,7 +195,7 @@ class Layer:
                          *[_ptr(keep[n]) for n in (
                              "w_router", "router_bias", "w_gate", "w_up", "w_down", "scale_gate",
                              "scale_up", "scale_down", "s_gate", "s_up", "s_down", "s_scale_gate",
-                             "s_scale_up", "s_scale_down", "shared_gate")])
+                             "s_scale_up", "s_scale_down", "shared_gate")], group_size)
         self.E, self.k, self.d, self.f, self.fs = E, top_k, d, f, fs
         self.convention, self.weight_dtype = convention, weight_dtype
         self._h = C.c_void_p()

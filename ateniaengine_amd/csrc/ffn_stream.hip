@@ -27,8 +27,10 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 struct StreamParams {
   const uint4* wa;      // gate (up phase) or down blocks
   const uint4* wb;      // up blocks (up phase only)
-  const float* sa;      // int8 row scales of wa, [G, n_rows]
+  const float* sa;      // int8 row scales of wa, [G, n_rows]; per-group: [G][strips][n_kgroups][16]
   const float* sb;
+  int group_blocks;     // per-group int8: 64-k blocks per scale group (0 = per-row scales)
+  int n_kgroups;        // per-group int8: scale groups along K
   int64_t w_stride_u4;  // uint4 between experts
   int n_rows;           // unpadded N
   int nkb;              // K blocks per strip
@@ -84,7 +86,11 @@ __device__ inline f32x4 mfma(bf16x8 a, bf16x8 b, f32x4 c) {
 // INT8: weights are int8 blocks (64 k per block) instead of bf16 blocks (32 k per block)
 // UP  : gate/up phase with SwiGLU epilogue, else down phase
 // WAVES: waves per workgroup = K slices of the strip
-template <int MT, bool INT8, bool UP, int WAVES>
+// PG  : int8 with one scale per output row and k group (Q8_0-style): every 64-k block is
+//       accumulated on its own and added to the running sum times the scale of its group,
+//       sum_g s[n, g] * (sum_{k in g} q[n, k] x[k]), which is the reference's
+//       sum_k (q * s) x (src/tensor/quantizer.rs:175-248) up to f32 rounding
+template <int MT, bool INT8, bool UP, int WAVES, bool PG>
 __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p) {
   constexpr int kWavesPerWg = WAVES;
   const int u = blockIdx.y;
@@ -157,13 +163,35 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p) 
   for (int n = 0; n < NACC; ++n)
 #pragma unroll
     for (int i = 0; i < MT; ++i) acc[n][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // Per-group scales of this lane's output row (column mm of the D layout), one per k group.
+  const float* psa = PG ? p.sa + (((size_t)e * gridDim.x + nb) * p.n_kgroups) * 16 + mm : nullptr;
+  const float* psb = PG && UP ? p.sb + (((size_t)e * gridDim.x + nb) * p.n_kgroups) * 16 + mm : nullptr;
 
   auto multiply = [&](const uint4 (&wa)[U], const uint4 (&wb)[UP ? U : 1],
                       const uint4 (&xa)[U][MT][AV], int kb) {
 #pragma unroll
     for (int j = 0; j < U; ++j) {
       if (kb + j < kb1) {
-        if (INT8) {
+        if (INT8 && PG) {
+          bf16x8 al, ah, bl, bh;
+          widen_i8x16(wa[j], al, ah);
+          if (UP) widen_i8x16(wb[j], bl, bh);
+          const int kg = (kb + j) / p.group_blocks;
+          const float s_a = psa[(size_t)kg * 16];
+          const float s_b = UP ? psb[(size_t)kg * 16] : 0.f;
+#pragma unroll
+          for (int i = 0; i < MT; ++i) {
+            uint4 x0 = xa[j][i][0], x1 = xa[j][i][AV - 1];
+            f32x4 ta = mfma(*(bf16x8*)&x0, al, f32x4{0.f, 0.f, 0.f, 0.f});
+            ta = mfma(*(bf16x8*)&x1, ah, ta);
+            acc[0][i] += ta * s_a;
+            if (UP) {
+              f32x4 tb = mfma(*(bf16x8*)&x0, bl, f32x4{0.f, 0.f, 0.f, 0.f});
+              tb = mfma(*(bf16x8*)&x1, bh, tb);
+              acc[NACC - 1][i] += tb * s_b;
+            }
+          }
+        } else if (INT8) {
           bf16x8 al, ah, bl, bh;
           widen_i8x16(wa[j], al, ah);
           if (UP) widen_i8x16(wb[j], bl, bh);
@@ -222,7 +250,7 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p) 
   // D layout: lane holds rows 4*kq + r (r = 0..3) of column mm.
   const int n = nb * 16 + mm;
   float sa = 1.f, sb = 1.f;
-  if (INT8) {
+  if (INT8 && !PG) {
     sa = n < p.n_rows ? p.sa[(size_t)e * p.n_rows + n] : 0.f;
     if (UP) sb = n < p.n_rows ? p.sb[(size_t)e * p.n_rows + n] : 0.f;
   }
@@ -354,10 +382,17 @@ hipError_t launch_stream(const StreamParams& p, int n_pad, int n_groups, int row
   // The down projection has few strips (d / 16) and a long K (f): eight K slices per strip
   // keep enough loads in flight; gate/up has 2f / 16 strips and uses four.
   constexpr int W = UP ? 4 : 8;
+  if (INT8 && p.group_blocks > 0) {
+    if (mt == 1)
+      ffn_stream_kernel<1, INT8, UP, W, INT8><<<grid, 64 * W, 0, s>>>(p);
+    else
+      ffn_stream_kernel<2, INT8, UP, W, INT8><<<grid, 64 * W, 0, s>>>(p);
+    return hipGetLastError();
+  }
   if (mt == 1)
-    ffn_stream_kernel<1, INT8, UP, W><<<grid, 64 * W, 0, s>>>(p);
+    ffn_stream_kernel<1, INT8, UP, W, false><<<grid, 64 * W, 0, s>>>(p);
   else
-    ffn_stream_kernel<2, INT8, UP, W><<<grid, 64 * W, 0, s>>>(p);
+    ffn_stream_kernel<2, INT8, UP, W, false><<<grid, 64 * W, 0, s>>>(p);
   return hipGetLastError();
 }
 
@@ -375,6 +410,8 @@ hipError_t launch_ffn_up(const FfnArgs& a, hipStream_t s) {
   p.wb = (const uint4*)a.up.w;
   p.sa = a.gate.scale;
   p.sb = a.up.scale;
+  p.group_blocks = a.gate.group_blocks;
+  p.n_kgroups = a.gate.n_kgroups;
   p.w_stride_u4 = a.gate.expert_stride / 16;
   p.n_rows = a.gate.n_rows;
   p.nkb = a.gate.k_pad / (int8 ? kKbInt8 : kKbBf16);
@@ -396,6 +433,8 @@ hipError_t launch_ffn_down(const FfnArgs& a, hipStream_t s) {
   p.wb = nullptr;
   p.sa = a.down.scale;
   p.sb = nullptr;
+  p.group_blocks = a.down.group_blocks;
+  p.n_kgroups = a.down.n_kgroups;
   p.w_stride_u4 = a.down.expert_stride / 16;
   p.n_rows = a.down.n_rows;
   p.nkb = a.down.k_pad / (int8 ? kKbInt8 : kKbBf16);
@@ -419,6 +458,8 @@ hipError_t launch_ffn_down_decode1(const FfnArgs& a, hipStream_t s) {
   p.wb = nullptr;
   p.sa = a.down.scale;
   p.sb = nullptr;
+  p.group_blocks = a.down.group_blocks;
+  p.n_kgroups = a.down.n_kgroups;
   p.w_stride_u4 = a.down.expert_stride / 16;
   p.n_rows = a.down.n_rows;
   p.nkb = a.down.k_pad / (int8 ? kKbInt8 : kKbBf16);

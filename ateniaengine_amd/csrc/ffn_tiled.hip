@@ -1005,6 +1005,7 @@ bool tiled_down_splits_tail(const WeightSet& down, int wdtype) {
 
 bool tiled_supported(const WeightSet& w, int wdtype) {
   if (wdtype == ATENIA_MOE_WEIGHT_F32) return false;
+  if (w.group_blocks > 0) return false;  // per-group scales: streaming kernels only
   return w.k_pad % TK == 0;
 }
 

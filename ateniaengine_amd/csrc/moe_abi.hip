@@ -83,6 +83,7 @@ struct AteniaMoeLayer {
   int f_kpad = 0;   // K padding of h rows (down projection)
   int fs_kpad = 0;
   int device = 0;
+  int group_size = 0;  // per-group int8: input elements per scale (0 = per-row scales)
 
   DevBuf w_router, router_bias, shared_gate;
   DevBuf wg, wu, wd, sg, su, sd;        // routed experts
@@ -198,6 +199,27 @@ int upload_f32(const float* host, size_t n, DevBuf& dst) {
   int rc = dst.ensure(n * 4);
   if (rc) return rc;
   HIP_TRY(hipMemcpy(dst.p, host, n * 4, hipMemcpyHostToDevice));
+  return ATENIA_MOE_OK;
+}
+
+// Per-group scales [G, n_rows, n_kgroups] (host) -> [G][n_pad / 16][n_kgroups][16] (device): the
+// 16 rows of a strip are adjacent for every k group, so a wavefront of the streaming kernel
+// fetches the scales of a group with one 64-byte read.  Rows past n_rows get scale 0.
+int upload_group_scales(const float* host, int G, int n_rows, int k_cols, int group_size,
+                        DevBuf& dst, WeightSet& ws) {
+  const int ng = (k_cols + group_size - 1) / group_size;
+  const int n_pad = round_up(n_rows, 16);
+  std::vector<float> re((size_t)G * n_pad * ng, 0.0f);
+  for (int g = 0; g < G; ++g)
+    for (int n = 0; n < n_rows; ++n)
+      for (int kg = 0; kg < ng; ++kg)
+        re[(((size_t)g * (n_pad / 16) + n / 16) * ng + kg) * 16 + n % 16] =
+            host[((size_t)g * n_rows + n) * ng + kg];
+  int rc = upload_f32(re.data(), re.size(), dst);
+  if (rc) return rc;
+  ws.scale = dst.as<float>();
+  ws.group_blocks = group_size / kKbInt8;
+  ws.n_kgroups = ng;
   return ATENIA_MOE_OK;
 }
 
@@ -441,6 +463,7 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   // One token, up to two experts, no shared expert, whole pipeline requested: the down launch
   // finishes the combine as well (same bits as the two launches, one launch less).
   const bool fuse1 = first <= kStageFfn && last >= kStageCombine &&
+                     L->group_size == 0 &&
                      ffn_down_decode1_supported(T, L->k, L->wdtype, tiled, L->fs > 0);
   if (first <= kStageFfn) {
     if (fuse1) {
@@ -537,11 +560,17 @@ int atenia_moe_hip_layer_create(const AteniaMoeLayerDesc* D, AteniaMoeLayer** ou
   if (D->convention != ATENIA_MOE_CONVENTION_ATENIA &&
       D->convention != ATENIA_MOE_CONVENTION_HUGGINGFACE_QWEN)
     return fail(ATENIA_MOE_ERR_DIM, "unknown convention %d", D->convention);
-  if (D->weight_dtype < 0 || D->weight_dtype > 2)
+  if (D->weight_dtype < 0 || D->weight_dtype > ATENIA_MOE_WEIGHT_INT8_PER_GROUP)
     return fail(ATENIA_MOE_ERR_DIM, "unknown weight dtype %d", D->weight_dtype);
+  const bool per_group = D->weight_dtype == ATENIA_MOE_WEIGHT_INT8_PER_GROUP;
+  if (per_group && (D->group_size <= 0 || D->group_size % kKbInt8 != 0))
+    return fail(ATENIA_MOE_ERR_DIM, "per-group int8 needs group_size > 0 and a multiple of %d (got %d)",
+                kKbInt8, D->group_size);
+  if (per_group && !D->w_up)
+    return fail(ATENIA_MOE_ERR_UNSUPPORTED, "per-group int8 takes separate gate and up tensors");
   if (!D->w_router || !D->w_gate || !D->w_down)
     return fail(ATENIA_MOE_ERR_DIM, "router / gate / down weights are required");
-  const bool int8 = D->weight_dtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
+  const bool int8 = D->weight_dtype == ATENIA_MOE_WEIGHT_INT8_W8A16 || per_group;
   if (int8 && (!D->scale_gate || !D->scale_up || !D->scale_down))
     return fail(ATENIA_MOE_ERR_DIM, "int8 weights need per-row scales");
   if (D->d_ff_shared > 0) {
@@ -564,7 +593,9 @@ int atenia_moe_hip_layer_create(const AteniaMoeLayerDesc* D, AteniaMoeLayer** ou
   L->f = D->d_ff;
   L->fs = D->d_ff_shared;
   L->conv = D->convention;
-  L->wdtype = D->weight_dtype;
+  // Per-group int8 is stored and streamed like per-row int8; only the scales differ.
+  L->wdtype = per_group ? ATENIA_MOE_WEIGHT_INT8_W8A16 : D->weight_dtype;
+  L->group_size = per_group ? D->group_size : 0;
   const int KB = L->wdtype == ATENIA_MOE_WEIGHT_F32 ? 1 : kb_of(L->wdtype);
   L->d_kpad = round_up(L->d, KB);
   L->f_kpad = round_up(L->f, KB);
@@ -596,7 +627,12 @@ int atenia_moe_hip_layer_create(const AteniaMoeLayerDesc* D, AteniaMoeLayer** ou
   if ((rc = upload_family(D->w_down, d * f, L->E, L->d, L->f, L->wdtype, L->wd, L->down,
                           staging)))
     return bail(rc);
-  if (int8) {
+  if (per_group) {
+    const int gs = L->group_size;
+    if ((rc = upload_group_scales(D->scale_gate, L->E, L->f, L->d, gs, L->sg, L->gate))) return bail(rc);
+    if ((rc = upload_group_scales(D->scale_up, L->E, L->f, L->d, gs, L->su, L->up))) return bail(rc);
+    if ((rc = upload_group_scales(D->scale_down, L->E, L->d, L->f, gs, L->sd, L->down))) return bail(rc);
+  } else if (int8) {
     if ((rc = upload_f32(D->scale_gate, E * f, L->sg))) return bail(rc);
     if ((rc = upload_f32(D->scale_up, E * f, L->su))) return bail(rc);
     if ((rc = upload_f32(D->scale_down, E * d, L->sd))) return bail(rc);
@@ -614,7 +650,12 @@ int atenia_moe_hip_layer_create(const AteniaMoeLayerDesc* D, AteniaMoeLayer** ou
     if ((rc = upload_family(D->s_down, d * fs, 1, L->d, L->fs, L->wdtype, L->swd, L->s_down,
                             staging)))
       return bail(rc);
-    if (int8) {
+    if (per_group) {
+      const int gs = L->group_size;
+      if ((rc = upload_group_scales(D->s_scale_gate, 1, L->fs, L->d, gs, L->ssg, L->s_gate))) return bail(rc);
+      if ((rc = upload_group_scales(D->s_scale_up, 1, L->fs, L->d, gs, L->ssu, L->s_up))) return bail(rc);
+      if ((rc = upload_group_scales(D->s_scale_down, 1, L->d, L->fs, gs, L->ssd, L->s_down))) return bail(rc);
+    } else if (int8) {
       if ((rc = upload_f32(D->s_scale_gate, fs, L->ssg))) return bail(rc);
       if ((rc = upload_f32(D->s_scale_up, fs, L->ssu))) return bail(rc);
       if ((rc = upload_f32(D->s_scale_down, d, L->ssd))) return bail(rc);
@@ -625,6 +666,10 @@ int atenia_moe_hip_layer_create(const AteniaMoeLayerDesc* D, AteniaMoeLayer** ou
   }
   // Algorithmic bytes of one routed expert as stored (weights + int8 scales).
   L->bytes_per_expert = (int64_t)(3 * d * f * eb) + (int8 ? (int64_t)(2 * f + d) * 4 : 0);
+  if (per_group)  // one scale per row and group instead of one per row
+    L->bytes_per_expert = (int64_t)(3 * d * f * eb) +
+                          ((int64_t)2 * f * ((d + L->group_size - 1) / L->group_size) +
+                           (int64_t)d * ((f + L->group_size - 1) / L->group_size)) * 4;
   if (D->max_tokens_hint > 0 && (rc = ensure_workspace(L, D->max_tokens_hint))) return bail(rc);
   if (hipDeviceSynchronize() != hipSuccess)
     return bail(fail(ATENIA_MOE_ERR_SYNC, "device synchronisation failed after upload"));
@@ -1047,6 +1092,30 @@ int atenia_moe_hip_layer_info(const AteniaMoeLayer* L, int64_t info[8]) {
   info[5] = L->conv;
   info[6] = L->wdtype;
   info[7] = L->bytes_per_expert;
+  return ATENIA_MOE_OK;
+}
+
+int atenia_moe_quantize_per_group_i8(const float* w, size_t rows, size_t cols, size_t group_size,
+                                     int8_t* q_out, float* scales_out) {
+  if (!w || !q_out || !scales_out) return fail(ATENIA_MOE_ERR_DIM, "null pointer");
+  if (group_size == 0) return fail(ATENIA_MOE_ERR_DIM, "group_size must be > 0");
+  const size_t ng = (cols + group_size - 1) / group_size;
+  for (size_t r = 0; r < rows; ++r)
+    for (size_t g = 0; g < ng; ++g) {
+      const size_t c0 = g * group_size, c1 = std::min(cols, c0 + group_size);
+      float max_abs = 0.0f;
+      for (size_t c = c0; c < c1; ++c) {
+        const float v = std::fabs(w[r * cols + c]);
+        if (v > max_abs) max_abs = v;
+      }
+      const float sc = std::max(max_abs / 127.0f, 1e-12f);
+      scales_out[r * ng + g] = sc;
+      for (size_t c = c0; c < c1; ++c) {
+        float qf = std::round(w[r * cols + c] / sc);  // half away from zero, like f32::round
+        qf = std::min(127.0f, std::max(-127.0f, qf));
+        q_out[r * cols + c] = (int8_t)(int32_t)qf;
+      }
+    }
   return ATENIA_MOE_OK;
 }
 

@@ -38,7 +38,10 @@ struct GroupDesc {
 // One expert projection family as stored on the device.
 struct WeightSet {
   const void* w;            // blocks (bf16/int8) or row-major f32
-  const float* scale;       // int8: per output row, [G, N] (unpadded N stride = n_rows)
+  const float* scale;       // int8: per output row, [G, N] (unpadded N stride = n_rows);
+                            // per-group int8: [G][n_pad / 16][n_kgroups][16] (see group_blocks)
+  int group_blocks;         // per-group int8: 64-k blocks per scale group (0 = one scale per row)
+  int n_kgroups;            // per-group int8: scale groups along K
   int64_t expert_stride;    // elements (f32) or bytes (blocked) between experts
   int n_rows;               // N (unpadded)
   int n_pad;                // padded N

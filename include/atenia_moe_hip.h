@@ -52,6 +52,10 @@ extern "C" {
 #define ATENIA_MOE_WEIGHT_BF16 1       /* TensorStorage::CpuBf16, raw u16 bit patterns          */
 #define ATENIA_MOE_WEIGHT_INT8_W8A16 2 /* per-output-row int8 + f32 scales
                                           (src/tensor/disk_tier.rs:231-259)                     */
+/* int8 with one f32 scale per output row and per group of `group_size` consecutive input
+ * elements (Q8_0-style; the reference's per-group scheme, src/tensor/quantizer.rs:175-248, laid
+ * out for [out, in] weights): scales are [.., rows, ceil(cols / group_size)]. */
+#define ATENIA_MOE_WEIGHT_INT8_PER_GROUP 3
 
 /* Element type of device activations handed to `forward_device`. */
 #define ATENIA_MOE_ACT_F32 0
@@ -111,6 +115,11 @@ typedef struct AteniaMoeLayerDesc {
   const float* s_scale_up;   /* int8 only: f32 [f_s]                                     */
   const float* s_scale_down; /* int8 only: f32 [d]                                       */
   const float* shared_gate; /* f32 [d] sigmoid gate vector (src/moe/layer.rs:436-443) or NULL */
+  int32_t group_size;       /* ATENIA_MOE_WEIGHT_INT8_PER_GROUP only: input elements per scale,
+                               a multiple of 64 (128 = the reference's production value); the
+                               scale arrays are then [E, f, ceil(d/gs)], [E, f, ceil(d/gs)],
+                               [E, d, ceil(f/gs)] and [f_s, ..] / [d, ceil(f_s/gs)] for the
+                               shared expert.  0 otherwise.                               */
 } AteniaMoeLayerDesc;
 
 /* 1 when a gfx950 device is present and usable, else 0.  Replaces `cuda_available()`
@@ -119,6 +128,14 @@ int atenia_moe_hip_available(void);
 
 /* Human-readable text of the calling thread's most recent failure ("" if none). */
 const char* atenia_moe_hip_last_error_string(void);
+
+/* Per-group symmetric int8 quantisation of a row-major [rows, cols] weight, groups of
+ * `group_size` consecutive elements of a row: scale = max(max|w| / 127, 1e-12), q = round(w /
+ * scale) clamped to [-127, 127]; scales out: [rows, ceil(cols / group_size)].  The arithmetic of
+ * absmax_per_group_symmetric (src/tensor/quantizer.rs:175-248), which walks a [K, N] weight in
+ * groups along K; here K is the row's own direction.  Host function. */
+int atenia_moe_quantize_per_group_i8(const float* w, size_t rows, size_t cols, size_t group_size,
+                                     int8_t* q_out, float* scales_out);
 
 /* Uploads the layer once; the handle owns the device copies, as the reference registry owns
  * its `Arc<RealMoeLayer>` (src/moe/graph_op.rs:228-232).  Replaces the per-call H->D upload of

@@ -24,6 +24,7 @@
  *              ora_numerical_metrics, ora_layer_forward_f64, ora_permute
  *              (brute force), ora_matvec_f32acc, ora_rms_norm_gamma,
  *              ora_block_forward, ora_v3_validate, ora_v3_route,
+ *              ora_absmax_per_group_symmetric, ora_int8_to_bf16_per_group,
  *              ora_v3_layer_forward (router and block output against the
  *              HuggingFace f64 fixture; its f32 combine is this build's choice,
  *              see the function).
@@ -611,6 +612,50 @@ void ora_int8_to_bf16_per_channel(const int8_t* q, const float* scales, size_t k
                                   uint16_t* out_bf16) {
   for (size_t i = 0; i < k * n; ++i)
     out_bf16[i] = ora_f32_to_bf16_bits((float)q[i] * scales[i % n]);
+}
+
+/* ---- quantizer.rs:175-248 : absmax_per_group_symmetric ---------------------------------
+ * weights [K, N] row-major, groups of `group_size` consecutive k for every column n:
+ * scales[g * N + n] = max(max_{k in g} |w[k, n]| / 127, 1e-12); q[k, n] = round(w / scale)
+ * clamped to [-127, 127] (f32 division, f32::round = half away from zero).
+ * Pinned by closed forms (a group's largest element maps to +-127; an all-zero group gets the
+ * 1e-12 floor; an outlier only coarsens its own group) and the round-trip bound |w - q s| <= s/2. */
+void ora_absmax_per_group_symmetric(const float* w, size_t k, size_t n, size_t group_size,
+                                    int8_t* q, float* scales) {
+  size_t ng = k == 0 ? 0 : (k + group_size - 1) / group_size;
+  for (size_t g = 0; g < ng; ++g) {
+    size_t lo = g * group_size, hi = (g + 1) * group_size < k ? (g + 1) * group_size : k;
+    for (size_t col = 0; col < n; ++col) {
+      float max_abs = 0.0f;
+      for (size_t row = lo; row < hi; ++row) {
+        float v = fabsf(w[row * n + col]);
+        if (v > max_abs) max_abs = v;
+      }
+      float sc = max_abs / 127.0f;
+      scales[g * n + col] = sc > 1e-12f ? sc : 1e-12f;
+    }
+  }
+  for (size_t row = 0; row < k; ++row) {
+    size_t g = row / group_size;
+    for (size_t col = 0; col < n; ++col) {
+      float qf = roundf(w[row * n + col] / scales[g * n + col]);
+      if (qf < -127.0f) qf = -127.0f;
+      if (qf > 127.0f) qf = 127.0f;
+      q[row * n + col] = (int8_t)(int32_t)qf;
+    }
+  }
+}
+
+/* int8_to_bf16.cu:91-110 : per-group dequantisation to truncated bf16 (the reference's GPU form). */
+void ora_int8_to_bf16_per_group(const int8_t* q, const float* scales, size_t k, size_t n,
+                                size_t group_size, uint16_t* out) {
+  for (size_t idx = 0; idx < k * n; ++idx) {
+    size_t row = idx / n, col = idx % n;
+    float f = (float)q[idx] * scales[(row / group_size) * n + col];
+    uint32_t bits;
+    memcpy(&bits, &f, 4);
+    out[idx] = (uint16_t)(bits >> 16);
+  }
 }
 
 /* ---- numerical.rs:40-88 : comparison metrics, f64 accumulation ----------- */

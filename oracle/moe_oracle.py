@@ -113,6 +113,8 @@ def lib():
         L.ora_dequantize_per_row_i8.argtypes = [P, P, Z, Z, P]
         L.ora_absmax_per_channel_symmetric.argtypes = [P, Z, Z, P, P]
         L.ora_int8_to_bf16_per_channel.argtypes = [P, P, Z, Z, P]
+        L.ora_absmax_per_group_symmetric.argtypes = [P, Z, Z, Z, P, P]
+        L.ora_int8_to_bf16_per_group.argtypes = [P, P, Z, Z, Z, P]
         L.ora_numerical_metrics.argtypes = [P, P, Z, P]
         L.ora_numerical_metrics.restype = C.c_int
         L.ora_layer_forward_f64.argtypes = [P, P, P, P]
@@ -446,6 +448,25 @@ def int8_to_bf16_per_channel(q, scales) -> np.ndarray:
     k, n = q.shape
     out = np.empty((k, n), dtype=np.uint16)
     lib().ora_int8_to_bf16_per_channel(_p(q), _p(scales), k, n, _p(out))
+    return out
+
+
+def absmax_per_group_symmetric(w, group_size: int):
+    """quantizer.rs:175-248 on a [K, N] weight: (q [K, N] i8, scales [ceil(K/gs), N])."""
+    w = _f32(w)
+    k, n = w.shape
+    q = np.empty((k, n), dtype=np.int8)
+    s = np.empty(((k + group_size - 1) // group_size, n), dtype=np.float32)
+    lib().ora_absmax_per_group_symmetric(_p(w), k, n, group_size, _p(q), _p(s))
+    return q, s
+
+
+def int8_to_bf16_per_group(q, scales, group_size: int) -> np.ndarray:
+    q = np.ascontiguousarray(q, dtype=np.int8)
+    scales = _f32(scales)
+    k, n = q.shape
+    out = np.empty((k, n), dtype=np.uint16)
+    lib().ora_int8_to_bf16_per_group(_p(q), _p(scales), k, n, group_size, _p(out))
     return out
 
 

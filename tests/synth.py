@@ -33,7 +33,7 @@ def make_weights(seed, E, d, f, f_s=0, gated=False, w_std=0.02, router_std=None,
     return W
 
 
-def build_pair(ora, W, top_k, convention, weight_dtype, max_tokens_hint=0):
+def build_pair(ora, W, top_k, convention, weight_dtype, max_tokens_hint=0, group_size=128):
     """Returns (oracle Layer on the stored values, capi Layer)."""
     proj = ["w_gate", "w_up", "w_down"] + (["s_gate", "s_up", "s_down"] if "s_gate" in W else [])
     stored, dev, scales = {}, {}, {}
@@ -43,6 +43,12 @@ def build_pair(ora, W, top_k, convention, weight_dtype, max_tokens_hint=0):
             stored[name] = dev[name] = w
         elif weight_dtype == capi.WEIGHT_BF16:
             dev[name], stored[name] = bf16_round_trip(w)
+        elif weight_dtype == capi.WEIGHT_INT8_PER_GROUP:
+            q, s = capi.quantize_per_group_i8(w, group_size)
+            dev[name], scales[name] = q, s
+            # the dequantised weight the reference computes with: q * scale of the element's group
+            s_full = np.repeat(s, group_size, axis=-1)[..., :w.shape[-1]]
+            stored[name] = (q.astype(np.float32) * s_full).astype(np.float32)
         else:
             q, s = capi.quantize_per_row_i8(w)
             dev[name], scales[name] = q, s
@@ -57,8 +63,10 @@ def build_pair(ora, W, top_k, convention, weight_dtype, max_tokens_hint=0):
                              w_down=stored["w_down"], s_gate=stored.get("s_gate"),
                              s_up=stored.get("s_up"), s_down=stored.get("s_down"), **common)
     kw = {}
-    if weight_dtype == capi.WEIGHT_INT8_W8A16:
-        kw = dict(scale_gate=scales["w_gate"], scale_up=scales["w_up"],
+    if weight_dtype in (capi.WEIGHT_INT8_W8A16, capi.WEIGHT_INT8_PER_GROUP):
+        if weight_dtype == capi.WEIGHT_INT8_PER_GROUP:
+            kw["group_size"] = group_size
+        kw.update(scale_gate=scales["w_gate"], scale_up=scales["w_up"],
                   scale_down=scales["w_down"])
         if "s_gate" in W:
             kw.update(s_scale_gate=scales["s_gate"], s_scale_up=scales["s_up"],
