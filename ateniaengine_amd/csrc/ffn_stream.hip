@@ -27,7 +27,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 struct StreamParams {
   const uint4* wa;      // gate (up phase) or down blocks
   const uint4* wb;      // up blocks (up phase only)
-  const float* sa;      // int8 row scales of wa, [G, n_rows]; per-group: [G][strips][n_kgroups][16]
+  const float* sa;      // int8 row scales of wa, [G, n_rows]; per-group: [G][n_kgroups][n_pad]
   const float* sb;
   int group_blocks;     // per-group int8: 64-k blocks per scale group (0 = per-row scales)
   int n_kgroups;        // per-group int8: scale groups along K
@@ -121,15 +121,27 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p) 
   constexpr int AV = INT8 ? 2 : 1;       // 16-byte activation pieces per block and row tile
   uint4 wA0[U], wB0[UP ? U : 1], wA1[U], wB1[UP ? U : 1];
   uint4 xa0[U][MT][AV], xa1[U][MT][AV];
-  auto load_w = [&](uint4 (&wa)[U], uint4 (&wb)[UP ? U : 1], int kb) {
+  // Per-group scales of this lane's output row (column mm of the D layout), one per k group;
+  // they are requested together with the weight blocks they belong to.
+  const size_t n_pad_s = (size_t)gridDim.x * 16;  // scale rows per k group
+  const float* psa = PG ? p.sa + (size_t)e * p.n_kgroups * n_pad_s + nb * 16 + mm : nullptr;
+  const float* psb = PG && UP ? p.sb + (size_t)e * p.n_kgroups * n_pad_s + nb * 16 + mm : nullptr;
+  float sA0[PG ? U : 1], sB0[PG && UP ? U : 1], sA1[PG ? U : 1], sB1[PG && UP ? U : 1];
+  auto load_w = [&](uint4 (&wa)[U], uint4 (&wb)[UP ? U : 1], float (&sa)[PG ? U : 1],
+                    float (&sb)[PG && UP ? U : 1], int kb) {
 #pragma unroll
     for (int j = 0; j < U; ++j) {
       const int kk = min(kb + j, kb1 - 1);  // clamped: a batch past the end is loaded, not used
       wa[j] = load_stream(pa + (size_t)kk * 64);
       if (UP) wb[j] = load_stream(pb + (size_t)kk * 64);
+      if (PG) {
+        const int kg = kk / p.group_blocks;
+        sa[j] = psa[(size_t)kg * n_pad_s];
+        if (UP) sb[j] = psb[(size_t)kg * n_pad_s];
+      }
     }
   };
-  if (kb0 < kb1) load_w(wA0, wB0, kb0);
+  if (kb0 < kb1) load_w(wA0, wB0, sA0, sB0, kb0);
 
   // Token rows of the A operand.  Lanes whose row lies past the end of the group read the
   // group's first row instead: an MFMA output row depends on its own input row only, and
@@ -163,11 +175,8 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p) 
   for (int n = 0; n < NACC; ++n)
 #pragma unroll
     for (int i = 0; i < MT; ++i) acc[n][i] = f32x4{0.f, 0.f, 0.f, 0.f};
-  // Per-group scales of this lane's output row (column mm of the D layout), one per k group.
-  const float* psa = PG ? p.sa + (((size_t)e * gridDim.x + nb) * p.n_kgroups) * 16 + mm : nullptr;
-  const float* psb = PG && UP ? p.sb + (((size_t)e * gridDim.x + nb) * p.n_kgroups) * 16 + mm : nullptr;
-
   auto multiply = [&](const uint4 (&wa)[U], const uint4 (&wb)[UP ? U : 1],
+                      const float (&sa)[PG ? U : 1], const float (&sb)[PG && UP ? U : 1],
                       const uint4 (&xa)[U][MT][AV], int kb) {
 #pragma unroll
     for (int j = 0; j < U; ++j) {
@@ -176,9 +185,8 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p) 
           bf16x8 al, ah, bl, bh;
           widen_i8x16(wa[j], al, ah);
           if (UP) widen_i8x16(wb[j], bl, bh);
-          const int kg = (kb + j) / p.group_blocks;
-          const float s_a = psa[(size_t)kg * 16];
-          const float s_b = UP ? psb[(size_t)kg * 16] : 0.f;
+          const float s_a = sa[PG ? j : 0];
+          const float s_b = UP ? sb[PG && UP ? j : 0] : 0.f;
 #pragma unroll
           for (int i = 0; i < MT; ++i) {
             uint4 x0 = xa[j][i][0], x1 = xa[j][i][AV - 1];
@@ -219,15 +227,15 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p) 
   if (kb0 < kb1) load_x(xa0, kb0);
   for (int kb = kb0; kb < kb1; kb += 2 * U) {
     if (kb + U < kb1) {
-      load_w(wA1, wB1, kb + U);
+      load_w(wA1, wB1, sA1, sB1, kb + U);
       load_x(xa1, kb + U);
     }
-    multiply(wA0, wB0, xa0, kb);
+    multiply(wA0, wB0, sA0, sB0, xa0, kb);
     if (kb + 2 * U < kb1) {
-      load_w(wA0, wB0, kb + 2 * U);
+      load_w(wA0, wB0, sA0, sB0, kb + 2 * U);
       load_x(xa0, kb + 2 * U);
     }
-    if (kb + U < kb1) multiply(wA1, wB1, xa1, kb + U);
+    if (kb + U < kb1) multiply(wA1, wB1, sA1, sB1, xa1, kb + U);
   }
 
   // Reduce the four K-slices through LDS; wave 0 finishes.
@@ -510,6 +518,52 @@ __global__ void repack_blocks_kernel(const uint8_t* __restrict__ src, uint4* __r
   dst[slot] = *(const uint4*)buf;
 }
 }  // namespace
+
+namespace {
+// One thread converts one 16-byte lane slot of an int8 block (row r = lane % 16, 16 consecutive
+// k) into the two lane slots of the bf16 block layout that hold the same elements.
+__global__ void dequant_group_blocks_kernel(const uint4* __restrict__ q,
+                                            const float* __restrict__ scales,
+                                            uint4* __restrict__ out, int n_pad, int nkb8,
+                                            int group_blocks, int n_kgroups, size_t total) {
+  const size_t slot = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (slot >= total) return;
+  const int lane = (int)(slot & 63);
+  const size_t blk = slot >> 6;
+  const int kb = (int)(blk % nkb8);
+  const size_t strip = blk / nkb8;                 // g * (n_pad / 16) + nb
+  const int nb = (int)(strip % (n_pad / 16));
+  const size_t g = strip / (n_pad / 16);
+  const int row = nb * 16 + (lane & 15), q4 = lane >> 4;
+  const float sc = scales[(g * n_kgroups + kb / group_blocks) * n_pad + row];
+  const uint4 v = q[slot];
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+  uint32_t o[8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float f0 = (float)(int8_t)(w[i] & 0xff) * sc, f1 = (float)(int8_t)((w[i] >> 8) & 0xff) * sc;
+    const float f2 = (float)(int8_t)((w[i] >> 16) & 0xff) * sc, f3 = (float)(int8_t)(w[i] >> 24) * sc;
+    o[2 * i] = (uint32_t)bf16_rne(f0) | ((uint32_t)bf16_rne(f1) << 16);
+    o[2 * i + 1] = (uint32_t)bf16_rne(f2) | ((uint32_t)bf16_rne(f3) << 16);
+  }
+  // int8 block kb, k offset 16 * q4 -> bf16 block 2 kb + q4 / 2, k offsets 8 * (2 (q4 % 2) + h)
+  const size_t oblk = (strip * (size_t)(2 * nkb8) + (size_t)(2 * kb + (q4 >> 1))) * 64;
+  const int olane = (lane & 15) + 16 * (2 * (q4 & 1));
+  out[oblk + olane] = make_uint4(o[0], o[1], o[2], o[3]);
+  out[oblk + olane + 16] = make_uint4(o[4], o[5], o[6], o[7]);
+}
+}  // namespace
+
+hipError_t launch_dequant_group_blocks(const void* q_blocks, const float* scales, void* bf16_blocks,
+                                       int G, int n_pad, int k_pad, int group_blocks, int n_kgroups,
+                                       hipStream_t s) {
+  const int nkb8 = k_pad / kKbInt8;
+  const size_t total = (size_t)G * (n_pad / 16) * nkb8 * 64;
+  if (total == 0) return hipSuccess;
+  dequant_group_blocks_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(
+      (const uint4*)q_blocks, scales, (uint4*)bf16_blocks, n_pad, nkb8, group_blocks, n_kgroups, total);
+  return hipGetLastError();
+}
 
 hipError_t launch_repack_blocks(const void* src, void* dst, int n_rows, int k_cols, int n_pad,
                                 int k_pad, int elem_bytes, hipStream_t s) {

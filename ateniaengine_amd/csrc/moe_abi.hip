@@ -102,6 +102,10 @@ struct AteniaMoeLayer {
   int v3_n_group = 0, v3_topk_group = 0, v3_norm = 0;
   double v3_scale = 1.0;
   DevBuf v3_bias, logits;
+  // per-group int8: bf16 copies for the MFMA-tiled (prefill) kernels, made on first use
+  DevBuf pg_wg, pg_wu, pg_wd, pg_swg, pg_swu, pg_swd;
+  WeightSet gate_b{}, up_b{}, down_b{}, s_gate_b{}, s_up_b{}, s_down_b{};
+  bool pg_ready = false;
   int normed_T = 0;     // rows of xn the last block forward wrote
   int last_T = 0;
   int stage_T[4] = {-1, -1, -1, -1};  // token count each pipeline stage last completed for
@@ -202,9 +206,10 @@ int upload_f32(const float* host, size_t n, DevBuf& dst) {
   return ATENIA_MOE_OK;
 }
 
-// Per-group scales [G, n_rows, n_kgroups] (host) -> [G][n_pad / 16][n_kgroups][16] (device): the
-// 16 rows of a strip are adjacent for every k group, so a wavefront of the streaming kernel
-// fetches the scales of a group with one 64-byte read.  Rows past n_rows get scale 0.
+// Per-group scales [G, n_rows, n_kgroups] (host) -> [G][n_kgroups][n_pad] (device): for a fixed
+// k group the rows are adjacent, so the 16 rows of a strip are one 64-byte read for the
+// streaming kernel and a row tile is contiguous for the dequantising kernel.  Rows past n_rows
+// get scale 0.
 int upload_group_scales(const float* host, int G, int n_rows, int k_cols, int group_size,
                         DevBuf& dst, WeightSet& ws) {
   const int ng = (k_cols + group_size - 1) / group_size;
@@ -213,13 +218,28 @@ int upload_group_scales(const float* host, int G, int n_rows, int k_cols, int gr
   for (int g = 0; g < G; ++g)
     for (int n = 0; n < n_rows; ++n)
       for (int kg = 0; kg < ng; ++kg)
-        re[(((size_t)g * (n_pad / 16) + n / 16) * ng + kg) * 16 + n % 16] =
-            host[((size_t)g * n_rows + n) * ng + kg];
+        re[((size_t)g * ng + kg) * n_pad + n] = host[((size_t)g * n_rows + n) * ng + kg];
   int rc = upload_f32(re.data(), re.size(), dst);
   if (rc) return rc;
   ws.scale = dst.as<float>();
   ws.group_blocks = group_size / kKbInt8;
   ws.n_kgroups = ng;
+  return ATENIA_MOE_OK;
+}
+
+// bf16 copy of a per-group int8 family (made on the first batch that takes the MFMA-tiled
+// kernels): same rows and K padding, bf16 blocks, value = bf16(q * scale of its group).
+int make_bf16_copy(const WeightSet& q, int G, DevBuf& dst, WeightSet& out) {
+  out = q;
+  out.scale = nullptr;
+  out.group_blocks = 0;
+  out.n_kgroups = 0;
+  out.expert_stride = (int64_t)q.n_pad * q.k_pad * 2;  // bytes
+  int rc = dst.ensure((size_t)G * out.expert_stride);
+  if (rc) return rc;
+  out.w = dst.p;
+  HIP_TRY(launch_dequant_group_blocks(q.w, q.scale, dst.p, G, q.n_pad, q.k_pad, q.group_blocks,
+                                      q.n_kgroups, nullptr));
   return ATENIA_MOE_OK;
 }
 
@@ -389,8 +409,29 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   const void* a_x = f32w ? d_x : (need_xb ? (const void*)L->xb.p : d_x);
   const int a_stride = f32w ? L->d : L->d_kpad;
 
+  // Per-group int8 and a batch for the MFMA-tiled kernels: those take one scale per row, so the
+  // layer keeps a bf16 copy of its experts (q * group scale, rounded to bf16 -- the form the
+  // reference's GPU path multiplies with, src/cuda/int8_to_bf16.cu:91-110) for such batches;
+  // decode batches stream the int8 weights themselves.
+  const bool pg_prefill = L->group_size > 0 && T > stream_max_tokens() && L->d_kpad % 64 == 0 &&
+                          L->f_kpad % 64 == 0 && (L->fs == 0 || L->fs_kpad % 64 == 0);
+  if (pg_prefill && !L->pg_ready) {
+    int rc = make_bf16_copy(L->gate, L->E, L->pg_wg, L->gate_b);
+    if (!rc) rc = make_bf16_copy(L->up, L->E, L->pg_wu, L->up_b);
+    if (!rc) rc = make_bf16_copy(L->down, L->E, L->pg_wd, L->down_b);
+    if (!rc && L->fs > 0) {
+      rc = make_bf16_copy(L->s_gate, 1, L->pg_swg, L->s_gate_b);
+      if (!rc) rc = make_bf16_copy(L->s_up, 1, L->pg_swu, L->s_up_b);
+      if (!rc) rc = make_bf16_copy(L->s_down, 1, L->pg_swd, L->s_down_b);
+    }
+    if (rc) return rc;
+    HIP_TRY(hipDeviceSynchronize());
+    L->pg_ready = true;
+  }
+  const int ffn_dtype = pg_prefill ? ATENIA_MOE_WEIGHT_BF16 : L->wdtype;
+
   FfnArgs fa{};
-  fa.wdtype = L->wdtype;
+  fa.wdtype = ffn_dtype;
   fa.g.offsets = L->offsets.as<int32_t>();
   fa.g.active = L->active.as<int32_t>();
   fa.g.n_active = L->n_active.as<int32_t>();
@@ -398,9 +439,9 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   fa.g.pair_div = L->k;
   fa.n_groups_max = (int)std::min<long long>(L->E, (long long)T * L->k);
   fa.rows_max = T;
-  fa.gate = L->gate;
-  fa.up = L->up;
-  fa.down = L->down;
+  fa.gate = pg_prefill ? L->gate_b : L->gate;
+  fa.up = pg_prefill ? L->up_b : L->up;
+  fa.down = pg_prefill ? L->down_b : L->down;
   fa.x = a_x;
   fa.x_stride = a_stride;
   fa.h = L->h.p;
@@ -409,15 +450,15 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   fa.y_stride = L->d;
   // Tiled (MFMA-bound) kernels once an expert can see more rows than the streaming kernel
   // keeps in registers; below that the weights are streamed once (HBM-bound).
-  const bool tiled = T > stream_max_tokens() && tiled_supported(L->gate, L->wdtype) &&
-                     tiled_supported(L->down, L->wdtype);
+  const bool tiled = T > stream_max_tokens() && tiled_supported(fa.gate, ffn_dtype) &&
+                     tiled_supported(fa.down, ffn_dtype);
   fa.use_tiled = tiled;
   fa.tile_group = L->tile_group.as<int32_t>();
   fa.tile_m0 = L->tile_m0.as<int32_t>();
   fa.n_tiles = L->shared_desc.as<int32_t>() + 4;
   fa.max_row_tiles = (int)(((size_t)T * L->k + kTileM - 1) / kTileM +
                            std::min<long long>(L->E, (long long)T * L->k));
-  const bool split_tail = tiled && tiled_down_splits_tail(L->down, L->wdtype);
+  const bool split_tail = tiled && tiled_down_splits_tail(fa.down, ffn_dtype);
   fa.y_parts = split_tail ? kMaxYParts : 1;
   fa.y_part_stride = (size_t)T * L->k * L->d;
   fa.part_flags = split_tail ? L->part_flags.as<uint8_t>() : nullptr;
@@ -435,16 +476,16 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
     fsd.g.pair_div = 1;
     fsd.n_groups_max = 1;
     fsd.rows_max = T;
-    fsd.gate = L->s_gate;
-    fsd.up = L->s_up;
-    fsd.down = L->s_down;
+    fsd.gate = pg_prefill ? L->s_gate_b : L->s_gate;
+    fsd.up = pg_prefill ? L->s_up_b : L->s_up;
+    fsd.down = pg_prefill ? L->s_down_b : L->s_down;
     fsd.h = L->hs.p;
     fsd.h_stride = L->fs_kpad;
     fsd.y = L->ys.as<float>();
     fsd.y_parts = 1;
     fsd.part_flags = nullptr;
-    fsd.use_tiled = T > stream_max_tokens() && tiled_supported(L->s_gate, L->wdtype) &&
-                    tiled_supported(L->s_down, L->wdtype);
+    fsd.use_tiled = T > stream_max_tokens() && tiled_supported(fsd.gate, ffn_dtype) &&
+                    tiled_supported(fsd.down, ffn_dtype);
     fsd.tile_group = L->s_tile_group.as<int32_t>();
     fsd.tile_m0 = L->s_tile_m0.as<int32_t>();
     fsd.n_tiles = L->shared_desc.as<int32_t>() + 5;

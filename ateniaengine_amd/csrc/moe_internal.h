@@ -39,7 +39,7 @@ struct GroupDesc {
 struct WeightSet {
   const void* w;            // blocks (bf16/int8) or row-major f32
   const float* scale;       // int8: per output row, [G, N] (unpadded N stride = n_rows);
-                            // per-group int8: [G][n_pad / 16][n_kgroups][16] (see group_blocks)
+                            // per-group int8: [G][n_kgroups][n_pad] (see group_blocks)
   int group_blocks;         // per-group int8: 64-k blocks per scale group (0 = one scale per row)
   int n_kgroups;            // per-group int8: scale groups along K
   int64_t expert_stride;    // elements (f32) or bytes (blocked) between experts
@@ -185,5 +185,10 @@ hipError_t launch_rmsnorm_gamma(const NormArgs& a, hipStream_t s);
 hipError_t launch_repack_blocks(const void* src, void* dst, int n_rows, int k_cols, int n_pad,
                                 int k_pad, int elem_bytes, hipStream_t s);
 hipError_t launch_fill_i32(int32_t* p, int n, int32_t v, int32_t step, hipStream_t s);
+// Per-group int8 blocks + scales [G][n_kgroups][n_pad] -> bf16 blocks of the same matrix:
+// value = bf16_rne((float)q * scale[row, k group]).
+hipError_t launch_dequant_group_blocks(const void* q_blocks, const float* scales, void* bf16_blocks,
+                                       int G, int n_pad, int k_pad, int group_blocks, int n_kgroups,
+                                       hipStream_t s);
 
 }  // namespace atenia_moe

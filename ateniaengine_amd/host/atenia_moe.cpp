@@ -381,9 +381,20 @@ int pack(const std::vector<const std::vector<float>*>& mats, size_t rows, size_t
     }
     return 0;
   }
+  if (s == MoeWeightStorage::Int8PerGroup) {  // quantizer.rs:175-248 along each row
+    const size_t ng = (cols + kInt8GroupSize - 1) / kInt8GroupSize;
+    out.i8.resize(n * per);
+    out.scale.resize(n * rows * ng);
+    for (size_t i = 0; i < n; ++i) {
+      int rc = atenia_moe_quantize_per_group_i8(mats[i]->data(), rows, cols, kInt8GroupSize,
+                                                &out.i8[i * per], &out.scale[i * rows * ng]);
+      if (rc) return rc;
+    }
+    return 0;
+  }
   out.i8.resize(n * per);  // per output row (disk_tier.rs:231-248)
   out.scale.resize(n * rows);
-  bool have_pre = pre.size() == n;
+  bool have_pre = pre.size() == n && s == MoeWeightStorage::Int8W8A16;
   for (size_t i = 0; have_pre && i < n; ++i)
     have_pre = pre[i] && pre[i]->rows == rows && pre[i]->cols == cols;
   for (size_t i = 0; i < n; ++i) {
@@ -440,7 +451,9 @@ Result<void*, MoeLayerError> RealMoeLayer::handle_for(MoeExecutionConvention con
   desc.w_gate = pg.data(storage);
   desc.w_up = pu.data(storage);
   desc.w_down = pd.data(storage);
-  if (storage == MoeWeightStorage::Int8W8A16) {
+  const bool int8 = storage == MoeWeightStorage::Int8W8A16 || storage == MoeWeightStorage::Int8PerGroup;
+  if (storage == MoeWeightStorage::Int8PerGroup) desc.group_size = (int32_t)kInt8GroupSize;
+  if (int8) {
     desc.scale_gate = pg.scale.data();
     desc.scale_up = pu.scale.data();
     desc.scale_down = pd.scale.data();
@@ -455,7 +468,7 @@ Result<void*, MoeLayerError> RealMoeLayer::handle_for(MoeExecutionConvention con
     desc.s_gate = sg.data(storage);
     desc.s_up = su.data(storage);
     desc.s_down = sd.data(storage);
-    if (storage == MoeWeightStorage::Int8W8A16) {
+    if (int8) {
       desc.s_scale_gate = sg.scale.data();
       desc.s_scale_up = su.scale.data();
       desc.s_scale_down = sd.scale.data();

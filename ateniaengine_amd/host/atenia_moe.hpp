@@ -160,7 +160,10 @@ struct V3RouterConfig {  // src/moe/v3_router.rs:59-72
 };
 
 // How the layer's expert weights are stored in HBM.
-enum class MoeWeightStorage { F32 = 0, Bf16 = 1, Int8W8A16 = 2 };
+// Int8PerGroup: one scale per output row and group of kInt8GroupSize input elements (the
+// reference's per-group scheme, src/tensor/quantizer.rs:175-248).
+enum class MoeWeightStorage { F32 = 0, Bf16 = 1, Int8W8A16 = 2, Int8PerGroup = 3 };
+constexpr size_t kInt8GroupSize = 128;
 
 // A per-output-row symmetric int8 weight [rows, cols]: w[r, c] = q[r, c] * scales[r]
 // (src/tensor/disk_tier.rs:225-262; the payload of the reference's qint8 tier files).

@@ -29,6 +29,9 @@ CONFIGS = {
                          zipf=False, sweep=(1, 16, 128, 512, 4096)),
     "mixtral_int8": dict(d=4096, E=8, k=2, f=14336, fs=0, gated=False, conv=0, wd="int8",
                          zipf=False, sweep=(1, 16, 4096)),
+    # per-group int8 (one scale per output row and 128 input elements, Q8_0-style)
+    "mixtral_int8g": dict(d=4096, E=8, k=2, f=14336, fs=0, gated=False, conv=0, wd="int8g",
+                          zipf=False, sweep=(1, 16, 4096)),
     "qwen_bf16": dict(d=2048, E=60, k=4, f=1408, fs=5632, gated=True, conv=1, wd="bf16",
                       zipf=False, sweep=(1, 256, 8192)),
     "deepseek_bf16": dict(d=2048, E=64, k=6, f=1408, fs=2816, gated=False, conv=1, wd="bf16",
@@ -42,6 +45,7 @@ CONFIGS = {
 D_MODEL, N_EXPERTS, TOP_K, D_FF = 4096, 8, 2, 14336
 D_FF_SHARED = 0
 W_BYTES = 2
+GROUP = 0  # per-group int8: input elements per scale
 W_STD = 0.02
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, GB/s
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, TFLOP/s
@@ -123,12 +127,16 @@ def measure(torch, np, capi, layer, T, steps, warmup, seed):
     U = active / steps  # experts with at least one token (mean over steps)
 
     eb = W_BYTES  # bytes per stored weight
-    sc = 4 if W_BYTES == 1 else 0  # int8: one f32 scale per output row
+    # int8: one f32 scale per output row, or per output row and group of GROUP input elements
+    sc_up = (4 * (-(-D_MODEL // GROUP) if GROUP else 1)) if W_BYTES == 1 else 0
+    sc_down = (4 * (-(-D_FF // GROUP) if GROUP else 1)) if W_BYTES == 1 else 0
+    sc_sdown = (4 * (-(-D_FF_SHARED // GROUP) if GROUP and D_FF_SHARED else 1)) if W_BYTES == 1 else 0
     fs = D_FF_SHARED
     # the shared expert (if any) runs as a second launch of the same kernels; both launches
     # of a stage are timed together, so their bytes / flops are added together too
-    bytes_up = U * (2 * D_FF * D_MODEL * eb + 2 * D_FF * sc) + 2 * fs * D_MODEL * eb + 2 * fs * sc
-    bytes_down = U * (D_MODEL * D_FF * eb + D_MODEL * sc) + fs * D_MODEL * eb + (D_MODEL * sc if fs else 0)
+    bytes_up = U * (2 * D_FF * D_MODEL * eb + 2 * D_FF * sc_up) + 2 * fs * D_MODEL * eb + 2 * fs * sc_up
+    bytes_down = (U * (D_MODEL * D_FF * eb + D_MODEL * sc_down) + fs * D_MODEL * eb +
+                  (D_MODEL * sc_sdown if fs else 0))
     bytes_fwd = bytes_up + bytes_down + N_EXPERTS * D_MODEL * 4 + T * D_MODEL * (2 + 4)
     P = T * TOP_K
     flops_up = 4.0 * P * D_MODEL * D_FF + 4.0 * T * D_MODEL * fs
@@ -235,11 +243,12 @@ def main():
         print("bench.py: no gfx950 device; the HIP path has no fallback", file=sys.stderr)
         sys.exit(3)
     torch.cuda.set_device(0)
-    global D_MODEL, N_EXPERTS, TOP_K, D_FF, D_FF_SHARED, W_BYTES, CONFIG_NAME
+    global D_MODEL, N_EXPERTS, TOP_K, D_FF, D_FF_SHARED, W_BYTES, CONFIG_NAME, GROUP
     cfg = CONFIGS[a.config]
     CONFIG_NAME = a.config
     D_MODEL, N_EXPERTS, TOP_K, D_FF, D_FF_SHARED = cfg["d"], cfg["E"], cfg["k"], cfg["f"], cfg["fs"]
-    W_BYTES = 1 if cfg["wd"] == "int8" else 2
+    W_BYTES = 1 if cfg["wd"] in ("int8", "int8g") else 2
+    GROUP = 128 if cfg["wd"] == "int8g" else 0
     if a.tokens <= 0:
         a.tokens = max(cfg["sweep"])
     if a.sweep == "all":
@@ -256,22 +265,26 @@ def main():
         kw["router_bias"] = (-1.2 * np.log(rank)).astype(np.float32)
     if shared is not None and cfg["gated"]:
         kw["shared_gate"] = shared[3]
-    if cfg["wd"] == "int8":
-        # per-output-row int8 of the bf16-valued weights, 0.1 % of rows scaled x8 first
+    if cfg["wd"] in ("int8", "int8g"):
+        # int8 of the bf16-valued weights (per output row, or per row and 128-element group),
+        # 0.1 % of rows scaled x8 first
         rng = np.random.default_rng(a.seed + 1)
+        per_group = cfg["wd"] == "int8g"
+        if per_group:
+            kw["group_size"] = 128
 
         def q8(bits):
             w = upcast(np, bits)
             rows = w.reshape(-1, w.shape[-1])
             rows[rng.choice(rows.shape[0], size=rows.shape[0] // 1000, replace=False)] *= 8.0
-            return capi.quantize_per_row_i8(w)
+            return capi.quantize_per_group_i8(w, 128) if per_group else capi.quantize_per_row_i8(w)
         (gate, sg), (up, su), (down, sd) = q8(gate), q8(up), q8(down)
         kw.update(scale_gate=sg, scale_up=su, scale_down=sd)
         if shared is not None:
             (g_, a1), (u_, a2), (d_, a3) = q8(shared[0]), q8(shared[1]), q8(shared[2])
             shared = (g_, u_, d_, shared[3])
             kw.update(s_scale_gate=a1, s_scale_up=a2, s_scale_down=a3)
-        wdt = capi.WEIGHT_INT8_W8A16
+        wdt = capi.WEIGHT_INT8_PER_GROUP if per_group else capi.WEIGHT_INT8_W8A16
     else:
         wdt = capi.WEIGHT_BF16
     if shared is not None:

@@ -363,6 +363,9 @@ int main(int argc, char** argv) {
     auto i8 = layer_from(*mix, MoeWeightStorage::Int8W8A16).forward_auto(mix->input).unwrap();
     CHECK(metrics(b16, f32).max_abs_diff <= 3e-2 * scale, "bf16 storage: %g of %g", metrics(b16, f32).max_abs_diff, scale);
     CHECK(metrics(i8, f32).max_abs_diff <= 3e-2 * scale, "int8 storage: %g of %g", metrics(i8, f32).max_abs_diff, scale);
+    auto i8g = layer_from(*mix, MoeWeightStorage::Int8PerGroup).forward_auto(mix->input).unwrap();
+    CHECK(metrics(i8g, f32).max_abs_diff <= 3e-2 * scale, "per-group int8 storage: %g of %g",
+          metrics(i8g, f32).max_abs_diff, scale);
   });
   printf("%d tests, %d failed\n", g_run, g_failed);
   return g_failed ? 1 : 0;

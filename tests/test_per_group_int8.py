@@ -70,7 +70,7 @@ def test_library_quantiser_equals_the_oracle_on_the_transpose(ora, rows, cols, g
 # ---- the layer on the GPU ---------------------------------------------------------------------
 @pytest.mark.gpu
 @pytest.mark.parametrize("gs", [64, 128])
-@pytest.mark.parametrize("T", [1, 16, 33, 150])
+@pytest.mark.parametrize("T", [1, 16, 33, 150, 700])
 def test_per_group_layer_against_oracle_on_dequantised_weights(ora, T, gs):
     d, f = 384, 640
     W = S.make_weights(60 + T, 8, d, f, f_s=256, gated=True, router_std=1.0 / np.sqrt(d), outlier_frac=0.002)
