@@ -567,7 +567,8 @@ __global__ __launch_bounds__(kTokenThreads) void router_token_kernel(
 
   // Work items: (row, k slice).  With few rows each row is split over several waves so that
   // all 16 waves stream the router matrix.  Partial results meet in LDS; under the exactness
-  // certificate their order of addition cannot change the sum.
+  // certificate their order of addition cannot change the sum (or, under the interval
+  // certificate below, cannot change what the sum rounds to).
   const int KS = R >= NW ? 1 : NW / R;              // k slices per row
   const int slice = ((d + KS - 1) / KS + 3) & ~3;   // multiple of 4 for float4 loads
   const bool vec_ok = (d & 3) == 0;
@@ -622,6 +623,24 @@ __global__ __launch_bounds__(kTokenThreads) void router_token_kernel(
     // Exact in every order iff sum|p| < 2^(q+53); asum itself carries a relative error of
     // at most d * 2^-53, covered by the margin.
     bool exact = qmin == kNoLsb || (qmin > -2000 && asum * 1.000001 < ldexp(1.0, qmin + 53));
+    if (!exact) {
+      // Second certificate, for operands that are not exact in every order (f32-valued rows):
+      // any order of d exact products summed in f64 lands within g = d * 2^-53 * sum|p| of the
+      // true sum (standard bound, 1 / (1 - d u) absorbed by the margin), so this sum and the
+      // reference's sequential one differ by at most 2 g.  If both ends of [acc - 2g, acc + 2g]
+      // round to the same f32 (the same f32 sigmoid for the gate row), the reference's result is
+      // that value, whatever its order.  Rounding is monotone; the two extra units of 2^-53
+      // cover the roundings of acc -/+ e themselves.
+      const double e = asum * ((double)(2 * d + 4) * 1.1102230246251565e-16) * 1.0001;
+      const double lo = acc - e, hi = acc + e;
+      if (row_lo + tid < E) {
+        const float flo = (float)lo, fhi = (float)hi;
+        exact = flo == fhi && isfinite(flo);
+      } else {
+        const float glo = (float)(1.0 / (1.0 + exp(-lo))), ghi = (float)(1.0 / (1.0 + exp(-hi)));
+        exact = glo == ghi;
+      }
+    }
     sAcc[tid] = acc;
     if (!exact) *sBad = 1;
   }

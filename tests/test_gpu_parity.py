@@ -383,3 +383,24 @@ def test_combine_is_bit_exact_given_expert_outputs(ora, wd, T, shared):
             if shared:
                 o = o + ys[t]
             assert out[t].tobytes() == o.tobytes()
+
+
+@pytest.mark.parametrize("E,k,d,T,gated", [(8, 2, 4096, 512, False), (60, 4, 2048, 300, True),
+                                           (64, 6, 1024, 97, False)])
+def test_router_f32_valued_rows_on_blocked_layers(ora, E, k, d, T, gated):
+    """f32-valued activations on a bf16 layer (what a reference caller hands over): sums of such
+    products are not exact in every order, so the per-token kernel either proves that its sum and
+    the reference's sequential one round to the same f32 (interval certificate) or recomputes
+    sequentially.  Routing must equal the oracle's for every token either way."""
+    W = S.make_weights(E + d, E, d, 16, f_s=16 if gated else 0, gated=gated,
+                       router_std=1.0 / np.sqrt(d))
+    conv = capi.CONVENTION_HUGGINGFACE_QWEN if gated else capi.CONVENTION_ATENIA
+    oL, gL = S.build_pair(ora, W, k, conv, capi.WEIGHT_BF16)
+    rng = np.random.default_rng(T)
+    x = rng.standard_normal((T, d)).astype(np.float32)
+    x *= np.exp2(rng.integers(-3, 4, size=(T, 1))).astype(np.float32)
+    with gL:
+        idx, w = gL.route(x)
+        o_idx, o_w = oL.route_tokens(x)
+        assert (idx == o_idx).all(), f"{(idx != o_idx).any(axis=1).sum()} tokens routed differently"
+        assert ulp_diff(w, o_w).max() <= 1
