@@ -364,9 +364,12 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   pa.shared_n_tiles = L->shared_desc.as<int32_t>() + 5;
   ra.fuse_permute = last >= kStagePermute ? &pa : nullptr;
   const bool v3 = L->v3_n_group > 0;
-  if (v3) {
+  if (v3 || L->E > 31) {
     int rc = L->logits.ensure((size_t)L->cap_tokens * L->E * 4);
     if (rc) return rc;
+    ra.logits_tmp = L->logits.as<float>();
+  }
+  if (v3) {
     ra.logits_out = L->logits.as<float>();
     ra.shared_gate = nullptr;  // the V3 block adds its shared experts ungated
   }

@@ -70,6 +70,9 @@ struct RouterArgs {
   const struct PermuteArgs* fuse_permute;  // null = do not fuse
   // non-null: write the raw logits [T, E] here and leave idx / w alone (another kernel routes)
   float* logits_out;
+  // scratch [T, E] the launcher may use to split the work of few tokens over more workgroups
+  // (null = none)
+  float* logits_tmp;
 };
 // *fused_permute is set to 1 when the launch also produced the expert grouping.
 hipError_t launch_router(const RouterArgs& a, hipStream_t s, int* fused_permute);

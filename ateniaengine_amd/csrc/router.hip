@@ -523,6 +523,56 @@ struct FusedGrouping {
   int32_t *tile_group, *tile_m0, *n_tiles, *shared_n_tiles;
 };
 
+// The expert grouping of ONE token from its selection flags (what kernel 2 would produce).
+__device__ inline void write_single_token_grouping(const FusedGrouping& fg, const int32_t* sel,
+                                                   int E, int k) {
+  int run = 0;
+  for (int e = 0; e < E; ++e) {
+    const int c = sel[e] ? 1 : 0;
+    fg.counts[e] = c;
+    fg.offsets[e] = run;
+    if (c && run < k) {
+      fg.active[run] = e;
+      fg.perm[run] = run;
+      fg.inv[run] = run;
+      fg.tile_group[run] = e;
+      fg.tile_m0[run] = 0;
+      ++run;
+    }
+  }
+  fg.offsets[E] = run;
+  *fg.n_active = run;
+  *fg.n_tiles = run;
+  *fg.shared_n_tiles = 1;
+  fg.shared_offsets[0] = 0;
+  fg.shared_offsets[1] = 1;
+}
+
+// Softmax + top-k from logits that another launch left in HBM: used when the rows of the
+// router matrix were spread over several workgroups per token (many experts, few tokens), so
+// no single workgroup holds all logits of a token.  256 / E tokens per workgroup.
+constexpr int kSelectThreads = 256;
+__global__ __launch_bounds__(kSelectThreads) void softmax_select_kernel(
+    const float* __restrict__ logits, int T, int E, int k, int renorm,
+    int32_t* __restrict__ idx_out, float* __restrict__ w_out, int32_t* __restrict__ status,
+    FusedGrouping fg) {
+  __shared__ double sExp[kSelectThreads];
+  __shared__ float sWt[kSelectThreads];
+  __shared__ int32_t sSel[kSelectThreads];
+  const int TT = kSelectThreads / E;
+  const int tid = threadIdx.x;
+  const int tl = tid / E, r = tid - tl * E;
+  const int t = blockIdx.x * TT + tl;
+  const bool on = tl < TT && t < T;
+  const int ts = on ? t : 0, ls = on ? tl : 0;
+  softmax_topk(on, r, E, k, renorm, ts, logits + (size_t)ts * E, sExp + ls * E, sWt + ls * E,
+               sSel + ls * E, idx_out, w_out, status);
+  if (fg.counts) {  // T == 1
+    __syncthreads();
+    if (tid == 0) write_single_token_grouping(fg, sSel, E, k);
+  }
+}
+
 template <typename XT>
 __global__ __launch_bounds__(kTokenThreads) void router_token_kernel(
     const XT* __restrict__ x, int T, int d, int E, int k, int renorm,
@@ -672,28 +722,7 @@ __global__ __launch_bounds__(kTokenThreads) void router_token_kernel(
   softmax_topk(tid < E, tid, E, k, renorm, t, sLogit, sExp, sWt, sSel, idx_out, w_out, status);
   if (fg.counts) {  // T == 1: the grouping of a single token follows from its top-k
     __syncthreads();
-    if (tid == 0) {
-      int run = 0;
-      for (int e = 0; e < E; ++e) {
-        const int c = sSel[e] ? 1 : 0;
-        fg.counts[e] = c;
-        fg.offsets[e] = run;
-        if (c && run < k) {
-          fg.active[run] = e;
-          fg.perm[run] = run;
-          fg.inv[run] = run;
-          fg.tile_group[run] = e;
-          fg.tile_m0[run] = 0;
-          ++run;
-        }
-      }
-      fg.offsets[E] = run;
-      *fg.n_active = run;
-      *fg.n_tiles = run;
-      *fg.shared_n_tiles = 1;
-      fg.shared_offsets[0] = 0;
-      fg.shared_offsets[1] = 1;
-    }
+    if (tid == 0) write_single_token_grouping(fg, sSel, E, k);
   }
 }
 
@@ -712,6 +741,13 @@ hipError_t launch_router(const RouterArgs& a, hipStream_t s, int* fused_permute)
     size_t smem = ((size_t)R + a.E + 2 * np) * 8 + (size_t)a.d * 4 + (size_t)a.E * 12 + 4 +
                   np * 4 + (size_t)a.d * 2 + 16;
     if (smem <= 64 * 1024) {
+      // Many rows, few tokens: one workgroup per token would stream the whole stacked matrix
+      // through a single CU.  The rows are spread over workgroups instead (four rows each, a
+      // row split over four waves), the logits go to HBM, and the selection runs as a second,
+      // tiny launch -- the caller's own one (logits_out) or softmax_select_kernel here.
+      const bool spread = R > 32 && (a.logits_out || (a.logits_tmp && a.T <= 32 &&
+                                                      a.E <= kSelectThreads));
+      float* lg = a.logits_out ? a.logits_out : (spread ? a.logits_tmp : nullptr);
       FusedGrouping fg{};
       if (a.T == 1 && a.fuse_permute && !a.logits_out) {
         const PermuteArgs& pa = *a.fuse_permute;
@@ -720,19 +756,24 @@ hipError_t launch_router(const RouterArgs& a, hipStream_t s, int* fused_permute)
                            pa.shared_n_tiles};
         if (fused_permute) *fused_permute = 1;
       }
-      // Four rows per workgroup (a row split over four waves) once the rows can be spread over
-      // workgroups, i.e. when the logits leave the kernel: the few tokens this kernel serves
-      // then keep R / 4 workgroups streaming the router matrix instead of one.
-      const int row_blocks = a.logits_out && R > 32 ? (R + 3) / 4 : 1;
+      const FusedGrouping fg_token = spread ? FusedGrouping{} : fg;
+      const int row_blocks = spread ? (R + 3) / 4 : 1;
       const dim3 grid(a.T, row_blocks);
       if (a.x_is_bf16)
         router_token_kernel<uint16_t><<<grid, kTokenThreads, smem, s>>>(
             (const uint16_t*)a.x, a.T, a.d, a.E, a.k, a.renorm, a.w_router, a.router_bias,
-            a.shared_gate, a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status, a.logits_out, fg);
+            a.shared_gate, a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status, lg, fg_token);
       else
         router_token_kernel<float><<<grid, kTokenThreads, smem, s>>>(
             (const float*)a.x, a.T, a.d, a.E, a.k, a.renorm, a.w_router, a.router_bias,
-            a.shared_gate, a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status, a.logits_out, fg);
+            a.shared_gate, a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status, lg, fg_token);
+      if (spread && !a.logits_out) {
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        const int TT = kSelectThreads / a.E;
+        softmax_select_kernel<<<(a.T + TT - 1) / TT, kSelectThreads, 0, s>>>(
+            lg, a.T, a.E, a.k, a.renorm, a.idx, a.w, a.status, fg);
+      }
       return hipGetLastError();
     }
   }

@@ -55,9 +55,9 @@ CONFIG_NAME = "mixtral_bf16"
 # (FETCH_SIZE counts 2 KiB units, WRITE_SIZE KiB): profiles/
 # ffn_kernels_mixtral_bf16_T4096_T1_hbm_counters.txt.  Keyed by (config, tokens per step).
 MEASURED_HBM_TRAFFIC = {
-    ("mixtral_bf16", 4096): {"expert_gate_up": 2537805.9 * 2048 + 229376.0 * 1024,
-                             "expert_down": 1262351.6 * 2048 + 169317.5 * 1024},
-    ("mixtral_bf16", 1): {"expert_gate_up": 229446.8 * 2048, "expert_down": 114935.2 * 2048},
+    ("mixtral_bf16", 4096): {"expert_gate_up": 2545230.2 * 2048 + 229376.0 * 1024,
+                             "expert_down": 1262441.1 * 2048 + 169318.0 * 1024},
+    ("mixtral_bf16", 1): {"expert_gate_up": 229446.8 * 2048, "expert_down": 114941.2 * 2048},
 }
 
 
