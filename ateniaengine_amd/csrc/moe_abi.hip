@@ -143,7 +143,7 @@ int stream_max_tokens() {
   static const int v = [] {
     const char* e = getenv("ATENIA_MOE_STREAM_MAX_TOKENS");
     int n = e ? atoi(e) : 0;
-    return n > 0 ? n : 32;
+    return n > 0 ? n : 48;
   }();
   return v;
 }

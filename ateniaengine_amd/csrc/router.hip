@@ -782,6 +782,19 @@ hipError_t launch_router(const RouterArgs& a, hipStream_t s, int* fused_permute)
     return a.x_is_bf16 ? dispatch_router_batch<uint16_t>(a, R, s)
                        : dispatch_router_batch<float>(a, R, s);
   }
+  // More than 64 rows with softmax routing: the same row-block launch into the scratch logits,
+  // then the selection as a second launch.
+  if (a.logits_tmp && a.E <= kSelectThreads && a.d % 4 == 0 && (!a.xb || a.d_pad % 4 == 0)) {
+    RouterArgs b = a;
+    b.logits_out = a.logits_tmp;
+    hipError_t e = a.x_is_bf16 ? dispatch_router_batch<uint16_t>(b, R, s)
+                               : dispatch_router_batch<float>(b, R, s);
+    if (e != hipSuccess) return e;
+    const int TT = kSelectThreads / a.E;
+    softmax_select_kernel<<<(a.T + TT - 1) / TT, kSelectThreads, 0, s>>>(
+        a.logits_tmp, a.T, a.E, a.k, a.renorm, a.idx, a.w, a.status, FusedGrouping{});
+    return hipGetLastError();
+  }
   int TT = kRouterThreads / R;
   if (TT < 1) TT = 1;
   // Keep enough blocks in flight for small batches.

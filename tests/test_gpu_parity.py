@@ -88,6 +88,12 @@ def test_golden_qwen_decomp_router(ora):
 
 # ---- router: bit-exact indices ---------------------------------------------------------
 ROUTER_CASES = [
+    # more than 64 rows with softmax routing: row blocks + selection launch at every batch size
+    (128, 8, 512, 1, 0, True, False, False),
+    (128, 8, 512, 40, 0, True, False, False),
+    (128, 8, 512, 700, 0, True, False, False),
+    (160, 6, 256, 3000, 1, True, False, True),
+    (100, 4, 260, 900, 0, False, False, False),
     # E, k, d, T, conv, bf16-valued inputs, bias, gated shared
     (8, 2, 1024, 64, 0, False, False, False),
     (8, 2, 4096, 33, 0, True, False, False),
