@@ -46,6 +46,7 @@ D_MODEL, N_EXPERTS, TOP_K, D_FF = 4096, 8, 2, 14336
 D_FF_SHARED = 0
 W_BYTES = 2
 GROUP = 0  # per-group int8: input elements per scale
+GRAPH = False  # --graph: also time small batches replayed from HIP graphs
 W_STD = 0.02
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, GB/s
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, TFLOP/s
@@ -109,6 +110,29 @@ def measure(torch, np, capi, layer, T, steps, warmup, seed):
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
 
+    # The same steps replayed from HIP graphs (one per input buffer), as a serving loop would
+    # issue them: no per-launch host work between the kernels of a step.
+    graph_ms = None
+    if GRAPH and T <= 64:
+        side = torch.cuda.Stream()
+        graphs = []
+        with torch.cuda.stream(side):
+            for i in range(n_buf):
+                g_ = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g_, stream=side):
+                    layer.forward_device(xs[i].data_ptr(), capi.ACT_BF16, T, out.data_ptr(),
+                                         torch.cuda.current_stream().cuda_stream)
+                graphs.append(g_)
+        torch.cuda.synchronize()
+        for i in range(warmup):
+            graphs[i % n_buf].replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            graphs[i % n_buf].replay()
+        torch.cuda.synchronize()
+        graph_ms = (time.perf_counter() - t0) * 1e3 / steps
+
     # Per-stage durations: HIP events recorded by the library on the launch stream.
     layer.set_profiling(True)
     acc = np.zeros(capi.N_STAGES, dtype=np.float64)
@@ -144,6 +168,7 @@ def measure(torch, np, capi, layer, T, steps, warmup, seed):
     flops_fwd = T * (2.0 * D_MODEL * N_EXPERTS + 6.0 * TOP_K * D_MODEL * D_FF + 6.0 * D_MODEL * fs)
     r = dict(
         tokens=T, ms_per_step=wall_ms, tokens_per_s=T / (wall_ms * 1e-3),
+        graph_replay_ms_per_step=graph_ms,
         active_experts=U,
         stage_ms={n: float(v) for n, v in zip(capi.STAGES, stage_ms)},
         stage_launches={n: int(v) for n, v in zip(capi.STAGES, launches)},
@@ -225,6 +250,8 @@ def main():
                     help="tokens of the CPU-baseline sample (0 = skip)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (reference point for HBM counters)")
+    ap.add_argument("--graph", action="store_true",
+                    help="also time batches of up to 64 tokens replayed from HIP graphs")
     ap.add_argument("--block", action="store_true",
                     help="also time the decoder-layer FFN block entry point (norm + layer + residual)")
     ap.add_argument("--seed", type=int, default=1234)
@@ -243,7 +270,8 @@ def main():
         print("bench.py: no gfx950 device; the HIP path has no fallback", file=sys.stderr)
         sys.exit(3)
     torch.cuda.set_device(0)
-    global D_MODEL, N_EXPERTS, TOP_K, D_FF, D_FF_SHARED, W_BYTES, CONFIG_NAME, GROUP
+    global D_MODEL, N_EXPERTS, TOP_K, D_FF, D_FF_SHARED, W_BYTES, CONFIG_NAME, GROUP, GRAPH
+    GRAPH = a.graph
     cfg = CONFIGS[a.config]
     CONFIG_NAME = a.config
     D_MODEL, N_EXPERTS, TOP_K, D_FF, D_FF_SHARED = cfg["d"], cfg["E"], cfg["k"], cfg["f"], cfg["fs"]

@@ -59,3 +59,65 @@ class DeviceArray:
             self.free()
         except Exception:
             pass
+
+
+class Stream:
+    """A HIP stream created through the runtime (default priority)."""
+
+    def __init__(self):
+        h = hip()
+        h.hipStreamCreate.argtypes = [C.POINTER(C.c_void_p)]
+        h.hipStreamDestroy.argtypes = [C.c_void_p]
+        h.hipStreamSynchronize.argtypes = [C.c_void_p]
+        p = C.c_void_p()
+        rc = h.hipStreamCreate(C.byref(p))
+        if rc:
+            raise RuntimeError(f"hipStreamCreate failed: {rc}")
+        self.ptr = p.value
+
+    def synchronize(self):
+        rc = hip().hipStreamSynchronize(self.ptr)
+        if rc:
+            raise RuntimeError(f"hipStreamSynchronize failed: {rc}")
+
+    def close(self):
+        if self.ptr:
+            hip().hipStreamDestroy(self.ptr)
+            self.ptr = None
+
+
+class Graph:
+    """Capture of the work launched on a stream between begin() and end(), replayable."""
+
+    def __init__(self, stream):
+        h = hip()
+        h.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+        h.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+        h.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_void_p,
+                                          C.c_size_t]
+        h.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+        h.hipGraphExecDestroy.argtypes = [C.c_void_p]
+        h.hipGraphDestroy.argtypes = [C.c_void_p]
+        self.stream, self.graph, self.exe = stream, C.c_void_p(), C.c_void_p()
+
+    def begin(self):
+        rc = hip().hipStreamBeginCapture(self.stream.ptr, 0)  # hipStreamCaptureModeGlobal
+        if rc:
+            raise RuntimeError(f"hipStreamBeginCapture failed: {rc}")
+
+    def end(self):
+        rc = hip().hipStreamEndCapture(self.stream.ptr, C.byref(self.graph))
+        rc = rc or hip().hipGraphInstantiate(C.byref(self.exe), self.graph, None, None, 0)
+        if rc:
+            raise RuntimeError(f"graph capture / instantiate failed: {rc}")
+
+    def launch(self):
+        rc = hip().hipGraphLaunch(self.exe, self.stream.ptr)
+        if rc:
+            raise RuntimeError(f"hipGraphLaunch failed: {rc}")
+
+    def close(self):
+        if self.exe:
+            hip().hipGraphExecDestroy(self.exe)
+            hip().hipGraphDestroy(self.graph)
+            self.exe = None
