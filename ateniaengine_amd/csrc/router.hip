@@ -77,6 +77,7 @@ __device__ inline void softmax_topk(bool on, int r, int E, int k, int renorm, in
   float my_logit = 0.f;
   if (on) {
     float mx = -INFINITY;
+#pragma unroll 8
     for (int e = 0; e < E; ++e) mx = fmaxf(mx, lg[e]);  // skips NaN like f32::max
     my_logit = lg[r];
     ex[r] = exp((double)(my_logit - mx));                // f32 subtraction, then f64 exp
@@ -85,6 +86,7 @@ __device__ inline void softmax_topk(bool on, int r, int E, int k, int renorm, in
   float my_w = 0.f;
   if (on) {
     double sum = 0.0;
+#pragma unroll 8
     for (int e = 0; e < E; ++e) sum += ex[e];            // sequential fold, e ascending
     double inv = sum > 0.0 ? 1.0 / sum : 0.0;
     my_w = (float)(ex[r] * inv);
@@ -98,6 +100,7 @@ __device__ inline void softmax_topk(bool on, int r, int E, int k, int renorm, in
   bool selected = false;
   if (on) {
     int rank = 0;  // experts that sort before me under (weight desc, index asc)
+#pragma unroll 8
     for (int e = 0; e < E; ++e) {
       float we = wt[e];
       rank += (we > my_w) || (we == my_w && e < r);
@@ -524,28 +527,36 @@ struct FusedGrouping {
 };
 
 // The expert grouping of ONE token from its selection flags (what kernel 2 would produce).
+// Called by the threads e = 0..E-1 of the workgroup (sel in LDS, already synchronised): thread e
+// counts the selected experts before it and writes its own entries.
 __device__ inline void write_single_token_grouping(const FusedGrouping& fg, const int32_t* sel,
-                                                   int E, int k) {
-  int run = 0;
-  for (int e = 0; e < E; ++e) {
-    const int c = sel[e] ? 1 : 0;
-    fg.counts[e] = c;
-    fg.offsets[e] = run;
-    if (c && run < k) {
-      fg.active[run] = e;
-      fg.perm[run] = run;
-      fg.inv[run] = run;
-      fg.tile_group[run] = e;
-      fg.tile_m0[run] = 0;
-      ++run;
-    }
+                                                   int e, int E, int k) {
+  if (e >= E) return;
+  int run = 0, total = 0;
+#pragma unroll 8
+  for (int o = 0; o < E; ++o) {
+    const int c = sel[o] ? 1 : 0;
+    run += o < e ? c : 0;
+    total += c;
   }
-  fg.offsets[E] = run;
-  *fg.n_active = run;
-  *fg.n_tiles = run;
-  *fg.shared_n_tiles = 1;
-  fg.shared_offsets[0] = 0;
-  fg.shared_offsets[1] = 1;
+  const int c = sel[e] ? 1 : 0;
+  fg.counts[e] = c;
+  fg.offsets[e] = run;
+  if (c && run < k) {
+    fg.active[run] = e;
+    fg.perm[run] = run;
+    fg.inv[run] = run;
+    fg.tile_group[run] = e;
+    fg.tile_m0[run] = 0;
+  }
+  if (e == 0) {
+    fg.offsets[E] = total;
+    *fg.n_active = total;
+    *fg.n_tiles = total;
+    *fg.shared_n_tiles = 1;
+    fg.shared_offsets[0] = 0;
+    fg.shared_offsets[1] = 1;
+  }
 }
 
 // Softmax + top-k from logits that another launch left in HBM: used when the rows of the
@@ -557,7 +568,7 @@ __global__ __launch_bounds__(kSelectThreads) void softmax_select_kernel(
     int32_t* __restrict__ idx_out, float* __restrict__ w_out, int32_t* __restrict__ status,
     FusedGrouping fg) {
   __shared__ double sExp[kSelectThreads];
-  __shared__ float sWt[kSelectThreads];
+  __shared__ float sWt[kSelectThreads], sLg[kSelectThreads];
   __shared__ int32_t sSel[kSelectThreads];
   const int TT = kSelectThreads / E;
   const int tid = threadIdx.x;
@@ -565,11 +576,13 @@ __global__ __launch_bounds__(kSelectThreads) void softmax_select_kernel(
   const int t = blockIdx.x * TT + tl;
   const bool on = tl < TT && t < T;
   const int ts = on ? t : 0, ls = on ? tl : 0;
-  softmax_topk(on, r, E, k, renorm, ts, logits + (size_t)ts * E, sExp + ls * E, sWt + ls * E,
-               sSel + ls * E, idx_out, w_out, status);
-  if (fg.counts) {  // T == 1
+  sLg[tid] = on ? logits[(size_t)t * E + r] : 0.f;  // one coalesced read; the folds walk LDS
+  __syncthreads();
+  softmax_topk(on, r, E, k, renorm, ts, sLg + ls * E, sExp + ls * E, sWt + ls * E, sSel + ls * E,
+               idx_out, w_out, status);
+  if (fg.counts) {  // T == 1: the workgroup holds token 0 only
     __syncthreads();
-    if (tid == 0) write_single_token_grouping(fg, sSel, E, k);
+    write_single_token_grouping(fg, sSel, tid, E, k);
   }
 }
 
@@ -722,7 +735,7 @@ __global__ __launch_bounds__(kTokenThreads) void router_token_kernel(
   softmax_topk(tid < E, tid, E, k, renorm, t, sLogit, sExp, sWt, sSel, idx_out, w_out, status);
   if (fg.counts) {  // T == 1: the grouping of a single token follows from its top-k
     __syncthreads();
-    if (tid == 0) write_single_token_grouping(fg, sSel, E, k);
+    write_single_token_grouping(fg, sSel, tid, E, k);
   }
 }
 
