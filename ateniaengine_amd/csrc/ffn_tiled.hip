@@ -981,13 +981,10 @@ hipError_t launch_tiled_dma(TiledParams p, int max_row_tiles, hipStream_t s) {
 
 template <bool INT8, bool UP>
 hipError_t launch_tiled(const TiledParams& p, int max_row_tiles, hipStream_t s) {
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)ffn_tiled_kernel<INT8, UP>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-    if (e != hipSuccess) return e;
-    attr_set = true;
-  }
+  static const hipError_t attr_rc =  // set once per instantiation, thread-safe
+      hipFuncSetAttribute((const void*)ffn_tiled_kernel<INT8, UP>,
+                          hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+  if (attr_rc != hipSuccess) return attr_rc;
   // Upper bound of the grid; workgroups past the real tile count return at once.
   int n_wg = max_row_tiles * p.n_col_tiles;
   n_wg = (n_wg + 7) / 8 * 8;

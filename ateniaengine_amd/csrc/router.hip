@@ -29,6 +29,8 @@
 
 #include "moe_internal.h"
 
+#include <mutex>
+
 namespace atenia_moe {
 
 namespace {
@@ -486,12 +488,18 @@ hipError_t launch_router_batch(const RouterArgs& a, hipStream_t s) {
   size_t dot_bytes = (size_t)(TT + RW) * LD * 8;
   size_t post_bytes = (((size_t)TT * R + 1) / 2) * 8 + (size_t)TT * a.E * (8 + 4 + 1) + TT * 8 + 16;
   size_t smem = dot_bytes > post_bytes ? dot_bytes : post_bytes;
-  static size_t attr_bytes = 0;  // per instantiation: largest size the attribute was set for
-  if (smem > 64 * 1024 && smem > attr_bytes) {
-    hipError_t e = hipFuncSetAttribute((const void*)router_batch_kernel<XT, RPT, TPT, KC>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) return e;
-    attr_bytes = smem;
+  if (smem > 64 * 1024) {
+    // per instantiation: largest size the attribute was set for (layers may launch from
+    // several host threads)
+    static std::mutex attr_mu;
+    static size_t attr_bytes = 0;
+    std::lock_guard<std::mutex> lock(attr_mu);
+    if (smem > attr_bytes) {
+      hipError_t e = hipFuncSetAttribute((const void*)router_batch_kernel<XT, RPT, TPT, KC>,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+      if (e != hipSuccess) return e;
+      attr_bytes = smem;
+    }
   }
   const int blocks = (a.T + TT - 1) / TT;
   const int row_blocks = (R + RW - 1) / RW;
