@@ -41,7 +41,13 @@ EXPORTS = (
     "atenia_moe_hip_layer_block_forward", "atenia_moe_hip_layer_block_forward_device",
     "atenia_moe_hip_layer_last_normed", "atenia_moe_hip_layer_set_v3_router",
     "atenia_moe_quantize_per_group_i8",
+    "atenia_moe_absmax_per_channel_symmetric", "atenia_moe_absmax_per_group_symmetric",
+    "atenia_moe_int8_to_bf16_per_channel_launch_device",
+    "atenia_moe_int8_to_bf16_per_group_launch_device",
 )
+# the reference's own names for the two dequantisation launchers (src/cuda/int8_to_bf16.rs:63-81)
+REFERENCE_NAMED_EXPORTS = ("int8_to_bf16_per_channel_launch_device",
+                           "int8_to_bf16_per_group_launch_device")
 
 
 class MoeHipError(RuntimeError):
@@ -107,6 +113,13 @@ def lib():
         L.atenia_moe_hip_layer_last_normed.argtypes = [P, P]
         L.atenia_moe_quantize_per_group_i8.argtypes = [P, C.c_size_t, C.c_size_t, C.c_size_t, P, P]
         L.atenia_moe_hip_layer_set_v3_router.argtypes = [P, C.c_int, C.c_int, C.c_double, C.c_int, P]
+        L.atenia_moe_absmax_per_channel_symmetric.argtypes = [P, C.c_size_t, C.c_size_t, P, P]
+        L.atenia_moe_absmax_per_group_symmetric.argtypes = [P, C.c_size_t, C.c_size_t, C.c_size_t, P, P]
+        L.atenia_moe_int8_to_bf16_per_channel_launch_device.argtypes = [P, P, P, C.c_int, C.c_int, P]
+        L.atenia_moe_int8_to_bf16_per_group_launch_device.argtypes = [P, P, P, C.c_int, C.c_int,
+                                                                      C.c_int, P]
+        L.int8_to_bf16_per_channel_launch_device.argtypes = [P, P, P, C.c_int, C.c_int]
+        L.int8_to_bf16_per_group_launch_device.argtypes = [P, P, P, C.c_int, C.c_int, C.c_int]
         L.atenia_moe_router_launch_device.argtypes = [P, P, C.c_int, C.c_int, P, P, P]
         L.atenia_moe_permute_launch_device.argtypes = [P, C.c_int, P, P, P, P]
         L.atenia_moe_expert_ffn_launch_device.argtypes = [P, P, C.c_int, C.c_int, P]
@@ -151,6 +164,45 @@ def quantize_per_group_i8(w, group_size: int):
     s = np.empty(w.shape[:-1] + ((cols + group_size - 1) // group_size,), dtype=np.float32)
     _check(lib().atenia_moe_quantize_per_group_i8(_ptr(w), rows, cols, group_size, _ptr(q), _ptr(s)))
     return q, s
+
+
+def absmax_per_channel_symmetric(w):
+    """[K, N] weight -> (q [K, N] int8, scales [N]), one scale per column
+    (src/tensor/quantizer.rs:67-117)."""
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    k, n = w.shape
+    q = np.empty((k, n), dtype=np.int8)
+    s = np.empty(n, dtype=np.float32)
+    _check(lib().atenia_moe_absmax_per_channel_symmetric(_ptr(w), k, n, _ptr(q), _ptr(s)))
+    return q, s
+
+
+def absmax_per_group_symmetric(w, group_size: int):
+    """[K, N] weight -> (q [K, N] int8, scales [ceil(K/gs), N]), groups along K
+    (src/tensor/quantizer.rs:175-248)."""
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    k, n = w.shape
+    q = np.empty((k, n), dtype=np.int8)
+    s = np.empty(((k + group_size - 1) // group_size, n), dtype=np.float32)
+    _check(lib().atenia_moe_absmax_per_group_symmetric(_ptr(w), k, n, group_size, _ptr(q), _ptr(s)))
+    return q, s
+
+
+def int8_to_bf16_launch_device(d_int8, d_scales, d_bf16, k: int, n: int, group_size: int = 0,
+                               stream=None, reference_symbol: bool = False) -> int:
+    """Launches the device dequantisation of a [K, N] int8 weight (device pointers as ints);
+    group_size 0 = one scale per column.  Returns the launcher's status code unchanged, as the
+    reference's wrapper receives it (src/cuda/int8_to_bf16.rs).  `reference_symbol` goes through
+    the entry points that carry the reference's own names (default stream)."""
+    L = lib()
+    if reference_symbol:
+        if group_size:
+            return L.int8_to_bf16_per_group_launch_device(d_int8, d_scales, d_bf16, k, n, group_size)
+        return L.int8_to_bf16_per_channel_launch_device(d_int8, d_scales, d_bf16, k, n)
+    if group_size:
+        return L.atenia_moe_int8_to_bf16_per_group_launch_device(d_int8, d_scales, d_bf16, k, n,
+                                                                 group_size, stream)
+    return L.atenia_moe_int8_to_bf16_per_channel_launch_device(d_int8, d_scales, d_bf16, k, n, stream)
 
 
 def f32_to_bf16_trunc(a) -> np.ndarray:

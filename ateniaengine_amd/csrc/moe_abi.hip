@@ -1182,6 +1182,34 @@ int atenia_moe_quantize_per_row_i8(const float* w, size_t rows, size_t cols, int
   return ATENIA_MOE_OK;
 }
 
+int atenia_moe_absmax_per_group_symmetric(const float* w, size_t k, size_t n, size_t group_size,
+                                          int8_t* q, float* scales) {
+  if (!w || !q || !scales) return fail(ATENIA_MOE_ERR_DIM, "null pointer");
+  if (group_size == 0) return fail(ATENIA_MOE_ERR_DIM, "group size must be positive");
+  // one pass per group of rows: column maxima into the group's scale row, then the quotients
+  for (size_t k0 = 0; k0 < k; k0 += group_size) {
+    const size_t k1 = k0 + group_size < k ? k0 + group_size : k;
+    float* sc = scales + (k0 / group_size) * n;
+    for (size_t c = 0; c < n; ++c) sc[c] = 0.0f;
+    for (size_t r = k0; r < k1; ++r)
+      for (size_t c = 0; c < n; ++c) sc[c] = fmaxf(sc[c], fabsf(w[r * n + c]));
+    for (size_t c = 0; c < n; ++c) sc[c] = fmaxf(sc[c] / 127.0f, 1e-12f);
+    for (size_t r = k0; r < k1; ++r)
+      for (size_t c = 0; c < n; ++c) {
+        float v = roundf(w[r * n + c] / sc[c]);
+        v = v < -127.0f ? -127.0f : (v > 127.0f ? 127.0f : v);
+        q[r * n + c] = (int8_t)v;
+      }
+  }
+  return ATENIA_MOE_OK;
+}
+
+int atenia_moe_absmax_per_channel_symmetric(const float* w, size_t k, size_t n, int8_t* q,
+                                            float* scales) {
+  // one group spanning all of K
+  return atenia_moe_absmax_per_group_symmetric(w, k, n, k > 0 ? k : 1, q, scales);
+}
+
 int atenia_moe_f32_to_bf16_trunc(const float* src, size_t n, uint16_t* dst) {
   if (!src || !dst) return fail(ATENIA_MOE_ERR_DIM, "null pointer");
   for (size_t i = 0; i < n; ++i) {

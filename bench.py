@@ -235,6 +235,45 @@ def measure_block(torch, np, capi, layer, T, steps, warmup, seed):
     return res
 
 
+def measure_dequant(torch, capi, steps, warmup, seed):
+    """The INT8 -> BF16 dequantisation launchers on one Mixtral expert projection ([K, N] =
+    [4096, 14336] and its transpose), timed with events on the launch stream.  Algorithmic bytes
+    per launch: K*N int8 read + 2*K*N bf16 written + the scales."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    stream = torch.cuda.current_stream().cuda_stream
+    res = []
+    for k, n in ((D_MODEL, D_FF), (D_FF, D_MODEL)):
+        # six weight / output pairs in rotation (1 GB in all), so that no launch finds its
+        # operands in the 256 MB Infinity Cache
+        qs = [torch.randint(-127, 128, (k, n), generator=g, device="cuda", dtype=torch.int8)
+              for _ in range(6)]
+        outs = [torch.empty((k, n), device="cuda", dtype=torch.bfloat16) for _ in range(6)]
+        for gs in (0, 128):
+            ng = (k + gs - 1) // gs if gs else 1
+            sc = torch.rand((ng, n), generator=g, device="cuda", dtype=torch.float32) * 1e-3 + 1e-4
+
+            def fn(i):
+                rc = capi.int8_to_bf16_launch_device(qs[i % 6].data_ptr(), sc.data_ptr(),
+                                                     outs[i % 6].data_ptr(), k, n, group_size=gs,
+                                                     stream=stream)
+                if rc != 0:
+                    raise RuntimeError(f"dequant launch failed: {rc}")
+            for i in range(warmup):
+                fn(i)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for i in range(steps):
+                fn(i)
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1) / steps
+            nbytes = 3.0 * k * n + 4.0 * ng * n
+            res.append({"k": k, "n": n, "group_size": gs, "us": ms * 1e3, "algorithmic_bytes": nbytes,
+                        "gbs": nbytes / ms / 1e6, "hbm_frac": nbytes / ms / 1e6 / PEAK_HBM_GBS})
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -254,6 +293,8 @@ def main():
                     help="also time batches of up to 64 tokens replayed from HIP graphs")
     ap.add_argument("--block", action="store_true",
                     help="also time the decoder-layer FFN block entry point (norm + layer + residual)")
+    ap.add_argument("--dequant", action="store_true",
+                    help="also time the INT8 -> BF16 dequantisation launchers")
     ap.add_argument("--seed", type=int, default=1234)
     a = ap.parse_args()
     if a.gpus != 1:
@@ -399,6 +440,8 @@ def main():
     }
     if block is not None:
         line["block"] = block
+    if a.dequant:
+        line["dequant"] = measure_dequant(torch, capi, max(a.steps, 50), a.warmup, a.seed)
     print(json.dumps(line))
 
 

@@ -286,8 +286,38 @@ int atenia_moe_hip_layer_info(const AteniaMoeLayer* layer, int64_t info[8]);
  * q = clamp(round_half_away(w * (1/scale)), -127, 127). */
 int atenia_moe_quantize_per_row_i8(const float* w, size_t rows, size_t cols, int8_t* q,
                                    float* scales);
+/* Symmetric int8 quantisation of a row-major [K, N] weight in the reference's own orientation
+ * (K = input, N = output channel): one scale per column (`absmax_per_channel_symmetric`,
+ * src/tensor/quantizer.rs:67-117; scales [N]) or per column and group of `group_size`
+ * consecutive k (`absmax_per_group_symmetric`, src/tensor/quantizer.rs:175-248; scales
+ * [ceil(K / group_size), N]): scale = max(max|w| / 127, 1e-12), q = clamp(round(w / scale)). */
+int atenia_moe_absmax_per_channel_symmetric(const float* w, size_t k, size_t n, int8_t* q,
+                                            float* scales);
+int atenia_moe_absmax_per_group_symmetric(const float* w, size_t k, size_t n, size_t group_size,
+                                          int8_t* q, float* scales);
 /* f32 -> bf16 bit patterns by truncation (`f32_to_bf16_bits`, src/tensor/tensor.rs:306-308). */
 int atenia_moe_f32_to_bf16_trunc(const float* src, size_t n, uint16_t* dst);
+
+/* INT8 -> BF16 dequantisation on the device ----------------------------------------------- */
+
+/* out[k, n] = truncate_to_bf16((float)q[k, n] * scales[n]) over a row-major [K, N] int8 weight;
+ * device pointers, asynchronous on `stream` (a hipStream_t; NULL = the default stream).
+ * Returns 0, a negative value for bad arguments (-1 null pointer, -2 group_size <= 0) or the
+ * runtime's launch status; k * n <= 0 is a no-op.  Replaces
+ * `int8_to_bf16_per_channel_launch_device` (src/cuda/int8_to_bf16.cu:42-71). */
+int atenia_moe_int8_to_bf16_per_channel_launch_device(const void* d_int8, const float* d_scales,
+                                                      void* d_bf16, int k, int n, void* stream);
+/* Same with scales [ceil(K / group_size), N]: scale of (k, n) = scales[(k / group_size) * N + n].
+ * Replaces `int8_to_bf16_per_group_launch_device` (src/cuda/int8_to_bf16.cu:112-141). */
+int atenia_moe_int8_to_bf16_per_group_launch_device(const void* d_int8, const float* d_scales,
+                                                    void* d_bf16, int k, int n, int group_size,
+                                                    void* stream);
+/* The same two launchers under the reference's own symbol names and argument lists (default
+ * stream), so that its FFI block (src/cuda/int8_to_bf16.rs:63-81) binds without a change. */
+int int8_to_bf16_per_channel_launch_device(const void* d_int8, const float* d_scales,
+                                           void* d_bf16, int k, int n);
+int int8_to_bf16_per_group_launch_device(const void* d_int8, const float* d_scales, void* d_bf16,
+                                         int k, int n, int group_size);
 
 #ifdef __cplusplus
 }

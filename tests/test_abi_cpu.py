@@ -17,6 +17,11 @@ def test_library_exports_every_declared_symbol():
     L = capi.lib()
     for name in declared:
         assert hasattr(L, name), f"{name} is declared but not exported"
+    # the two dequantisation launchers that keep the reference's symbol names
+    plain = set(re.findall(r"^int (int8_to_bf16_\w+)\s*\(", header, flags=re.M))
+    assert plain == set(capi.REFERENCE_NAMED_EXPORTS)
+    for name in plain:
+        assert hasattr(L, name), f"{name} is declared but not exported"
 
 
 def test_last_error_string_and_bad_handles():
@@ -35,6 +40,37 @@ def test_host_quantiser_matches_oracle(ora):
     q, s = capi.quantize_per_row_i8(w)
     oq, os_ = ora.quantize_per_row_i8(w)
     assert (q == oq).all() and s.tobytes() == os_.tobytes()
+
+
+def test_host_kn_quantisers_match_oracle(ora):
+    """[K, N]-oriented quantisers (src/tensor/quantizer.rs:67-117, 175-248) against the oracle,
+    with an all-zero column, an outlier and a ragged last group."""
+    rng = np.random.default_rng(2)
+    w = (rng.standard_normal((200, 37)) * 0.02).astype(np.float32)
+    w[:, 3] = 0
+    w[17, 5] *= 40
+    q, s = capi.absmax_per_channel_symmetric(w)
+    oq, os_ = ora.absmax_per_channel_symmetric(w)
+    assert (q == oq).all() and s.tobytes() == os_.tobytes()
+    for gs in (1, 64, 128, 200, 512):
+        q, s = capi.absmax_per_group_symmetric(w, gs)
+        oq, os_ = ora.absmax_per_group_symmetric(w, gs)
+        assert (q == oq).all() and s.tobytes() == os_.tobytes(), gs
+    # the known-answer case of the reference's own test (quantizer.rs:969-993)
+    q, s = capi.absmax_per_channel_symmetric(np.array([[2.0], [-4.0], [6.0], [-127.0]], np.float32))
+    assert s.tolist() == [1.0] and q.reshape(-1).tolist() == [2, -4, 6, -127]
+
+
+def test_dequant_launchers_check_their_arguments():
+    """Argument checks run before anything touches the GPU: empty shapes are a no-op (0), a
+    non-positive group size is -2 (src/cuda/int8_to_bf16.cu:57-59, 122), null pointers -1."""
+    assert capi.int8_to_bf16_launch_device(None, None, None, 0, 16) == 0
+    assert capi.int8_to_bf16_launch_device(None, None, None, 16, 0, group_size=8) == 0
+    L = capi.lib()
+    assert L.atenia_moe_int8_to_bf16_per_group_launch_device(None, None, None, 4, 4, 0, None) == -2
+    assert L.int8_to_bf16_per_group_launch_device(None, None, None, 4, 4, -1) == -2
+    assert capi.int8_to_bf16_launch_device(None, None, None, 4, 4) == -1
+    assert capi.int8_to_bf16_launch_device(None, None, None, 4, 4, reference_symbol=True) == -1
 
 
 def test_host_bf16_truncation_matches_oracle(ora):
