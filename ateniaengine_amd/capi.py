@@ -19,6 +19,7 @@ CONVENTION_ATENIA = 0
 CONVENTION_HUGGINGFACE_QWEN = 1
 WEIGHT_F32, WEIGHT_BF16, WEIGHT_INT8_W8A16, WEIGHT_INT8_PER_GROUP = 0, 1, 2, 3
 ACT_F32, ACT_BF16 = 0, 1
+POLICY_CERTIFIED, POLICY_STRICT, POLICY_FAST = 0, 1, 2
 NORM_GRAPH_F32, NORM_F64 = 0, 1
 OK, ERR_SYNC, ERR_LAUNCH = 0, 1, 2
 ERR_DIM, ERR_K, ERR_NON_FINITE, ERR_OOM, ERR_HANDLE, ERR_UNSUPPORTED = -1, -2, -3, -4, -5, -6
@@ -44,6 +45,7 @@ EXPORTS = (
     "atenia_moe_absmax_per_channel_symmetric", "atenia_moe_absmax_per_group_symmetric",
     "atenia_moe_int8_to_bf16_per_channel_launch_device",
     "atenia_moe_int8_to_bf16_per_group_launch_device",
+    "atenia_moe_hip_layer_set_numeric_policy",
 )
 # the reference's own names for the two dequantisation launchers (src/cuda/int8_to_bf16.rs:63-81)
 REFERENCE_NAMED_EXPORTS = ("int8_to_bf16_per_channel_launch_device",
@@ -113,6 +115,7 @@ def lib():
         L.atenia_moe_hip_layer_last_normed.argtypes = [P, P]
         L.atenia_moe_quantize_per_group_i8.argtypes = [P, C.c_size_t, C.c_size_t, C.c_size_t, P, P]
         L.atenia_moe_hip_layer_set_v3_router.argtypes = [P, C.c_int, C.c_int, C.c_double, C.c_int, P]
+        L.atenia_moe_hip_layer_set_numeric_policy.argtypes = [P, C.c_int]
         L.atenia_moe_absmax_per_channel_symmetric.argtypes = [P, C.c_size_t, C.c_size_t, P, P]
         L.atenia_moe_absmax_per_group_symmetric.argtypes = [P, C.c_size_t, C.c_size_t, C.c_size_t, P, P]
         L.atenia_moe_int8_to_bf16_per_channel_launch_device.argtypes = [P, P, P, C.c_int, C.c_int, P]
@@ -293,6 +296,11 @@ class Layer:
         _check(lib().atenia_moe_hip_layer_set_v3_router(self._h, n_group, topk_group,
                                                         routed_scaling_factor, int(norm_topk_prob),
                                                         _ptr(b)))
+
+    def set_numeric_policy(self, policy: int):
+        """Expert arithmetic of an f32 layer from the next forward on: POLICY_CERTIFIED (f64
+        accumulation), POLICY_STRICT / POLICY_FAST (f32 accumulation); numeric_policy.rs:36-75."""
+        _check(lib().atenia_moe_hip_layer_set_numeric_policy(self._h, policy))
 
     # The decoder layer's FFN block around the op: out = x1 + MoE(RMSNorm(x1) * gamma).
     def block_forward(self, x1, gamma, eps: float, norm_policy: int = NORM_GRAPH_F32) -> np.ndarray:

@@ -8,6 +8,13 @@
 // Only the order of the f64 additions differs from the CPU path (k is tiled), which moves a
 // result by ~1e-16 relative before the final f32 rounding.  This path exists for parity
 // with f32 checkpoints (1e-5 bar); it is FMA-bound and not the throughput path.
+//
+// F32ACC: the reference's other expert arithmetic (`matvec_f32`, src/moe/dense.rs:120-140, used
+// under NumericPolicy::Strict and as the result `Fast` falls back to): the three projections
+// accumulate in f32, acc = acc + w * x with the product and the sum rounded separately, c
+// ascending.  A thread walks the k tiles in order, so its f32 sequence IS the reference's; the
+// file is compiled without contraction so that no product is fused into the sum.  silu stays
+// f64 -> f32 and the router stays f64 on every policy (src/moe/numeric_policy.rs:24-29).
 #include "moe_internal.h"
 
 namespace atenia_moe {
@@ -17,7 +24,7 @@ namespace {
 constexpr int kTile = 32;
 constexpr int kLdT = kTile + 1;
 
-template <bool UP>
+template <bool UP, bool F32ACC>
 __global__ __launch_bounds__(256) void ffn_f32_kernel(
     const float* __restrict__ wa, const float* __restrict__ wb, int64_t w_stride, int n_rows,
     int k_cols, const float* __restrict__ a, int a_stride, float* __restrict__ out,
@@ -47,6 +54,7 @@ __global__ __launch_bounds__(256) void ffn_f32_kernel(
   const float* wbe = UP ? wb + (size_t)e * w_stride : nullptr;
 
   double acc_a[4] = {0, 0, 0, 0}, acc_b[4] = {0, 0, 0, 0};
+  float facc_a[4] = {0.f, 0.f, 0.f, 0.f}, facc_b[4] = {0.f, 0.f, 0.f, 0.f};
   for (int k0 = 0; k0 < k_cols; k0 += kTile) {
     __syncthreads();
     for (int j = tid; j < kTile * kTile; j += 256) {
@@ -60,6 +68,22 @@ __global__ __launch_bounds__(256) void ffn_f32_kernel(
       if (UP) sBb[r * kLdT + c] = ok ? wbe[(size_t)n * k_cols + kk] : 0.f;
     }
     __syncthreads();
+    if (F32ACC) {
+      // tile columns past k_cols hold +0.0: acc + 0 * 0 leaves every sum as it was (a sum that
+      // starts at +0.0 never becomes -0.0)
+#pragma unroll 8
+      for (int c = 0; c < kTile; ++c) {
+        const float ba = sBa[tx * kLdT + c];
+        const float bb = UP ? sBb[tx * kLdT + c] : 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float av = sA[(ty * 4 + i) * kLdT + c];
+          facc_a[i] = facc_a[i] + ba * av;  // two roundings (no contraction in this file)
+          if (UP) facc_b[i] = facc_b[i] + bb * av;
+        }
+      }
+      continue;
+    }
 #pragma unroll 8
     for (int c = 0; c < kTile; ++c) {
       double ba = (double)sBa[tx * kLdT + c];
@@ -79,14 +103,14 @@ __global__ __launch_bounds__(256) void ffn_f32_kernel(
     int pos = m0 + ty * 4 + i;
     if (pos >= cnt) continue;
     if (UP) {
-      float gate = (float)acc_a[i];
-      float up = (float)acc_b[i];
+      float gate = F32ACC ? facc_a[i] : (float)acc_a[i];
+      float up = F32ACC ? facc_b[i] : (float)acc_b[i];
       double gd = (double)gate;
       float s = (float)(gd / (1.0 + exp(-gd)));
       out[(size_t)(base + pos) * out_stride + n] = __fmul_rn(s, up);
     } else {
       int pair = g.perm[base + pos];
-      out[(size_t)pair * out_stride + n] = (float)acc_a[i];
+      out[(size_t)pair * out_stride + n] = F32ACC ? facc_a[i] : (float)acc_a[i];
     }
   }
 }
@@ -96,19 +120,19 @@ __global__ __launch_bounds__(256) void ffn_f32_kernel(
 hipError_t launch_ffn_up_f32(const FfnArgs& a, hipStream_t s) {
   dim3 grid((a.gate.n_rows + kTile - 1) / kTile, a.n_groups_max,
             (a.rows_max + kTile - 1) / kTile);
-  ffn_f32_kernel<true><<<grid, 256, 0, s>>>((const float*)a.gate.w, (const float*)a.up.w,
-                                            a.gate.expert_stride, a.gate.n_rows, a.gate.k_cols,
-                                            (const float*)a.x, a.x_stride, (float*)a.h,
-                                            a.h_stride, a.g);
+  auto k = a.f32_accumulate ? ffn_f32_kernel<true, true> : ffn_f32_kernel<true, false>;
+  k<<<grid, 256, 0, s>>>((const float*)a.gate.w, (const float*)a.up.w, a.gate.expert_stride,
+                         a.gate.n_rows, a.gate.k_cols, (const float*)a.x, a.x_stride, (float*)a.h,
+                         a.h_stride, a.g);
   return hipGetLastError();
 }
 
 hipError_t launch_ffn_down_f32(const FfnArgs& a, hipStream_t s) {
   dim3 grid((a.down.n_rows + kTile - 1) / kTile, a.n_groups_max,
             (a.rows_max + kTile - 1) / kTile);
-  ffn_f32_kernel<false><<<grid, 256, 0, s>>>((const float*)a.down.w, nullptr,
-                                             a.down.expert_stride, a.down.n_rows, a.down.k_cols,
-                                             (const float*)a.h, a.h_stride, a.y, a.y_stride, a.g);
+  auto k = a.f32_accumulate ? ffn_f32_kernel<false, true> : ffn_f32_kernel<false, false>;
+  k<<<grid, 256, 0, s>>>((const float*)a.down.w, nullptr, a.down.expert_stride, a.down.n_rows,
+                         a.down.k_cols, (const float*)a.h, a.h_stride, a.y, a.y_stride, a.g);
   return hipGetLastError();
 }
 

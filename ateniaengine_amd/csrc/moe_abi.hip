@@ -116,6 +116,7 @@ struct AteniaMoeLayer {
   std::mutex mu;
 
   bool profiling = false;
+  int policy = ATENIA_MOE_POLICY_CERTIFIED;  // expert arithmetic of f32 layers
   hipEvent_t ev[ATENIA_MOE_N_STAGES] = {};
   bool ev_valid = false;
   int32_t launches[ATENIA_MOE_N_STAGES] = {};
@@ -435,6 +436,7 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
 
   FfnArgs fa{};
   fa.wdtype = ffn_dtype;
+  fa.f32_accumulate = L->policy != ATENIA_MOE_POLICY_CERTIFIED;
   fa.g.offsets = L->offsets.as<int32_t>();
   fa.g.active = L->active.as<int32_t>();
   fa.g.n_active = L->n_active.as<int32_t>();
@@ -1088,6 +1090,16 @@ int atenia_moe_hip_layer_last_expert_outputs(AteniaMoeLayer* L, float* y_host,
   if (y_shared_host && L->fs > 0)
     HIP_TRY(hipMemcpy(y_shared_host, L->ys.p, (size_t)L->last_T * L->d * 4,
                       hipMemcpyDeviceToHost));
+  return ATENIA_MOE_OK;
+}
+
+int atenia_moe_hip_layer_set_numeric_policy(AteniaMoeLayer* L, int policy) {
+  if (!valid_handle(L)) return fail(ATENIA_MOE_ERR_HANDLE, "invalid layer handle");
+  if (policy != ATENIA_MOE_POLICY_CERTIFIED && policy != ATENIA_MOE_POLICY_STRICT &&
+      policy != ATENIA_MOE_POLICY_FAST)
+    return fail(ATENIA_MOE_ERR_DIM, "unknown numeric policy %d", policy);
+  std::lock_guard<std::mutex> lock(L->mu);
+  L->policy = policy;
   return ATENIA_MOE_OK;
 }
 

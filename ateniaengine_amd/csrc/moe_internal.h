@@ -111,6 +111,7 @@ hipError_t launch_permute(const PermuteArgs& a, hipStream_t s, int* n_launches);
 
 struct FfnArgs {
   int wdtype;          // ATENIA_MOE_WEIGHT_*
+  int f32_accumulate;  // f32 weights only: the projections accumulate in f32 (Strict / Fast)
   GroupDesc g;
   int n_groups_max;    // upper bound of *n_active (grid sizing)
   int rows_max;        // upper bound of rows in any one group (grid sizing)

@@ -2,6 +2,10 @@
 // interface each part follows).
 #include "atenia_moe.hpp"
 
+#include <algorithm>
+#include <cstdlib>
+#include <cctype>
+#include <atomic>
 #include <cmath>
 #include <cstring>
 #include <map>
@@ -413,6 +417,106 @@ int pack(const std::vector<const std::vector<float>*>& mats, size_t rows, size_t
 
 // The C-ABI handle for (convention, with shared expert), created and uploaded on first use.
 // Caller holds dev_->mu.
+// ---- numeric policy -----------------------------------------------------------------------------
+const char* as_str(NumericPolicy p) {
+  switch (p) {
+    case NumericPolicy::Strict: return "strict";
+    case NumericPolicy::Fast: return "fast";
+    default: return "certified";
+  }
+}
+
+std::optional<NumericPolicy> numeric_policy_from_str(const std::string& s) {
+  size_t b = 0, e = s.size();
+  while (b < e && std::isspace((unsigned char)s[b])) ++b;
+  while (e > b && std::isspace((unsigned char)s[e - 1])) --e;
+  std::string t = s.substr(b, e - b);
+  for (auto& c : t) c = (char)std::tolower((unsigned char)c);
+  if (t == "certified" || t == "f64") return NumericPolicy::Certified;
+  if (t == "strict" || t == "f32") return NumericPolicy::Strict;
+  if (t == "fast") return NumericPolicy::Fast;
+  return std::nullopt;
+}
+
+namespace {
+constexpr int kPolicyUnset = 255;
+std::atomic<int> g_policy_override{kPolicyUnset};
+NumericPolicy policy_from_env() {  // read once (src/moe/numeric_policy.rs:99-116)
+  static const NumericPolicy p = [] {
+    const char* e = std::getenv("ATENIA_NUMERIC_POLICY");
+    auto v = e ? numeric_policy_from_str(e) : std::nullopt;
+    return v ? *v : NumericPolicy::Certified;
+  }();
+  return p;
+}
+}  // namespace
+
+NumericPolicy numeric_policy() {
+  const int o = g_policy_override.load(std::memory_order_relaxed);
+  if (o != kPolicyUnset) return o == 1 ? NumericPolicy::Strict : o == 2 ? NumericPolicy::Fast : NumericPolicy::Certified;
+  return policy_from_env();
+}
+void set_numeric_policy(NumericPolicy p) { g_policy_override.store((int)p, std::memory_order_relaxed); }
+void clear_numeric_policy_override() { g_policy_override.store(kPolicyUnset, std::memory_order_relaxed); }
+
+std::optional<NumericalMetrics> NumericalMetrics::compute(const std::vector<float>& atenia,
+                                                          const std::vector<float>& reference) {
+  if (atenia.empty() || atenia.size() != reference.size()) return std::nullopt;
+  auto argmax = [](const std::vector<float>& v) {
+    size_t best = 0;
+    double bv = (double)v[0];
+    for (size_t i = 1; i < v.size(); ++i)
+      if ((double)v[i] > bv) {
+        bv = (double)v[i];
+        best = i;
+      }
+    return best;
+  };
+  NumericalMetrics m;
+  m.len = atenia.size();
+  double sum_abs = 0.0, sum_sq = 0.0;
+  for (size_t i = 0; i < m.len; ++i) {
+    const double dd = (double)atenia[i] - (double)reference[i];
+    const double ad = std::fabs(dd);
+    if (ad > m.max_abs_diff) m.max_abs_diff = ad;
+    sum_abs += ad;
+    sum_sq += dd * dd;
+  }
+  m.mean_abs_diff = sum_abs / (double)m.len;
+  m.rmse = std::sqrt(sum_sq / (double)m.len);
+  m.argmax_match = argmax(atenia) == argmax(reference);
+  return m;
+}
+
+PolicyCertificate PolicyCertificate::compare(NumericPolicy policy,
+                                             const std::vector<std::vector<float>>& reference_rows,
+                                             const std::vector<std::vector<float>>& candidate_rows,
+                                             const std::vector<uint32_t>& reference_tokens,
+                                             const std::vector<uint32_t>& candidate_tokens) {
+  const size_t rows = std::min(reference_rows.size(), candidate_rows.size());
+  double max_abs = 0.0, sum_abs = 0.0, sum_sq = 0.0;
+  size_t argmax_ok = 0, counted = 0;
+  for (size_t i = 0; i < rows; ++i) {
+    auto m = NumericalMetrics::compute(candidate_rows[i], reference_rows[i]);
+    if (!m) continue;
+    max_abs = std::max(max_abs, m->max_abs_diff);
+    sum_abs += m->mean_abs_diff;
+    sum_sq += m->rmse * m->rmse;
+    if (m->argmax_match) ++argmax_ok;
+    ++counted;
+  }
+  const double denom = (double)std::max<size_t>(counted, 1);
+  PolicyCertificate c;
+  c.policy = policy;
+  c.rows = counted;
+  c.max_abs_diff = max_abs;
+  c.mean_abs_diff = sum_abs / denom;
+  c.rmse = std::sqrt(sum_sq / denom);
+  c.argmax_match_rate = (double)argmax_ok / denom;
+  c.tokens_match = reference_tokens == candidate_tokens;
+  return c;
+}
+
 Result<void*, MoeLayerError> RealMoeLayer::handle_for(MoeExecutionConvention convention,
                                                       bool with_shared) const {
   typedef Result<void*, MoeLayerError> R;
@@ -557,6 +661,7 @@ Result<std::vector<float>, MoeLayerError> RealMoeLayer::run(const std::vector<fl
   if (hr.is_err()) return R::Err(hr.error());
   AteniaMoeLayer* h = (AteniaMoeLayer*)hr.value();
   std::vector<float> out(x.size());
+  (void)atenia_moe_hip_layer_set_numeric_policy(h, (int)numeric_policy());
   const int rc = atenia_moe_hip_layer_forward(h, x.data(), (int)(x.size() / d), out.data());
   if (rc == ATENIA_MOE_ERR_NON_FINITE) return R::Err(non_finite_error(h));
   if (rc == ATENIA_MOE_ERR_DIM) return R::Err(dense_dim_error("x", d, x.size()));
@@ -590,6 +695,7 @@ Result<std::vector<float>, MoeLayerError> RealMoeLayer::ffn_block(
   if (hr.is_err()) return R::Err(hr.error());
   AteniaMoeLayer* h = (AteniaMoeLayer*)hr.value();
   std::vector<float> out(x1.size());
+  (void)atenia_moe_hip_layer_set_numeric_policy(h, (int)numeric_policy());
   const int rc = atenia_moe_hip_layer_block_forward(h, x1.data(), (int)(x1.size() / d), gamma.data(),
                                                     eps, (int)norm_policy, out.data());
   if (rc == ATENIA_MOE_ERR_NON_FINITE) return R::Err(non_finite_error(h));

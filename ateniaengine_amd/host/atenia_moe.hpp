@@ -163,6 +163,53 @@ struct V3RouterConfig {  // src/moe/v3_router.rs:59-72
 // Int8PerGroup: one scale per output row and group of kInt8GroupSize input elements (the
 // reference's per-group scheme, src/tensor/quantizer.rs:175-248).
 enum class MoeWeightStorage { F32 = 0, Bf16 = 1, Int8W8A16 = 2, Int8PerGroup = 3 };
+
+// ---- numeric policy (src/moe/numeric_policy.rs) -----------------------------------------------
+// Arithmetic of the expert projections of f32 layers: Certified = f64 accumulation (default and
+// fallback), Strict = f32 accumulation, Fast = f32 on the GPU (here: the Strict arithmetic, which
+// is what the reference's Fast falls back to).  The router is f64 under every policy.  Process
+// global like the reference's: resolved once from ATENIA_NUMERIC_POLICY={certified,strict,fast}
+// (also f64 / f32), overridable in-process; anything unknown means Certified.
+enum class NumericPolicy { Certified = 0, Strict = 1, Fast = 2 };
+const char* as_str(NumericPolicy p);
+std::optional<NumericPolicy> numeric_policy_from_str(const std::string& s);
+inline bool ffn_uses_f32(NumericPolicy p) { return p != NumericPolicy::Certified; }
+inline bool ffn_uses_cuda(NumericPolicy p) { return p == NumericPolicy::Fast; }  // "on the GPU"
+NumericPolicy numeric_policy();
+void set_numeric_policy(NumericPolicy p);
+void clear_numeric_policy_override();
+
+// Comparison of an output with a reference in f64 (src/moe/numerical.rs:22-88): nullopt when
+// the lengths differ or are zero; argmax = first index of the largest value.
+struct NumericalMetrics {
+  size_t len = 0;
+  double max_abs_diff = 0.0, mean_abs_diff = 0.0, rmse = 0.0;
+  bool argmax_match = false;
+  static std::optional<NumericalMetrics> compute(const std::vector<float>& atenia,
+                                                 const std::vector<float>& reference);
+  bool passes(double tolerance) const { return max_abs_diff < tolerance && argmax_match; }
+};
+
+// By-tolerance certificate of a non-Certified policy against Certified rows
+// (src/moe/numeric_policy.rs:132-196): worst max |diff| over the rows, means of the per-row mean
+// |diff| and of the squared rmse (root taken at the end), share of rows whose argmax agrees, and
+// whether the token sequences are identical.  Rows that are empty or differ in length are
+// skipped, as NumericalMetrics::compute returns None for them.
+struct PolicyCertificate {
+  NumericPolicy policy = NumericPolicy::Certified;
+  size_t rows = 0;
+  double max_abs_diff = 0.0, mean_abs_diff = 0.0, rmse = 0.0, argmax_match_rate = 0.0;
+  bool tokens_match = false;
+  static PolicyCertificate compare(NumericPolicy policy,
+                                   const std::vector<std::vector<float>>& reference_rows,
+                                   const std::vector<std::vector<float>>& candidate_rows,
+                                   const std::vector<uint32_t>& reference_tokens,
+                                   const std::vector<uint32_t>& candidate_tokens);
+  bool passes(double tolerance) const {
+    return argmax_match_rate >= 1.0 && tokens_match && max_abs_diff <= tolerance;
+  }
+};
+constexpr double STRICT_LOGIT_TOLERANCE = 0.5;
 constexpr size_t kInt8GroupSize = 128;
 
 // A per-output-row symmetric int8 weight [rows, cols]: w[r, c] = q[r, c] * scales[r]

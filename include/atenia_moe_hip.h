@@ -275,6 +275,21 @@ int atenia_moe_hip_layer_set_profiling(AteniaMoeLayer* layer, int enabled);
 int atenia_moe_hip_layer_stage_ms(AteniaMoeLayer* layer, float ms[ATENIA_MOE_N_STAGES]);
 int atenia_moe_hip_layer_stage_launches(AteniaMoeLayer* layer, int32_t n[ATENIA_MOE_N_STAGES]);
 
+/* Expert arithmetic of a layer with f32 weights, the reference's NumericPolicy
+ * (src/moe/numeric_policy.rs:36-75; selection in `matvec_policy`, src/moe/dense.rs:159-168):
+ *   CERTIFIED  f64 accumulation (default; the bit-exact reference arithmetic)
+ *   STRICT     f32 accumulation, product and sum rounded separately, columns ascending
+ *              (`matvec_f32`, src/moe/dense.rs:120-140)
+ *   FAST       f32 on the GPU; the reference sends each projection through `cuda_matmul` and
+ *              falls back to the Strict arithmetic, which is what this library computes
+ * The router accumulates in f64 under every policy, so routing never changes.  Layers stored
+ * as bf16 / int8 multiply on the matrix cores with f32 accumulation whatever the policy; the
+ * call is accepted for them and changes nothing.  Takes effect from the next forward. */
+#define ATENIA_MOE_POLICY_CERTIFIED 0
+#define ATENIA_MOE_POLICY_STRICT 1
+#define ATENIA_MOE_POLICY_FAST 2
+int atenia_moe_hip_layer_set_numeric_policy(AteniaMoeLayer* layer, int policy);
+
 /* Layer facts a host needs to size buffers: writes E, k, d, f, f_s, convention,
  * weight_dtype, bytes of expert weights per routed expert as stored in HBM. */
 int atenia_moe_hip_layer_info(const AteniaMoeLayer* layer, int64_t info[8]);

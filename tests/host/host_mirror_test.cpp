@@ -231,6 +231,60 @@ int main(int argc, char** argv) {
     CHECK(thrown, "node accepted a bad input dim");
     CHECK(get_real_moe_layer(id) != nullptr && get_real_moe_layer(id + 1000) == nullptr, "registry lookup");
   });
+  // src/moe/numeric_policy.rs:208-251 and tests/numeric_policy_test.rs, same cases
+  run_test("policy_classification_is_correct", [] {
+    CHECK(!ffn_uses_f32(NumericPolicy::Certified) && !ffn_uses_cuda(NumericPolicy::Certified), "certified");
+    CHECK(ffn_uses_f32(NumericPolicy::Strict) && !ffn_uses_cuda(NumericPolicy::Strict), "strict");
+    CHECK(ffn_uses_f32(NumericPolicy::Fast) && ffn_uses_cuda(NumericPolicy::Fast), "fast");
+    CHECK(std::string(as_str(NumericPolicy::Strict)) == "strict" && std::string(as_str(NumericPolicy::Fast)) == "fast" &&
+              std::string(as_str(NumericPolicy::Certified)) == "certified", "as_str");
+  });
+  run_test("policy_from_str_unknown_is_none_known_ok", [] {
+    CHECK(numeric_policy_from_str("certified") == NumericPolicy::Certified, "certified");
+    CHECK(numeric_policy_from_str("STRICT") == NumericPolicy::Strict, "case");
+    CHECK(numeric_policy_from_str(" fast \n") == NumericPolicy::Fast, "trim");
+    CHECK(numeric_policy_from_str("f64") == NumericPolicy::Certified && numeric_policy_from_str("f32") == NumericPolicy::Strict, "aliases");
+    CHECK(!numeric_policy_from_str("garbage").has_value() && !numeric_policy_from_str("").has_value(), "unknown");
+  });
+  run_test("policy_override_selects_and_clears", [] {
+    clear_numeric_policy_override();
+    const NumericPolicy from_env = numeric_policy();  // Certified unless ATENIA_NUMERIC_POLICY says otherwise
+    const char* env = getenv("ATENIA_NUMERIC_POLICY");
+    CHECK(env || from_env == NumericPolicy::Certified, "no override and no env must mean Certified");
+    set_numeric_policy(NumericPolicy::Strict);
+    CHECK(numeric_policy() == NumericPolicy::Strict, "strict");
+    set_numeric_policy(NumericPolicy::Fast);
+    CHECK(numeric_policy() == NumericPolicy::Fast, "fast");
+    set_numeric_policy(NumericPolicy::Certified);
+    CHECK(numeric_policy() == NumericPolicy::Certified, "certified");
+    clear_numeric_policy_override();
+    CHECK(numeric_policy() == from_env, "cleared");
+  });
+  run_test("policy_certificate_passes_on_identical_and_fails_on_token_mismatch", [] {
+    std::vector<std::vector<float>> r = {{1.0f, 2.0f, 0.5f}, {0.1f, 0.2f, 9.0f}};
+    std::vector<uint32_t> toks = {1, 2};
+    auto c = PolicyCertificate::compare(NumericPolicy::Strict, r, r, toks, toks);
+    CHECK(c.passes(STRICT_LOGIT_TOLERANCE) && c.argmax_match_rate == 1.0 && c.max_abs_diff == 0.0 && c.rows == 2, "identical");
+    std::vector<std::vector<float>> cand = {{1.0001f, 2.0f, 0.5f}, {0.1f, 0.2f, 9.0001f}};
+    auto c2 = PolicyCertificate::compare(NumericPolicy::Strict, r, cand, toks, toks);
+    CHECK(c2.passes(STRICT_LOGIT_TOLERANCE) && c2.max_abs_diff > 9e-5 && c2.max_abs_diff < 1.1e-4, "tiny drift: %g", c2.max_abs_diff);
+    // mean of the per-row means, root of the mean of the per-row squared rmse
+    const double d0 = (double)1.0001f - 1.0, d1 = (double)9.0001f - 9.0;
+    CHECK(std::fabs(c2.mean_abs_diff - (d0 / 3 + d1 / 3) / 2) < 1e-12, "mean_abs_diff %g", c2.mean_abs_diff);
+    CHECK(std::fabs(c2.rmse - std::sqrt((d0 * d0 / 3 + d1 * d1 / 3) / 2)) < 1e-12, "rmse %g", c2.rmse);
+    auto c3 = PolicyCertificate::compare(NumericPolicy::Strict, r, r, toks, {1, 3});
+    CHECK(!c3.passes(STRICT_LOGIT_TOLERANCE), "token mismatch");
+    std::vector<std::vector<float>> flip = {{2.0f, 1.0f, 0.5f}, {0.1f, 0.2f, 9.0f}};
+    auto c4 = PolicyCertificate::compare(NumericPolicy::Strict, r, flip, toks, toks);
+    CHECK(!c4.passes(STRICT_LOGIT_TOLERANCE) && c4.argmax_match_rate == 0.5, "argmax flip");
+    // rows of different length are skipped, as NumericalMetrics::compute returns None
+    std::vector<std::vector<float>> ragged = {{1.0f, 2.0f}, {0.1f, 0.2f, 9.0f}};
+    auto c5 = PolicyCertificate::compare(NumericPolicy::Fast, r, ragged, toks, toks);
+    CHECK(c5.rows == 1 && c5.policy == NumericPolicy::Fast, "skipped rows");
+    CHECK(!NumericalMetrics::compute({}, {}).has_value() && !NumericalMetrics::compute({1.f}, {1.f, 2.f}).has_value(), "None cases");
+    auto m = NumericalMetrics::compute({1.f, 5.f, 5.f}, {1.f, 5.f, 4.f}).value();
+    CHECK(m.argmax_match && m.max_abs_diff == 1.0 && m.passes(1.5) && !m.passes(1.0), "first maximum wins; gate is strict");
+  });
   if (no_gpu) {
     run_test("forward_without_device_fails_loudly", [] {
       RealMoeLayer l = layer_from(synthetic(4, 2, 8, 16));
@@ -308,6 +362,56 @@ int main(int argc, char** argv) {
         CHECK(std::fabs(w[t * fx.k + s] - ow[s]) <= 1.2e-7f * std::fabs(ow[s]), "routing weight");
       }
     }
+  });
+  run_test("strict_policy_accumulates_in_f32_like_the_reference", [&] {
+    // f32 layer under Strict / Fast: the oracle's f32-accumulating expert (dense.rs:120-140);
+    // routing must not move; Certified afterwards is the f64 result again.
+    Fixture fx = synthetic(4, 2, 64, 96);
+    RealMoeLayer layer = layer_from(fx);
+    const int T = 6, d = fx.d;
+    std::vector<float> x = seeded(21, (size_t)T * d);
+    OraLayer ol = ora_of(fx, 0);
+    auto oracle_rows = [&](int policy) {
+      std::vector<float> out((size_t)T * d);
+      for (int t = 0; t < T; ++t) {
+        std::vector<float> ow(fx.k);
+        std::vector<int32_t> oi(fx.k);
+        int32_t err = 0;
+        CHECK(ora_layer_forward_with(&ol, x.data() + (size_t)t * d, 0, policy, out.data() + (size_t)t * d,
+                                     oi.data(), ow.data(), &err) == 0, "oracle");
+      }
+      return out;
+    };
+    const std::vector<float> want_cert = oracle_rows(0), want_strict = oracle_rows(1);
+    CHECK(metrics(want_cert, want_strict).max_abs_diff > 0.0, "the two arithmetics should differ somewhere");
+    std::vector<int32_t> idx_cert, idx_strict;
+    clear_numeric_policy_override();
+    auto cert = layer.forward(x).unwrap();
+    layer.route(x, MoeExecutionConvention::Atenia, &idx_cert).unwrap();
+    for (NumericPolicy p : {NumericPolicy::Strict, NumericPolicy::Fast}) {
+      set_numeric_policy(p);
+      auto got = layer.forward(x).unwrap();
+      layer.route(x, MoeExecutionConvention::Atenia, &idx_strict).unwrap();
+      size_t differ = 0;
+      for (size_t i = 0; i < got.size(); ++i) differ += memcmp(&got[i], &want_strict[i], 4) != 0;
+      // bit for bit, up to the last ulp of the device's f64 exp inside silu
+      CHECK(differ * 1000 <= got.size(), "%zu of %zu elements differ from the f32-accumulating oracle", differ, got.size());
+      CHECK(metrics(got, want_strict).max_abs_diff <= 1e-6 * (1.0 + metrics(want_strict, std::vector<float>(got.size(), 0.f)).max_abs_diff), "drift");
+      CHECK(idx_strict == idx_cert, "routing moved under %s", as_str(p));
+    }
+    set_numeric_policy(NumericPolicy::Certified);
+    auto again = layer.forward(x).unwrap();
+    CHECK(memcmp(again.data(), cert.data(), cert.size() * 4) == 0, "Certified after Strict differs from Certified before");
+    CHECK(metrics(cert, want_cert).max_abs_diff < 1e-5, "certified vs oracle");
+    clear_numeric_policy_override();
+    // the certificate the reference's harness would form
+    std::vector<std::vector<float>> ref_rows, cand_rows;
+    for (int t = 0; t < T; ++t) {
+      ref_rows.emplace_back(want_cert.begin() + (size_t)t * d, want_cert.begin() + (size_t)(t + 1) * d);
+      cand_rows.emplace_back(want_strict.begin() + (size_t)t * d, want_strict.begin() + (size_t)(t + 1) * d);
+    }
+    auto cert_c = PolicyCertificate::compare(NumericPolicy::Strict, ref_rows, cand_rows, {1, 2}, {1, 2});
+    CHECK(cert_c.passes(STRICT_LOGIT_TOLERANCE), "strict certificate: max %g argmax %g", cert_c.max_abs_diff, cert_c.argmax_match_rate);
   });
   run_test("identical_experts_reproduce_single_expert", [&] {
     Fixture fx = synthetic(4, 2, 8, 16, true);
