@@ -33,6 +33,7 @@ struct StreamParams {
   int n_kgroups;        // per-group int8: scale groups along K
   int64_t w_stride_u4;  // uint4 between experts
   int n_rows;           // unpadded N
+  int n_pad;            // N padded to whole 16-row strips
   int nkb;              // K blocks per strip
   const uint16_t* a;    // bf16 rows: x [T, a_stride] (up) or h [rows, a_stride] (down)
   int a_stride;
@@ -90,10 +91,18 @@ __device__ inline f32x4 mfma(bf16x8 a, bf16x8 b, f32x4 c) {
 //       accumulated on its own and added to the running sum times the scale of its group,
 //       sum_g s[n, g] * (sum_{k in g} q[n, k] x[k]), which is the reference's
 //       sum_k (q * s) x (src/tensor/quantizer.rs:175-248) up to f32 rounding
+// A second parameter set rides along for the shared expert: the workgroups with blockIdx.y ==
+// shared_y stream the shared expert's strips (its own weights, width, input and output rows)
+// in the same launch as the routed experts', one launch less per phase for layers that have one.
 template <int MT, bool INT8, bool UP, int WAVES, bool PG>
-__global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p) {
+__global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p_routed,
+                                                                StreamParams p_shared,
+                                                                int shared_y) {
   constexpr int kWavesPerWg = WAVES;
-  const int u = blockIdx.y;
+  const bool sh = (int)blockIdx.y == shared_y;
+  const StreamParams& p = sh ? p_shared : p_routed;
+  if ((int)blockIdx.x * 16 >= p.n_pad) return;  // the grid spans the wider of the two
+  const int u = sh ? 0 : blockIdx.y;
   if (u >= *p.g.n_active) return;
   const int e = p.g.active[u];
   const int base = p.g.offsets[e];
@@ -123,7 +132,7 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p) 
   uint4 xa0[U][MT][AV], xa1[U][MT][AV];
   // Per-group scales of this lane's output row (column mm of the D layout), one per k group;
   // they are requested together with the weight blocks they belong to.
-  const size_t n_pad_s = (size_t)gridDim.x * 16;  // scale rows per k group
+  const size_t n_pad_s = (size_t)p.n_pad;  // scale rows per k group
   const float* psa = PG ? p.sa + (size_t)e * p.n_kgroups * n_pad_s + nb * 16 + mm : nullptr;
   const float* psb = PG && UP ? p.sb + (size_t)e * p.n_kgroups * n_pad_s + nb * 16 + mm : nullptr;
   float sA0[PG ? U : 1], sB0[PG && UP ? U : 1], sA1[PG ? U : 1], sB1[PG && UP ? U : 1];
@@ -382,25 +391,28 @@ __global__ __launch_bounds__(1024) void ffn_down_decode1_kernel(StreamParams p, 
 }
 
 template <bool INT8, bool UP>
-hipError_t launch_stream(const StreamParams& p, int n_pad, int n_groups, int rows_max,
-                         hipStream_t s) {
+hipError_t launch_stream(const StreamParams& p, int n_groups, int rows_max, hipStream_t s,
+                         const StreamParams* shared) {
   // Up to 32 rows per expert per workgroup; larger groups take more workgroups along z.
   int mt = rows_max <= 16 ? 1 : 2;
-  dim3 grid(n_pad / 16, n_groups, (rows_max + 16 * mt - 1) / (16 * mt));
+  const StreamParams ps = shared ? *shared : p;
+  const int shared_y = shared ? n_groups : -1;
+  const int n_pad = shared && shared->n_pad > p.n_pad ? shared->n_pad : p.n_pad;
+  dim3 grid(n_pad / 16, n_groups + (shared ? 1 : 0), (rows_max + 16 * mt - 1) / (16 * mt));
   // The down projection has few strips (d / 16) and a long K (f): eight K slices per strip
   // keep enough loads in flight; gate/up has 2f / 16 strips and uses four.
   constexpr int W = UP ? 4 : 8;
   if (INT8 && p.group_blocks > 0) {
     if (mt == 1)
-      ffn_stream_kernel<1, INT8, UP, W, INT8><<<grid, 64 * W, 0, s>>>(p);
+      ffn_stream_kernel<1, INT8, UP, W, INT8><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
     else
-      ffn_stream_kernel<2, INT8, UP, W, INT8><<<grid, 64 * W, 0, s>>>(p);
+      ffn_stream_kernel<2, INT8, UP, W, INT8><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
     return hipGetLastError();
   }
   if (mt == 1)
-    ffn_stream_kernel<1, INT8, UP, W, false><<<grid, 64 * W, 0, s>>>(p);
+    ffn_stream_kernel<1, INT8, UP, W, false><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
   else
-    ffn_stream_kernel<2, INT8, UP, W, false><<<grid, 64 * W, 0, s>>>(p);
+    ffn_stream_kernel<2, INT8, UP, W, false><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
   return hipGetLastError();
 }
 
@@ -409,9 +421,8 @@ hipError_t launch_stream(const StreamParams& p, int n_pad, int n_groups, int row
 hipError_t launch_ffn_up_f32(const FfnArgs& a, hipStream_t s);
 hipError_t launch_ffn_down_f32(const FfnArgs& a, hipStream_t s);
 
-hipError_t launch_ffn_up(const FfnArgs& a, hipStream_t s) {
-  if (a.wdtype == ATENIA_MOE_WEIGHT_F32) return launch_ffn_up_f32(a, s);
-  if (a.use_tiled) return launch_ffn_up_tiled(a, s);
+namespace {
+StreamParams stream_params_up(const FfnArgs& a) {
   const bool int8 = a.wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
   StreamParams p;
   p.wa = (const uint4*)a.gate.w;
@@ -422,19 +433,16 @@ hipError_t launch_ffn_up(const FfnArgs& a, hipStream_t s) {
   p.n_kgroups = a.gate.n_kgroups;
   p.w_stride_u4 = a.gate.expert_stride / 16;
   p.n_rows = a.gate.n_rows;
+  p.n_pad = a.gate.n_pad;
   p.nkb = a.gate.k_pad / (int8 ? kKbInt8 : kKbBf16);
   p.a = (const uint16_t*)a.x;
   p.a_stride = a.x_stride;
   p.out = a.h;
   p.out_stride = a.h_stride;
   p.g = a.g;
-  return int8 ? launch_stream<true, true>(p, a.gate.n_pad, a.n_groups_max, a.rows_max, s)
-              : launch_stream<false, true>(p, a.gate.n_pad, a.n_groups_max, a.rows_max, s);
+  return p;
 }
-
-hipError_t launch_ffn_down(const FfnArgs& a, hipStream_t s) {
-  if (a.wdtype == ATENIA_MOE_WEIGHT_F32) return launch_ffn_down_f32(a, s);
-  if (a.use_tiled) return launch_ffn_down_tiled(a, s);
+StreamParams stream_params_down(const FfnArgs& a) {
   const bool int8 = a.wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
   StreamParams p;
   p.wa = (const uint4*)a.down.w;
@@ -445,14 +453,50 @@ hipError_t launch_ffn_down(const FfnArgs& a, hipStream_t s) {
   p.n_kgroups = a.down.n_kgroups;
   p.w_stride_u4 = a.down.expert_stride / 16;
   p.n_rows = a.down.n_rows;
+  p.n_pad = a.down.n_pad;
   p.nkb = a.down.k_pad / (int8 ? kKbInt8 : kKbBf16);
   p.a = (const uint16_t*)a.h;
   p.a_stride = a.h_stride;
   p.out = a.y;
   p.out_stride = a.y_stride;
   p.g = a.g;
-  return int8 ? launch_stream<true, false>(p, a.down.n_pad, a.n_groups_max, a.rows_max, s)
-              : launch_stream<false, false>(p, a.down.n_pad, a.n_groups_max, a.rows_max, s);
+  return p;
+}
+// The shared expert can ride in the routed experts' launch when both stream (no tiles, no f32
+// weights), are stored alike and see the same rows bound.
+bool can_fuse_shared(const FfnArgs& a, const FfnArgs* sh) {
+  return sh && a.wdtype != ATENIA_MOE_WEIGHT_F32 && sh->wdtype == a.wdtype && !a.use_tiled &&
+         !sh->use_tiled && sh->rows_max == a.rows_max &&
+         (sh->gate.group_blocks > 0) == (a.gate.group_blocks > 0);
+}
+}  // namespace
+
+bool ffn_stream_fuses_shared(const FfnArgs& a, const FfnArgs& shared) {
+  return can_fuse_shared(a, &shared);
+}
+
+hipError_t launch_ffn_up(const FfnArgs& a, hipStream_t s, const FfnArgs* shared) {
+  if (a.wdtype == ATENIA_MOE_WEIGHT_F32) return launch_ffn_up_f32(a, s);
+  if (a.use_tiled) return launch_ffn_up_tiled(a, s);
+  const bool int8 = a.wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
+  const StreamParams p = stream_params_up(a);
+  StreamParams ps;
+  const bool fuse = can_fuse_shared(a, shared);
+  if (fuse) ps = stream_params_up(*shared);
+  return int8 ? launch_stream<true, true>(p, a.n_groups_max, a.rows_max, s, fuse ? &ps : nullptr)
+              : launch_stream<false, true>(p, a.n_groups_max, a.rows_max, s, fuse ? &ps : nullptr);
+}
+
+hipError_t launch_ffn_down(const FfnArgs& a, hipStream_t s, const FfnArgs* shared) {
+  if (a.wdtype == ATENIA_MOE_WEIGHT_F32) return launch_ffn_down_f32(a, s);
+  if (a.use_tiled) return launch_ffn_down_tiled(a, s);
+  const bool int8 = a.wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
+  const StreamParams p = stream_params_down(a);
+  StreamParams ps;
+  const bool fuse = can_fuse_shared(a, shared);
+  if (fuse) ps = stream_params_down(*shared);
+  return int8 ? launch_stream<true, false>(p, a.n_groups_max, a.rows_max, s, fuse ? &ps : nullptr)
+              : launch_stream<false, false>(p, a.n_groups_max, a.rows_max, s, fuse ? &ps : nullptr);
 }
 
 bool ffn_down_decode1_supported(int T, int k, int wdtype, bool tiled, bool shared) {
@@ -461,21 +505,7 @@ bool ffn_down_decode1_supported(int T, int k, int wdtype, bool tiled, bool share
 
 hipError_t launch_ffn_down_decode1(const FfnArgs& a, hipStream_t s) {
   const bool int8 = a.wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
-  StreamParams p;
-  p.wa = (const uint4*)a.down.w;
-  p.wb = nullptr;
-  p.sa = a.down.scale;
-  p.sb = nullptr;
-  p.group_blocks = a.down.group_blocks;
-  p.n_kgroups = a.down.n_kgroups;
-  p.w_stride_u4 = a.down.expert_stride / 16;
-  p.n_rows = a.down.n_rows;
-  p.nkb = a.down.k_pad / (int8 ? kKbInt8 : kKbBf16);
-  p.a = (const uint16_t*)a.h;
-  p.a_stride = a.h_stride;
-  p.out = a.y;
-  p.out_stride = a.y_stride;
-  p.g = a.g;
+  const StreamParams p = stream_params_down(a);
   const dim3 grid(a.down.n_pad / 16);
   const int threads = 64 * 8 * a.fuse_k;
   if (int8)

@@ -497,10 +497,12 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
     fsd.max_row_tiles = (T + kTileM - 1) / kTileM;
   }
 
+  // Small batches stream both the routed experts and the shared one: one launch per phase.
+  const bool fuse_shared = L->fs > 0 && ffn_stream_fuses_shared(fa, fsd);
   if (first <= kStageFfn) {
-    HIP_TRY(launch_ffn_up(fa, s));
+    HIP_TRY(launch_ffn_up(fa, s, fuse_shared ? &fsd : nullptr));
     L->launches[2] = 1;
-    if (L->fs > 0) {
+    if (L->fs > 0 && !fuse_shared) {
       HIP_TRY(launch_ffn_up(fsd, s));
       L->launches[2] = 2;
     }
@@ -519,10 +521,10 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
       fa.fuse_k = L->k;
       HIP_TRY(launch_ffn_down_decode1(fa, s));
     } else {
-      HIP_TRY(launch_ffn_down(fa, s));
+      HIP_TRY(launch_ffn_down(fa, s, fuse_shared ? &fsd : nullptr));
     }
     L->launches[3] = 1;
-    if (L->fs > 0) {
+    if (L->fs > 0 && !fuse_shared) {
       HIP_TRY(launch_ffn_down(fsd, s));
       L->launches[3] = 2;
     }
