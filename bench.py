@@ -285,7 +285,7 @@ def main():
                     help="headline batch size T (default: the config's largest)")
     ap.add_argument("--decode-tokens", type=int, default=1, help="decode batch (0 = skip)")
     ap.add_argument("--sweep", type=str, default="", help="extra batch sizes, comma separated")
-    ap.add_argument("--cpu-tokens", type=int, default=16,
+    ap.add_argument("--cpu-tokens", type=int, default=1024,
                     help="tokens of the CPU-baseline sample (0 = skip)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (reference point for HBM counters)")
