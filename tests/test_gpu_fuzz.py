@@ -1,0 +1,50 @@
+"""Seeded random layer shapes through the whole pipeline: expert counts from 1 to 70, any top-k,
+widths that are not multiples of the kernels' tile sizes, batch sizes on both sides of every
+kernel-selection threshold, all three storage types and both conventions.  Same bars as the
+fixed cases of test_gpu_parity.py (routing and grouping bit-exact, outputs within tolerance, and
+within 1e-3 of the NumPy model of the blocked kernels' arithmetic)."""
+import numpy as np
+import pytest
+
+from ateniaengine_amd import capi
+from tests import synth as S
+from tests.test_gpu_parity import TOL_BF16_TOY, TOL_F32, check_layer
+
+pytestmark = pytest.mark.gpu
+
+
+def _cases(n, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(n):
+        E = int(rng.choice([1, 2, 3, 5, 8, 17, 33, 60, 64, 65, 70]))
+        k = int(rng.integers(1, min(E, 8) + 1))
+        d = int(rng.choice([8, 24, 37, 64, 100, 128, 200, 256, 320]))
+        f = int(rng.choice([8, 20, 33, 64, 96, 130, 256, 400]))
+        shared = bool(rng.integers(0, 2))
+        fs = int(rng.choice([16, 50, 128, 272])) if shared else 0
+        gated = shared and bool(rng.integers(0, 2))
+        conv = int(rng.integers(0, 2)) if shared else 0
+        wd = [capi.WEIGHT_F32, capi.WEIGHT_BF16, capi.WEIGHT_INT8_W8A16][i % 3]
+        T = int(rng.choice([1, 2, 3, 15, 16, 17, 31, 32, 33, 47, 48, 49, 63, 64, 65, 127, 128, 129,
+                            255, 256, 257, 300, 511, 513, 800, 1100]))
+        if wd == capi.WEIGHT_F32:
+            T = min(T, 130)  # the f32 path is the slow one on both sides
+        out.append(pytest.param(E, k, d, f, fs, gated, conv, wd, T, 1000 + i,
+                                id=f"{i}-E{E}k{k}d{d}f{f}s{fs}g{int(gated)}c{conv}w{wd}T{T}"))
+    return out
+
+
+@pytest.mark.parametrize("E,k,d,f,fs,gated,conv,wd,T,seed", _cases(150, 20240607))
+def test_random_layer(ora, E, k, d, f, fs, gated, conv, wd, T, seed):
+    W = S.make_weights(seed, E, d, f, f_s=fs, gated=gated, router_std=1.0 / np.sqrt(d),
+                       outlier_frac=0.01 if wd == capi.WEIGHT_INT8_W8A16 else 0.0)
+    oL, gL = S.build_pair(ora, W, k, conv, wd)
+    with gL:
+        x = S.make_tokens(seed + 1, T, d, bf16=wd != capi.WEIGHT_F32)
+        tol = TOL_F32 if wd == capi.WEIGHT_F32 else TOL_BF16_TOY
+        sample = None if T <= 64 else sorted(set(np.linspace(0, T - 1, 48).astype(int).tolist()))
+        check_layer(ora, oL, gL, x, tol, sample=sample)
+        # a second, smaller batch on the same handle (grow-only workspace, stale state)
+        T2 = max(1, T // 3)
+        check_layer(ora, oL, gL, x[:T2], tol, sample=None if T2 <= 64 else range(0, T2, max(1, T2 // 40)))
