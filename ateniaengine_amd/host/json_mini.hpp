@@ -59,11 +59,22 @@ class Parser {
     p_ = end_;
     return Value();
   }
+  // Containers nest by recursion; a header or config that nests deeper than any real one is
+  // rejected instead of being followed down the stack.
+  static constexpr int kMaxDepth = 64;
+  int depth_ = 0;
+  struct DepthGuard {
+    int& d;
+    explicit DepthGuard(int& x) : d(x) { ++d; }
+    ~DepthGuard() { --d; }
+  };
   Value value() {
     ws();
     if (p_ >= end_) return fail();
     Value v;
     const char c = *p_;
+    if ((c == '{' || c == '[') && depth_ >= kMaxDepth) return fail();
+    DepthGuard guard(depth_);
     if (c == '{') {
       ++p_;
       v.kind = Value::Object;

@@ -704,6 +704,13 @@ int main(int argc, char** argv) {
     spit(work + "/wrong_len.safetensors", le64(wrong_len.size()) + wrong_len + std::string(8, '\0'));
     auto rd = SafetensorsReader::open(work + "/wrong_len.safetensors");
     CHECK(rd.is_ok() && !rd.value().to_vec_f32("a"), "byte range that disagrees with shape x dtype");
+    // nesting far beyond any real header must be refused, not followed down the stack
+    const std::string deep = "{\"a\":" + std::string(200000, '[') + "}";
+    spit(work + "/deep.safetensors", le64(deep.size()) + deep);
+    CHECK(SafetensorsReader::open(work + "/deep.safetensors").is_err(), "deeply nested header");
+    CHECK(MoeConfig::from_json_str(std::string(200000, '[')).is_err(), "deeply nested config");
+    CHECK(MoeConfig::from_json_str("{\"num_local_experts\": " + std::string(100, '[') + "8" + std::string(100, ']') + "}").is_err() ||
+              true, "moderate nesting either parses or is refused");
     const std::string empty = "{}";
     spit(work + "/empty.safetensors", le64(empty.size()) + empty);
     auto e = SafetensorsReader::open(work + "/empty.safetensors");
