@@ -464,15 +464,20 @@ StreamParams stream_params_down(const FfnArgs& a) {
 }
 // The shared expert can ride in the routed experts' launch when both stream (no tiles, no f32
 // weights), are stored alike and see the same rows bound.
-bool can_fuse_shared(const FfnArgs& a, const FfnArgs* sh) {
-  return sh && a.wdtype != ATENIA_MOE_WEIGHT_F32 && sh->wdtype == a.wdtype && !a.use_tiled &&
-         !sh->use_tiled && sh->rows_max == a.rows_max &&
-         (sh->gate.group_blocks > 0) == (a.gate.group_blocks > 0);
+// In the down phase a strip's K is the expert's width: a shared expert much wider than the
+// routed ones would make its strips the launch's critical path (measured: Qwen1.5-MoE, shared
+// 4x as wide, 20 us fused against 18 us as two launches), so it keeps its own launch then.
+bool can_fuse_shared(const FfnArgs& a, const FfnArgs* sh, bool down_phase) {
+  if (!(sh && a.wdtype != ATENIA_MOE_WEIGHT_F32 && sh->wdtype == a.wdtype && !a.use_tiled &&
+        !sh->use_tiled && sh->rows_max == a.rows_max &&
+        (sh->gate.group_blocks > 0) == (a.gate.group_blocks > 0)))
+    return false;
+  return !down_phase || sh->down.k_pad <= 2 * a.down.k_pad;
 }
 }  // namespace
 
-bool ffn_stream_fuses_shared(const FfnArgs& a, const FfnArgs& shared) {
-  return can_fuse_shared(a, &shared);
+bool ffn_stream_fuses_shared(const FfnArgs& a, const FfnArgs& shared, bool down_phase) {
+  return can_fuse_shared(a, &shared, down_phase);
 }
 
 hipError_t launch_ffn_up(const FfnArgs& a, hipStream_t s, const FfnArgs* shared) {
@@ -481,7 +486,7 @@ hipError_t launch_ffn_up(const FfnArgs& a, hipStream_t s, const FfnArgs* shared)
   const bool int8 = a.wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
   const StreamParams p = stream_params_up(a);
   StreamParams ps;
-  const bool fuse = can_fuse_shared(a, shared);
+  const bool fuse = can_fuse_shared(a, shared, false);
   if (fuse) ps = stream_params_up(*shared);
   return int8 ? launch_stream<true, true>(p, a.n_groups_max, a.rows_max, s, fuse ? &ps : nullptr)
               : launch_stream<false, true>(p, a.n_groups_max, a.rows_max, s, fuse ? &ps : nullptr);
@@ -493,7 +498,7 @@ hipError_t launch_ffn_down(const FfnArgs& a, hipStream_t s, const FfnArgs* share
   const bool int8 = a.wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
   const StreamParams p = stream_params_down(a);
   StreamParams ps;
-  const bool fuse = can_fuse_shared(a, shared);
+  const bool fuse = can_fuse_shared(a, shared, true);
   if (fuse) ps = stream_params_down(*shared);
   return int8 ? launch_stream<true, false>(p, a.n_groups_max, a.rows_max, s, fuse ? &ps : nullptr)
               : launch_stream<false, false>(p, a.n_groups_max, a.rows_max, s, fuse ? &ps : nullptr);

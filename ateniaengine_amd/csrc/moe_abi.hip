@@ -498,11 +498,12 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   }
 
   // Small batches stream both the routed experts and the shared one: one launch per phase.
-  const bool fuse_shared = L->fs > 0 && ffn_stream_fuses_shared(fa, fsd);
+  const bool fuse_shared_up = L->fs > 0 && ffn_stream_fuses_shared(fa, fsd, false);
+  const bool fuse_shared_down = L->fs > 0 && ffn_stream_fuses_shared(fa, fsd, true);
   if (first <= kStageFfn) {
-    HIP_TRY(launch_ffn_up(fa, s, fuse_shared ? &fsd : nullptr));
+    HIP_TRY(launch_ffn_up(fa, s, fuse_shared_up ? &fsd : nullptr));
     L->launches[2] = 1;
-    if (L->fs > 0 && !fuse_shared) {
+    if (L->fs > 0 && !fuse_shared_up) {
       HIP_TRY(launch_ffn_up(fsd, s));
       L->launches[2] = 2;
     }
@@ -521,10 +522,10 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
       fa.fuse_k = L->k;
       HIP_TRY(launch_ffn_down_decode1(fa, s));
     } else {
-      HIP_TRY(launch_ffn_down(fa, s, fuse_shared ? &fsd : nullptr));
+      HIP_TRY(launch_ffn_down(fa, s, fuse_shared_down ? &fsd : nullptr));
     }
     L->launches[3] = 1;
-    if (L->fs > 0 && !fuse_shared) {
+    if (L->fs > 0 && !fuse_shared_down) {
       HIP_TRY(launch_ffn_down(fsd, s));
       L->launches[3] = 2;
     }

@@ -151,11 +151,11 @@ bool tiled_supported(const WeightSet& w, int wdtype);
 bool tiled_down_splits_tail(const WeightSet& down, int wdtype);
 hipError_t launch_ffn_up_tiled(const FfnArgs& a, hipStream_t s);
 hipError_t launch_ffn_down_tiled(const FfnArgs& a, hipStream_t s);
-// `shared` (may be null): the shared expert's arguments; when ffn_stream_fuses_shared(a, *shared)
-// holds, its work is done by the same launch and the caller must not launch it again.
+// `shared` (may be null): the shared expert's arguments; when ffn_stream_fuses_shared(a, *shared,
+// phase) holds, its work is done by the same launch and the caller must not launch it again.
 hipError_t launch_ffn_up(const FfnArgs& a, hipStream_t s, const FfnArgs* shared = nullptr);
 hipError_t launch_ffn_down(const FfnArgs& a, hipStream_t s, const FfnArgs* shared = nullptr);
-bool ffn_stream_fuses_shared(const FfnArgs& a, const FfnArgs& shared);
+bool ffn_stream_fuses_shared(const FfnArgs& a, const FfnArgs& shared, bool down_phase);
 // One token, at most two experts per token, blocked (bf16 / int8) weights: the down projection
 // of all the token's experts and the weighted combine in one launch.
 bool ffn_down_decode1_supported(int T, int k, int wdtype, bool tiled, bool shared);
