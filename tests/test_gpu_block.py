@@ -140,3 +140,27 @@ def test_tiny_mixtral_logits_with_gpu_blocks(ora, policy):
             L.close()
     assert np.abs(got - want).max() < 1e-6
     assert np.array_equal(got.argmax(-1), want.argmax(-1))
+
+
+@pytest.mark.parametrize("name,conv", [("mixtral_scale", capi.CONVENTION_ATENIA),
+                                       ("qwen_scale", capi.CONVENTION_HUGGINGFACE_QWEN)])
+@pytest.mark.parametrize("policy", [capi.NORM_GRAPH_F32, capi.NORM_F64])
+def test_scale_fixture_logits_with_gpu_blocks(ora, name, conv, policy):
+    """The reference's topology fixtures (tests/moe_scale_cert_test.rs) with the GPU as every
+    layer's FFN block: grouped-head Mixtral, and Qwen2-MoE with its sigmoid-gated shared expert."""
+    cfg, t = TM.load(name)
+    layers = {}
+
+    def block(layer, x1, gamma, eps):
+        if layer not in layers:
+            layers[layer] = capi.Layer(top_k=TM.top_k(cfg), convention=conv,
+                                       weight_dtype=capi.WEIGHT_F32, **TM.moe_arrays(t, layer))
+        return layers[layer].block_forward(x1, gamma, eps, policy)
+
+    try:
+        got, want = TM.logits(block, name), TM.hf_logits(name)
+    finally:
+        for L in layers.values():
+            L.close()
+    assert np.abs(got - want).max() < 1e-6, np.abs(got - want).max()
+    assert np.array_equal(got.argmax(-1), want.argmax(-1))

@@ -102,6 +102,50 @@ def test_tiny_mixtral_logits_match_hf(ora, policy):
     assert np.array_equal(got.argmax(-1), want.argmax(-1))
 
 
+# Topology fixtures of the reference's tests/moe_scale_cert_test.rs: Mixtral with grouped heads
+# (8 experts, top-2, renormalised) and Qwen2-MoE (16 experts, top-4 raw weights, sigmoid-gated
+# shared expert).  The block's convention is what differs between them.
+SCALE_CONVENTION = {"mixtral_scale": "ATENIA", "qwen_scale": "HUGGINGFACE_QWEN"}
+
+
+@pytest.mark.parametrize("name", TM.SCALE)
+@pytest.mark.parametrize("policy", [0, 1])
+def test_scale_fixture_logits_match_hf(ora, name, policy):
+    cfg, t = TM.load(name)
+    conv = getattr(ora, SCALE_CONVENTION[name])
+
+    def block(layer, x1, gamma, eps):
+        L = ora.Layer(top_k=TM.top_k(cfg), convention=conv, **TM.moe_arrays(t, layer))
+        return L.block_forward(x1, gamma, eps, policy)[0]
+
+    got, want = TM.logits(block, name), TM.hf_logits(name)
+    assert np.abs(got - want).max() < 1e-6, np.abs(got - want).max()
+    assert np.array_equal(got.argmax(-1), want.argmax(-1))
+
+
+def test_qwen_scale_detects_the_wrong_convention(ora):
+    """Renormalised weights, an ungated shared expert or no shared expert at all each miss the
+    HuggingFace logits by far more than the tolerance."""
+    cfg, t = TM.load("qwen_scale")
+    want = TM.hf_logits("qwen_scale")
+
+    def with_(conv, drop_gate=False, drop_shared=False):
+        def block(layer, x1, gamma, eps):
+            a = TM.moe_arrays(t, layer)
+            if drop_gate or drop_shared:
+                a.pop("shared_gate")
+            if drop_shared:
+                for n in ("s_gate", "s_up", "s_down"):
+                    a.pop(n)
+            return ora.Layer(top_k=TM.top_k(cfg), convention=conv, **a).block_forward(x1, gamma, eps, 0)[0]
+        return np.abs(TM.logits(block, "qwen_scale") - want).max()
+
+    assert with_(ora.HUGGINGFACE_QWEN) < 1e-6
+    assert with_(ora.ATENIA) > 1e-4                               # renormalised + ungated
+    assert with_(ora.HUGGINGFACE_QWEN, drop_gate=True) > 1e-4     # raw weights, ungated shared
+    assert with_(ora.HUGGINGFACE_QWEN, drop_shared=True) > 1e-4   # no shared expert
+
+
 def test_tiny_mixtral_detects_a_broken_block(ora):
     """The fixture has teeth: no residual, no normalisation, or raw (not renormalised) top-k
     weights each move the logits far beyond the tolerance.  (Its gamma vectors are all ones, so
