@@ -143,11 +143,13 @@ def test_tiny_mixtral_logits_with_gpu_blocks(ora, policy):
 
 
 @pytest.mark.parametrize("name,conv", [("mixtral_scale", capi.CONVENTION_ATENIA),
-                                       ("qwen_scale", capi.CONVENTION_HUGGINGFACE_QWEN)])
+                                       ("qwen_scale", capi.CONVENTION_HUGGINGFACE_QWEN),
+                                       ("deepseek_scale", capi.CONVENTION_HUGGINGFACE_QWEN)])
 @pytest.mark.parametrize("policy", [capi.NORM_GRAPH_F32, capi.NORM_F64])
 def test_scale_fixture_logits_with_gpu_blocks(ora, name, conv, policy):
     """The reference's topology fixtures (tests/moe_scale_cert_test.rs) with the GPU as every
-    layer's FFN block: grouped-head Mixtral, and Qwen2-MoE with its sigmoid-gated shared expert."""
+    layer's FFN block: grouped-head Mixtral, Qwen2-MoE with its sigmoid-gated shared expert, and
+    DeepSeek-V2 (top-6 of 16, two fused shared experts, latent attention in the NumPy part)."""
     cfg, t = TM.load(name)
     layers = {}
 
