@@ -417,6 +417,114 @@ int pack(const std::vector<const std::vector<float>*>& mats, size_t rows, size_t
 
 // The C-ABI handle for (convention, with shared expert), created and uploaded on first use.
 // Caller holds dev_->mu.
+// ---- unit-level forwards of MoeDenseExpert / MoeDenseLayer ---------------------------------------
+namespace {
+// The routed experts as a RealMoeLayer with k experts per token; `renormalize` picks the
+// convention (there is no shared expert, so the conventions differ in nothing else).
+Result<std::vector<float>, MoeSparseError> run_routed(const MoeDenseLayer& layer,
+                                                       const std::vector<float>& x, size_t k,
+                                                       bool renormalize,
+                                                       std::vector<int32_t>* indices,
+                                                       std::vector<float>* weights) {
+  typedef Result<std::vector<float>, MoeSparseError> R;
+  MoeSparseError e{MoeSparseError::Dense};
+  if (x.size() != layer.d_model) {
+    e.dense = MoeDenseError{MoeDenseError::DimMismatch, "router input", layer.d_model, x.size()};
+    return R::Err(e);
+  }
+  if (k == 0) return R::Err(MoeSparseError{MoeSparseError::ZeroK});
+  if (k > layer.num_experts()) {
+    MoeSparseError ke{MoeSparseError::KExceedsExperts};
+    ke.k = k;
+    ke.num_experts = layer.num_experts();
+    return R::Err(ke);
+  }
+  auto cfg = MoeLayerConfig::make(layer.num_experts(), k, false, layer.d_model, layer.d_ff);
+  auto fail_device = [&](const std::string& text) {
+    // no counterpart in the reference (it computes on the CPU): reported as a shape error text
+    static thread_local std::string keep;
+    keep = text;
+    e.dense = MoeDenseError{MoeDenseError::DimMismatch, keep.c_str(), 0, 0};
+    return R::Err(e);
+  };
+  if (cfg.is_err()) return fail_device(cfg.error().to_string());
+  auto real = RealMoeLayer::assemble(cfg.value(), layer, std::nullopt, std::nullopt);
+  if (real.is_err()) return fail_device(real.error().to_string());
+  const MoeExecutionConvention conv =
+      renormalize ? MoeExecutionConvention::Atenia : MoeExecutionConvention::HuggingFaceQwen;
+  auto out = real.value().forward_with(x, conv);
+  if (out.is_err()) {
+    if (out.error().kind == MoeLayerError::Sparse) return R::Err(out.error().sparse);
+    return fail_device(out.error().to_string());
+  }
+  if (indices || weights) {
+    std::vector<int32_t> idx;
+    auto w = real.value().route(x, conv, &idx);
+    if (w.is_err()) return fail_device(w.error().to_string());
+    if (indices) *indices = idx;
+    if (weights) *weights = w.value();
+  }
+  return R::Ok(out.value());
+}
+}  // namespace
+
+Result<MoeSparseForwardOutput, MoeSparseError> MoeDenseLayer::forward_sparse_with(
+    const std::vector<float>& x, size_t k, bool renormalize) const {
+  typedef Result<MoeSparseForwardOutput, MoeSparseError> R;
+  std::vector<int32_t> idx;
+  auto out = run_routed(*this, x, k, renormalize, &idx, nullptr);
+  if (out.is_err()) return R::Err(out.error());
+  MoeSparseForwardOutput r;
+  r.output = out.value();
+  r.selected_experts.assign(idx.begin(), idx.end());
+  return R::Ok(std::move(r));
+}
+
+Result<MoeSparseForwardOutput, MoeSparseError> MoeDenseLayer::forward_sparse(
+    const std::vector<float>& x, size_t k) const {
+  return forward_sparse_with(x, k, true);
+}
+
+Result<MoeRouterOutput, MoeDenseError> MoeDenseLayer::route(const std::vector<float>& x) const {
+  typedef Result<MoeRouterOutput, MoeDenseError> R;
+  if (x.size() != d_model)
+    return R::Err(MoeDenseError{MoeDenseError::DimMismatch, "router input", d_model, x.size()});
+  // all experts, raw weights: the selection lists them in ascending order
+  std::vector<float> w;
+  auto out = run_routed(*this, x, num_experts(), false, nullptr, &w);
+  if (out.is_err()) {
+    if (out.error().kind == MoeSparseError::NonFiniteWeight)  // softmax of non-finite logits
+      return R::Ok(MoeRouterOutput{std::vector<float>(num_experts(), std::nanf(""))});
+    return R::Err(out.error().dense);
+  }
+  return R::Ok(MoeRouterOutput{std::move(w)});
+}
+
+Result<std::vector<float>, MoeDenseError> MoeDenseLayer::forward(const std::vector<float>& x) const {
+  typedef Result<std::vector<float>, MoeDenseError> R;
+  if (x.size() != d_model)
+    return R::Err(MoeDenseError{MoeDenseError::DimMismatch, "router input", d_model, x.size()});
+  auto out = run_routed(*this, x, num_experts(), false, nullptr, nullptr);
+  if (out.is_err()) {
+    if (out.error().kind == MoeSparseError::NonFiniteWeight)
+      return R::Ok(std::vector<float>(d_model, std::nanf("")));
+    return R::Err(out.error().dense);
+  }
+  return R::Ok(out.value());
+}
+
+Result<std::vector<float>, MoeDenseError> MoeDenseExpert::forward(const std::vector<float>& x) const {
+  typedef Result<std::vector<float>, MoeDenseError> R;
+  if (x.size() != d_model)
+    return R::Err(MoeDenseError{MoeDenseError::DimMismatch, "expert input", d_model, x.size()});
+  // a one-expert layer with a zero router: its single routing weight is exactly 1
+  auto layer = MoeDenseLayer::make(d_model, d_ff, std::vector<float>(d_model, 0.f), {*this}, 1);
+  if (layer.is_err()) return R::Err(layer.error());
+  auto out = run_routed(layer.value(), x, 1, true, nullptr, nullptr);
+  if (out.is_err()) return R::Err(out.error().dense);
+  return R::Ok(out.value());
+}
+
 // ---- numeric policy -----------------------------------------------------------------------------
 const char* as_str(NumericPolicy p) {
   switch (p) {

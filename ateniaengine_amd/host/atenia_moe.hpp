@@ -238,6 +238,24 @@ struct MoeDenseExpert {
                                                     std::vector<float> w_gate,
                                                     std::vector<float> w_up,
                                                     std::vector<float> w_down);
+  // y = W_down (silu(W_gate x) * (W_up x)) for one token (src/moe/dense.rs:253-270), on the
+  // device under the active numeric policy.  Unit-level entry: it uploads the expert for the
+  // call; layers that run many tokens go through RealMoeLayer / the registry.
+  Result<std::vector<float>, MoeDenseError> forward(const std::vector<float>& x) const;
+};
+
+// src/moe/dense.rs:189-201 and src/moe/sparse.rs:195-201
+struct MoeRouterOutput {
+  std::vector<float> weights;  // one per expert, softmax of the router logits
+  float weight_sum() const {
+    float s = 0.f;
+    for (float w : weights) s += w;
+    return s;
+  }
+};
+struct MoeSparseForwardOutput {
+  std::vector<float> output;
+  std::vector<size_t> selected_experts;  // ascending
 };
 
 struct MoeDenseLayer {
@@ -250,6 +268,20 @@ struct MoeDenseLayer {
                                                    std::vector<MoeDenseExpert> experts,
                                                    size_t conceptual_top_k);
   size_t num_experts() const { return experts.size(); }
+  // One token through the routed experts, on the device (unit-level entries like
+  // MoeDenseExpert::forward: the layer is uploaded for the call).
+  //   route                softmax(W_router x)                      src/moe/dense.rs:325-337
+  //   forward              every expert, weighted by its softmax weight   :341-359
+  //   forward_sparse[_with] top-k experts, renormalised or raw weights     src/moe/sparse.rs:206-238
+  // A non-finite router weight makes forward() return NaNs, as the reference's arithmetic does,
+  // and forward_sparse an error, as its validation does.
+  Result<MoeRouterOutput, MoeDenseError> route(const std::vector<float>& x) const;
+  Result<std::vector<float>, MoeDenseError> forward(const std::vector<float>& x) const;
+  Result<MoeSparseForwardOutput, MoeSparseError> forward_sparse(const std::vector<float>& x,
+                                                                size_t k) const;
+  Result<MoeSparseForwardOutput, MoeSparseError> forward_sparse_with(const std::vector<float>& x,
+                                                                     size_t k,
+                                                                     bool renormalize) const;
 };
 
 class RealMoeLayer {

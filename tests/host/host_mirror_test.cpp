@@ -33,6 +33,8 @@ int ora_block_forward(const OraLayer* L, const float* x1, size_t n_tokens, const
 void ora_expert_forward(const float* w_gate, const float* w_up, const float* w_down, size_t d, size_t f,
                         const float* x, float* out, int policy);
 void ora_seeded(uint64_t seed, size_t n, float* out);
+void ora_matvec(const float* w, size_t rows, size_t cols, const float* x, float* y);
+void ora_softmax(const float* logits, size_t n, float* out);
 }
 
 static int g_failed = 0, g_run = 0;
@@ -412,6 +414,66 @@ int main(int argc, char** argv) {
     }
     auto cert_c = PolicyCertificate::compare(NumericPolicy::Strict, ref_rows, cand_rows, {1, 2}, {1, 2});
     CHECK(cert_c.passes(STRICT_LOGIT_TOLERANCE), "strict certificate: max %g argmax %g", cert_c.max_abs_diff, cert_c.argmax_match_rate);
+  });
+  run_test("dense_layer_unit_forwards_match_the_oracle", [&] {
+    // MoeDenseExpert::forward, MoeDenseLayer::{route, forward, forward_sparse[_with]} as the
+    // reference's in-module tests use them (src/moe/dense.rs:405-470, src/moe/sparse.rs:341-397)
+    Fixture fx = synthetic(6, 2, 16, 24);
+    RealMoeLayer rl = layer_from(fx);
+    const MoeDenseLayer& layer = rl.routed;
+    const std::vector<float> x = seeded(5, fx.d);
+    OraLayer ol = ora_of(fx, 0);
+    // one expert
+    for (int e : {0, 5}) {
+      std::vector<float> want(fx.d);
+      ora_expert_forward(fx.gate.data() + (size_t)e * fx.f * fx.d, fx.up.data() + (size_t)e * fx.f * fx.d,
+                         fx.down.data() + (size_t)e * fx.d * fx.f, fx.d, fx.f, x.data(), want.data(), 0);
+      auto got = layer.experts[e].forward(x).unwrap();
+      CHECK(metrics(got, want).max_abs_diff <= 1e-6, "expert %d: %g", e, metrics(got, want).max_abs_diff);
+    }
+    // router weights
+    std::vector<float> lg(fx.E), sm(fx.E);
+    ora_matvec(fx.w_router.data(), fx.E, fx.d, x.data(), lg.data());
+    ora_softmax(lg.data(), fx.E, sm.data());
+    auto ro = layer.route(x).unwrap();
+    CHECK(ro.weights.size() == (size_t)fx.E, "one weight per expert");
+    for (int e = 0; e < fx.E; ++e)
+      CHECK(std::fabs(ro.weights[e] - sm[e]) <= 1.2e-7f * sm[e], "weight %d: %g vs %g", e, ro.weights[e], sm[e]);
+    CHECK(std::fabs(ro.weight_sum() - 1.0f) < 1e-5f, "weights sum to one");
+    // sparse, both conventions, against the oracle; selected experts ascending
+    for (int conv = 0; conv < 2; ++conv) {
+      std::vector<float> want(fx.d), ow(fx.k);
+      std::vector<int32_t> oi(fx.k);
+      int32_t err = 0;
+      CHECK(ora_layer_forward_with(&ol, x.data(), conv, 0, want.data(), oi.data(), ow.data(), &err) == 0, "oracle");
+      auto sp = layer.forward_sparse_with(x, fx.k, conv == 0).unwrap();
+      CHECK(metrics(sp.output, want).max_abs_diff <= 1e-6, "sparse conv %d: %g", conv, metrics(sp.output, want).max_abs_diff);
+      CHECK(sp.selected_experts.size() == (size_t)fx.k, "k experts");
+      for (int s = 0; s < fx.k; ++s) CHECK((int32_t)sp.selected_experts[s] == oi[s], "selected expert %d", s);
+    }
+    auto sp_default = layer.forward_sparse(x, fx.k).unwrap();
+    auto sp_renorm = layer.forward_sparse_with(x, fx.k, true).unwrap();
+    CHECK(sp_default.output == sp_renorm.output, "forward_sparse renormalises");
+    // k = E with raw weights is the dense forward (sparse.rs "k_equals_num_experts" test)
+    auto dense = layer.forward(x).unwrap();
+    auto all = layer.forward_sparse_with(x, fx.E, false).unwrap();
+    CHECK(dense == all.output, "dense forward == sparse with every expert and raw weights");
+    std::vector<float> manual(fx.d, 0.f);
+    for (int e = 0; e < fx.E; ++e) {
+      auto y = layer.experts[e].forward(x).unwrap();
+      for (int c = 0; c < fx.d; ++c) manual[c] += ro.weights[e] * y[c];
+    }
+    CHECK(metrics(dense, manual).max_abs_diff <= 1e-6, "dense forward vs manual weighted sum");
+    // errors: dimension first, then k (the order of route() and top_k_routing_with())
+    auto e1 = layer.forward_sparse(std::vector<float>(3, 0.f), 0);
+    CHECK(e1.is_err() && e1.error().kind == MoeSparseError::Dense && e1.error().dense.kind == MoeDenseError::DimMismatch &&
+              e1.error().dense.expected == (size_t)fx.d && e1.error().dense.actual == 3, "dim before k");
+    CHECK(layer.forward_sparse(x, 0).error().kind == MoeSparseError::ZeroK, "zero k");
+    auto e3 = layer.forward_sparse(x, fx.E + 1).error();
+    CHECK(e3.kind == MoeSparseError::KExceedsExperts && e3.k == (size_t)fx.E + 1 && e3.num_experts == (size_t)fx.E, "k > E");
+    CHECK(e3.to_string() == "moe-sparse: k (7) exceeds num_experts (6)", "%s", e3.to_string().c_str());
+    auto e4 = layer.experts[0].forward(std::vector<float>(2, 0.f)).error();
+    CHECK(e4.kind == MoeDenseError::DimMismatch && std::string(e4.what) == "expert input", "expert input dim");
   });
   run_test("identical_experts_reproduce_single_expert", [&] {
     Fixture fx = synthetic(4, 2, 8, 16, true);
