@@ -525,6 +525,116 @@ Result<std::vector<float>, MoeDenseError> MoeDenseExpert::forward(const std::vec
   return R::Ok(out.value());
 }
 
+// ---- MoeDenseLayer registry and the decomposed graph ops -----------------------------------------
+namespace {
+std::mutex& dense_registry_mutex() {
+  static std::mutex m;
+  return m;
+}
+std::vector<std::shared_ptr<const MoeDenseLayer>>& dense_registry() {
+  static std::vector<std::shared_ptr<const MoeDenseLayer>> r;
+  return r;
+}
+MoeSparseError no_such_layer() {
+  MoeSparseError e{MoeSparseError::Dense};
+  e.dense = MoeDenseError{MoeDenseError::NoExperts};
+  return e;
+}
+MoeSparseError from_dense(const MoeDenseError& d) {
+  MoeSparseError e{MoeSparseError::Dense};
+  e.dense = d;
+  return e;
+}
+}  // namespace
+
+uint32_t register_layer(MoeDenseLayer layer) {
+  std::lock_guard<std::mutex> lock(dense_registry_mutex());
+  dense_registry().push_back(std::make_shared<const MoeDenseLayer>(std::move(layer)));
+  return (uint32_t)(dense_registry().size() - 1);
+}
+
+std::shared_ptr<const MoeDenseLayer> get_layer(uint32_t layer_id) {
+  std::lock_guard<std::mutex> lock(dense_registry_mutex());
+  return layer_id < dense_registry().size() ? dense_registry()[layer_id] : nullptr;
+}
+
+Result<std::vector<float>, MoeSparseError> execute_sparse_reference(uint32_t layer_id,
+                                                                    const std::vector<float>& input,
+                                                                    size_t k) {
+  typedef Result<std::vector<float>, MoeSparseError> R;
+  auto layer = get_layer(layer_id);
+  if (!layer) return R::Err(no_such_layer());
+  auto out = layer->forward_sparse(input, k);
+  if (out.is_err()) return R::Err(out.error());
+  return R::Ok(out.value().output);
+}
+
+Result<DynamicDispatchOutput, MoeSparseError> execute_dynamic_dispatch(
+    uint32_t layer_id, const std::vector<float>& input, const std::vector<float>& selection) {
+  typedef Result<DynamicDispatchOutput, MoeSparseError> R;
+  auto layer = get_layer(layer_id);
+  if (!layer) return R::Err(no_such_layer());
+  if (selection.size() % 2 != 0)
+    return R::Err(from_dense(MoeDenseError{MoeDenseError::DimMismatch,
+                                           "dispatch selection (must be [idx, w, ...])", 0,
+                                           selection.size() % 2}));
+  const size_t pairs = selection.size() / 2, d = layer->d_model, E = layer->num_experts();
+  DynamicDispatchOutput r;
+  r.output.assign(d, 0.0f);
+  for (size_t p = 0; p < pairs; ++p) {
+    const float idx_f = selection[2 * p], weight = selection[2 * p + 1];
+    if (!std::isfinite(idx_f) || idx_f < 0.0f) {
+      MoeSparseError e{MoeSparseError::NegativeWeight};
+      e.index = 2 * p;
+      return R::Err(e);
+    }
+    const size_t idx = (size_t)idx_f;
+    if (idx >= E) {
+      MoeSparseError e{MoeSparseError::KExceedsExperts};
+      e.k = idx + 1;
+      e.num_experts = E;
+      return R::Err(e);
+    }
+    auto y = layer->experts[idx].forward(input);  // only the listed experts run
+    if (y.is_err()) return R::Err(from_dense(y.error()));
+    volatile float prod;  // product and sum rounded separately, as the reference's f32 loop
+    for (size_t c = 0; c < d; ++c) {
+      prod = weight * y.value()[c];
+      r.output[c] = r.output[c] + prod;
+    }
+    r.executed_experts.push_back(idx);
+  }
+  return R::Ok(std::move(r));
+}
+
+std::optional<float> expert_weight_in_selection(const std::vector<float>& selection,
+                                                uint32_t expert_id) {
+  for (size_t p = 0; p + 1 < selection.size(); p += 2)
+    if ((uint32_t)selection[p] == expert_id) return selection[p + 1];
+  return std::nullopt;
+}
+
+Result<std::pair<std::vector<float>, bool>, MoeSparseError> execute_conditional_expert(
+    uint32_t layer_id, uint32_t expert_id, const std::vector<float>& input,
+    const std::vector<float>& selection) {
+  typedef Result<std::pair<std::vector<float>, bool>, MoeSparseError> R;
+  auto layer = get_layer(layer_id);
+  if (!layer) return R::Err(no_such_layer());
+  if (expert_id >= layer->num_experts()) {
+    MoeSparseError e{MoeSparseError::KExceedsExperts};
+    e.k = (size_t)expert_id + 1;
+    e.num_experts = layer->num_experts();
+    return R::Err(e);
+  }
+  auto w = expert_weight_in_selection(selection, expert_id);
+  if (!w) return R::Ok(std::make_pair(std::vector<float>(layer->d_model, 0.0f), false));
+  auto y = layer->experts[expert_id].forward(input);
+  if (y.is_err()) return R::Err(from_dense(y.error()));
+  std::vector<float> scaled = y.value();
+  for (auto& v : scaled) v = v * *w;
+  return R::Ok(std::make_pair(std::move(scaled), true));
+}
+
 // ---- numeric policy -----------------------------------------------------------------------------
 const char* as_str(NumericPolicy p) {
   switch (p) {

@@ -352,6 +352,32 @@ class RealMoeLayer {
   Result<void*, MoeLayerError> handle_for(MoeExecutionConvention convention, bool with_shared) const;
 };
 
+// ---- registry of MoeDenseLayer and the decomposed graph ops (src/moe/graph_op.rs:28-205) -------
+// Behind NodeType::MoeSparseReference / MoeDynamicDispatch / ConditionalExpert: the selection
+// arrives as data, a flat [idx0, w0, idx1, w1, ...] f32 tensor (what MoeTopK emits), and only the
+// listed experts run -- here on the device, one MoeDenseExpert::forward per listed expert; the
+// weighted sum over the handful of listed experts is formed on the host in the listed order, as
+// the reference forms it.
+uint32_t register_layer(MoeDenseLayer layer);
+std::shared_ptr<const MoeDenseLayer> get_layer(uint32_t layer_id);
+// forward_sparse(input, k).output of a registered layer; an unknown id is Dense(NoExperts).
+Result<std::vector<float>, MoeSparseError> execute_sparse_reference(uint32_t layer_id,
+                                                                    const std::vector<float>& input,
+                                                                    size_t k);
+struct DynamicDispatchOutput {
+  std::vector<float> output;
+  std::vector<size_t> executed_experts;  // in the order of the selection
+};
+Result<DynamicDispatchOutput, MoeSparseError> execute_dynamic_dispatch(
+    uint32_t layer_id, const std::vector<float>& input, const std::vector<float>& selection);
+std::optional<float> expert_weight_in_selection(const std::vector<float>& selection,
+                                                uint32_t expert_id);
+// (weight * expert(input), true) when expert_id is in the selection, else (zeros, false) without
+// running the expert.
+Result<std::pair<std::vector<float>, bool>, MoeSparseError> execute_conditional_expert(
+    uint32_t layer_id, uint32_t expert_id, const std::vector<float>& input,
+    const std::vector<float>& selection);
+
 // ---- registry and graph op --------------------------------------------------------------------
 // Process-global, grow-only, ids stable per process (src/moe/graph_op.rs:221-232).
 uint32_t register_real_moe_layer(RealMoeLayer layer);

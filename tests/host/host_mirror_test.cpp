@@ -475,6 +475,67 @@ int main(int argc, char** argv) {
     auto e4 = layer.experts[0].forward(std::vector<float>(2, 0.f)).error();
     CHECK(e4.kind == MoeDenseError::DimMismatch && std::string(e4.what) == "expert input", "expert input dim");
   });
+  run_test("decomposed_graph_ops_match_the_sparse_reference", [&] {
+    // tests/moe_dynamic_dispatch_test.rs and tests/moe_conditional_expert_test.rs, same checks
+    Fixture fx = synthetic(6, 2, 16, 24);
+    RealMoeLayer rl = layer_from(fx);
+    const uint32_t id = register_layer(rl.routed);
+    auto layer = get_layer(id);
+    CHECK(layer && layer->num_experts() == 6 && !get_layer(id + 1000), "registry");
+    const std::vector<float> x = seeded(9, fx.d);
+    const size_t k = 2;
+    auto reference = execute_sparse_reference(id, x, k).unwrap();
+    auto sp = layer->forward_sparse(x, k).unwrap();
+    CHECK(reference == sp.output, "graph op == forward_sparse");
+    // the selection as MoeTopK emits it: [idx0, w0, idx1, w1], renormalised weights
+    auto ro = layer->route(x).unwrap();
+    double sum = 0;
+    for (size_t e : sp.selected_experts) sum += (double)ro.weights[e];
+    std::vector<float> selection;
+    for (size_t e : sp.selected_experts) {
+      selection.push_back((float)e);
+      selection.push_back((float)((double)ro.weights[e] * (1.0 / sum)));
+    }
+    auto dd = execute_dynamic_dispatch(id, x, selection).unwrap();
+    CHECK(metrics(dd.output, reference).max_abs_diff < 1e-5, "dispatch vs sparse reference: %g",
+          metrics(dd.output, reference).max_abs_diff);
+    CHECK(dd.executed_experts == sp.selected_experts && dd.executed_experts.size() < layer->num_experts(),
+          "only the selected experts run");
+    auto dd2 = execute_dynamic_dispatch(id, x, selection).unwrap();
+    CHECK(dd.output == dd2.output, "deterministic");
+    // conditional experts: one node per expert, contributions summed
+    std::vector<float> conditional(fx.d, 0.f);
+    size_t executed = 0, skipped = 0;
+    for (uint32_t e = 0; e < 6; ++e) {
+      auto ce = execute_conditional_expert(id, e, x, selection).unwrap();
+      CHECK(ce.first.size() == (size_t)fx.d, "contribution length");
+      if (ce.second) {
+        ++executed;
+        for (int c = 0; c < fx.d; ++c) conditional[c] += ce.first[c];
+      } else {
+        ++skipped;
+        for (float v : ce.first) CHECK(v == 0.0f, "a skipped expert contributes zeros");
+      }
+    }
+    CHECK(executed == k && skipped == 6 - k, "exactly k experts execute");
+    CHECK(metrics(conditional, dd.output).max_abs_diff < 1e-6, "conditional pipeline == dynamic dispatch");
+    CHECK(metrics(conditional, reference).max_abs_diff < 1e-5, "conditional pipeline == sparse reference");
+    auto one = execute_conditional_expert(id, (uint32_t)sp.selected_experts[0], x, {(float)sp.selected_experts[0], 0.6f}).unwrap();
+    auto y0 = layer->experts[sp.selected_experts[0]].forward(x).unwrap();
+    for (int c = 0; c < fx.d; ++c) CHECK(std::fabs(one.first[c] - 0.6f * y0[c]) < 1e-6, "weight * expert output");
+    CHECK(expert_weight_in_selection(selection, (uint32_t)sp.selected_experts[1]).value() == selection[3] &&
+              !expert_weight_in_selection(selection, 99).has_value(), "weight lookup");
+    // errors (dispatch_rejects_bad_selection / unknown layer / expert out of range)
+    CHECK(execute_dynamic_dispatch(id, x, {0.0f, 0.5f, 1.0f}).is_err(), "odd selection length");
+    auto bad = execute_dynamic_dispatch(id, x, {99.0f, 1.0f}).error();
+    CHECK(bad.kind == MoeSparseError::KExceedsExperts && bad.k == 100 && bad.num_experts == 6, "index out of range");
+    CHECK(execute_dynamic_dispatch(id, x, {-1.0f, 1.0f}).error().kind == MoeSparseError::NegativeWeight, "negative index");
+    auto unk = execute_dynamic_dispatch(0xffffffffu, x, {0.0f, 1.0f});
+    CHECK(unk.is_err() && unk.error().kind == MoeSparseError::Dense && unk.error().dense.kind == MoeDenseError::NoExperts, "unknown layer");
+    CHECK(execute_conditional_expert(0xffffffffu, 0, x, {0.0f, 1.0f}).is_err(), "unknown layer");
+    CHECK(execute_conditional_expert(id, 6, x, {0.0f, 1.0f}).error().kind == MoeSparseError::KExceedsExperts, "expert out of range");
+    CHECK(execute_sparse_reference(0xffffffffu, x, 2).is_err(), "unknown layer");
+  });
   run_test("identical_experts_reproduce_single_expert", [&] {
     Fixture fx = synthetic(4, 2, 8, 16, true);
     RealMoeLayer layer = layer_from(fx);
