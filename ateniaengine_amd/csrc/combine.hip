@@ -20,6 +20,14 @@ namespace atenia_moe {
 
 namespace {
 
+// Expert outputs are read exactly once: a streaming (non-temporal) load leaves the caches to the
+// kernels around this one.
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+__device__ inline float4 load_once(const float* p) {
+  const f32x4_t v = __builtin_nontemporal_load((const f32x4_t*)p);
+  return make_float4(v.x, v.y, v.z, v.w);
+}
+
 __global__ __launch_bounds__(256) void combine_kernel(int T, int k, int d,
                                                       const float* __restrict__ w,
                                                       const float* __restrict__ y, int y_stride,
@@ -40,7 +48,7 @@ __global__ __launch_bounds__(256) void combine_kernel(int T, int k, int d,
     const int y_parts = part_flags ? part_flags[((size_t)t * k + slot) * flag_cols + c / 256] : 1;
     float v[4] = {0.f, 0.f, 0.f, 0.f};
     if (vec) {
-      float4 q = *(const float4*)yr;
+      float4 q = load_once(yr);
       v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
       for (int part = 1; part < y_parts; ++part) {
         q = *(const float4*)(yr + part * y_part_stride);
@@ -61,7 +69,7 @@ __global__ __launch_bounds__(256) void combine_kernel(int T, int k, int d,
     const float* yr = y_shared + (size_t)t * y_stride + c;
     float v[4] = {0.f, 0.f, 0.f, 0.f};
     if (vec) {
-      float4 q = *(const float4*)yr;
+      float4 q = load_once(yr);
       v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
     } else {
       for (int j = 0; j < 4 && c + j < d; ++j) v[j] = yr[j];
