@@ -12,6 +12,8 @@
 // Small batches (P <= 1024 pairs) take one launch of one block.  Larger ones take three:
 // per-block histograms, one block that scans them, and a scatter pass that recomputes each
 // block's stable ranks.
+#include <algorithm>
+
 #include "moe_internal.h"
 
 namespace atenia_moe {
@@ -157,34 +159,56 @@ __global__ __launch_bounds__(kPermuteBlock) void permute_hist_kernel(
     blk_counts[(size_t)blockIdx.x * E + j] = sm[j];
 }
 
-// One block: for every expert, turn the per-block counts into per-block bases.
+// One block: for every expert, turn the per-block counts into per-block bases.  The blocks are
+// cut into nseg contiguous segments and thread (segment, expert) walks its own segment, so the
+// two passes over the nblk x E table take nblk / nseg dependent steps instead of nblk (96 blocks
+// of 1024 pairs at 16384 tokens x 6: 39 us when one thread per expert walked them all).
 __global__ __launch_bounds__(kPermuteBlock) void permute_scan_kernel(
     int E, int nblk, int T, int32_t* __restrict__ blk_counts, int32_t* counts,
     int32_t* offsets, int32_t* active, int32_t* n_active, int32_t* shared_offsets, TileOut to) {
-  extern __shared__ int32_t sm[];  // [E] totals, [E+1] offsets
+  extern __shared__ int32_t sm[];  // [E] totals, [E+1] offsets, [nseg][E] segment sums
   int32_t* sTot = sm;
   int32_t* sOff = sm + E;
-  for (int e = threadIdx.x; e < E; e += kPermuteBlock) {
+  int32_t* sSeg = sOff + E + 1;
+  int nseg = kPermuteBlock / E;
+  if (nseg > nblk) nseg = nblk;
+  if (nseg < 1) nseg = 1;
+  const int bps = (nblk + nseg - 1) / nseg;  // blocks per segment
+  const int tid = threadIdx.x;
+  const int seg = tid / E, e = tid - seg * E;
+  const bool on = seg < nseg;
+  const int b_lo = seg * bps, b_hi = min(nblk, b_lo + bps);
+  if (on) {
     int run = 0;
-    for (int b = 0; b < nblk; ++b) run += blk_counts[(size_t)b * E + e];
-    sTot[e] = run;
-    counts[e] = run;
+    for (int b = b_lo; b < b_hi; ++b) run += blk_counts[(size_t)b * E + e];
+    sSeg[seg * E + e] = run;
+  }
+  __syncthreads();
+  if (tid < E) {  // totals; the segment sums become exclusive prefixes over the segments
+    int run = 0;
+    for (int sg = 0; sg < nseg; ++sg) {
+      const int c = sSeg[sg * E + tid];
+      sSeg[sg * E + tid] = run;
+      run += c;
+    }
+    sTot[tid] = run;
+    counts[tid] = run;
   }
   __syncthreads();
   if (threadIdx.x == 0) {
     int run = 0;
-    for (int e = 0; e < E; ++e) {
-      sOff[e] = run;
-      run += sTot[e];
+    for (int ee = 0; ee < E; ++ee) {
+      sOff[ee] = run;
+      run += sTot[ee];
     }
     sOff[E] = run;
   }
   __syncthreads();
   finish_offsets(E, sTot, offsets, active, n_active, shared_offsets, T, to);
-  for (int e = threadIdx.x; e < E; e += kPermuteBlock) {
-    int run = sOff[e];
-    for (int b = 0; b < nblk; ++b) {
-      int c = blk_counts[(size_t)b * E + e];
+  if (on) {
+    int run = sOff[e] + sSeg[seg * E + e];
+    for (int b = b_lo; b < b_hi; ++b) {
+      const int c = blk_counts[(size_t)b * E + e];
       blk_counts[(size_t)b * E + e] = run;  // becomes the block's base for expert e
       run += c;
     }
@@ -230,7 +254,8 @@ hipError_t launch_permute(const PermuteArgs& a, hipStream_t s, int* n_launches) 
   const int nblk = (P + kPermuteBlock - 1) / kPermuteBlock;
   permute_hist_kernel<<<nblk, kPermuteBlock, (size_t)E * sizeof(int32_t), s>>>(a.idx, P, E,
                                                                                  a.blk_counts);
-  permute_scan_kernel<<<1, kPermuteBlock, ((size_t)2 * E + 1) * sizeof(int32_t), s>>>(
+  const int nseg = std::max(1, std::min(nblk, kPermuteBlock / E));
+  permute_scan_kernel<<<1, kPermuteBlock, ((size_t)2 * E + 1 + (size_t)nseg * E) * sizeof(int32_t), s>>>(
       E, nblk, a.T, a.blk_counts, a.counts, a.offsets, a.active, a.n_active, a.shared_offsets,
       to);
   permute_scatter_kernel<<<nblk, kPermuteBlock, ((size_t)kWaves * E + E) * sizeof(int32_t), s>>>(
