@@ -138,15 +138,28 @@ int device_cu_count() {
   return v;
 }
 
-// Largest batch served by the weight-streaming expert kernels (tuning knob:
-// ATENIA_MOE_STREAM_MAX_TOKENS, read once per process).
-int stream_max_tokens() {
+// Largest batch served by the weight-streaming expert kernels when set from outside (tuning
+// knob: ATENIA_MOE_STREAM_MAX_TOKENS, read once per process); 0 = the built-in rule below.
+int stream_max_tokens_override() {
   static const int v = [] {
     const char* e = getenv("ATENIA_MOE_STREAM_MAX_TOKENS");
     int n = e ? atoi(e) : 0;
-    return n > 0 ? n : 48;
+    return n > 0 ? n : 0;
   }();
   return v;
+}
+constexpr int kStreamMaxTokens = 48;
+// Whether a batch of T tokens whose experts see rows_num / rows_den rows each on average
+// (T * k / E) is served by the weight-streaming kernels.  Those pass
+// over an expert's weights once per 32 of its rows, while the tiled kernels cost about the same
+// from 49 tokens to a few hundred, so beyond 48 tokens the choice goes by the average rows per
+// expert.  Measured cross-overs on MI355X: about 9 rows for bf16 weights (Qwen1.5-MoE shape
+// T = 140, DeepSeek-V2-Lite shape T = 100), about 24 for int8 (Mixtral shape T = 100), whose tiled
+// kernel widens every weight in the VALU however few rows it multiplies.
+bool batch_streams(int T, long long rows_num, long long rows_den, bool int8) {
+  if (const int n = stream_max_tokens_override()) return T <= n;
+  if (T <= kStreamMaxTokens) return true;
+  return rows_num <= rows_den * (int8 ? 24 : 9);
 }
 // Largest batch routed by the one-workgroup-per-token router kernel (tuning knob:
 // ATENIA_MOE_ROUTER_TOKEN_MAX, read once per process).
@@ -417,7 +430,9 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   // layer keeps a bf16 copy of its experts (q * group scale, rounded to bf16 -- the form the
   // reference's GPU path multiplies with, src/cuda/int8_to_bf16.cu:91-110) for such batches;
   // decode batches stream the int8 weights themselves.
-  const bool pg_prefill = L->group_size > 0 && T > stream_max_tokens() && L->d_kpad % 64 == 0 &&
+  const bool int8w = L->wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
+  const bool routed_streams = batch_streams(T, (long long)T * L->k, L->E, int8w);
+  const bool pg_prefill = L->group_size > 0 && !routed_streams && L->d_kpad % 64 == 0 &&
                           L->f_kpad % 64 == 0 && (L->fs == 0 || L->fs_kpad % 64 == 0);
   if (pg_prefill && !L->pg_ready) {
     int rc = make_bf16_copy(L->gate, L->E, L->pg_wg, L->gate_b);
@@ -455,7 +470,7 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   fa.y_stride = L->d;
   // Tiled (MFMA-bound) kernels once an expert can see more rows than the streaming kernel
   // keeps in registers; below that the weights are streamed once (HBM-bound).
-  const bool tiled = T > stream_max_tokens() && tiled_supported(fa.gate, ffn_dtype) &&
+  const bool tiled = !routed_streams && tiled_supported(fa.gate, ffn_dtype) &&
                      tiled_supported(fa.down, ffn_dtype);
   fa.use_tiled = tiled;
   fa.tile_group = L->tile_group.as<int32_t>();
@@ -489,7 +504,10 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
     fsd.y = L->ys.as<float>();
     fsd.y_parts = 1;
     fsd.part_flags = nullptr;
-    fsd.use_tiled = T > stream_max_tokens() && tiled_supported(fsd.gate, ffn_dtype) &&
+    // The shared expert follows the routed ones (it then rides in their launches): it is small
+    // next to E routed experts, so its extra passes (one per 32 tokens) cost less than the
+    // launches of its own that the tiled form would need.
+    fsd.use_tiled = !routed_streams && tiled_supported(fsd.gate, ffn_dtype) &&
                     tiled_supported(fsd.down, ffn_dtype);
     fsd.tile_group = L->s_tile_group.as<int32_t>();
     fsd.tile_m0 = L->s_tile_m0.as<int32_t>();

@@ -241,11 +241,15 @@ LAYER_CASES = [
     ("ragged_bf16", 5, 2, 40, 44, 0, False, 0, capi.WEIGHT_BF16, TOL_BF16_TOY),
     ("ragged_int8", 5, 3, 72, 100, 36, True, 1, capi.WEIGHT_INT8_W8A16, TOL_BF16_TOY),
     ("ragged_mid_int8", 5, 3, 200, 360, 136, True, 1, capi.WEIGHT_INT8_W8A16, TOL_BF16_TOY),
+    # many experts: few rows each, so batches of 90 / 150 tokens still take the streaming kernels
+    # (several row slices per expert, the shared expert's T rows riding in the same launches)
+    ("wide_bf16", 40, 2, 128, 96, 64, True, 1, capi.WEIGHT_BF16, TOL_BF16),
+    ("wide_int8", 40, 3, 128, 96, 0, False, 0, capi.WEIGHT_INT8_W8A16, TOL_BF16),
 ]
 
 
 @pytest.mark.parametrize("name,E,k,d,f,f_s,gated,conv,wd,tol", LAYER_CASES)
-@pytest.mark.parametrize("T", [1, 7, 16, 40, 150, 700])
+@pytest.mark.parametrize("T", [1, 7, 16, 40, 90, 150, 700])
 def test_layer_forward(ora, name, E, k, d, f, f_s, gated, conv, wd, tol, T):
     W = S.make_weights(zlib.crc32(name.encode()) % 1000, E, d, f, f_s=f_s, gated=gated,
                        outlier_frac=0.01 if wd == capi.WEIGHT_INT8_W8A16 else 0.0)
