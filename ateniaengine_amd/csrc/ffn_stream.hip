@@ -109,8 +109,16 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p_r
   const int cnt = p.g.offsets[e + 1] - base;
   const int m0 = blockIdx.z * 16 * MT;
   if (m0 >= cnt) return;
+  // 16-row tiles of this slice that hold rows.  The others are not loaded: their A registers
+  // stay zero and their MFMAs run on zeros.  (The MFMAs are deliberately not branched around:
+  // with a branch between an MFMA and the VALU instruction that reads its result, hipcc 7.2
+  // leaves out the wait states on the taken path and the per-group form read stale sums.)
+  const int mt_live = min(MT, (cnt - m0 + 15) >> 4);
   const int nb = blockIdx.x;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  // The wave id as a scalar: everything derived from it (k range, loop bounds, the guards around
+  // the MFMAs) is then a scalar branch.  Left as a vector value the compiler predicates those
+  // guards through EXEC, which MFMA instructions do not obey.
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int kq = lane >> 4, mm = lane & 15;
   constexpr int KB = INT8 ? kKbInt8 : kKbBf16;  // k per block
   constexpr int NACC = UP ? 2 : 1;
@@ -130,6 +138,12 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p_r
   constexpr int AV = INT8 ? 2 : 1;       // 16-byte activation pieces per block and row tile
   uint4 wA0[U], wB0[UP ? U : 1], wA1[U], wB1[UP ? U : 1];
   uint4 xa0[U][MT][AV], xa1[U][MT][AV];
+#pragma unroll
+  for (int j = 0; j < U; ++j)
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int v = 0; v < AV; ++v) xa0[j][i][v] = xa1[j][i][v] = make_uint4(0u, 0u, 0u, 0u);
   // Per-group scales of this lane's output row (column mm of the D layout), one per k group;
   // they are requested together with the weight blocks they belong to.
   const size_t n_pad_s = (size_t)p.n_pad;  // scale rows per k group
@@ -173,9 +187,11 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p_r
       const int kk = min(kb + j, kb1 - 1);
 #pragma unroll
       for (int i = 0; i < MT; ++i)
+        if (i < mt_live) {
 #pragma unroll
-        for (int v = 0; v < AV; ++v)
-          xa[j][i][v] = *((const uint4*)(arow[i] + (size_t)kk * KB) + v);
+          for (int v = 0; v < AV; ++v)
+            xa[j][i][v] = *((const uint4*)(arow[i] + (size_t)kk * KB) + v);
+        }
     }
   };
 
@@ -303,7 +319,10 @@ __global__ __launch_bounds__(1024) void ffn_down_decode1_kernel(StreamParams p, 
                                                                const float* residual, float* out) {
   constexpr int KS = 8;  // K slices per expert, as in the separate down launch
   const int nb = blockIdx.x;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  // The wave id as a scalar: everything derived from it (k range, loop bounds, the guards around
+  // the MFMAs) is then a scalar branch.  Left as a vector value the compiler predicates those
+  // guards through EXEC, which MFMA instructions do not obey.
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int kq = lane >> 4, mm = lane & 15;
   const int j = wave / KS, slice = wave - j * KS;
   constexpr int KB = INT8 ? kKbInt8 : kKbBf16;

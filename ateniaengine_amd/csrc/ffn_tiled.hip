@@ -200,7 +200,9 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_kernel(TiledParams p) {
   const int cnt = p.g.offsets[e + 1] - base;
   const int rows_here = min(TM, cnt - tm0);
 
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = threadIdx.x, lane = tid & 63;
+  // scalar wave id: guards around MFMAs must be scalar branches (MFMA does not obey EXEC)
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int kq = lane >> 4, mm = lane & 15;
   const int wm = wave >> 1, wn = wave & 1;
   constexpr int BROWS = UP ? 128 : 256;  // distinct weight rows per tile

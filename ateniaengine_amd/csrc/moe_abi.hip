@@ -148,11 +148,11 @@ int stream_max_tokens_override() {
   }();
   return v;
 }
-constexpr int kStreamMaxTokens = 48;
+constexpr int kStreamMaxTokens = 56;
 // Whether a batch of T tokens whose experts see rows_num / rows_den rows each on average
 // (T * k / E) is served by the weight-streaming kernels.  Those pass
 // over an expert's weights once per 32 of its rows, while the tiled kernels cost about the same
-// from 49 tokens to a few hundred, so beyond 48 tokens the choice goes by the average rows per
+// from about 50 tokens to a few hundred, so beyond 56 tokens the choice goes by the average rows per
 // expert.  Measured cross-overs on MI355X: about 9 rows for bf16 weights (Qwen1.5-MoE shape
 // T = 140, DeepSeek-V2-Lite shape T = 100), about 24 for int8 (Mixtral shape T = 100), whose tiled
 // kernel widens every weight in the VALU however few rows it multiplies.

@@ -244,7 +244,7 @@ LAYER_CASES = [
     # many experts: few rows each, so batches of 90 / 150 tokens still take the streaming kernels
     # (several row slices per expert, the shared expert's T rows riding in the same launches)
     ("wide_bf16", 40, 2, 128, 96, 64, True, 1, capi.WEIGHT_BF16, TOL_BF16),
-    ("wide_int8", 40, 3, 128, 96, 0, False, 0, capi.WEIGHT_INT8_W8A16, TOL_BF16),
+    ("wide_int8", 40, 3, 128, 352, 0, False, 0, capi.WEIGHT_INT8_W8A16, TOL_BF16),
 ]
 
 

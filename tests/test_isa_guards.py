@@ -1,0 +1,109 @@
+"""Checks on the gfx950 assembly hipcc generates for the MFMA kernels (no GPU needed: hipcc
+cross-compiles).  Two code shapes gave wrong numbers on the device while this library was built,
+both silently:
+
+* an MFMA inside an EXEC-masked region.  MFMA instructions ignore EXEC, so a guard that the
+  compiler turned into lane predication (because it could not prove the condition wave-uniform,
+  e.g. one derived from ``threadIdx.x >> 6``) only holds while the compiler also keeps the
+  ``s_cbranch_execz`` around the block; when it dropped one, clamped duplicate weight blocks were
+  multiplied in and outputs came out 4x too large.  The kernels now derive such conditions from a
+  ``readfirstlane`` wave id, which makes them scalar branches.
+* a branch between an MFMA and the VALU instruction that reads its result.  hipcc 7.2 counts the
+  required wait states along the fall-through path only; on the taken path the read saw stale
+  accumulator values.
+
+Both are properties of the generated code, so they are asserted on the generated code."""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "ateniaengine_amd", "csrc")
+HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-w", "-Xclang", "-target-feature",
+         "-Xclang", "-packed-fp32-ops", "--cuda-device-only", "-S"]
+
+_EXEC_OPEN = ("s_and_saveexec", "s_andn2_saveexec", "s_or_saveexec", "s_and_b64 exec", "s_xor_b64 exec",
+              "s_andn2_b64 exec")
+_EXEC_CLOSE = ("s_or_b64 exec", "s_mov_b64 exec", "s_endpgm")
+
+
+def _assembly(tmp_path_factory, name):
+    out = tmp_path_factory.mktemp("isa") / (name + ".s")
+    r = subprocess.run([HIPCC] + FLAGS + ["-o", str(out), os.path.join(CSRC, name)],
+                       capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0, r.stderr[-2000:]
+    return [ln.strip() for ln in open(out).read().split("\n")]
+
+
+@pytest.fixture(scope="module", params=["ffn_stream.hip", "ffn_tiled.hip"])
+def asm(request, tmp_path_factory):
+    if not os.path.exists(HIPCC):
+        pytest.skip("hipcc not found")
+    return request.param, _assembly(tmp_path_factory, request.param)
+
+
+def test_no_mfma_under_an_exec_mask(asm):
+    name, lines = asm
+    masked, hits, total = False, [], 0
+    for no, ln in enumerate(lines, 1):
+        if ln.startswith(_EXEC_OPEN):
+            masked = True
+        elif ln.startswith(_EXEC_CLOSE):
+            masked = False
+        elif ln.startswith("v_mfma"):
+            total += 1
+            if masked:
+                hits.append((no, ln))
+    assert total > 100, f"{name}: expected the MFMA kernels in the assembly, found {total} MFMAs"
+    assert not hits, f"{name}: MFMA inside an EXEC-masked region (MFMA ignores EXEC): {hits[:5]}"
+
+
+def _regs(operand):
+    m = re.fullmatch(r"([va])\[(\d+):(\d+)\]", operand)
+    if m:
+        return {(m.group(1), i) for i in range(int(m.group(2)), int(m.group(3)) + 1)}
+    m = re.fullmatch(r"([va])(\d+)", operand)
+    return {(m.group(1), int(m.group(2)))} if m else set()
+
+
+def test_no_branch_between_an_mfma_and_the_valu_read_of_its_result(asm):
+    """For every branch that directly follows an MFMA: the first instructions at the branch
+    target must not be plain VALU / LDS / memory reads of that MFMA's destination registers
+    (an MFMA reading it as its own accumulator again is the hardware's back-to-back case)."""
+    name, lines = asm
+    labels = {ln[:-1]: i for i, ln in enumerate(lines) if ln.endswith(":") and ln.startswith(".LBB")}
+    labels.update({ln.split(":")[0]: i for i, ln in enumerate(lines) if ln.startswith(".LBB") and ":" in ln})
+    bad = []
+    for i, ln in enumerate(lines):
+        if not ln.startswith("v_mfma"):
+            continue
+        dst = _regs(ln.split()[1].rstrip(","))
+        for j in range(i + 1, min(i + 3, len(lines))):
+            if lines[j].startswith("v_mfma"):
+                break
+            if lines[j].startswith("s_cbranch") or lines[j].startswith("s_branch"):
+                target = labels.get(lines[j].split()[-1])
+                if target is None:
+                    break
+                waited = 0
+                for t in lines[target + 1:target + 12]:
+                    if not t or t.startswith(";") or t.endswith(":"):
+                        continue
+                    if t.startswith("s_nop"):
+                        waited += int(t.split()[1]) + 1
+                    if waited >= 8 or t.startswith(("s_waitcnt", "s_barrier", "s_cbranch", "s_branch")):
+                        break
+                    ops = [o.strip().rstrip(",") for o in t.replace(",", " ").split()[1:]]
+                    reads = set().union(*[_regs(o) for o in ops[1:]]) if len(ops) > 1 else set()
+                    if t.startswith("v_mfma"):
+                        reads -= _regs(ops[-1]) if ops else set()   # accumulator operand
+                    if reads & dst:
+                        bad.append((i + 1, ln[:60], "->", target + 1, t[:60]))
+                        break
+                    waited += 1
+                break
+    assert not bad, f"{name}: result of an MFMA read right after a branch: {bad[:5]}"
