@@ -109,6 +109,11 @@ ROUTER_CASES = [
     (16, 2, 64, 600, 0, True, True, False),
     (63, 5, 128, 531, 1, True, False, True),
     (33, 2, 36, 19, 0, False, False, False),
+    # 33-64 tokens with more than 32 rows: rows spread over workgroups + selection launch; 65: not
+    (60, 4, 2048, 48, 1, True, False, True),
+    (64, 6, 2048, 64, 1, True, True, False),
+    (64, 6, 2048, 65, 1, True, True, False),
+    (40, 2, 96, 57, 0, False, False, False),
 ]
 
 
