@@ -335,7 +335,7 @@ __global__ __launch_bounds__(1024) void ffn_down_decode1_kernel(StreamParams p, 
     const int kb0 = slice * kb_per;
     const int kb1 = min(p.nkb, kb0 + kb_per);
     const uint4* pa = p.wa + (size_t)e * p.w_stride_u4 + (size_t)nb * p.nkb * 64 + lane;
-    constexpr int U = INT8 ? 2 : 4;
+    constexpr int U = 4;
     constexpr int AV = INT8 ? 2 : 1;
     uint4 wA0[U], wA1[U], xa0[U][AV], xa1[U][AV];
     auto load_w = [&](uint4 (&wa)[U], int kb) {
