@@ -94,14 +94,18 @@ __device__ inline f32x4 mfma(bf16x8 a, bf16x8 b, f32x4 c) {
 // A second parameter set rides along for the shared expert: the workgroups with blockIdx.y ==
 // shared_y stream the shared expert's strips (its own weights, width, input and output rows)
 // in the same launch as the routed experts', one launch less per phase for layers that have one.
-template <int MT, bool INT8, bool UP, int WAVES, bool PG>
+// S  : adjacent 16-row strips per workgroup (1 or 2).  With two, a wave multiplies the token
+//      rows it loaded with the blocks of both strips, which halves the activation traffic from
+//      L2 per weight byte -- what the streaming rate falls with once an expert has more than 16 rows.
+template <int MT, bool INT8, bool UP, int WAVES, bool PG, int S = 1>
 __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p_routed,
                                                                 StreamParams p_shared,
                                                                 int shared_y) {
   constexpr int kWavesPerWg = WAVES;
   const bool sh = (int)blockIdx.y == shared_y;
   const StreamParams& p = sh ? p_shared : p_routed;
-  if ((int)blockIdx.x * 16 >= p.n_pad) return;  // the grid spans the wider of the two
+  static_assert(S == 1 || !PG, "two strips per workgroup: per-row scales only");
+  if ((int)blockIdx.x * 16 * S >= p.n_pad) return;  // the grid spans the wider of the two
   const int u = sh ? 0 : blockIdx.y;
   if (u >= *p.g.n_active) return;
   const int e = p.g.active[u];
@@ -114,7 +118,7 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p_r
   // with a branch between an MFMA and the VALU instruction that reads its result, hipcc 7.2
   // leaves out the wait states on the taken path and the per-group form read stale sums.)
   const int mt_live = min(MT, (cnt - m0 + 15) >> 4);
-  const int nb = blockIdx.x;
+  const int nb = blockIdx.x * S;  // first strip; n_pad is a multiple of 16 * S (launcher)
   // The wave id as a scalar: everything derived from it (k range, loop bounds, the guards around
   // the MFMAs) is then a scalar branch.  Left as a vector value the compiler predicates those
   // guards through EXEC, which MFMA instructions do not obey.
@@ -129,6 +133,7 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p_r
   const uint4* pa = p.wa + (size_t)e * p.w_stride_u4 + (size_t)nb * p.nkb * 64 + lane;
   const uint4* pb = UP ? p.wb + (size_t)e * p.w_stride_u4 + (size_t)nb * p.nkb * 64 + lane
                        : nullptr;
+  const size_t strip_u4 = (size_t)p.nkb * 64;  // uint4 between adjacent strips
 
   // Software pipeline over batches of U weight blocks with two register buffers: the loads
   // of batch i+1 are in flight while batch i is multiplied.  The first batch is requested
@@ -136,7 +141,7 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p_r
   // memory latency after the workgroup does.
   constexpr int U = INT8 ? 2 : 4;        // blocks per batch
   constexpr int AV = INT8 ? 2 : 1;       // 16-byte activation pieces per block and row tile
-  uint4 wA0[U], wB0[UP ? U : 1], wA1[U], wB1[UP ? U : 1];
+  uint4 wA0[S][U], wB0[S][UP ? U : 1], wA1[S][U], wB1[S][UP ? U : 1];
   uint4 xa0[U][MT][AV], xa1[U][MT][AV];
 #pragma unroll
   for (int j = 0; j < U; ++j)
@@ -150,13 +155,16 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p_r
   const float* psa = PG ? p.sa + (size_t)e * p.n_kgroups * n_pad_s + nb * 16 + mm : nullptr;
   const float* psb = PG && UP ? p.sb + (size_t)e * p.n_kgroups * n_pad_s + nb * 16 + mm : nullptr;
   float sA0[PG ? U : 1], sB0[PG && UP ? U : 1], sA1[PG ? U : 1], sB1[PG && UP ? U : 1];
-  auto load_w = [&](uint4 (&wa)[U], uint4 (&wb)[UP ? U : 1], float (&sa)[PG ? U : 1],
+  auto load_w = [&](uint4 (&wa)[S][U], uint4 (&wb)[S][UP ? U : 1], float (&sa)[PG ? U : 1],
                     float (&sb)[PG && UP ? U : 1], int kb) {
 #pragma unroll
     for (int j = 0; j < U; ++j) {
       const int kk = min(kb + j, kb1 - 1);  // clamped: a batch past the end is loaded, not used
-      wa[j] = load_stream(pa + (size_t)kk * 64);
-      if (UP) wb[j] = load_stream(pb + (size_t)kk * 64);
+#pragma unroll
+      for (int t = 0; t < S; ++t) {
+        wa[t][j] = load_stream(pa + t * strip_u4 + (size_t)kk * 64);
+        if (UP) wb[t][j] = load_stream(pb + t * strip_u4 + (size_t)kk * 64);
+      }
       if (PG) {
         const int kg = kk / p.group_blocks;
         sa[j] = psa[(size_t)kg * n_pad_s];
@@ -195,12 +203,14 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p_r
     }
   };
 
-  f32x4 acc[NACC][MT];
+  f32x4 acc[NACC][S][MT];
 #pragma unroll
   for (int n = 0; n < NACC; ++n)
 #pragma unroll
-    for (int i = 0; i < MT; ++i) acc[n][i] = f32x4{0.f, 0.f, 0.f, 0.f};
-  auto multiply = [&](const uint4 (&wa)[U], const uint4 (&wb)[UP ? U : 1],
+    for (int t = 0; t < S; ++t)
+#pragma unroll
+      for (int i = 0; i < MT; ++i) acc[n][t][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  auto multiply = [&](const uint4 (&wa)[S][U], const uint4 (&wb)[S][UP ? U : 1],
                       const float (&sa)[PG ? U : 1], const float (&sb)[PG && UP ? U : 1],
                       const uint4 (&xa)[U][MT][AV], int kb) {
 #pragma unroll
@@ -208,8 +218,8 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p_r
       if (kb + j < kb1) {
         if (INT8 && PG) {
           bf16x8 al, ah, bl, bh;
-          widen_i8x16(wa[j], al, ah);
-          if (UP) widen_i8x16(wb[j], bl, bh);
+          widen_i8x16(wa[0][j], al, ah);
+          if (UP) widen_i8x16(wb[0][j], bl, bh);
           const float s_a = sa[PG ? j : 0];
           const float s_b = UP ? sb[PG && UP ? j : 0] : 0.f;
 #pragma unroll
@@ -217,33 +227,38 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p_r
             uint4 x0 = xa[j][i][0], x1 = xa[j][i][AV - 1];
             f32x4 ta = mfma(*(bf16x8*)&x0, al, f32x4{0.f, 0.f, 0.f, 0.f});
             ta = mfma(*(bf16x8*)&x1, ah, ta);
-            acc[0][i] += ta * s_a;
+            acc[0][0][i] += ta * s_a;
             if (UP) {
               f32x4 tb = mfma(*(bf16x8*)&x0, bl, f32x4{0.f, 0.f, 0.f, 0.f});
               tb = mfma(*(bf16x8*)&x1, bh, tb);
-              acc[NACC - 1][i] += tb * s_b;
+              acc[NACC - 1][0][i] += tb * s_b;
             }
           }
         } else if (INT8) {
-          bf16x8 al, ah, bl, bh;
-          widen_i8x16(wa[j], al, ah);
-          if (UP) widen_i8x16(wb[j], bl, bh);
 #pragma unroll
-          for (int i = 0; i < MT; ++i) {
-            uint4 x0 = xa[j][i][0], x1 = xa[j][i][AV - 1];
-            acc[0][i] = mfma(*(bf16x8*)&x0, al, acc[0][i]);
-            acc[0][i] = mfma(*(bf16x8*)&x1, ah, acc[0][i]);
-            if (UP) {
-              acc[NACC - 1][i] = mfma(*(bf16x8*)&x0, bl, acc[NACC - 1][i]);
-              acc[NACC - 1][i] = mfma(*(bf16x8*)&x1, bh, acc[NACC - 1][i]);
+          for (int t = 0; t < S; ++t) {
+            bf16x8 al, ah, bl, bh;
+            widen_i8x16(wa[t][j], al, ah);
+            if (UP) widen_i8x16(wb[t][j], bl, bh);
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+              uint4 x0 = xa[j][i][0], x1 = xa[j][i][AV - 1];
+              acc[0][t][i] = mfma(*(bf16x8*)&x0, al, acc[0][t][i]);
+              acc[0][t][i] = mfma(*(bf16x8*)&x1, ah, acc[0][t][i]);
+              if (UP) {
+                acc[NACC - 1][t][i] = mfma(*(bf16x8*)&x0, bl, acc[NACC - 1][t][i]);
+                acc[NACC - 1][t][i] = mfma(*(bf16x8*)&x1, bh, acc[NACC - 1][t][i]);
+              }
             }
           }
         } else {
 #pragma unroll
-          for (int i = 0; i < MT; ++i) {
-            acc[0][i] = mfma(xa[j][i][0], wa[j], acc[0][i]);
-            if (UP) acc[NACC - 1][i] = mfma(xa[j][i][0], wb[j], acc[NACC - 1][i]);
-          }
+          for (int t = 0; t < S; ++t)
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+              acc[0][t][i] = mfma(xa[j][i][0], wa[t][j], acc[0][t][i]);
+              if (UP) acc[NACC - 1][t][i] = mfma(xa[j][i][0], wb[t][j], acc[NACC - 1][t][i]);
+            }
         }
       }
     }
@@ -264,12 +279,14 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p_r
   }
 
   // Reduce the four K-slices through LDS; wave 0 finishes.
-  __shared__ f32x4 red[kWavesPerWg - 1][NACC][MT][64];
+  __shared__ f32x4 red[kWavesPerWg - 1][NACC][S][MT][64];
   if (wave > 0) {
 #pragma unroll
     for (int n = 0; n < NACC; ++n)
 #pragma unroll
-      for (int i = 0; i < MT; ++i) red[wave - 1][n][i][lane] = acc[n][i];
+      for (int t = 0; t < S; ++t)
+#pragma unroll
+        for (int i = 0; i < MT; ++i) red[wave - 1][n][t][i][lane] = acc[n][t][i];
   }
   __syncthreads();
   if (wave != 0) return;
@@ -278,29 +295,34 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p_r
 #pragma unroll
     for (int n = 0; n < NACC; ++n)
 #pragma unroll
-      for (int i = 0; i < MT; ++i) acc[n][i] += red[w][n][i][lane];
+      for (int t = 0; t < S; ++t)
+#pragma unroll
+        for (int i = 0; i < MT; ++i) acc[n][t][i] += red[w][n][t][i][lane];
 
   // D layout: lane holds rows 4*kq + r (r = 0..3) of column mm.
-  const int n = nb * 16 + mm;
-  float sa = 1.f, sb = 1.f;
-  if (INT8 && !PG) {
-    sa = n < p.n_rows ? p.sa[(size_t)e * p.n_rows + n] : 0.f;
-    if (UP) sb = n < p.n_rows ? p.sb[(size_t)e * p.n_rows + n] : 0.f;
-  }
 #pragma unroll
-  for (int i = 0; i < MT; ++i) {
+  for (int t = 0; t < S; ++t) {
+    const int n = (nb + t) * 16 + mm;
+    float sa = 1.f, sb = 1.f;
+    if (INT8 && !PG) {
+      sa = n < p.n_rows ? p.sa[(size_t)e * p.n_rows + n] : 0.f;
+      if (UP) sb = n < p.n_rows ? p.sb[(size_t)e * p.n_rows + n] : 0.f;
+    }
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      int pos = m0 + 16 * i + 4 * kq + r;
-      if (pos >= cnt) continue;
-      if (UP) {
-        float g = acc[0][i][r] * sa;
-        float uu = acc[NACC - 1][i][r] * sb;
-        float h = (g / (1.f + __expf(-g))) * uu;
-        ((uint16_t*)p.out)[(size_t)(base + pos) * p.out_stride + n] = bf16_rne(h);
-      } else if (n < p.n_rows) {
-        int pair = p.g.perm[base + pos];
-        ((float*)p.out)[(size_t)pair * p.out_stride + n] = acc[0][i][r] * sa;
+    for (int i = 0; i < MT; ++i) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        int pos = m0 + 16 * i + 4 * kq + r;
+        if (pos >= cnt) continue;
+        if (UP) {
+          float g = acc[0][t][i][r] * sa;
+          float uu = acc[NACC - 1][t][i][r] * sb;
+          float h = (g / (1.f + __expf(-g))) * uu;
+          ((uint16_t*)p.out)[(size_t)(base + pos) * p.out_stride + n] = bf16_rne(h);
+        } else if (n < p.n_rows) {
+          int pair = p.g.perm[base + pos];
+          ((float*)p.out)[(size_t)pair * p.out_stride + n] = acc[0][t][i][r] * sa;
+        }
       }
     }
   }
@@ -417,7 +439,14 @@ hipError_t launch_stream(const StreamParams& p, int n_groups, int rows_max, hipS
   const StreamParams ps = shared ? *shared : p;
   const int shared_y = shared ? n_groups : -1;
   const int n_pad = shared && shared->n_pad > p.n_pad ? shared->n_pad : p.n_pad;
-  dim3 grid(n_pad / 16, n_groups + (shared ? 1 : 0), (rows_max + 16 * mt - 1) / (16 * mt));
+  // Two strips per workgroup once experts can have more than 16 rows (per-row scales only):
+  // int8 in both phases, bf16 in the down phase.  Measured at T = 48 on the Mixtral shape:
+  // int8 gate/up 177 -> 159 us, down 118 -> 97 us; bf16 down 170 -> 151 us, while the bf16
+  // gate/up form (218 registers) is slower, 299 -> 331 us, and keeps one strip.
+  const bool two = mt == 2 && (INT8 || !UP) && !(INT8 && p.group_blocks > 0) &&
+                   p.n_pad % 32 == 0 && (!shared || shared->n_pad % 32 == 0);
+  dim3 grid(n_pad / (two ? 32 : 16), n_groups + (shared ? 1 : 0),
+            (rows_max + 16 * mt - 1) / (16 * mt));
   // The down projection has few strips (d / 16) and a long K (f): eight K slices per strip
   // keep enough loads in flight; gate/up has 2f / 16 strips and uses four.
   constexpr int W = UP ? 4 : 8;
@@ -430,6 +459,8 @@ hipError_t launch_stream(const StreamParams& p, int n_groups, int rows_max, hipS
   }
   if (mt == 1)
     ffn_stream_kernel<1, INT8, UP, W, false><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
+  else if (two)
+    ffn_stream_kernel<2, INT8, UP, W, false, 2><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
   else
     ffn_stream_kernel<2, INT8, UP, W, false><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
   return hipGetLastError();

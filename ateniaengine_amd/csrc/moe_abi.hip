@@ -150,16 +150,17 @@ int stream_max_tokens_override() {
 }
 constexpr int kStreamMaxTokens = 56;
 // Whether a batch of T tokens whose experts see rows_num / rows_den rows each on average
-// (T * k / E) is served by the weight-streaming kernels.  Those pass
-// over an expert's weights once per 32 of its rows, while the tiled kernels cost about the same
-// from about 50 tokens to a few hundred, so beyond 56 tokens the choice goes by the average rows per
-// expert.  Measured cross-overs on MI355X: about 9 rows for bf16 weights (Qwen1.5-MoE shape
-// T = 140, DeepSeek-V2-Lite shape T = 100), about 24 for int8 (Mixtral shape T = 100), whose tiled
-// kernel widens every weight in the VALU however few rows it multiplies.
-bool batch_streams(int T, long long rows_num, long long rows_den, bool int8) {
+// (T * k / E) is served by the weight-streaming kernels.  Those pass over an expert's weights
+// once per 32 of its rows, while the tiled kernels cost about the same from about 50 tokens to a
+// few hundred, so beyond 56 tokens the choice goes by the average rows per expert.  Measured
+// cross-overs on MI355X: 15-21 rows for bf16 weights (Mixtral shape T = 85, Qwen1.5-MoE shape
+// T = 256, DeepSeek-V2-Lite shape T = 175), 35 for int8 with per-row scales (Mixtral shape
+// T = 140; its tiled kernel widens every weight in the VALU however few rows it multiplies),
+// about 26 for per-group int8 (one strip per workgroup in the streaming kernel).
+bool batch_streams(int T, long long rows_num, long long rows_den, int max_avg_rows) {
   if (const int n = stream_max_tokens_override()) return T <= n;
   if (T <= kStreamMaxTokens) return true;
-  return rows_num <= rows_den * (int8 ? 24 : 9);
+  return rows_num <= rows_den * max_avg_rows;
 }
 // Largest batch routed by the one-workgroup-per-token router kernel (tuning knob:
 // ATENIA_MOE_ROUTER_TOKEN_MAX, read once per process).
@@ -431,7 +432,8 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   // reference's GPU path multiplies with, src/cuda/int8_to_bf16.cu:91-110) for such batches;
   // decode batches stream the int8 weights themselves.
   const bool int8w = L->wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
-  const bool routed_streams = batch_streams(T, (long long)T * L->k, L->E, int8w);
+  const bool routed_streams =
+      batch_streams(T, (long long)T * L->k, L->E, !int8w ? 16 : L->group_size > 0 ? 24 : 32);
   const bool pg_prefill = L->group_size > 0 && !routed_streams && L->d_kpad % 64 == 0 &&
                           L->f_kpad % 64 == 0 && (L->fs == 0 || L->fs_kpad % 64 == 0);
   if (pg_prefill && !L->pg_ready) {
