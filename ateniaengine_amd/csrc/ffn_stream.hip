@@ -104,7 +104,6 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p_r
   constexpr int kWavesPerWg = WAVES;
   const bool sh = (int)blockIdx.y == shared_y;
   const StreamParams& p = sh ? p_shared : p_routed;
-  static_assert(S == 1 || !PG, "two strips per workgroup: per-row scales only");
   if ((int)blockIdx.x * 16 * S >= p.n_pad) return;  // the grid spans the wider of the two
   const int u = sh ? 0 : blockIdx.y;
   if (u >= *p.g.n_active) return;
@@ -154,9 +153,10 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p_r
   const size_t n_pad_s = (size_t)p.n_pad;  // scale rows per k group
   const float* psa = PG ? p.sa + (size_t)e * p.n_kgroups * n_pad_s + nb * 16 + mm : nullptr;
   const float* psb = PG && UP ? p.sb + (size_t)e * p.n_kgroups * n_pad_s + nb * 16 + mm : nullptr;
-  float sA0[PG ? U : 1], sB0[PG && UP ? U : 1], sA1[PG ? U : 1], sB1[PG && UP ? U : 1];
-  auto load_w = [&](uint4 (&wa)[S][U], uint4 (&wb)[S][UP ? U : 1], float (&sa)[PG ? U : 1],
-                    float (&sb)[PG && UP ? U : 1], int kb) {
+  constexpr int SP = PG ? S : 1, UA = PG ? U : 1, UB = PG && UP ? U : 1;
+  float sA0[SP][UA], sB0[SP][UB], sA1[SP][UA], sB1[SP][UB];
+  auto load_w = [&](uint4 (&wa)[S][U], uint4 (&wb)[S][UP ? U : 1], float (&sa)[SP][UA],
+                    float (&sb)[SP][UB], int kb) {
 #pragma unroll
     for (int j = 0; j < U; ++j) {
       const int kk = min(kb + j, kb1 - 1);  // clamped: a batch past the end is loaded, not used
@@ -167,8 +167,11 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p_r
       }
       if (PG) {
         const int kg = kk / p.group_blocks;
-        sa[j] = psa[(size_t)kg * n_pad_s];
-        if (UP) sb[j] = psb[(size_t)kg * n_pad_s];
+#pragma unroll
+        for (int t = 0; t < SP; ++t) {
+          sa[t][j] = psa[(size_t)kg * n_pad_s + 16 * t];
+          if (UP) sb[t][UB > 1 ? j : 0] = psb[(size_t)kg * n_pad_s + 16 * t];
+        }
       }
     }
   };
@@ -211,27 +214,30 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p_r
 #pragma unroll
       for (int i = 0; i < MT; ++i) acc[n][t][i] = f32x4{0.f, 0.f, 0.f, 0.f};
   auto multiply = [&](const uint4 (&wa)[S][U], const uint4 (&wb)[S][UP ? U : 1],
-                      const float (&sa)[PG ? U : 1], const float (&sb)[PG && UP ? U : 1],
+                      const float (&sa)[SP][UA], const float (&sb)[SP][UB],
                       const uint4 (&xa)[U][MT][AV], int kb) {
 #pragma unroll
     for (int j = 0; j < U; ++j) {
       if (kb + j < kb1) {
         if (INT8 && PG) {
-          bf16x8 al, ah, bl, bh;
-          widen_i8x16(wa[0][j], al, ah);
-          if (UP) widen_i8x16(wb[0][j], bl, bh);
-          const float s_a = sa[PG ? j : 0];
-          const float s_b = UP ? sb[PG && UP ? j : 0] : 0.f;
 #pragma unroll
-          for (int i = 0; i < MT; ++i) {
-            uint4 x0 = xa[j][i][0], x1 = xa[j][i][AV - 1];
-            f32x4 ta = mfma(*(bf16x8*)&x0, al, f32x4{0.f, 0.f, 0.f, 0.f});
-            ta = mfma(*(bf16x8*)&x1, ah, ta);
-            acc[0][0][i] += ta * s_a;
-            if (UP) {
-              f32x4 tb = mfma(*(bf16x8*)&x0, bl, f32x4{0.f, 0.f, 0.f, 0.f});
-              tb = mfma(*(bf16x8*)&x1, bh, tb);
-              acc[NACC - 1][0][i] += tb * s_b;
+          for (int t = 0; t < S; ++t) {
+            bf16x8 al, ah, bl, bh;
+            widen_i8x16(wa[t][j], al, ah);
+            if (UP) widen_i8x16(wb[t][j], bl, bh);
+            const float s_a = sa[PG ? t : 0][PG ? j : 0];
+            const float s_b = UP ? sb[PG ? t : 0][PG && UP ? j : 0] : 0.f;
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+              uint4 x0 = xa[j][i][0], x1 = xa[j][i][AV - 1];
+              f32x4 ta = mfma(*(bf16x8*)&x0, al, f32x4{0.f, 0.f, 0.f, 0.f});
+              ta = mfma(*(bf16x8*)&x1, ah, ta);
+              acc[0][t][i] += ta * s_a;
+              if (UP) {
+                f32x4 tb = mfma(*(bf16x8*)&x0, bl, f32x4{0.f, 0.f, 0.f, 0.f});
+                tb = mfma(*(bf16x8*)&x1, bh, tb);
+                acc[NACC - 1][t][i] += tb * s_b;
+              }
             }
           }
         } else if (INT8) {
@@ -439,12 +445,12 @@ hipError_t launch_stream(const StreamParams& p, int n_groups, int rows_max, hipS
   const StreamParams ps = shared ? *shared : p;
   const int shared_y = shared ? n_groups : -1;
   const int n_pad = shared && shared->n_pad > p.n_pad ? shared->n_pad : p.n_pad;
-  // Two strips per workgroup once experts can have more than 16 rows (per-row scales only):
-  // int8 in both phases, bf16 in the down phase.  Measured at T = 48 on the Mixtral shape:
+  // Two strips per workgroup once experts can have more than 16 rows:
+  // int8 (per-row and per-group scales) in both phases, bf16 in the down phase.  Measured at T = 48 on the Mixtral shape:
   // int8 gate/up 177 -> 159 us, down 118 -> 97 us; bf16 down 170 -> 151 us, while the bf16
   // gate/up form (218 registers) is slower, 299 -> 331 us, and keeps one strip.
-  const bool two = mt == 2 && (INT8 || !UP) && !(INT8 && p.group_blocks > 0) &&
-                   p.n_pad % 32 == 0 && (!shared || shared->n_pad % 32 == 0);
+  const bool two = mt == 2 && (INT8 || !UP) && p.n_pad % 32 == 0 &&
+                   (!shared || shared->n_pad % 32 == 0);
   dim3 grid(n_pad / (two ? 32 : 16), n_groups + (shared ? 1 : 0),
             (rows_max + 16 * mt - 1) / (16 * mt));
   // The down projection has few strips (d / 16) and a long K (f): eight K slices per strip
@@ -453,6 +459,8 @@ hipError_t launch_stream(const StreamParams& p, int n_groups, int rows_max, hipS
   if (INT8 && p.group_blocks > 0) {
     if (mt == 1)
       ffn_stream_kernel<1, INT8, UP, W, INT8><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
+    else if (two)
+      ffn_stream_kernel<2, INT8, UP, W, INT8, 2><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
     else
       ffn_stream_kernel<2, INT8, UP, W, INT8><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
     return hipGetLastError();

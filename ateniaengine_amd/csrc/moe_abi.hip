@@ -154,9 +154,9 @@ constexpr int kStreamMaxTokens = 56;
 // once per 32 of its rows, while the tiled kernels cost about the same from about 50 tokens to a
 // few hundred, so beyond 56 tokens the choice goes by the average rows per expert.  Measured
 // cross-overs on MI355X: 15-21 rows for bf16 weights (Mixtral shape T = 85, Qwen1.5-MoE shape
-// T = 256, DeepSeek-V2-Lite shape T = 175), 35 for int8 with per-row scales (Mixtral shape
-// T = 140; its tiled kernel widens every weight in the VALU however few rows it multiplies),
-// about 26 for per-group int8 (one strip per workgroup in the streaming kernel).
+// T = 256, DeepSeek-V2-Lite shape T = 175), 35 for int8 with per-row or per-group scales
+// (Mixtral shape T = 140; the tiled int8 kernel widens every weight in the VALU however few rows
+// it multiplies, and per-group layers run the tiled kernels on a bf16 copy).
 bool batch_streams(int T, long long rows_num, long long rows_den, int max_avg_rows) {
   if (const int n = stream_max_tokens_override()) return T <= n;
   if (T <= kStreamMaxTokens) return true;
@@ -433,7 +433,7 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   // decode batches stream the int8 weights themselves.
   const bool int8w = L->wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
   const bool routed_streams =
-      batch_streams(T, (long long)T * L->k, L->E, !int8w ? 16 : L->group_size > 0 ? 24 : 32);
+      batch_streams(T, (long long)T * L->k, L->E, int8w ? 32 : 16);
   const bool pg_prefill = L->group_size > 0 && !routed_streams && L->d_kpad % 64 == 0 &&
                           L->f_kpad % 64 == 0 && (L->fs == 0 || L->fs_kpad % 64 == 0);
   if (pg_prefill && !L->pg_ready) {
