@@ -449,15 +449,18 @@ hipError_t launch_stream(const StreamParams& p, int n_groups, int rows_max, hipS
   // int8 (per-row and per-group scales) in both phases, bf16 in the down phase.  Measured at T = 48 on the Mixtral shape:
   // int8 gate/up 177 -> 159 us, down 118 -> 97 us; bf16 down 170 -> 151 us, while the bf16
   // gate/up form (218 registers) is slower, 299 -> 331 us, and keeps one strip.
-  const bool two = mt == 2 && (INT8 || !UP) && p.n_pad % 32 == 0 &&
-                   (!shared || shared->n_pad % 32 == 0);
+  // With a single row tile only the int8 down phase gains (T = 16: 86 -> 77 us), from 4 rows on.
+  const bool two = (mt == 2 ? (INT8 || !UP) : (INT8 && !UP && rows_max >= 4)) &&
+                   p.n_pad % 32 == 0 && (!shared || shared->n_pad % 32 == 0);
   dim3 grid(n_pad / (two ? 32 : 16), n_groups + (shared ? 1 : 0),
             (rows_max + 16 * mt - 1) / (16 * mt));
   // The down projection has few strips (d / 16) and a long K (f): eight K slices per strip
   // keep enough loads in flight; gate/up has 2f / 16 strips and uses four.
   constexpr int W = UP ? 4 : 8;
   if (INT8 && p.group_blocks > 0) {
-    if (mt == 1)
+    if (mt == 1 && two)
+      ffn_stream_kernel<1, INT8, UP, W, INT8, 2><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
+    else if (mt == 1)
       ffn_stream_kernel<1, INT8, UP, W, INT8><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
     else if (two)
       ffn_stream_kernel<2, INT8, UP, W, INT8, 2><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
@@ -465,7 +468,9 @@ hipError_t launch_stream(const StreamParams& p, int n_groups, int rows_max, hipS
       ffn_stream_kernel<2, INT8, UP, W, INT8><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
     return hipGetLastError();
   }
-  if (mt == 1)
+  if (mt == 1 && two)
+    ffn_stream_kernel<1, INT8, UP, W, false, 2><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
+  else if (mt == 1)
     ffn_stream_kernel<1, INT8, UP, W, false><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
   else if (two)
     ffn_stream_kernel<2, INT8, UP, W, false, 2><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
