@@ -56,9 +56,9 @@ CONFIG_NAME = "mixtral_bf16"
 # (FETCH_SIZE counts 2 KiB units, WRITE_SIZE KiB): profiles/
 # ffn_kernels_mixtral_bf16_T4096_T1_hbm_counters.txt.  Keyed by (config, tokens per step).
 MEASURED_HBM_TRAFFIC = {
-    ("mixtral_bf16", 4096): {"expert_gate_up": 2530461.5 * 2048 + 229376.0 * 1024,
-                             "expert_down": 1261823.8 * 2048 + 169318.0 * 1024},
-    ("mixtral_bf16", 1): {"expert_gate_up": 229450.4 * 2048, "expert_down": 114941.2 * 2048},
+    ("mixtral_bf16", 4096): {"expert_gate_up": 2534048.7 * 2048 + 229376.0 * 1024,
+                             "expert_down": 1261307.5 * 2048 + 169317.3 * 1024},
+    ("mixtral_bf16", 1): {"expert_gate_up": 229448.8 * 2048, "expert_down": 114935.2 * 2048},
 }
 
 
