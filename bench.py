@@ -26,16 +26,16 @@ sys.path.insert(0, ROOT)
 # reported with --config.
 CONFIGS = {
     "mixtral_bf16": dict(d=4096, E=8, k=2, f=14336, fs=0, gated=False, conv=0, wd="bf16",
-                         zipf=False, sweep=(1, 16, 128, 512, 4096)),
+                         zipf=False, sweep=(1, 16, 32, 64, 128, 512, 4096)),
     "mixtral_int8": dict(d=4096, E=8, k=2, f=14336, fs=0, gated=False, conv=0, wd="int8",
-                         zipf=False, sweep=(1, 16, 4096)),
+                         zipf=False, sweep=(1, 16, 32, 64, 128, 4096)),
     # per-group int8 (one scale per output row and 128 input elements, Q8_0-style)
     "mixtral_int8g": dict(d=4096, E=8, k=2, f=14336, fs=0, gated=False, conv=0, wd="int8g",
-                          zipf=False, sweep=(1, 16, 4096)),
+                          zipf=False, sweep=(1, 16, 32, 64, 128, 4096)),
     "qwen_bf16": dict(d=2048, E=60, k=4, f=1408, fs=5632, gated=True, conv=1, wd="bf16",
-                      zipf=False, sweep=(1, 256, 8192)),
+                      zipf=False, sweep=(1, 16, 64, 128, 256, 8192)),
     "deepseek_bf16": dict(d=2048, E=64, k=6, f=1408, fs=2816, gated=False, conv=1, wd="bf16",
-                          zipf=True, sweep=(1, 1024, 16384)),
+                          zipf=True, sweep=(1, 16, 64, 1024, 16384)),
     # DeepSeek-V3 router shape (256 experts in 8 groups, top-8 of the 4 best groups) in front of
     # narrow experts: times the sigmoid / group-limited routing path, not a checkpoint shape.
     "v3route_bf16": dict(d=7168, E=256, k=8, f=256, fs=256, gated=False, conv=1, wd="bf16",
