@@ -10,8 +10,9 @@
 // The bound here is HBM: every weight byte of an active expert is read exactly once per
 // launch, straight from global memory into the MFMA B-operand registers (the weights are
 // stored in that register layout, see moe_internal.h), 1 KiB per wave per load, several
-// loads in flight.  A workgroup owns one 16-row strip of W_g and W_u (or of W_d); its four
-// waves split K and reduce through LDS.  Token rows (A operand) come from L2.
+// loads in flight.  A workgroup owns one or two adjacent 16-row strips of W_g and W_u (four
+// waves) or of W_d (eight waves); its waves split K and reduce through LDS.  Token rows (A
+// operand) come from L2.
 #include "moe_internal.h"
 
 #include "../../include/atenia_moe_hip.h"

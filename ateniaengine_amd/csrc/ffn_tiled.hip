@@ -2,23 +2,27 @@
 //
 //   gate/up : H[rows of e, f] = silu(X_e W_g^T) * (X_e W_u^T)     (src/moe/dense.rs:253-266)
 //   down    : Y[rows of e, d] = H_e W_d^T                         (src/moe/dense.rs:267-269)
-// on v_mfma_f32_16x16x32_bf16 with f32 accumulation.  The bound is the matrix pipeline.
+// on bf16 MFMA with f32 accumulation.  The bound is the matrix pipeline.
 //
-// A workgroup (4 waves, one per SIMD) owns a 256 x 256 output tile of one expert: 256
-// grouped token rows by 256 weight rows (gate/up phase: 128 gate rows plus the SAME 128 up
-// rows, so silu(g)*u is formed in registers).  Each wave owns 128 x 128 of it as 8 x 8 MFMA
-// tiles (256 accumulator registers); per 32-wide k step it reads 8 A and 8 B fragments from
-// LDS for 64 MFMAs, which keeps LDS at half its bandwidth.
+// A workgroup (4 waves, one per SIMD) owns a 256 x 256 output tile of one expert: 256 grouped
+// token rows by 256 weight rows (gate/up phase: 128 gate rows plus the SAME 128 up rows, so
+// silu(g)*u is formed in registers); each wave owns 128 x 128 of it.  Token rows are gathered
+// through the permutation while they are loaded (no permuted copy of X is ever written).
 //
-// LDS holds both operands as 1 KiB chunks already in MFMA register order (lane l owns bytes
-// 16*l), so every fragment read is one conflict-free ds_read_b128.  Weights are stored in HBM
-// in that same chunk layout (moe_internal.h), so a B chunk is a straight 1 KiB copy; token
-// rows are gathered through the permutation while they are loaded (no permuted copy of X is
-// ever written).  INT8 W8A16 weights are widened to bf16 on their way into LDS and the
-// per-row scale is applied to the accumulator.
-//
-// Two LDS stages of 64 k each: global loads of stage i+1 are issued into registers before
-// the MFMAs of stage i and stored to the other LDS buffer after them.
+// Three kernels share this tiling:
+//   ffn_tiled_pipe_kernel     bf16 weights, K a multiple of 64 and >= 128: 4 x 4 tiles of
+//                             v_mfma_f32_32x32x16_bf16 per wave, operands go global -> LDS
+//                             directly (global_load_lds_dwordx4) into a ring of three 64-k A
+//                             stages and four 32-k B stages, software-pipelined in units of 16
+//                             MFMAs with one barrier per 32-k step
+//   ffn_tiled_pipe_i8_kernel  INT8 W8A16, K >= 128: same pipeline, weights stay int8 into LDS and
+//                             are widened to bf16 in registers, row scale applied to the
+//                             accumulator
+//   ffn_tiled_kernel          fallback for other K: 8 x 8 tiles of v_mfma_f32_16x16x32_bf16 per
+//                             wave, two 64-k LDS stages filled through registers (int8 widened on
+//                             the way into LDS)
+// Weights are stored in HBM as 1 KiB blocks already in MFMA register order (moe_internal.h), so
+// a B chunk is a straight 1 KiB copy and every B fragment read is one ds_read_b128.
 #include <type_traits>
 
 #include "moe_internal.h"

@@ -428,9 +428,10 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   const int a_stride = f32w ? L->d : L->d_kpad;
 
   // Per-group int8 and a batch for the MFMA-tiled kernels: those take one scale per row, so the
-  // layer keeps a bf16 copy of its experts (q * group scale, rounded to bf16 -- the form the
-  // reference's GPU path multiplies with, src/cuda/int8_to_bf16.cu:91-110) for such batches;
-  // decode batches stream the int8 weights themselves.
+  // layer keeps a bf16 copy of its experts for such batches: q * group scale rounded to the
+  // nearest bf16 (the reference's GPU dequantiser truncates instead,
+  // src/cuda/int8_to_bf16.cu:91-110; rounding halves the error against the q * scale the
+  // reference's CPU path multiplies with).  Decode batches stream the int8 weights themselves.
   const bool int8w = L->wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
   const bool routed_streams =
       batch_streams(T, (long long)T * L->k, L->E, int8w ? 32 : 16);

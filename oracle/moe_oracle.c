@@ -28,10 +28,13 @@
  *              ora_v3_layer_forward (router and block output against the
  *              HuggingFace f64 fixture; its f32 combine is this build's choice,
  *              see the function).
- *   parity unpinned (no reference counterpart; defined by this build):
- *              the `router_bias` term of ora_route (the reference router has
- *              no bias, dense.rs:333).  With router_bias == NULL ora_route is
- *              pinned like the rest.
+ *   no reference counterpart: the `router_bias` term of ora_route (the
+ *              reference router has no bias, dense.rs:333).  Its arithmetic --
+ *              one f32 addition to the rounded logit, indexed by expert -- is
+ *              pinned by tests/test_oracle_router_bias.py against a NumPy
+ *              restatement built on the pinned softmax / top-k, with closed
+ *              forms and engineered ties.  With router_bias == NULL ora_route
+ *              is pinned like the rest.
  *   platform note: exp() is the host libm's; the reference uses Rust's
  *              f64::exp (also the platform libm).  Last-ulp differences of
  *              exp between platforms are not pinned by any fixture.
