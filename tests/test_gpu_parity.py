@@ -229,9 +229,14 @@ def check_layer(ora, oL, gL, x, tol, sample=None, model=True):
     assert worst <= tol, f"layer output off by {worst:.3e} (bar {tol})"
     if model and gL.weight_dtype != capi.WEIGHT_F32:
         rows = np.array(list(rows))
-        em = S.emulate_bf16_kernels(oL, x[rows], o_idx[rows], o_w[rows])
-        dist = max(S.rel_err(out[t], em[i]) for i, t in enumerate(rows))
-        assert dist <= TOL_MODEL, f"HIP path is {dist:.3e} away from its arithmetic model"
+        em, slack = S.emulate_bf16_kernels(oL, x[rows], o_idx[rows], o_w[rows], with_slack=True)
+        # per token: TOL_MODEL of its largest output, plus what a bf16 rounding flip of its
+        # fragile h elements can move (zero for all but a few tokens; see synth.py)
+        for i, t in enumerate(rows):
+            dist = float(np.abs(out[t].astype(np.float64) - em[i]).max())
+            bar = TOL_MODEL * float(np.abs(em[i]).max()) + slack[i]
+            assert dist <= bar, (f"token {t}: HIP path is {dist:.3e} away from its arithmetic "
+                                 f"model (bar {bar:.3e}, of which rounding flips {slack[i]:.3e})")
     return out, worst
 
 
@@ -250,6 +255,10 @@ LAYER_CASES = [
     # (several row slices per expert, the shared expert's T rows riding in the same launches)
     ("wide_bf16", 40, 2, 128, 96, 64, True, 1, capi.WEIGHT_BF16, TOL_BF16),
     ("wide_int8", 40, 3, 128, 352, 0, False, 0, capi.WEIGHT_INT8_W8A16, TOL_BF16),
+    # narrow experts: the down projection's K (96) is padded to one 128-k stage pair and the
+    # gate/up N is less than one column tile; at T = 700 one h element of one token sits on a bf16
+    # rounding midpoint (the arithmetic model's slack covers exactly that)
+    ("wide_narrow_int8", 40, 3, 128, 96, 0, False, 0, capi.WEIGHT_INT8_W8A16, TOL_BF16),
 ]
 
 
