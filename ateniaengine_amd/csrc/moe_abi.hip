@@ -76,6 +76,20 @@ int kb_of(int wdtype) { return wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16 ? kKbInt8 
 
 }  // namespace
 
+// Pointers into one workspace (device memory beyond the inputs and outputs of a forward).
+struct WsView {
+  int cap_tokens = 0;  // tokens the view was laid out for
+  int y_parts = 1;     // partial output buffers of the tiled down phase it has room for
+  uint16_t* xb = nullptr;
+  int32_t *idx = nullptr, *counts = nullptr, *offsets = nullptr, *active = nullptr,
+          *n_active = nullptr, *perm = nullptr, *inv = nullptr, *blk_counts = nullptr,
+          *shared_desc = nullptr, *ident = nullptr, *tile_group = nullptr, *tile_m0 = nullptr,
+          *s_tile_group = nullptr, *s_tile_m0 = nullptr;
+  float *w = nullptr, *sgate = nullptr, *y = nullptr, *ys = nullptr, *logits = nullptr;
+  void *h = nullptr, *hs = nullptr;
+  uint8_t* part_flags = nullptr;
+};
+
 struct AteniaMoeLayer {
   uint32_t magic = 0x4d6f4541u;
   int E = 0, k = 0, d = 0, f = 0, fs = 0, conv = 0, wdtype = 0;
@@ -91,17 +105,16 @@ struct AteniaMoeLayer {
   WeightSet gate{}, up{}, down{}, s_gate{}, s_up{}, s_down{};
   int64_t bytes_per_expert = 0;
 
-  // workspace (grow-only in tokens)
-  int cap_tokens = 0;
-  DevBuf x_in, out, xb, idx, w, sgate, counts, offsets, active, n_active, perm, inv, blk_counts,
-      shared_desc, ident, h, hs, y, ys, status, tile_group, tile_m0, s_tile_group, s_tile_m0,
-      part_flags;
+  // workspace (grow-only in tokens): one slab carved by ws_layout; `cur` is the view the most
+  // recent forward ran on (the handle's own, or the static scratch of the no-alloc entry point)
+  DevBuf slab, x_in, out, status;
+  WsView ws{}, cur{};
   DevBuf xn, gamma_in;  // block forward: normalised rows [T, d] f32; gamma of the host variant
   // DeepSeek-V3 routing (off while v3_n_group == 0): the router kernels leave raw logits in
   // `logits` and v3_route_kernel decides from them
   int v3_n_group = 0, v3_topk_group = 0, v3_norm = 0;
   double v3_scale = 1.0;
-  DevBuf v3_bias, logits;
+  DevBuf v3_bias;
   // per-group int8: bf16 copies for the MFMA-tiled (prefill) kernels, made on first use
   DevBuf pg_wg, pg_wu, pg_wd, pg_swg, pg_swu, pg_swd;
   WeightSet gate_b{}, up_b{}, down_b{}, s_gate_b{}, s_up_b{}, s_down_b{};
@@ -114,6 +127,12 @@ struct AteniaMoeLayer {
 
   hipStream_t stream = nullptr;
   std::mutex mu;
+  // Ordering of asynchronous forwards on one handle: every forward records `done` at its end and
+  // a forward on another stream waits for it first, so two streams never use the workspace at
+  // the same time (skipped while a stream is being captured into a graph).
+  hipEvent_t done = nullptr;
+  hipStream_t done_stream = nullptr;
+  bool done_valid = false;
 
   bool profiling = false;
   int policy = ATENIA_MOE_POLICY_CERTIFIED;  // expert arithmetic of f32 layers
@@ -258,52 +277,107 @@ int make_bf16_copy(const WeightSet& q, int G, DevBuf& dst, WeightSet& out) {
   return ATENIA_MOE_OK;
 }
 
-int ensure_workspace(AteniaMoeLayer* L, int T) {
-  if (T <= L->cap_tokens) return ATENIA_MOE_OK;
+// Lays a workspace for T tokens out from `base` (256-byte aligned pieces) and returns its size;
+// with v == nullptr only the size is computed.  y_parts: partial output buffers of the down phase.
+size_t ws_layout(const AteniaMoeLayer* L, int T, int y_parts, uint8_t* base, WsView* v) {
   const size_t P = (size_t)T * L->k;
   const bool f32w = L->wdtype == ATENIA_MOE_WEIGHT_F32;
   const size_t act = f32w ? 4 : 2;
-  int rc = 0;
-#define ENS(buf, bytes)                 \
-  if ((rc = L->buf.ensure(bytes))) return rc;
-  ENS(x_in, (size_t)T * L->d * 4)
-  ENS(out, (size_t)T * L->d * 4)
-  if (!f32w) ENS(xb, (size_t)T * L->d_kpad * 2)
-  ENS(idx, P * 4)
-  ENS(w, P * 4)
-  ENS(sgate, (size_t)T * 4)
-  ENS(counts, (size_t)L->E * 4)
-  ENS(offsets, (size_t)(L->E + 1) * 4)
-  ENS(active, (size_t)L->E * 4)
-  ENS(n_active, 4)
-  ENS(perm, P * 4)
-  ENS(inv, P * 4)
-  ENS(blk_counts, ((P + kPermuteBlock - 1) / kPermuteBlock) * L->E * 4)
-  ENS(shared_desc, 32)  // [0..1] offsets {0,T}, [2] active {0}, [3] n_active {1},
-                        // [4] routed row tiles, [5] shared row tiles
+  size_t off = 0;
+  auto take = [&](size_t bytes) {
+    uint8_t* p = base ? base + off : nullptr;
+    off += (bytes + 255) / 256 * 256;
+    return p;
+  };
+  WsView t{};
+  t.cap_tokens = T;
+  t.y_parts = y_parts;
+  if (!f32w) t.xb = (uint16_t*)take((size_t)T * L->d_kpad * 2);
+  t.idx = (int32_t*)take(P * 4);
+  t.w = (float*)take(P * 4);
+  t.sgate = (float*)take((size_t)T * 4);
+  t.counts = (int32_t*)take((size_t)L->E * 4);
+  t.offsets = (int32_t*)take((size_t)(L->E + 1) * 4);
+  t.active = (int32_t*)take((size_t)L->E * 4);
+  t.n_active = (int32_t*)take(4);
+  t.perm = (int32_t*)take(P * 4);
+  t.inv = (int32_t*)take(P * 4);
+  t.blk_counts = (int32_t*)take(((P + kPermuteBlock - 1) / kPermuteBlock) * L->E * 4);
+  // [0..1] offsets {0,T}, [2] active {0}, [3] n_active {1}, [4] routed row tiles, [5] shared row tiles
+  t.shared_desc = (int32_t*)take(32);
   const size_t max_tiles = (P + kTileM - 1) / kTileM + L->E;
-  ENS(tile_group, max_tiles * 4)
-  ENS(tile_m0, max_tiles * 4)
-  ENS(s_tile_group, ((size_t)T / kTileM + 1) * 4)
-  ENS(s_tile_m0, ((size_t)T / kTileM + 1) * 4)
-  ENS(ident, (size_t)T * 4)
-  ENS(h, P * (size_t)L->f_kpad * act)
-  ENS(y, kMaxYParts * P * (size_t)L->d * 4)  // partial buffers for k ranges of tail tiles
-  ENS(part_flags, P * (size_t)((L->d + 255) / 256))
+  t.tile_group = (int32_t*)take(max_tiles * 4);
+  t.tile_m0 = (int32_t*)take(max_tiles * 4);
+  t.s_tile_group = (int32_t*)take(((size_t)T / kTileM + 1) * 4);
+  t.s_tile_m0 = (int32_t*)take(((size_t)T / kTileM + 1) * 4);
+  t.ident = (int32_t*)take((size_t)T * 4);
+  t.logits = (float*)take((size_t)T * L->E * 4);
+  t.h = take(P * (size_t)L->f_kpad * act);
+  t.y = (float*)take((size_t)y_parts * P * L->d * 4);  // one buffer per k range of tail tiles
+  t.part_flags = (uint8_t*)take(P * (size_t)((L->d + 255) / 256));
   if (L->fs > 0) {
-    ENS(hs, (size_t)T * L->fs_kpad * act)
-    ENS(ys, (size_t)T * L->d * 4)
+    t.hs = take((size_t)T * L->fs_kpad * act);
+    t.ys = (float*)take((size_t)T * L->d * 4);
   }
-  ENS(status, 8)
-#undef ENS
-  HIP_TRY(launch_fill_i32(L->ident.as<int32_t>(), T, 0, 1, nullptr));
-  HIP_TRY(launch_fill_i32(L->s_tile_m0.as<int32_t>(), T / kTileM + 1, 0, kTileM, nullptr));
-  int32_t sd[8] = {0, 0, 0, 1, 0, 0, 0, 0};
-  HIP_TRY(hipMemcpy(L->shared_desc.p, sd, 32, hipMemcpyHostToDevice));
-  int32_t st[2] = {0, INT_MAX};
-  HIP_TRY(hipMemcpy(L->status.p, st, 8, hipMemcpyHostToDevice));
+  if (v) *v = t;
+  return off;
+}
+
+// What a workspace must hold before its first forward: the identity row list and the row tiles
+// of the shared expert, its group descriptor, and zeros in the K padding of the h rows (the
+// expert kernels multiply the padding with zero weights, which only helps if it is finite).
+// A kernel, not memsets, so that the no-alloc entry point stays capturable into a graph.
+__global__ void workspace_init_kernel(int32_t* ident, int T, int32_t* s_tile_group,
+                                      int32_t* s_tile_m0, int n_s_tiles, int32_t* shared_desc,
+                                      uint16_t* h, int h_rows, int f, int f_kpad, uint16_t* hs,
+                                      int fs, int fs_kpad) {
+  const int stride = gridDim.x * blockDim.x;
+  const int i0 = blockIdx.x * blockDim.x + threadIdx.x;
+  for (int i = i0; i < T; i += stride) ident[i] = i;
+  for (int i = i0; i < n_s_tiles; i += stride) {
+    s_tile_group[i] = 0;
+    s_tile_m0[i] = i * kTileM;
+  }
+  if (i0 < 8) shared_desc[i0] = i0 == 3 ? 1 : 0;
+  const int pad = f_kpad - f;
+  if (h && pad > 0)
+    for (long long i = i0; i < (long long)h_rows * pad; i += stride)
+      h[(i / pad) * f_kpad + f + (i % pad)] = 0;
+  const int spad = fs_kpad - fs;
+  if (hs && spad > 0)
+    for (long long i = i0; i < (long long)T * spad; i += stride)
+      hs[(i / spad) * fs_kpad + fs + (i % spad)] = 0;
+}
+
+hipError_t launch_workspace_init(const AteniaMoeLayer* L, const WsView& V, int T, hipStream_t s) {
+  const bool f32w = L->wdtype == ATENIA_MOE_WEIGHT_F32;  // f32 rows carry no K padding
+  const long long work = (long long)T * L->k * (f32w ? 0 : L->f_kpad - L->f) + T;
+  const int blocks = (int)std::min<long long>(256, (work + 255) / 256);
+  workspace_init_kernel<<<blocks, 256, 0, s>>>(
+      V.ident, T, V.s_tile_group, V.s_tile_m0, T / kTileM + 1, V.shared_desc,
+      f32w ? nullptr : (uint16_t*)V.h, T * L->k, L->f, L->f_kpad,
+      f32w ? nullptr : (uint16_t*)V.hs, L->fs, L->fs_kpad);
+  return hipGetLastError();
+}
+
+int ensure_workspace(AteniaMoeLayer* L, int T) {
+  if (T <= L->ws.cap_tokens) return ATENIA_MOE_OK;
+  // the slab may be in use by a forward still running on some stream
   HIP_TRY(hipDeviceSynchronize());
-  L->cap_tokens = T;
+  const size_t bytes = ws_layout(L, T, kMaxYParts, nullptr, nullptr);
+  L->ws = WsView{};
+  L->cur = WsView{};
+  for (int st = 0; st < 4; ++st) L->stage_T[st] = -1;
+  L->last_T = 0;
+  int rc = L->slab.ensure(bytes);
+  if (rc) return rc;
+  WsView v{};
+  ws_layout(L, T, kMaxYParts, (uint8_t*)L->slab.p, &v);
+  if ((rc = L->x_in.ensure((size_t)T * L->d * 4))) return rc;
+  if ((rc = L->out.ensure((size_t)T * L->d * 4))) return rc;
+  HIP_TRY(launch_workspace_init(L, v, T, nullptr));
+  HIP_TRY(hipDeviceSynchronize());
+  L->ws = v;
   return ATENIA_MOE_OK;
 }
 
@@ -323,8 +397,52 @@ enum { kStageRouter = 0, kStagePermute = 1, kStageFfn = 2, kStageCombine = 3 };
 // Runs stages first..last of the pipeline on `s`.  A stage reads what the stages before it
 // left in the handle's workspace, so a range that does not start at the router is only valid
 // after the earlier stages ran for the same n_tokens (checked) on the same activations.
+// Per-group int8: the bf16 copy of the experts that batches for the MFMA-tiled kernels run on.
+// Made at `create` when max_tokens_hint announces such batches, else by the first such batch.
+int ensure_pg_copy(AteniaMoeLayer* L) {
+  if (L->pg_ready) return ATENIA_MOE_OK;
+  int rc = make_bf16_copy(L->gate, L->E, L->pg_wg, L->gate_b);
+  if (!rc) rc = make_bf16_copy(L->up, L->E, L->pg_wu, L->up_b);
+  if (!rc) rc = make_bf16_copy(L->down, L->E, L->pg_wd, L->down_b);
+  if (!rc && L->fs > 0) {
+    rc = make_bf16_copy(L->s_gate, 1, L->pg_swg, L->s_gate_b);
+    if (!rc) rc = make_bf16_copy(L->s_up, 1, L->pg_swu, L->s_up_b);
+    if (!rc) rc = make_bf16_copy(L->s_down, 1, L->pg_swd, L->s_down_b);
+  }
+  if (rc) return rc;
+  HIP_TRY(hipDeviceSynchronize());
+  L->pg_ready = true;
+  return ATENIA_MOE_OK;
+}
+
+// Which expert kernels a batch of T tokens takes (a pure function of the layer and T).
+struct BatchPlan {
+  bool routed_streams;  // weight-streaming kernels (decode) instead of the tiled ones
+  bool pg_prefill;      // per-group int8 layer running the tiled kernels on its bf16 copy
+};
+BatchPlan plan_batch(const AteniaMoeLayer* L, int T) {
+  const bool int8w = L->wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
+  BatchPlan p;
+  p.routed_streams = batch_streams(T, (long long)T * L->k, L->E, int8w ? 32 : 16);
+  p.pg_prefill = L->group_size > 0 && !p.routed_streams && L->d_kpad % 64 == 0 &&
+                 L->f_kpad % 64 == 0 && (L->fs == 0 || L->fs_kpad % 64 == 0);
+  return p;
+}
+
+bool stream_is_capturing(hipStream_t s) {
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &st) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return st != hipStreamCaptureStatusNone;
+}
+
+// `view`: the workspace to run on (nullptr = the handle's own).  no_alloc: fail instead of
+// allocating anything.
 int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d_out,
-                hipStream_t s, int first, int last, const float* d_residual = nullptr) {
+                hipStream_t s, int first, int last, const float* d_residual = nullptr,
+                const WsView* view = nullptr, bool no_alloc = false) {
   for (int st = 0; st < first; ++st)
     if (L->stage_T[st] != T)
       return fail(ATENIA_MOE_ERR_DIM, "stage %d has not run for %d tokens on this handle", st, T);
@@ -332,6 +450,24 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   const bool f32w = L->wdtype == ATENIA_MOE_WEIGHT_F32;
   if (f32w && x_dtype != ATENIA_MOE_ACT_F32)
     return fail(ATENIA_MOE_ERR_UNSUPPORTED, "f32 weights need f32 activations");
+  if (first > kStageRouter && view == nullptr && L->cur.idx != L->ws.idx)
+    return fail(ATENIA_MOE_ERR_DIM, "the earlier stages ran on another workspace");
+  const WsView V = view ? *view : L->ws;
+  L->cur = V;
+  // A forward still running on another stream uses the same workspace: wait for it.
+  const bool capturing = stream_is_capturing(s);
+  if (!capturing && L->done_valid && L->done_stream != s) HIP_TRY(hipStreamWaitEvent(s, L->done, 0));
+  struct DoneMark {  // records the end of this call's work on every way out
+    AteniaMoeLayer* L;
+    hipStream_t s;
+    bool on;
+    ~DoneMark() {
+      if (on && hipEventRecord(L->done, s) == hipSuccess) {
+        L->done_valid = true;
+        L->done_stream = s;
+      }
+    }
+  } done_mark{L, s, !capturing && L->done != nullptr};
   StageTimer tm{L, s};
   for (int i = 0; i < ATENIA_MOE_N_STAGES; ++i) L->launches[i] = 0;
   tm.mark();  // ev[0]: start
@@ -351,41 +487,37 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   const bool gated = L->fs > 0 && L->conv == ATENIA_MOE_CONVENTION_HUGGINGFACE_QWEN &&
                      L->shared_gate.p != nullptr && L->v3_n_group == 0;
   ra.shared_gate = gated ? L->shared_gate.as<float>() : nullptr;
-  ra.idx = L->idx.as<int32_t>();
-  ra.w = L->w.as<float>();
-  ra.sgate = L->sgate.as<float>();
-  ra.xb = need_xb ? L->xb.as<uint16_t>() : nullptr;
+  ra.idx = V.idx;
+  ra.w = V.w;
+  ra.sgate = V.sgate;
+  ra.xb = need_xb ? V.xb : nullptr;
   ra.d_pad = L->d_kpad;
   ra.status = L->status.as<int32_t>();
   // f32-valued operands almost never satisfy the exactness test of the per-token kernel, so
   // f32 layers always take the sequential-order kernel.
   ra.token_kernel_max_tokens = f32w ? 0 : router_token_max();
   PermuteArgs pa{};
-  pa.idx = L->idx.as<int32_t>();
+  pa.idx = V.idx;
   pa.T = T;
   pa.k = L->k;
   pa.E = L->E;
-  pa.counts = L->counts.as<int32_t>();
-  pa.offsets = L->offsets.as<int32_t>();
-  pa.perm = L->perm.as<int32_t>();
-  pa.inv = L->inv.as<int32_t>();
-  pa.active = L->active.as<int32_t>();
-  pa.n_active = L->n_active.as<int32_t>();
-  pa.blk_counts = L->blk_counts.as<int32_t>();
-  pa.shared_offsets = L->shared_desc.as<int32_t>();
-  pa.tile_group = L->tile_group.as<int32_t>();
-  pa.tile_m0 = L->tile_m0.as<int32_t>();
-  pa.n_tiles = L->shared_desc.as<int32_t>() + 4;
-  pa.shared_n_tiles = L->shared_desc.as<int32_t>() + 5;
+  pa.counts = V.counts;
+  pa.offsets = V.offsets;
+  pa.perm = V.perm;
+  pa.inv = V.inv;
+  pa.active = V.active;
+  pa.n_active = V.n_active;
+  pa.blk_counts = V.blk_counts;
+  pa.shared_offsets = V.shared_desc;
+  pa.tile_group = V.tile_group;
+  pa.tile_m0 = V.tile_m0;
+  pa.n_tiles = V.shared_desc + 4;
+  pa.shared_n_tiles = V.shared_desc + 5;
   ra.fuse_permute = last >= kStagePermute ? &pa : nullptr;
   const bool v3 = L->v3_n_group > 0;
-  if (v3 || L->E > 31) {
-    int rc = L->logits.ensure((size_t)L->cap_tokens * L->E * 4);
-    if (rc) return rc;
-    ra.logits_tmp = L->logits.as<float>();
-  }
+  if (v3 || L->E > 31) ra.logits_tmp = V.logits;
   if (v3) {
-    ra.logits_out = L->logits.as<float>();
+    ra.logits_out = V.logits;
     ra.shared_gate = nullptr;  // the V3 block adds its shared experts ungated
   }
   int fused = 0;
@@ -394,7 +526,7 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
     L->launches[0] = 1;
     if (v3) {
       V3RouteArgs va{};
-      va.logits = L->logits.as<float>();
+      va.logits = V.logits;
       va.bias = L->v3_bias.as<float>();
       va.T = T;
       va.E = L->E;
@@ -403,8 +535,8 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
       va.topk_group = L->v3_topk_group;
       va.norm_topk_prob = L->v3_norm;
       va.routed_scaling_factor = L->v3_scale;
-      va.idx = L->idx.as<int32_t>();
-      va.w = L->w.as<float>();
+      va.idx = V.idx;
+      va.w = V.w;
       va.status = L->status.as<int32_t>();
       HIP_TRY(launch_v3_route(va, s));
       L->launches[0] = 2;
@@ -424,7 +556,7 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   tm.mark();  // ev[2]: permute done
   if (last < kStageFfn) return ATENIA_MOE_OK;
 
-  const void* a_x = f32w ? d_x : (need_xb ? (const void*)L->xb.p : d_x);
+  const void* a_x = f32w ? d_x : (need_xb ? (const void*)V.xb : d_x);
   const int a_stride = f32w ? L->d : L->d_kpad;
 
   // Per-group int8 and a batch for the MFMA-tiled kernels: those take one scale per row, so the
@@ -432,33 +564,25 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   // nearest bf16 (the reference's GPU dequantiser truncates instead,
   // src/cuda/int8_to_bf16.cu:91-110; rounding halves the error against the q * scale the
   // reference's CPU path multiplies with).  Decode batches stream the int8 weights themselves.
-  const bool int8w = L->wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
-  const bool routed_streams =
-      batch_streams(T, (long long)T * L->k, L->E, int8w ? 32 : 16);
-  const bool pg_prefill = L->group_size > 0 && !routed_streams && L->d_kpad % 64 == 0 &&
-                          L->f_kpad % 64 == 0 && (L->fs == 0 || L->fs_kpad % 64 == 0);
+  const BatchPlan plan = plan_batch(L, T);
+  const bool routed_streams = plan.routed_streams, pg_prefill = plan.pg_prefill;
+  if (pg_prefill && !L->pg_ready && no_alloc)
+    return fail(ATENIA_MOE_ERR_UNSUPPORTED,
+                "per-group int8: a batch of %d tokens needs the layer's bf16 copy, which is made by "
+                "the first such batch through an allocating entry point", T);
   if (pg_prefill && !L->pg_ready) {
-    int rc = make_bf16_copy(L->gate, L->E, L->pg_wg, L->gate_b);
-    if (!rc) rc = make_bf16_copy(L->up, L->E, L->pg_wu, L->up_b);
-    if (!rc) rc = make_bf16_copy(L->down, L->E, L->pg_wd, L->down_b);
-    if (!rc && L->fs > 0) {
-      rc = make_bf16_copy(L->s_gate, 1, L->pg_swg, L->s_gate_b);
-      if (!rc) rc = make_bf16_copy(L->s_up, 1, L->pg_swu, L->s_up_b);
-      if (!rc) rc = make_bf16_copy(L->s_down, 1, L->pg_swd, L->s_down_b);
-    }
+    int rc = ensure_pg_copy(L);
     if (rc) return rc;
-    HIP_TRY(hipDeviceSynchronize());
-    L->pg_ready = true;
   }
   const int ffn_dtype = pg_prefill ? ATENIA_MOE_WEIGHT_BF16 : L->wdtype;
 
   FfnArgs fa{};
   fa.wdtype = ffn_dtype;
   fa.f32_accumulate = L->policy != ATENIA_MOE_POLICY_CERTIFIED;
-  fa.g.offsets = L->offsets.as<int32_t>();
-  fa.g.active = L->active.as<int32_t>();
-  fa.g.n_active = L->n_active.as<int32_t>();
-  fa.g.perm = L->perm.as<int32_t>();
+  fa.g.offsets = V.offsets;
+  fa.g.active = V.active;
+  fa.g.n_active = V.n_active;
+  fa.g.perm = V.perm;
   fa.g.pair_div = L->k;
   fa.n_groups_max = (int)std::min<long long>(L->E, (long long)T * L->k);
   fa.rows_max = T;
@@ -467,44 +591,44 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   fa.down = pg_prefill ? L->down_b : L->down;
   fa.x = a_x;
   fa.x_stride = a_stride;
-  fa.h = L->h.p;
+  fa.h = V.h;
   fa.h_stride = L->f_kpad;
-  fa.y = L->y.as<float>();
+  fa.y = V.y;
   fa.y_stride = L->d;
   // Tiled (MFMA-bound) kernels once an expert can see more rows than the streaming kernel
   // keeps in registers; below that the weights are streamed once (HBM-bound).
   const bool tiled = !routed_streams && tiled_supported(fa.gate, ffn_dtype) &&
                      tiled_supported(fa.down, ffn_dtype);
   fa.use_tiled = tiled;
-  fa.tile_group = L->tile_group.as<int32_t>();
-  fa.tile_m0 = L->tile_m0.as<int32_t>();
-  fa.n_tiles = L->shared_desc.as<int32_t>() + 4;
+  fa.tile_group = V.tile_group;
+  fa.tile_m0 = V.tile_m0;
+  fa.n_tiles = V.shared_desc + 4;
   fa.max_row_tiles = (int)(((size_t)T * L->k + kTileM - 1) / kTileM +
                            std::min<long long>(L->E, (long long)T * L->k));
   const bool split_tail = tiled && tiled_down_splits_tail(fa.down, ffn_dtype);
-  fa.y_parts = split_tail ? kMaxYParts : 1;
+  fa.y_parts = split_tail ? std::min(kMaxYParts, V.y_parts) : 1;
   fa.y_part_stride = (size_t)T * L->k * L->d;
-  fa.part_flags = split_tail ? L->part_flags.as<uint8_t>() : nullptr;
+  fa.part_flags = split_tail ? V.part_flags : nullptr;
   fa.n_cus = device_cu_count();
   L->last_split = split_tail;
 
   FfnArgs fsd{};
   if (L->fs > 0) {
     fsd = fa;
-    const int32_t* sd = L->shared_desc.as<int32_t>();
+    const int32_t* sd = V.shared_desc;
     fsd.g.offsets = sd;
     fsd.g.active = sd + 2;
     fsd.g.n_active = sd + 3;
-    fsd.g.perm = L->ident.as<int32_t>();
+    fsd.g.perm = V.ident;
     fsd.g.pair_div = 1;
     fsd.n_groups_max = 1;
     fsd.rows_max = T;
     fsd.gate = pg_prefill ? L->s_gate_b : L->s_gate;
     fsd.up = pg_prefill ? L->s_up_b : L->s_up;
     fsd.down = pg_prefill ? L->s_down_b : L->s_down;
-    fsd.h = L->hs.p;
+    fsd.h = V.hs;
     fsd.h_stride = L->fs_kpad;
-    fsd.y = L->ys.as<float>();
+    fsd.y = V.ys;
     fsd.y_parts = 1;
     fsd.part_flags = nullptr;
     // The shared expert follows the routed ones (it then rides in their launches): it is small
@@ -512,9 +636,9 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
     // launches of its own that the tiled form would need.
     fsd.use_tiled = !routed_streams && tiled_supported(fsd.gate, ffn_dtype) &&
                     tiled_supported(fsd.down, ffn_dtype);
-    fsd.tile_group = L->s_tile_group.as<int32_t>();
-    fsd.tile_m0 = L->s_tile_m0.as<int32_t>();
-    fsd.n_tiles = L->shared_desc.as<int32_t>() + 5;
+    fsd.tile_group = V.s_tile_group;
+    fsd.tile_m0 = V.s_tile_m0;
+    fsd.n_tiles = V.shared_desc + 5;
     fsd.max_row_tiles = (T + kTileM - 1) / kTileM;
   }
 
@@ -537,7 +661,7 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
                      ffn_down_decode1_supported(T, L->k, L->wdtype, tiled, L->fs > 0);
   if (first <= kStageFfn) {
     if (fuse1) {
-      fa.fuse_w = L->w.as<float>();
+      fa.fuse_w = V.w;
       fa.fuse_out = d_out;
       fa.fuse_residual = d_residual;
       fa.fuse_k = L->k;
@@ -566,14 +690,14 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   ca.T = T;
   ca.k = L->k;
   ca.d = L->d;
-  ca.w = L->w.as<float>();
-  ca.y = L->y.as<float>();
+  ca.w = V.w;
+  ca.y = V.y;
   ca.y_stride = L->d;
   ca.part_flags = fa.part_flags;
   ca.flag_cols = (L->d + 255) / 256;
   ca.y_part_stride = fa.y_part_stride;
-  ca.y_shared = L->fs > 0 ? L->ys.as<float>() : nullptr;
-  ca.sgate = gated ? L->sgate.as<float>() : nullptr;
+  ca.y_shared = L->fs > 0 ? V.ys : nullptr;
+  ca.sgate = gated ? V.sgate : nullptr;
   ca.residual = d_residual;
   ca.out = d_out;
   HIP_TRY(launch_combine(ca, s));
@@ -740,7 +864,20 @@ int atenia_moe_hip_layer_create(const AteniaMoeLayerDesc* D, AteniaMoeLayer** ou
     L->bytes_per_expert = (int64_t)(3 * d * f * eb) +
                           ((int64_t)2 * f * ((d + L->group_size - 1) / L->group_size) +
                            (int64_t)d * ((f + L->group_size - 1) / L->group_size)) * 4;
-  if (D->max_tokens_hint > 0 && (rc = ensure_workspace(L, D->max_tokens_hint))) return bail(rc);
+  if ((rc = L->status.ensure(8))) return bail(rc);
+  {
+    const int32_t st[2] = {0, INT_MAX};
+    if (hipMemcpy(L->status.p, st, 8, hipMemcpyHostToDevice) != hipSuccess)
+      return bail(fail(ATENIA_MOE_ERR_LAUNCH, "status upload failed"));
+  }
+  if (hipEventCreateWithFlags(&L->done, hipEventDisableTiming) != hipSuccess)
+    return bail(fail(ATENIA_MOE_ERR_LAUNCH, "hipEventCreate failed"));
+  if (hipGetDevice(&L->device) != hipSuccess)
+    return bail(fail(ATENIA_MOE_ERR_LAUNCH, "hipGetDevice failed"));
+  if (D->max_tokens_hint > 0) {
+    if ((rc = ensure_workspace(L, D->max_tokens_hint))) return bail(rc);
+    if (plan_batch(L, D->max_tokens_hint).pg_prefill && (rc = ensure_pg_copy(L))) return bail(rc);
+  }
   if (hipDeviceSynchronize() != hipSuccess)
     return bail(fail(ATENIA_MOE_ERR_SYNC, "device synchronisation failed after upload"));
   *out_layer = L;
@@ -754,6 +891,7 @@ int atenia_moe_hip_layer_destroy(AteniaMoeLayer* L) {
     (void)hipDeviceSynchronize();
     if (L->ev_valid)
       for (auto& e : L->ev) (void)hipEventDestroy(e);
+    if (L->done) (void)hipEventDestroy(L->done);
     if (L->stream) (void)hipStreamDestroy(L->stream);
     L->magic = 0;
   }
@@ -802,7 +940,7 @@ int run_block(AteniaMoeLayer* L, const float* d_x1, int T, const float* d_gamma,
               int norm_policy, float* d_out, hipStream_t s) {
   int rc = ensure_workspace(L, T);
   if (rc) return rc;
-  if ((rc = L->xn.ensure((size_t)L->cap_tokens * L->d * 4))) return rc;
+  if ((rc = L->xn.ensure((size_t)L->ws.cap_tokens * L->d * 4))) return rc;
   NormArgs na{};
   na.x = d_x1;
   na.gamma = d_gamma;
@@ -894,8 +1032,9 @@ int atenia_moe_router_launch_device(AteniaMoeLayer* L, const void* d_x, int x_dt
   rc = run_forward(L, d_x, x_dtype, n_tokens, nullptr, s, kStageRouter, kStageRouter);
   if (rc) return rc;
   const size_t n = (size_t)n_tokens * L->k;
-  if (d_idx) HIP_TRY(hipMemcpyAsync(d_idx, L->idx.p, n * 4, hipMemcpyDeviceToDevice, s));
-  if (d_w) HIP_TRY(hipMemcpyAsync(d_w, L->w.p, n * 4, hipMemcpyDeviceToDevice, s));
+  const WsView& V = L->cur;
+  if (d_idx) HIP_TRY(hipMemcpyAsync(d_idx, V.idx, n * 4, hipMemcpyDeviceToDevice, s));
+  if (d_w) HIP_TRY(hipMemcpyAsync(d_w, V.w, n * 4, hipMemcpyDeviceToDevice, s));
   return ATENIA_MOE_OK;
 }
 
@@ -908,13 +1047,14 @@ int atenia_moe_permute_launch_device(AteniaMoeLayer* L, int n_tokens, int32_t* d
   rc = run_forward(L, nullptr, L->wdtype == ATENIA_MOE_WEIGHT_F32 ? ATENIA_MOE_ACT_F32 : ATENIA_MOE_ACT_BF16,
                    n_tokens, nullptr, s, kStagePermute, kStagePermute);
   if (rc) return rc;
+  const WsView& V = L->cur;
   if (d_counts)
-    HIP_TRY(hipMemcpyAsync(d_counts, L->counts.p, (size_t)L->E * 4, hipMemcpyDeviceToDevice, s));
+    HIP_TRY(hipMemcpyAsync(d_counts, V.counts, (size_t)L->E * 4, hipMemcpyDeviceToDevice, s));
   if (d_offsets)
-    HIP_TRY(hipMemcpyAsync(d_offsets, L->offsets.p, ((size_t)L->E + 1) * 4,
+    HIP_TRY(hipMemcpyAsync(d_offsets, V.offsets, ((size_t)L->E + 1) * 4,
                            hipMemcpyDeviceToDevice, s));
   if (d_perm)
-    HIP_TRY(hipMemcpyAsync(d_perm, L->perm.p, (size_t)n_tokens * L->k * 4,
+    HIP_TRY(hipMemcpyAsync(d_perm, V.perm, (size_t)n_tokens * L->k * 4,
                            hipMemcpyDeviceToDevice, s));
   return ATENIA_MOE_OK;
 }
@@ -1013,8 +1153,9 @@ int atenia_moe_hip_layer_route(AteniaMoeLayer* L, const float* x_host, int n_tok
   rc = read_status(L, L->stream, nullptr, nullptr);
   if (rc) return rc;
   const size_t P = (size_t)n_tokens * L->k;
-  HIP_TRY(hipMemcpy(idx_host, L->idx.p, P * 4, hipMemcpyDeviceToHost));
-  HIP_TRY(hipMemcpy(w_host, L->w.p, P * 4, hipMemcpyDeviceToHost));
+  const WsView& V = L->cur;
+  HIP_TRY(hipMemcpy(idx_host, V.idx, P * 4, hipMemcpyDeviceToHost));
+  HIP_TRY(hipMemcpy(w_host, V.w, P * 4, hipMemcpyDeviceToHost));
   return ATENIA_MOE_OK;
 }
 
@@ -1037,19 +1178,25 @@ int atenia_moe_hip_layer_permute(AteniaMoeLayer* L, const int32_t* idx_host, int
   std::lock_guard<std::mutex> lock(L->mu);
   int rc = ensure_workspace(L, n_tokens);
   if (rc) return rc;
-  HIP_TRY(hipMemcpyAsync(L->idx.p, idx_host, P * 4, hipMemcpyHostToDevice, L->stream));
+  const WsView& V = L->ws;
+  L->cur = V;
+  // the routing, the grouping and the row tiles no longer describe one forward
+  for (int st = 0; st < 4; ++st) L->stage_T[st] = -1;
+  L->last_T = 0;
+  if (L->done_valid && L->done_stream != L->stream) HIP_TRY(hipStreamWaitEvent(L->stream, L->done, 0));
+  HIP_TRY(hipMemcpyAsync(V.idx, idx_host, P * 4, hipMemcpyHostToDevice, L->stream));
   PermuteArgs pa{};
-  pa.idx = L->idx.as<int32_t>();
+  pa.idx = V.idx;
   pa.T = n_tokens;
   pa.k = L->k;
   pa.E = L->E;
-  pa.counts = L->counts.as<int32_t>();
-  pa.offsets = L->offsets.as<int32_t>();
-  pa.perm = L->perm.as<int32_t>();
-  pa.inv = L->inv.as<int32_t>();
-  pa.active = L->active.as<int32_t>();
-  pa.n_active = L->n_active.as<int32_t>();
-  pa.blk_counts = L->blk_counts.as<int32_t>();
+  pa.counts = V.counts;
+  pa.offsets = V.offsets;
+  pa.perm = V.perm;
+  pa.inv = V.inv;
+  pa.active = V.active;
+  pa.n_active = V.n_active;
+  pa.blk_counts = V.blk_counts;
   pa.shared_offsets = nullptr;
   pa.tile_group = nullptr;
   pa.tile_m0 = nullptr;
@@ -1058,10 +1205,9 @@ int atenia_moe_hip_layer_permute(AteniaMoeLayer* L, const int32_t* idx_host, int
   HIP_TRY(launch_permute(pa, L->stream, nullptr));
   if (hipStreamSynchronize(L->stream) != hipSuccess)
     return fail(ATENIA_MOE_ERR_SYNC, "stream synchronisation failed");
-  HIP_TRY(hipMemcpy(counts_host, L->counts.p, (size_t)L->E * 4, hipMemcpyDeviceToHost));
-  HIP_TRY(hipMemcpy(offsets_host, L->offsets.p, (size_t)(L->E + 1) * 4, hipMemcpyDeviceToHost));
-  HIP_TRY(hipMemcpy(perm_host, L->perm.p, P * 4, hipMemcpyDeviceToHost));
-  L->last_T = 0;  // the workspace no longer describes a forward
+  HIP_TRY(hipMemcpy(counts_host, V.counts, (size_t)L->E * 4, hipMemcpyDeviceToHost));
+  HIP_TRY(hipMemcpy(offsets_host, V.offsets, (size_t)(L->E + 1) * 4, hipMemcpyDeviceToHost));
+  HIP_TRY(hipMemcpy(perm_host, V.perm, P * 4, hipMemcpyDeviceToHost));
   return ATENIA_MOE_OK;
 }
 
@@ -1074,13 +1220,14 @@ int atenia_moe_hip_layer_last_routing(AteniaMoeLayer* L, int32_t* idx_host, floa
   if (hipDeviceSynchronize() != hipSuccess)
     return fail(ATENIA_MOE_ERR_SYNC, "device synchronisation failed");
   const size_t P = (size_t)L->last_T * L->k;
-  if (idx_host) HIP_TRY(hipMemcpy(idx_host, L->idx.p, P * 4, hipMemcpyDeviceToHost));
-  if (w_host) HIP_TRY(hipMemcpy(w_host, L->w.p, P * 4, hipMemcpyDeviceToHost));
+  const WsView& V = L->cur;
+  if (idx_host) HIP_TRY(hipMemcpy(idx_host, V.idx, P * 4, hipMemcpyDeviceToHost));
+  if (w_host) HIP_TRY(hipMemcpy(w_host, V.w, P * 4, hipMemcpyDeviceToHost));
   if (counts_host)
-    HIP_TRY(hipMemcpy(counts_host, L->counts.p, (size_t)L->E * 4, hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy(counts_host, V.counts, (size_t)L->E * 4, hipMemcpyDeviceToHost));
   if (offsets_host)
-    HIP_TRY(hipMemcpy(offsets_host, L->offsets.p, (size_t)(L->E + 1) * 4, hipMemcpyDeviceToHost));
-  if (perm_host) HIP_TRY(hipMemcpy(perm_host, L->perm.p, P * 4, hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy(offsets_host, V.offsets, (size_t)(L->E + 1) * 4, hipMemcpyDeviceToHost));
+  if (perm_host) HIP_TRY(hipMemcpy(perm_host, V.perm, P * 4, hipMemcpyDeviceToHost));
   return ATENIA_MOE_OK;
 }
 
@@ -1092,18 +1239,19 @@ int atenia_moe_hip_layer_last_expert_outputs(AteniaMoeLayer* L, float* y_host,
   if (hipDeviceSynchronize() != hipSuccess)
     return fail(ATENIA_MOE_ERR_SYNC, "device synchronisation failed");
   const size_t P = (size_t)L->last_T * L->k;
+  const WsView& V = L->cur;
   if (y_host) {
-    HIP_TRY(hipMemcpy(y_host, L->y.p, P * L->d * 4, hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy(y_host, V.y, P * L->d * 4, hipMemcpyDeviceToHost));
     if (L->last_split) {  // add the partial buffers the down phase wrote for split tail tiles
       const int fc = (L->d + 255) / 256;
       std::vector<uint8_t> flags(P * fc);
-      HIP_TRY(hipMemcpy(flags.data(), L->part_flags.p, flags.size(), hipMemcpyDeviceToHost));
+      HIP_TRY(hipMemcpy(flags.data(), V.part_flags, flags.size(), hipMemcpyDeviceToHost));
       std::vector<float> part(P * L->d);
       for (int i = 1; i < kMaxYParts; ++i) {
         bool any = false;
         for (uint8_t f : flags) any = any || f > i;
         if (!any) break;
-        HIP_TRY(hipMemcpy(part.data(), (const float*)L->y.p + (size_t)i * P * L->d, P * L->d * 4,
+        HIP_TRY(hipMemcpy(part.data(), (const float*)V.y + (size_t)i * P * L->d, P * L->d * 4,
                           hipMemcpyDeviceToHost));
         for (size_t pr = 0; pr < P; ++pr)
           for (int c = 0; c < L->d; ++c)
@@ -1112,7 +1260,7 @@ int atenia_moe_hip_layer_last_expert_outputs(AteniaMoeLayer* L, float* y_host,
     }
   }
   if (y_shared_host && L->fs > 0)
-    HIP_TRY(hipMemcpy(y_shared_host, L->ys.p, (size_t)L->last_T * L->d * 4,
+    HIP_TRY(hipMemcpy(y_shared_host, V.ys, (size_t)L->last_T * L->d * 4,
                       hipMemcpyDeviceToHost));
   return ATENIA_MOE_OK;
 }

@@ -30,8 +30,13 @@
  *
  * Threading: any thread may call; one handle is NOT re-entrant (it owns one workspace) and
  * calls on the same handle are serialised by an internal mutex, as the reference serialises
- * forwards behind its registry mutex (src/moe/graph_op.rs:304-316).  Different handles may
- * run concurrently.
+ * forwards behind its registry mutex (src/moe/graph_op.rs:304-316).  The asynchronous entry
+ * points keep that promise on the device as well: a call whose stream differs from the stream
+ * of the handle's previous call first waits (hipStreamWaitEvent) for that call's kernels, so
+ * two streams never use one workspace at the same time.  The one exception is a stream that is
+ * being captured into a HIP graph: no cross-stream wait is recorded there, and replays of graphs
+ * that hold calls on one handle must be ordered by the caller.  Different handles may run
+ * concurrently.
  */
 #ifndef ATENIA_MOE_HIP_H
 #define ATENIA_MOE_HIP_H

@@ -116,3 +116,30 @@ def test_one_handle_shared_by_threads_is_serialised(ora):
         for i in range(len(sizes)):
             for r in range(rounds):
                 assert got[i][r].tobytes() == want[i].tobytes(), f"{sizes[i]} tokens, round {r}"
+
+
+def test_one_handle_on_two_streams_is_ordered_on_the_device(ora):
+    """The asynchronous entry point on ONE handle from two streams, calls issued back to back
+    without any host synchronisation in between: the second stream must wait for the first
+    stream's kernels (they share the handle's workspace), so every output equals the result of the
+    same call made alone."""
+    wd, E, k, d, f, fs, _ = SHAPES[2]
+    W = S.make_weights(778, E, d, f, f_s=fs, gated=True, router_std=1.0 / np.sqrt(d))
+    _, gL = S.build_pair(ora, W, k, capi.CONVENTION_HUGGINGFACE_QWEN, wd, max_tokens_hint=700)
+    sizes = [700, 3, 260, 1, 64, 700]  # long and short calls alternate between the streams
+    xs = [S.make_tokens(60 + i, n, d) for i, n in enumerate(sizes)]
+    with gL:
+        want = [gL.forward(x).copy() for x in xs]
+        streams = [Stream(), Stream()]
+        dx = [DeviceArray.from_host(x) for x in xs]
+        for rep in range(3):
+            outs = [DeviceArray(x.shape, np.float32, fill=0) for x in xs]
+            for i, n in enumerate(sizes):
+                gL.forward_device(dx[i].ptr, capi.ACT_F32, n, outs[i].ptr, streams[i % 2].ptr)
+            for s in streams:
+                s.synchronize()
+            for i in range(len(sizes)):
+                assert outs[i].to_host().tobytes() == want[i].tobytes(), \
+                    f"repeat {rep}, call {i} ({sizes[i]} tokens)"
+        for s in streams:
+            s.close()
