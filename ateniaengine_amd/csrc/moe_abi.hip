@@ -127,9 +127,9 @@ struct AteniaMoeLayer {
 
   hipStream_t stream = nullptr;
   std::mutex mu;
-  // Ordering of asynchronous forwards on one handle: every forward records `done` at its end and
-  // a forward on another stream waits for it first, so two streams never use the workspace at
-  // the same time (skipped while a stream is being captured into a graph).
+  // Ordering of asynchronous forwards on one handle: a forward on another stream than the
+  // previous one (`done_stream`) first waits for that stream's work, so two streams never use
+  // the workspace at the same time (skipped while a stream is being captured into a graph).
   hipEvent_t done = nullptr;
   hipStream_t done_stream = nullptr;
   bool done_valid = false;
@@ -454,20 +454,24 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
     return fail(ATENIA_MOE_ERR_DIM, "the earlier stages ran on another workspace");
   const WsView V = view ? *view : L->ws;
   L->cur = V;
-  // A forward still running on another stream uses the same workspace: wait for it.
+  // A forward still running on another stream uses the same workspace: wait for it.  Nothing
+  // is recorded while calls stay on one stream (an event per forward would cost a decode step
+  // several microseconds); when the stream changes, the previous stream is marked now -- the
+  // mark covers everything submitted to it so far -- and the new one waits for the mark.  A
+  // previous stream that no longer exists cannot be marked; the device is drained instead.
   const bool capturing = stream_is_capturing(s);
-  if (!capturing && L->done_valid && L->done_stream != s) HIP_TRY(hipStreamWaitEvent(s, L->done, 0));
-  struct DoneMark {  // records the end of this call's work on every way out
-    AteniaMoeLayer* L;
-    hipStream_t s;
-    bool on;
-    ~DoneMark() {
-      if (on && hipEventRecord(L->done, s) == hipSuccess) {
-        L->done_valid = true;
-        L->done_stream = s;
+  if (!capturing) {
+    if (L->done_valid && L->done_stream != s) {
+      if (hipEventRecord(L->done, L->done_stream) == hipSuccess) {
+        HIP_TRY(hipStreamWaitEvent(s, L->done, 0));
+      } else {
+        (void)hipGetLastError();
+        HIP_TRY(hipDeviceSynchronize());
       }
     }
-  } done_mark{L, s, !capturing && L->done != nullptr};
+    L->done_valid = true;
+    L->done_stream = s;
+  }
   StageTimer tm{L, s};
   for (int i = 0; i < ATENIA_MOE_N_STAGES; ++i) L->launches[i] = 0;
   tm.mark();  // ev[0]: start
@@ -1183,7 +1187,7 @@ int atenia_moe_hip_layer_permute(AteniaMoeLayer* L, const int32_t* idx_host, int
   // the routing, the grouping and the row tiles no longer describe one forward
   for (int st = 0; st < 4; ++st) L->stage_T[st] = -1;
   L->last_T = 0;
-  if (L->done_valid && L->done_stream != L->stream) HIP_TRY(hipStreamWaitEvent(L->stream, L->done, 0));
+  HIP_TRY(hipDeviceSynchronize());  // a forward may still be using the workspace on some stream
   HIP_TRY(hipMemcpyAsync(V.idx, idx_host, P * 4, hipMemcpyHostToDevice, L->stream));
   PermuteArgs pa{};
   pa.idx = V.idx;
