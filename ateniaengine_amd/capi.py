@@ -46,6 +46,7 @@ EXPORTS = (
     "atenia_moe_int8_to_bf16_per_channel_launch_device",
     "atenia_moe_int8_to_bf16_per_group_launch_device",
     "atenia_moe_hip_layer_set_numeric_policy",
+    "atenia_moe_hip_layer_forward_device_noalloc",
 )
 # the reference's own names for the two dequantisation launchers (src/cuda/int8_to_bf16.rs:63-81)
 REFERENCE_NAMED_EXPORTS = ("int8_to_bf16_per_channel_launch_device",
@@ -97,6 +98,7 @@ def lib():
         L.atenia_moe_hip_layer_destroy.argtypes = [P]
         L.atenia_moe_hip_layer_forward.argtypes = [P, P, C.c_int, P]
         L.atenia_moe_hip_layer_forward_device.argtypes = [P, P, C.c_int, C.c_int, P, P]
+        L.atenia_moe_hip_layer_forward_device_noalloc.argtypes = [P, P, C.c_int, C.c_int, P, P]
         L.atenia_moe_hip_layer_status.argtypes = [P, P, P, P]
         L.atenia_moe_hip_layer_route.argtypes = [P, P, C.c_int, P, P]
         L.atenia_moe_hip_layer_permute.argtypes = [P, P, C.c_int, P, P, P]
@@ -287,6 +289,12 @@ class Layer:
         """Raw device pointers (ints); asynchronous on `stream`."""
         _check(lib().atenia_moe_hip_layer_forward_device(self._h, d_x, x_dtype, n_tokens, d_out,
                                                          stream))
+
+    def forward_device_noalloc(self, d_x: int, x_dtype: int, n_tokens: int, d_out: int,
+                               stream: int = 0):
+        """forward_device on the library's static workspace: the call allocates nothing."""
+        _check(lib().atenia_moe_hip_layer_forward_device_noalloc(self._h, d_x, x_dtype, n_tokens,
+                                                                 d_out, stream))
 
     def set_v3_router(self, n_group: int, topk_group: int, routed_scaling_factor: float,
                       norm_topk_prob: bool, e_score_correction_bias):

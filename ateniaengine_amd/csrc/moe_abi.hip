@@ -21,6 +21,15 @@
 
 using namespace atenia_moe;
 
+// Workspace of atenia_moe_hip_layer_forward_device_noalloc: device memory the library owns from
+// load time on, for callers that must not allocate.  Every GPU the library runs on holds its own
+// copy of the array at its own address for the life of the process.  In host code the NAME of the
+// array is only a stand-in for hipGetSymbolAddress -- it is not a device address and is never
+// passed to a kernel or a runtime call; resolve_static_scratch() below keeps the real address
+// per device.
+constexpr size_t kStaticScratchBytes = (size_t)16 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace {
 
 thread_local std::string g_last_error;
@@ -46,6 +55,31 @@ int hip_rc(hipError_t e, const char* what) {
     int rc__ = hip_rc((expr), #expr);               \
     if (rc__ != ATENIA_MOE_OK) return rc__;         \
   } while (0)
+
+// Device address of `scratch` on GPU `device`, looked up once per device with that device
+// current (each GPU has its own copy of the array).  *out may be nullptr to only warm the table.
+constexpr int kMaxDevices = 64;
+int resolve_static_scratch(int device, unsigned char** out) {
+  static std::mutex mu;
+  static unsigned char* table[kMaxDevices] = {};
+  if (device < 0 || device >= kMaxDevices)
+    return fail(ATENIA_MOE_ERR_UNSUPPORTED, "device ordinal %d out of range", device);
+  std::lock_guard<std::mutex> lock(mu);
+  if (!table[device]) {
+    int cur = -1;
+    HIP_TRY(hipGetDevice(&cur));
+    if (cur != device) HIP_TRY(hipSetDevice(device));
+    void* ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (cur != device) (void)hipSetDevice(cur);
+    if (e != hipSuccess || !ptr)
+      return fail(ATENIA_MOE_ERR_LAUNCH, "hipGetSymbolAddress(scratch) on device %d: %s", device,
+                  hipGetErrorString(e));
+    table[device] = (unsigned char*)ptr;
+  }
+  if (out) *out = table[device];
+  return ATENIA_MOE_OK;
+}
 
 struct DevBuf {
   void* p = nullptr;
@@ -427,6 +461,12 @@ BatchPlan plan_batch(const AteniaMoeLayer* L, int T) {
   p.pg_prefill = L->group_size > 0 && !p.routed_streams && L->d_kpad % 64 == 0 &&
                  L->f_kpad % 64 == 0 && (L->fs == 0 || L->fs_kpad % 64 == 0);
   return p;
+}
+
+// Partial output buffers the no-alloc workspace of a T-token batch needs (the tiled down phase
+// may split tail tiles over k; the streaming kernels write one buffer).
+int noalloc_y_parts(const AteniaMoeLayer* L, int T) {
+  return plan_batch(L, T).routed_streams || L->wdtype == ATENIA_MOE_WEIGHT_F32 ? 1 : kMaxYParts;
 }
 
 bool stream_is_capturing(hipStream_t s) {
@@ -878,6 +918,7 @@ int atenia_moe_hip_layer_create(const AteniaMoeLayerDesc* D, AteniaMoeLayer** ou
     return bail(fail(ATENIA_MOE_ERR_LAUNCH, "hipEventCreate failed"));
   if (hipGetDevice(&L->device) != hipSuccess)
     return bail(fail(ATENIA_MOE_ERR_LAUNCH, "hipGetDevice failed"));
+  if ((rc = resolve_static_scratch(L->device, nullptr))) return bail(rc);
   if (D->max_tokens_hint > 0) {
     if ((rc = ensure_workspace(L, D->max_tokens_hint))) return bail(rc);
     if (plan_batch(L, D->max_tokens_hint).pg_prefill && (rc = ensure_pg_copy(L))) return bail(rc);
@@ -918,6 +959,38 @@ int atenia_moe_hip_layer_forward_device(AteniaMoeLayer* L, const void* d_x, int 
   if (rc) return rc;
   return run_forward(L, d_x, x_dtype, n_tokens, d_out, (hipStream_t)stream, kStageRouter,
                      kStageCombine);
+}
+
+int atenia_moe_hip_layer_forward_device_noalloc(AteniaMoeLayer* L, const void* d_x, int x_dtype,
+                                                int n_tokens, float* d_out, void* stream) {
+  if (!valid_handle(L)) return fail(ATENIA_MOE_ERR_HANDLE, "invalid layer handle");
+  if (n_tokens < 0) return fail(ATENIA_MOE_ERR_DIM, "negative token count");
+  if (n_tokens == 0) return ATENIA_MOE_OK;
+  if (!d_x || !d_out) return fail(ATENIA_MOE_ERR_DIM, "null activation pointer");
+  if (x_dtype != ATENIA_MOE_ACT_F32 && x_dtype != ATENIA_MOE_ACT_BF16)
+    return fail(ATENIA_MOE_ERR_DIM, "unknown activation dtype %d", x_dtype);
+  if ((long long)n_tokens * L->k > (long long)INT_MAX / 4)
+    return fail(ATENIA_MOE_ERR_DIM, "too many tokens");
+  std::lock_guard<std::mutex> lock(L->mu);
+  const int y_parts = noalloc_y_parts(L, n_tokens);
+  const size_t need = ws_layout(L, n_tokens, y_parts, nullptr, nullptr);
+  if (need > kStaticScratchBytes)
+    return fail(ATENIA_MOE_ERR_UNSUPPORTED,
+                "a batch of %d tokens needs %zu bytes of workspace; the static buffer of the "
+                "no-alloc entry point holds %zu", n_tokens, need, kStaticScratchBytes);
+  int dev = -1;
+  HIP_TRY(hipGetDevice(&dev));
+  unsigned char* base = nullptr;  // the array's address on this GPU, never the array's name
+  int rc = resolve_static_scratch(dev, &base);
+  if (rc) return rc;
+  WsView v{};
+  ws_layout(L, n_tokens, y_parts, base, &v);
+  hipStream_t s = (hipStream_t)stream;
+  // The buffer keeps the last call's contents (possibly another layer's, laid out otherwise):
+  // what must start from a known state is rewritten by a kernel on the call's own stream.
+  HIP_TRY(launch_workspace_init(L, v, n_tokens, s));
+  return run_forward(L, d_x, x_dtype, n_tokens, d_out, s, kStageRouter, kStageCombine, nullptr, &v,
+                     true);
 }
 
 int atenia_moe_hip_layer_forward(AteniaMoeLayer* L, const float* x_host, int n_tokens,

@@ -162,6 +162,25 @@ int atenia_moe_hip_layer_forward(AteniaMoeLayer* layer, const float* x_host, int
 int atenia_moe_hip_layer_forward_device(AteniaMoeLayer* layer, const void* d_x, int x_dtype,
                                         int n_tokens, float* d_out, void* stream);
 
+/* atenia_moe_hip_layer_forward_device for callers that cannot allocate: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the
+ * reference.  Same op, same arguments and the same kernels, but the workspace (routing, grouping,
+ * the h rows, the per-pair expert outputs) is a 16 MiB buffer that lives in the library's own
+ * device image from load time on, one per GPU, instead of the handle's grow-on-demand
+ * allocation: the call makes no hipMalloc / hipFree and no allocating library call, whatever
+ * n_tokens was seen before.  A batch whose workspace does not fit (about T * top_k * (2 * d_ff +
+ * 4 * d_model) bytes for the streaming kernels that serve decode batches; the Mixtral shape fits
+ * up to 85 tokens, i.e. every batch those kernels take) is refused with ATENIA_MOE_ERR_UNSUPPORTED and a message that names both sizes; so
+ * is a per-group int8 batch large enough to need the layer's bf16 copy before an allocating
+ * call has made it.  All handles on one GPU share that GPU's buffer, which keeps the previous
+ * call's contents: the call rewrites what must start from a known state with a small kernel on
+ * `stream` (no memset nodes), and calls that overlap in time on one GPU -- different handles
+ * included -- race on it; order them on one stream or with events.  The status word of
+ * ..._layer_status and the taps (..._last_routing, ..._last_expert_outputs) work as after
+ * atenia_moe_hip_layer_forward_device until the next no-alloc call on the GPU. */
+int atenia_moe_hip_layer_forward_device_noalloc(AteniaMoeLayer* layer, const void* d_x, int x_dtype,
+                                                int n_tokens, float* d_out, void* stream);
+
 /* Switches the handle's router to DeepSeek-V3 routing (src/moe/v3_router.rs:36-52, 206-309):
  * scores = sigmoid(W_r x) instead of a softmax, selection on scores + e_score_correction_bias
  * ([E] f32, host) limited to the `topk_group` best of `n_group` expert groups (group score = its
