@@ -942,14 +942,85 @@ Result<std::vector<float>, MoeLayerError> RealMoeLayer::route(const std::vector<
   return R::Ok(std::move(w));
 }
 
+// ---- ResidentExpertLayer ----------------------------------------------------------------------
+ResidentExpertLayer ResidentExpertLayer::from_real_layer(const RealMoeLayer& layer, ExpertTier tier) {
+  ResidentExpertLayer r;
+  r.config = layer.config;
+  r.convention = layer.resolve_convention();
+  r.tier = tier;
+  r.layer_ = std::make_shared<RealMoeLayer>(layer);
+  return r;
+}
+
+namespace {
+size_t stored_bytes(MoeWeightStorage st, size_t d, size_t f) {
+  switch (st) {
+    case MoeWeightStorage::F32: return 3 * d * f * 4;
+    case MoeWeightStorage::Bf16: return 3 * d * f * 2;
+    case MoeWeightStorage::Int8W8A16: return 3 * d * f + (2 * f + d) * 4;
+    case MoeWeightStorage::Int8PerGroup:
+      return 3 * d * f + (2 * f * ((d + 127) / 128) + d * ((f + 127) / 128)) * 4;
+  }
+  return 0;
+}
+}  // namespace
+
+size_t ResidentExpertLayer::expert_bytes() const {
+  return stored_bytes(layer_->storage, config.d_model, config.d_ff);
+}
+size_t ResidentExpertLayer::shared_bytes() const {
+  if (!layer_->shared) return 0;
+  return stored_bytes(layer_->storage, config.d_model, layer_->shared->d_ff);
+}
+
+Result<std::vector<float>, MoeLayerError> ResidentExpertLayer::forward_batch(
+    const std::vector<float>& x, std::vector<ResidencyInfo>* infos) const {
+  using R = Result<std::vector<float>, MoeLayerError>;
+  auto out = layer_->forward_with(x, convention);
+  if (!out.is_ok() || !infos) return out;
+  std::vector<int32_t> idx;
+  auto w = layer_->route(x, convention, &idx);
+  if (!w.is_ok()) return R::Err(w.error());
+  const size_t k = config.experts_per_token, n = k ? idx.size() / k : 0;
+  infos->assign(n, ResidencyInfo{});
+  for (size_t t = 0; t < n; ++t) {
+    for (size_t s = 0; s < k; ++s) (*infos)[t].materialized_experts.push_back((size_t)idx[t * k + s]);
+    (*infos)[t].materialized_bytes = k * expert_bytes() + shared_bytes();
+  }
+  return out;
+}
+
+Result<std::pair<std::vector<float>, ResidencyInfo>, MoeLayerError> ResidentExpertLayer::forward(
+    const std::vector<float>& x) const {
+  using R = Result<std::pair<std::vector<float>, ResidencyInfo>, MoeLayerError>;
+  if (x.size() != config.d_model) {  // the reference's forward takes one row
+    MoeLayerError e{MoeLayerError::Binding};
+    e.binding.kind = MoeBindingError::Dense;
+    e.binding.dense.kind = MoeDenseError::DimMismatch;
+    e.binding.dense.what = "x";
+    e.binding.dense.expected = config.d_model;
+    e.binding.dense.actual = x.size();
+    return R::Err(e);
+  }
+  std::vector<ResidencyInfo> infos;
+  auto out = forward_batch(x, &infos);
+  if (!out.is_ok()) return R::Err(out.error());
+  return R::Ok({out.value(), infos.empty() ? ResidencyInfo{} : infos[0]});
+}
+
 // ---- registry -------------------------------------------------------------------------------
 namespace {
+// RegisteredMoe (src/moe/graph_op.rs:207-216): a RAM layer or a resident one, one id space.
+struct RegisteredMoe {
+  std::shared_ptr<RealMoeLayer> real;
+  std::shared_ptr<ResidentExpertLayer> resident;
+};
 std::mutex& registry_mutex() {
   static std::mutex m;
   return m;
 }
-std::vector<std::shared_ptr<RealMoeLayer>>& registry() {
-  static std::vector<std::shared_ptr<RealMoeLayer>> r;
+std::vector<RegisteredMoe>& registry() {
+  static std::vector<RegisteredMoe> r;
   return r;
 }
 MoeLayerError layer_not_found(uint32_t id) {
@@ -958,25 +1029,41 @@ MoeLayerError layer_not_found(uint32_t id) {
   e.binding.layer_id = id;
   return e;
 }
+bool lookup(uint32_t layer_id, RegisteredMoe* out) {
+  std::lock_guard<std::mutex> lock(registry_mutex());
+  if (layer_id >= registry().size()) return false;
+  *out = registry()[layer_id];
+  return true;
+}
 }  // namespace
 
 uint32_t register_real_moe_layer(RealMoeLayer layer) {
   std::lock_guard<std::mutex> lock(registry_mutex());
-  registry().push_back(std::make_shared<RealMoeLayer>(std::move(layer)));
+  registry().push_back({std::make_shared<RealMoeLayer>(std::move(layer)), nullptr});
   return (uint32_t)(registry().size() - 1);
 }
 
-std::shared_ptr<const RealMoeLayer> get_real_moe_layer(uint32_t layer_id) {
+uint32_t register_resident_moe_layer(std::shared_ptr<ResidentExpertLayer> layer, size_t) {
   std::lock_guard<std::mutex> lock(registry_mutex());
-  if (layer_id >= registry().size()) return nullptr;
-  return registry()[layer_id];
+  registry().push_back({nullptr, std::move(layer)});
+  return (uint32_t)(registry().size() - 1);
+}
+
+// A resident id answers None here, as in the reference (graph_op.rs:294-299).
+std::shared_ptr<const RealMoeLayer> get_real_moe_layer(uint32_t layer_id) {
+  RegisteredMoe m;
+  if (!lookup(layer_id, &m)) return nullptr;
+  return m.real;
 }
 
 Result<std::vector<float>, MoeLayerError> execute_real_moe_layer(uint32_t layer_id,
                                                                  const std::vector<float>& input) {
-  auto layer = get_real_moe_layer(layer_id);
-  if (!layer) return Result<std::vector<float>, MoeLayerError>::Err(layer_not_found(layer_id));
-  return layer->forward_auto(input);  // whole batch, one call into the device library
+  RegisteredMoe m;
+  if (!lookup(layer_id, &m)) return Result<std::vector<float>, MoeLayerError>::Err(layer_not_found(layer_id));
+  // whole batch, one call into the device library; a resident layer drops its evidence here
+  // as the reference's execute_moe_row does (graph_op.rs:304-316)
+  if (m.resident) return m.resident->forward_batch(input);
+  return m.real->forward_auto(input);
 }
 
 Result<std::vector<float>, MoeLayerError> execute_real_moe_layer_with(

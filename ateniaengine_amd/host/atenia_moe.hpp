@@ -378,8 +378,49 @@ Result<std::pair<std::vector<float>, bool>, MoeSparseError> execute_conditional_
     uint32_t layer_id, uint32_t expert_id, const std::vector<float>& input,
     const std::vector<float>& selection);
 
+// ---- ResidentExpertLayer (src/moe/residency.rs:66-109, 586-614, 706-791) -------------------------
+// The reference keeps a layer's experts in a residency tier (RAM f32, bf16 RAM, NVMe) and
+// resolves the selected ones per token; its DeepSeek decoders call ResidentExpertLayer::forward
+// directly and its registry holds such layers next to the RAM ones (graph_op.rs:234-247).  With
+// every expert resident in HBM the tiers collapse to one, `Hbm`: nothing is materialised per
+// token, so the evidence the reference returns with each forward is what the kernels read --
+// the selected experts and their stored bytes.
+enum class ExpertTier { Hbm };
+struct ResidencyInfo {
+  std::vector<size_t> materialized_experts;  // routed experts the token used, ascending
+  size_t materialized_bytes = 0;             // their stored bytes, plus the shared expert's
+};
+class ResidentExpertLayer {
+ public:
+  MoeLayerConfig config;
+  MoeExecutionConvention convention = MoeExecutionConvention::Atenia;
+  ExpertTier tier = ExpertTier::Hbm;
+
+  // The layer's weights go to the device in the layer's own storage type on first use;
+  // convention = layer.resolve_convention(), as the reference's constructor takes it.
+  static ResidentExpertLayer from_real_layer(const RealMoeLayer& layer, ExpertTier tier = ExpertTier::Hbm);
+  size_t num_experts() const { return config.num_experts; }
+  // Bytes of one routed expert / of the shared expert as stored in HBM.
+  size_t expert_bytes() const;
+  size_t shared_bytes() const;
+  // One token [d_model]: output and evidence; equal to RealMoeLayer::forward_with under
+  // `convention` (src/moe/residency.rs:732-791).
+  Result<std::pair<std::vector<float>, ResidencyInfo>, MoeLayerError> forward(
+      const std::vector<float>& x) const;
+  // A flat batch [n * d_model] in one device call; infos (optional) receives one entry per row.
+  Result<std::vector<float>, MoeLayerError> forward_batch(const std::vector<float>& x,
+                                                          std::vector<ResidencyInfo>* infos = nullptr) const;
+
+ private:
+  std::shared_ptr<RealMoeLayer> layer_;
+};
+
 // ---- registry and graph op --------------------------------------------------------------------
 // Process-global, grow-only, ids stable per process (src/moe/graph_op.rs:221-232).
+// Resident layers share the id space with the RAM ones (graph_op.rs:207-216, 234-247);
+// cache_capacity is accepted for signature parity: with one HBM tier there is no expert cache.
+uint32_t register_resident_moe_layer(std::shared_ptr<ResidentExpertLayer> layer,
+                                     size_t cache_capacity = 0);
 uint32_t register_real_moe_layer(RealMoeLayer layer);
 std::shared_ptr<const RealMoeLayer> get_real_moe_layer(uint32_t layer_id);
 Result<std::vector<float>, MoeLayerError> execute_real_moe_layer(uint32_t layer_id,

@@ -582,6 +582,47 @@ int main(int argc, char** argv) {
           r.error().to_string().c_str());
     CHECK(layer.forward_auto(seeded(5, 8)).is_ok(), "the handle must stay usable after an error");
   });
+  // ResidentExpertLayer::forward == RealMoeLayer::forward_with under the resolved convention, with
+  // the evidence the reference returns (src/moe/residency.rs:732-791); a resident layer shares the
+  // registry with the RAM ones and is invisible to get_real_moe_layer (graph_op.rs:234-247, 294-299).
+  run_test("resident_expert_layer_equals_real_layer_and_registers", [&] {
+    RealMoeLayer real = layer_from(*q15);  // shared expert + sigmoid gate => HuggingFaceQwen
+    auto res = std::make_shared<ResidentExpertLayer>(ResidentExpertLayer::from_real_layer(real));
+    CHECK(res->convention == MoeExecutionConvention::HuggingFaceQwen && res->tier == ExpertTier::Hbm, "resolved");
+    CHECK(res->num_experts() == real.num_experts(), "experts");
+    auto want = real.forward_with(q15->input, real.resolve_convention()).unwrap();
+    auto got = res->forward(q15->input).unwrap();
+    CHECK(got.first == want, "resident forward differs from the RAM layer's");
+    std::vector<int32_t> idx;
+    real.route(q15->input, real.resolve_convention(), &idx).unwrap();
+    CHECK(got.second.materialized_experts.size() == idx.size(), "k experts reported");
+    for (size_t i = 0; i < idx.size(); ++i) {
+      CHECK(got.second.materialized_experts[i] == (size_t)idx[i], "expert %zu", i);
+      CHECK(i == 0 || idx[i] > idx[i - 1], "ascending");
+    }
+    const size_t d = real.config.d_model, f = real.config.d_ff, fs = real.shared->d_ff;
+    CHECK(got.second.materialized_bytes == idx.size() * 3 * d * f * 4 + 3 * d * fs * 4, "bytes %zu",
+          got.second.materialized_bytes);
+    // hf_ref of the fixture through the resident layer as well
+    CHECK(metrics(got.first, q15->hf_ref).max_abs_diff <= 1e-5, "hf_ref: %g",
+          metrics(got.first, q15->hf_ref).max_abs_diff);
+    // a row of the wrong length is the dense DimMismatch of the reference's forward
+    auto bad = res->forward(std::vector<float>(d + 1, 0.f));
+    CHECK(bad.is_err() && bad.error().kind == MoeLayerError::Binding, "wrong length refused");
+    // batch of rows == row by row, infos per row
+    std::vector<float> xb = q15->input;
+    auto x2 = seeded(91, d);
+    xb.insert(xb.end(), x2.begin(), x2.end());
+    std::vector<ResidencyInfo> infos;
+    auto yb = res->forward_batch(xb, &infos).unwrap();
+    auto y2 = res->forward(x2).unwrap();
+    CHECK(infos.size() == 2 && std::equal(y2.first.begin(), y2.first.end(), yb.begin() + d), "batch rows");
+    CHECK(infos[1].materialized_experts == y2.second.materialized_experts, "row evidence");
+    const uint32_t id = register_resident_moe_layer(res, 4);
+    CHECK(execute_real_moe_layer(id, q15->input).unwrap() == want, "graph op on a resident id");
+    CHECK(get_real_moe_layer(id) == nullptr, "a resident id is not a RealMoeLayer");
+    CHECK(moe_real_layer_reference_node(id, xb) == yb, "executor arm, flat batch");
+  });
   run_test("bf16_and_int8_storage_track_f32", [&] {
     auto f32 = layer_from(*mix).forward_auto(mix->input).unwrap();
     double scale = 0;
