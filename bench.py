@@ -5,8 +5,9 @@ Workload (the headline configuration): Mixtral-8x7B-shape layer, d_model 4096, 8
 renormalisation, expert d_ff 14336, bf16 weights resident in HBM (2.8 GB), bf16 activations
 already on the device.  A step is one layer forward over one batch of T tokens through the
 C ABI (`atenia_moe_hip_layer_forward_device`).  The default run times the prefill point
-T=4096 (the headline tokens/s, MFMA-bound) and the decode point T=1 (HBM-bound);
-`--sweep 1,16,128,512,4096` adds more batch sizes.
+T=4096 (the headline tokens/s, MFMA-bound) and the decode points T=1 and T=16 (HBM-bound);
+`--sweep 128,512` adds more batch sizes, `--config` picks another layer shape (tiny_f32 is the
+reference's own CPU-runnable case on the GPU's f32 path).
 
 Prints ONE JSON line.  `roofline` describes the dominant kernel of the headline batch, timed
 live with HIP events on the launch stream; `decode.roofline` the same for T=1;
@@ -25,6 +26,10 @@ sys.path.insert(0, ROOT)
 # Benchmark configurations.  The headline metric is quoted on mixtral_bf16; the others are
 # reported with --config.
 CONFIGS = {
+    # Tiny f32 layer (f32 storage, f64 accumulation: the reference's certified arithmetic on the
+    # GPU), T = 64: the configuration the reference's own CPU path is quoted on.
+    "tiny_f32": dict(d=1024, E=8, k=2, f=2048, fs=0, gated=False, conv=0, wd="f32",
+                     zipf=False, sweep=(64,)),
     "mixtral_bf16": dict(d=4096, E=8, k=2, f=14336, fs=0, gated=False, conv=0, wd="bf16",
                          zipf=False, sweep=(1, 16, 32, 64, 128, 512, 4096)),
     "mixtral_int8": dict(d=4096, E=8, k=2, f=14336, fs=0, gated=False, conv=0, wd="int8",
@@ -51,25 +56,42 @@ W_STD = 0.02
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, GB/s
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, TFLOP/s
 CONFIG_NAME = "mixtral_bf16"
-# HBM bytes per launch (read + written) of the expert kernels, measured with rocprofv3 --pmc
-# FETCH_SIZE / WRITE_SIZE and scaled by what the same counters read for a 1 GiB device copy
-# (FETCH_SIZE counts 2 KiB units, WRITE_SIZE KiB): profiles/
-# ffn_kernels_mixtral_bf16_T4096_T1_hbm_counters.txt.  Keyed by (config, tokens per step).
-MEASURED_HBM_TRAFFIC = {
-    ("mixtral_bf16", 4096): {"expert_gate_up": 2534048.7 * 2048 + 229376.0 * 1024,
-                             "expert_down": 1261307.5 * 2048 + 169317.3 * 1024},
-    ("mixtral_bf16", 1): {"expert_gate_up": 229448.8 * 2048, "expert_down": 114935.2 * 2048},
-}
+ACT = 1  # element type of the device activations: capi.ACT_BF16, or capi.ACT_F32 for f32 layers
+# Arithmetic type the expert kernels compute in, per storage type.
+DTYPE = {"bf16": "bf16", "int8": "bf16 (int8 weights widened in registers, W8A16)",
+         "int8g": "bf16 (int8 weights widened in registers, W8A16)", "f32": "f64"}
 
 
-def make_weights(torch, np, seed):
-    """~N(0, 0.02) weights generated on the GPU, truncated to bf16 (the reference's storage
-    convention, src/tensor/tensor.rs:306-308), returned as host uint16 arrays."""
+def measured_hbm_traffic():
+    """HBM bytes per launch (read + written) of the expert kernels as rocprofv3 measured them:
+    the `traffic <config> <tokens> <stage> <bytes>` lines that rocprof_summary.py writes into the
+    counter summaries under profiles/ (FETCH_SIZE / WRITE_SIZE passes scaled by a plain device
+    copy of known size).  {(config, tokens): {stage: bytes}}; empty when no summary is there."""
+    import glob
+    out = {}
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*hbm_counters*.txt"))):
+        with open(path) as fh:
+            for ln in fh:
+                f = ln.split()
+                if len(f) == 5 and f[0] == "traffic":
+                    out.setdefault((f[1], int(f[2])), {})[f[3]] = float(f[4])
+    return out
+
+
+MEASURED_HBM_TRAFFIC = measured_hbm_traffic()
+
+
+def make_weights(torch, np, seed, f32=False):
+    """~N(0, 0.02) weights generated on the GPU.  bf16 / int8 configurations: truncated to bf16
+    (the reference's storage convention, src/tensor/tensor.rs:306-308), returned as host uint16
+    arrays.  f32 configuration: the f32 values themselves."""
     g = torch.Generator(device="cuda")
     g.manual_seed(seed)
 
     def bf16_bits(shape):
         w = torch.randn(shape, generator=g, device="cuda", dtype=torch.float32) * W_STD
+        if f32:
+            return w.cpu().numpy()
         bits = (w.view(torch.int32) >> 16).to(torch.int16)
         return bits.cpu().numpy().view(np.uint16)
 
@@ -85,6 +107,8 @@ def make_weights(torch, np, seed):
 
 
 def upcast(np, bits):
+    if bits.dtype == np.float32:
+        return bits
     return (bits.astype(np.uint32) << 16).view(np.float32)
 
 
@@ -94,12 +118,14 @@ def measure(torch, np, capi, layer, T, steps, warmup, seed):
     g = torch.Generator(device="cuda")
     g.manual_seed(seed + T)
     xs = [torch.randn((T, D_MODEL), generator=g, device="cuda", dtype=torch.float32)
-          .to(torch.bfloat16) for _ in range(n_buf)]
+          for _ in range(n_buf)]
+    if ACT == capi.ACT_BF16:
+        xs = [x.to(torch.bfloat16) for x in xs]
     out = torch.empty((T, D_MODEL), device="cuda", dtype=torch.float32)
     stream = torch.cuda.current_stream().cuda_stream
 
     def step(i):
-        layer.forward_device(xs[i % n_buf].data_ptr(), capi.ACT_BF16, T, out.data_ptr(), stream)
+        layer.forward_device(xs[i % n_buf].data_ptr(), ACT, T, out.data_ptr(), stream)
 
     for i in range(warmup):
         step(i)
@@ -120,7 +146,7 @@ def measure(torch, np, capi, layer, T, steps, warmup, seed):
             for i in range(n_buf):
                 g_ = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(g_, stream=side):
-                    layer.forward_device(xs[i].data_ptr(), capi.ACT_BF16, T, out.data_ptr(),
+                    layer.forward_device(xs[i].data_ptr(), ACT, T, out.data_ptr(),
                                          torch.cuda.current_stream().cuda_stream)
                 graphs.append(g_)
         torch.cuda.synchronize()
@@ -161,7 +187,8 @@ def measure(torch, np, capi, layer, T, steps, warmup, seed):
     bytes_up = U * (2 * D_FF * D_MODEL * eb + 2 * D_FF * sc_up) + 2 * fs * D_MODEL * eb + 2 * fs * sc_up
     bytes_down = (U * (D_MODEL * D_FF * eb + D_MODEL * sc_down) + fs * D_MODEL * eb +
                   (D_MODEL * sc_sdown if fs else 0))
-    bytes_fwd = bytes_up + bytes_down + N_EXPERTS * D_MODEL * 4 + T * D_MODEL * (2 + 4)
+    bytes_fwd = (bytes_up + bytes_down + N_EXPERTS * D_MODEL * 4 +
+                 T * D_MODEL * ((2 if ACT == capi.ACT_BF16 else 4) + 4))
     P = T * TOP_K
     flops_up = 4.0 * P * D_MODEL * D_FF + 4.0 * T * D_MODEL * fs
     flops_down = 2.0 * P * D_MODEL * D_FF + 2.0 * T * D_MODEL * fs
@@ -184,7 +211,8 @@ def measure(torch, np, capi, layer, T, steps, warmup, seed):
         ("expert_gate_up", up_ms, bytes_up, flops_up) if up_ms >= down_ms
         else ("expert_down", down_ms, bytes_down, flops_down))
     # HBM-bound while the weights outweigh the arithmetic: below ~300 rows per expert.
-    hbm_bound = (dom_flops / (PEAK_BF16_TFLOPS * 1e12)) < (dom_bytes / (PEAK_HBM_GBS * 1e9))
+    hbm_bound = W_BYTES == 4 or ((dom_flops / (PEAK_BF16_TFLOPS * 1e12)) <
+                                 (dom_bytes / (PEAK_HBM_GBS * 1e9)))
     if hbm_bound:
         ach = dom_bytes / (dom_ms * 1e-3) / 1e9
         r["roofline"] = dict(bound="hbm", kernel=dom, achieved=ach, peak=PEAK_HBM_GBS,
@@ -283,10 +311,15 @@ def main():
                     help="layer shape (the headline metric is quoted on mixtral_bf16)")
     ap.add_argument("--tokens", type=int, default=0,
                     help="headline batch size T (default: the config's largest)")
-    ap.add_argument("--decode-tokens", type=int, default=1, help="decode batch (0 = skip)")
+    ap.add_argument("--decode-tokens", type=str, default="1,16",
+                    help="decode batch sizes, comma separated (empty = skip); reported as "
+                         "`decode` (the first) and `decode<T>` (the others)")
     ap.add_argument("--sweep", type=str, default="", help="extra batch sizes, comma separated")
-    ap.add_argument("--cpu-tokens", type=int, default=1024,
-                    help="tokens of the CPU-baseline sample (0 = skip)")
+    ap.add_argument("--cpu-tokens", type=int, default=-1,
+                    help="tokens of the CPU-baseline sample (0 = skip; default: about 12 s of "
+                         "CPU work on 16 cores)")
+    ap.add_argument("--host-steps", type=int, default=3,
+                    help="timed calls of the host-buffer entry point on the headline batch (0 = skip)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (reference point for HBM counters)")
     ap.add_argument("--graph", action="store_true",
@@ -311,29 +344,38 @@ def main():
         print("bench.py: no gfx950 device; the HIP path has no fallback", file=sys.stderr)
         sys.exit(3)
     torch.cuda.set_device(0)
-    global D_MODEL, N_EXPERTS, TOP_K, D_FF, D_FF_SHARED, W_BYTES, CONFIG_NAME, GROUP, GRAPH
+    global D_MODEL, N_EXPERTS, TOP_K, D_FF, D_FF_SHARED, W_BYTES, CONFIG_NAME, GROUP, GRAPH, ACT
     GRAPH = a.graph
     cfg = CONFIGS[a.config]
     CONFIG_NAME = a.config
     D_MODEL, N_EXPERTS, TOP_K, D_FF, D_FF_SHARED = cfg["d"], cfg["E"], cfg["k"], cfg["f"], cfg["fs"]
-    W_BYTES = 1 if cfg["wd"] in ("int8", "int8g") else 2
+    f32w = cfg["wd"] == "f32"
+    W_BYTES = 4 if f32w else 1 if cfg["wd"] in ("int8", "int8g") else 2
+    ACT = capi.ACT_F32 if f32w else capi.ACT_BF16
     GROUP = 128 if cfg["wd"] == "int8g" else 0
     if a.tokens <= 0:
         a.tokens = max(cfg["sweep"])
+    decode_ts = [int(t) for t in a.decode_tokens.split(",") if t]
+    decode_ts = [t for t in decode_ts if t != a.tokens and (t in cfg["sweep"] or a.decode_tokens != "1,16")]
     if a.sweep == "all":
-        a.sweep = ",".join(str(t) for t in cfg["sweep"] if t not in (a.tokens, a.decode_tokens))
-    router, gate, up, down, shared = make_weights(torch, np, a.seed)
+        a.sweep = ",".join(str(t) for t in cfg["sweep"] if t != a.tokens and t not in decode_ts)
+    router, gate, up, down, shared = make_weights(torch, np, a.seed, f32=f32w)
     router_f32 = upcast(np, router)
     if cfg["zipf"]:  # logits ~ N(0,1) plus a log-Zipf(1.2) bias: skewed expert load
         router_f32 = router_f32 * np.float32(1.0 / (W_STD * np.sqrt(D_MODEL)))
         router_f32 = upcast(np, capi.f32_to_bf16_trunc(router_f32))
-    tmax = max([a.tokens, a.decode_tokens] + [int(t) for t in a.sweep.split(",") if t])
+    tmax = max([a.tokens] + decode_ts + [int(t) for t in a.sweep.split(",") if t])
     kw = dict(w_router=router_f32, top_k=TOP_K, convention=cfg["conv"], max_tokens_hint=tmax)
     if cfg["zipf"]:
         rank = np.random.default_rng(a.seed).permutation(N_EXPERTS) + 1.0
         kw["router_bias"] = (-1.2 * np.log(rank)).astype(np.float32)
     if shared is not None and cfg["gated"]:
         kw["shared_gate"] = shared[3]
+    # what the CPU path computes with: the stored values, upcast / dequantised to f32
+    stored = dict(w_gate=upcast(np, gate), w_up=upcast(np, up), w_down=upcast(np, down))
+    if shared is not None:
+        stored.update(s_gate=upcast(np, shared[0]), s_up=upcast(np, shared[1]),
+                      s_down=upcast(np, shared[2]))
     if cfg["wd"] in ("int8", "int8g"):
         # int8 of the bf16-valued weights (per output row, or per row and 128-element group),
         # 0.1 % of rows scaled x8 first
@@ -342,20 +384,24 @@ def main():
         if per_group:
             kw["group_size"] = 128
 
-        def q8(bits):
+        def q8(bits, name):
             w = upcast(np, bits)
             rows = w.reshape(-1, w.shape[-1])
             rows[rng.choice(rows.shape[0], size=rows.shape[0] // 1000, replace=False)] *= 8.0
-            return capi.quantize_per_group_i8(w, 128) if per_group else capi.quantize_per_row_i8(w)
-        (gate, sg), (up, su), (down, sd) = q8(gate), q8(up), q8(down)
+            q, sc = capi.quantize_per_group_i8(w, 128) if per_group else capi.quantize_per_row_i8(w)
+            full = np.repeat(sc, 128, axis=-1)[..., :w.shape[-1]] if per_group else sc[..., None]
+            stored[name] = q.astype(np.float32) * full
+            return q, sc
+        (gate, sg), (up, su), (down, sd) = q8(gate, "w_gate"), q8(up, "w_up"), q8(down, "w_down")
         kw.update(scale_gate=sg, scale_up=su, scale_down=sd)
         if shared is not None:
-            (g_, a1), (u_, a2), (d_, a3) = q8(shared[0]), q8(shared[1]), q8(shared[2])
+            (g_, a1), (u_, a2), (d_, a3) = (q8(shared[0], "s_gate"), q8(shared[1], "s_up"),
+                                            q8(shared[2], "s_down"))
             shared = (g_, u_, d_, shared[3])
             kw.update(s_scale_gate=a1, s_scale_up=a2, s_scale_down=a3)
         wdt = capi.WEIGHT_INT8_PER_GROUP if per_group else capi.WEIGHT_INT8_W8A16
     else:
-        wdt = capi.WEIGHT_BF16
+        wdt = capi.WEIGHT_F32 if f32w else capi.WEIGHT_BF16
     if shared is not None:
         kw.update(s_gate=shared[0], s_up=shared[1], s_down=shared[2])
     layer = capi.Layer(w_gate=gate, w_up=up, w_down=down, weight_dtype=wdt, **kw)
@@ -374,10 +420,10 @@ def main():
         del src, dst
 
     head, x_head, out_head = measure(torch, np, capi, layer, a.tokens, a.steps, a.warmup, a.seed)
-    decode = None
-    if a.decode_tokens > 0:
-        decode, _, _ = measure(torch, np, capi, layer, a.decode_tokens, max(a.steps, 50),
-                               max(a.warmup, 10), a.seed)
+    decodes = {}
+    for t in decode_ts:
+        decodes[t], _, _ = measure(torch, np, capi, layer, t, max(a.steps, 50), max(a.warmup, 10),
+                                   a.seed)
     sweep = []
     for t in [int(t) for t in a.sweep.split(",") if t]:
         r, _, _ = measure(torch, np, capi, layer, t, a.steps if t >= 512 else max(a.steps, 50),
@@ -388,23 +434,40 @@ def main():
     if a.block:
         block = [measure_block(torch, np, capi, layer, t, a.steps if t >= 512 else max(a.steps, 50),
                                a.warmup, a.seed)
-                 for t in sorted({a.tokens, a.decode_tokens} | {int(t) for t in a.sweep.split(",") if t})
+                 for t in sorted({a.tokens} | set(decode_ts) | {int(t) for t in a.sweep.split(",") if t})
                  if t > 0]
+
+    # The entry point a caller of the reference's op reaches: [T * d] f32 in host memory in and
+    # out (src/amg/graph.rs:5572-5589 hands a Vec<f32> over).  PCIe-inclusive, never `value`.
+    host = None
+    if a.host_steps > 0:
+        xh = x_head.to(torch.float32).cpu().numpy()
+        layer.forward(xh)
+        t0 = time.perf_counter()
+        for _ in range(a.host_steps):
+            layer.forward(xh)
+        host_ms = (time.perf_counter() - t0) * 1e3 / a.host_steps
+        host = dict(tokens=a.tokens, forward_host_ms=host_ms, tokens_per_s=a.tokens / (host_ms * 1e-3),
+                    host_bytes_moved=2.0 * a.tokens * D_MODEL * 4,
+                    note="atenia_moe_hip_layer_forward: pageable host buffers in and out, synchronous")
 
     cpu = None
     parity = None
-    if a.cpu_tokens > 0 and a.config == "mixtral_bf16":
+    if a.cpu_tokens != 0:
         from oracle import moe_oracle as ora  # checker + reported CPU baseline only
-        n = min(a.cpu_tokens, a.tokens)
+        flops_tok = 2.0 * D_MODEL * N_EXPERTS + 6.0 * TOP_K * D_MODEL * D_FF + 6.0 * D_MODEL * D_FF_SHARED
+        n = a.cpu_tokens if a.cpu_tokens > 0 else int(1024 * 704.7e6 / flops_tok)
+        n = max(1, min(n, a.tokens))
         # the headline batch, recomputed once so `out_head` matches `x_head`
-        layer.forward_device(x_head.data_ptr(), capi.ACT_BF16, a.tokens, out_head.data_ptr(),
+        layer.forward_device(x_head.data_ptr(), ACT, a.tokens, out_head.data_ptr(),
                              torch.cuda.current_stream().cuda_stream)
         torch.cuda.synchronize()
         idx_gpu, *_ = layer.last_routing(a.tokens)
         xs = x_head[:n].to(torch.float32).cpu().numpy()
         got = out_head[:n].cpu().numpy()
-        oL = ora.Layer(w_router=router_f32, w_gate=upcast(np, gate), w_up=upcast(np, up),
-                       w_down=upcast(np, down), top_k=TOP_K, convention=ora.ATENIA)
+        oL = ora.Layer(w_router=router_f32, top_k=TOP_K, convention=cfg["conv"],
+                       shared_gate=kw.get("shared_gate"), router_bias=kw.get("router_bias"),
+                       **stored)
         cores = ora.hw_threads()
         ora.set_threads(cores)
         oL.execute(xs[:1])  # warm the pages
@@ -425,19 +488,23 @@ def main():
         "metric": "Mixtral-shape MoE layer tok/s; decode HBM GB/s and prefill MFMA TFLOPS",
         "value": head["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": a.steps,
         "warmup": a.warmup, "ms_per_step": head["ms_per_step"], "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "scaling": "weak", "vs_baseline": None, "dtype": DTYPE[cfg["wd"]], "data": "synthetic",
         "config": {"workload": f"{a.config}: MoE layer, d_model={D_MODEL}, experts={N_EXPERTS}, "
                                f"top_k={TOP_K}, d_ff={D_FF}, shared d_ff={D_FF_SHARED}, "
-                               f"{cfg['wd']} weights resident in HBM, bf16 activations, "
+                               f"{cfg['wd']} weights resident in HBM, "
+                               f"{'f32' if f32w else 'bf16'} activations, "
                                f"T={a.tokens} tokens per step",
                    "tokens_per_step": a.tokens},
         "roofline": head["roofline"],
         "cpu_baseline": cpu,
         "prefill": head,
-        "decode": decode,
+        "decode": decodes.get(decode_ts[0]) if decode_ts else None,
         "sweep": sweep,
         "parity": parity,
+        "host_entry": host,
     }
+    for t in decode_ts[1:]:
+        line[f"decode{t}"] = decodes[t]
     if block is not None:
         line["block"] = block
     if a.dequant:
