@@ -13,7 +13,8 @@ from typing import Optional
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libatenia_moe_hip.so")
+# ATENIA_MOE_HIP_LIBRARY names another build of the library (same ABI) to load instead.
+LIB_PATH = os.environ.get("ATENIA_MOE_HIP_LIBRARY") or os.path.join(_HERE, "libatenia_moe_hip.so")
 
 CONVENTION_ATENIA = 0
 CONVENTION_HUGGINGFACE_QWEN = 1

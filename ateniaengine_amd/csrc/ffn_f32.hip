@@ -6,8 +6,9 @@
 //   h    = (f32)(silu_f64(gate)) * up        -- an f32 product
 //   y    = (f32) sum_f64(W_d h)
 // Only the order of the f64 additions differs from the CPU path (k is tiled), which moves a
-// result by ~1e-16 relative before the final f32 rounding.  This path exists for parity
-// with f32 checkpoints (1e-5 bar); it is FMA-bound and not the throughput path.
+// result by ~1e-16 relative before the final f32 rounding.  Two forms: the f64 matrix cores
+// (ffn_f32_mfma_kernel, K a multiple of 8) and a scalar tile kernel for every other shape and
+// for the f32-accumulating policies.
 //
 // F32ACC: the reference's other expert arithmetic (`matvec_f32`, src/moe/dense.rs:120-140, used
 // under NumericPolicy::Strict and as the result `Fast` falls back to): the three projections
@@ -15,6 +16,8 @@
 // ascending.  A thread walks the k tiles in order, so its f32 sequence IS the reference's; the
 // file is compiled without contraction so that no product is fused into the sum.  silu stays
 // f64 -> f32 and the router stays f64 on every policy (src/moe/numeric_policy.rs:24-29).
+#include <cstdlib>
+
 #include "moe_internal.h"
 
 namespace atenia_moe {
@@ -115,9 +118,192 @@ __global__ __launch_bounds__(256) void ffn_f32_kernel(
   }
 }
 
+// ---- certified arithmetic on the f64 matrix cores ---------------------------------------------
+// v_mfma_f64_16x16x4_f64: D[16 x 16] += A[16 x 4] * B[4 x 16] in f64.  Lane l supplies
+// A[l % 16][l / 16] and B[l / 16][l % 16] (one double each) and holds D[4 * r + l / 16][l % 16],
+// r = 0..3 (rows interleaved, unlike the f32 forms).  Here A = 16 weight rows, B = 16 token rows
+// (transposed), so a lane's four results are weight rows l / 16, +4, +8, +12 of one token.
+//
+// f32 operands widen to f64 exactly and every product of two f32 values is exact in f64, so the
+// only difference from the reference's c-ascending sum is the order of the f64 additions
+// (~1e-16 relative before the f32 rounding) -- the same statement as for the scalar kernel above,
+// at the matrix cores' rate.
+//
+// A workgroup owns a strip of 16 weight rows (gate and up strips in the gate/up phase) of one
+// expert and up to MT * 16 of its token rows; its four waves split K and add their partial sums
+// in wave order through LDS.  A lane loads 8 consecutive k of "its" row per step (rows l % 16,
+// k chunk l / 16: four lanes cover one full 128-byte line of the row) for both operands; MFMA t
+// of the step contracts element t of every lane's chunk, i.e. k = k0 + 8 * (l / 16) + t -- any
+// partition of k into groups of four is as good as another as long as A and B agree.
+typedef __attribute__((__vector_size__(4 * sizeof(double)))) double f64x4;
+
+// KS: waves that share one strip's K (4: one strip per workgroup, partial sums meet in LDS;
+// 1: four strips per workgroup, one per wave, no reduction -- better when K is short).
+template <bool UP, int MT, int KS>
+__global__ __launch_bounds__(256) void ffn_f32_mfma_kernel(
+    const float* __restrict__ wa, const float* __restrict__ wb, int64_t w_stride, int n_rows,
+    int k_cols, const float* __restrict__ a, int a_stride, float* __restrict__ out,
+    int out_stride, GroupDesc g) {
+  const int u = blockIdx.y;
+  if (u >= *g.n_active) return;
+  const int e = g.active[u];
+  const int base = g.offsets[e];
+  const int cnt = g.offsets[e + 1] - base;
+  const int m0 = blockIdx.z * 16 * MT;
+  if (m0 >= cnt) return;
+  const int mt_live = __builtin_amdgcn_readfirstlane(min(MT, (cnt - m0 + 15) >> 4));
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int n0 = (blockIdx.x * (4 / KS) + wave / KS) * 16;
+  if (KS == 1 && n0 >= n_rows) return;  // whole wave past the last strip (no barrier follows)
+  const int kslice = wave % KS;
+  const int r16 = lane & 15, q = lane >> 4;
+  constexpr int NACC = UP ? 2 : 1;
+
+  // weight row of this lane (clamped: rows past n_rows are computed and never stored)
+  const int nrow = min(n0 + r16, n_rows - 1);
+  const float* pa = wa + (size_t)e * w_stride + (size_t)nrow * k_cols + 8 * q;
+  const float* pb = UP ? wb + (size_t)e * w_stride + (size_t)nrow * k_cols + 8 * q : nullptr;
+  const float* px[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) {
+    int pos = m0 + 16 * i + r16;
+    if (pos >= cnt) pos = m0;  // an output column depends on its own token only; never stored
+    const int row = UP ? g.perm[base + pos] / g.pair_div : base + pos;
+    px[i] = a + (size_t)row * a_stride + 8 * q;
+  }
+
+  // K in steps of 32 (8 per lane chunk), the steps dealt to the KS waves in contiguous runs
+  const int nsteps = (k_cols + 31) / 32;
+  const int per = (nsteps + KS - 1) / KS;
+  const int s0 = kslice * per, s1 = min(nsteps, s0 + per);
+  f64x4 acc[NACC][MT];
+#pragma unroll
+  for (int n = 0; n < NACC; ++n)
+#pragma unroll
+    for (int i = 0; i < MT; ++i) acc[n][i] = f64x4{0.0, 0.0, 0.0, 0.0};
+
+  struct Chunk {
+    float4 lo, hi;
+  };
+  auto load8 = [&](const float* p, int st) {
+    Chunk c;
+    if (st * 32 + 8 * q < k_cols) {  // k_cols is a multiple of 8: a chunk is whole or absent
+      c.lo = *(const float4*)(p + (size_t)st * 32);
+      c.hi = *(const float4*)(p + (size_t)st * 32 + 4);
+    } else {
+      c.lo = c.hi = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    return c;
+  };
+  auto elem = [](const Chunk& c, int t) {
+    const float v[8] = {c.lo.x, c.lo.y, c.lo.z, c.lo.w, c.hi.x, c.hi.y, c.hi.z, c.hi.w};
+    return (double)v[t];
+  };
+  Chunk wA[2], wB[2], xs[2][MT] = {};
+  auto load_step = [&](int buf, int st) {
+    wA[buf] = load8(pa, st);
+    if (UP) wB[buf] = load8(pb, st);
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+      if (i < mt_live) xs[buf][i] = load8(px[i], st);
+  };
+  auto multiply = [&](int buf) {
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      const double va = elem(wA[buf], t);
+      const double vb = UP ? elem(wB[buf], t) : 0.0;
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        if (i >= mt_live) continue;  // scalar branch: a 16-row tile without rows costs no MFMAs
+        const double vx = elem(xs[buf][i], t);
+        acc[0][i] = __builtin_amdgcn_mfma_f64_16x16x4f64(va, vx, acc[0][i], 0, 0, 0);
+        if (UP) acc[NACC - 1][i] = __builtin_amdgcn_mfma_f64_16x16x4f64(vb, vx, acc[NACC - 1][i], 0, 0, 0);
+      }
+    }
+  };
+  if (s0 < s1) load_step(0, s0);
+  for (int st = s0; st < s1; st += 2) {
+    if (st + 1 < s1) load_step(1, st + 1);
+    multiply(0);
+    if (st + 2 < s1) load_step(0, st + 2);
+    if (st + 1 < s1) multiply(1);
+  }
+
+  if (KS > 1) {  // partial sums of waves 1..3 to LDS, wave 0 adds them in wave order
+    __shared__ f64x4 red[KS > 1 ? KS - 1 : 1][NACC][MT][64];
+    if (wave > 0) {
+#pragma unroll
+      for (int n = 0; n < NACC; ++n)
+#pragma unroll
+        for (int i = 0; i < MT; ++i) red[wave - 1][n][i][lane] = acc[n][i];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int w = 0; w < KS - 1; ++w)
+#pragma unroll
+      for (int n = 0; n < NACC; ++n)
+#pragma unroll
+        for (int i = 0; i < MT; ++i) acc[n][i] += red[w][n][i][lane];
+  }
+
+#pragma unroll
+  for (int i = 0; i < MT; ++i) {
+    const int pos = m0 + 16 * i + r16;  // the lane's token
+    if (pos >= cnt) continue;
+    const int pair = UP ? 0 : g.perm[base + pos];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int n = n0 + 4 * r + q;
+      if (n >= n_rows) continue;
+      if (UP) {
+        const float gate = (float)acc[0][i][r];
+        const float up = (float)acc[NACC - 1][i][r];
+        const double gd = (double)gate;
+        const float sv = (float)(gd / (1.0 + exp(-gd)));
+        out[(size_t)(base + pos) * out_stride + n] = __fmul_rn(sv, up);
+      } else {
+        out[(size_t)pair * out_stride + n] = (float)acc[0][i][r];
+      }
+    }
+  }
+}
+
+// The matrix-core form needs whole 8-element chunks and 16-byte aligned rows.
+bool mfma_f64_ok(const FfnArgs& a, bool up) {
+  const int k = up ? a.gate.k_cols : a.down.k_cols;
+  const int stride = up ? a.x_stride : a.h_stride;
+  const void* act = up ? a.x : a.h;
+  return !a.f32_accumulate && k % 8 == 0 && stride % 4 == 0 && ((uintptr_t)act & 15) == 0;
+}
+
+// Four waves on one strip's K, or one strip per wave (tuning knob ATENIA_MOE_F32_KSPLIT = 0 / 1,
+// read once per process; default: split unless K is a few steps only).
+bool mfma_f64_splits_k(int n_rows, int k_cols) {
+  static const int forced = [] {
+    const char* e = getenv("ATENIA_MOE_F32_KSPLIT");
+    return e ? atoi(e) : -1;
+  }();
+  if (forced >= 0) return forced != 0;
+  (void)n_rows;
+  return k_cols >= 128;  // measured at d = 1024, f = 2048, T = 64: gate/up 53 against 59 us, down 32 against 69
+}
+
 }  // namespace
 
 hipError_t launch_ffn_up_f32(const FfnArgs& a, hipStream_t s) {
+  if (mfma_f64_ok(a, true)) {
+    const int mt = a.rows_max <= 16 ? 1 : 2;
+    const bool split = mfma_f64_splits_k(a.gate.n_rows, a.gate.k_cols);
+    const int strips = (a.gate.n_rows + 15) / 16;
+    dim3 grid(split ? strips : (strips + 3) / 4, a.n_groups_max, (a.rows_max + 16 * mt - 1) / (16 * mt));
+    auto k = split ? (mt == 1 ? ffn_f32_mfma_kernel<true, 1, 4> : ffn_f32_mfma_kernel<true, 2, 4>)
+                   : (mt == 1 ? ffn_f32_mfma_kernel<true, 1, 1> : ffn_f32_mfma_kernel<true, 2, 1>);
+    k<<<grid, 256, 0, s>>>((const float*)a.gate.w, (const float*)a.up.w, a.gate.expert_stride,
+                           a.gate.n_rows, a.gate.k_cols, (const float*)a.x, a.x_stride,
+                           (float*)a.h, a.h_stride, a.g);
+    return hipGetLastError();
+  }
   dim3 grid((a.gate.n_rows + kTile - 1) / kTile, a.n_groups_max,
             (a.rows_max + kTile - 1) / kTile);
   auto k = a.f32_accumulate ? ffn_f32_kernel<true, true> : ffn_f32_kernel<true, false>;
@@ -128,6 +314,17 @@ hipError_t launch_ffn_up_f32(const FfnArgs& a, hipStream_t s) {
 }
 
 hipError_t launch_ffn_down_f32(const FfnArgs& a, hipStream_t s) {
+  if (mfma_f64_ok(a, false)) {
+    const int mt = a.rows_max <= 16 ? 1 : 2;
+    const bool split = mfma_f64_splits_k(a.down.n_rows, a.down.k_cols);
+    const int strips = (a.down.n_rows + 15) / 16;
+    dim3 grid(split ? strips : (strips + 3) / 4, a.n_groups_max, (a.rows_max + 16 * mt - 1) / (16 * mt));
+    auto k = split ? (mt == 1 ? ffn_f32_mfma_kernel<false, 1, 4> : ffn_f32_mfma_kernel<false, 2, 4>)
+                   : (mt == 1 ? ffn_f32_mfma_kernel<false, 1, 1> : ffn_f32_mfma_kernel<false, 2, 1>);
+    k<<<grid, 256, 0, s>>>((const float*)a.down.w, nullptr, a.down.expert_stride, a.down.n_rows,
+                           a.down.k_cols, (const float*)a.h, a.h_stride, a.y, a.y_stride, a.g);
+    return hipGetLastError();
+  }
   dim3 grid((a.down.n_rows + kTile - 1) / kTile, a.n_groups_max,
             (a.rows_max + kTile - 1) / kTile);
   auto k = a.f32_accumulate ? ffn_f32_kernel<false, true> : ffn_f32_kernel<false, false>;

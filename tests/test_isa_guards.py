@@ -39,7 +39,7 @@ def _assembly(tmp_path_factory, name):
     return [ln.strip() for ln in open(out).read().split("\n")]
 
 
-@pytest.fixture(scope="module", params=["ffn_stream.hip", "ffn_tiled.hip"])
+@pytest.fixture(scope="module", params=["ffn_stream.hip", "ffn_tiled.hip", "ffn_f32.hip"])
 def asm(request, tmp_path_factory):
     if not os.path.exists(HIPCC):
         pytest.skip("hipcc not found")
@@ -68,7 +68,7 @@ def test_no_mfma_under_an_exec_mask(asm):
             total += 1
             if masked:
                 hits.append((no, ln))
-    assert total > 100, f"{name}: expected the MFMA kernels in the assembly, found {total} MFMAs"
+    assert total > (30 if name == "ffn_f32.hip" else 100), f"{name}: expected the MFMA kernels in the assembly, found {total} MFMAs"
     assert not hits, f"{name}: MFMA inside an EXEC-masked region (MFMA ignores EXEC): {hits[:5]}"
 
 
