@@ -139,7 +139,7 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p_r
   // of batch i+1 are in flight while batch i is multiplied.  The first batch is requested
   // before the dependent look-ups (perm -> token row) below, so the weight stream starts one
   // memory latency after the workgroup does.
-  constexpr int U = INT8 ? 2 : 4;        // blocks per batch
+  constexpr int U = INT8 ? (MT == 1 && S == 1 && !PG ? 4 : 2) : 4;  // blocks per batch
   constexpr int AV = INT8 ? 2 : 1;       // 16-byte activation pieces per block and row tile
   uint4 wA0[S][U], wB0[S][UP ? U : 1], wA1[S][U], wB1[S][UP ? U : 1];
   uint4 xa0[U][MT][AV], xa1[U][MT][AV];
