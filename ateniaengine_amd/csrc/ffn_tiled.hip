@@ -64,6 +64,8 @@ struct TiledParams {
   const int32_t* tile_group;  // [n_tiles] expert of each row tile
   const int32_t* tile_m0;     // [n_tiles] first row (relative to the group) of each row tile
   const int32_t* n_tiles;     // [1]
+  const int32_t* tile_rows;   // [n_tiles] rows of each tile, or null: min(TM, rows left)
+  const int32_t* tile_li;     // [n_tiles] index inside the expert | (its tiles << 16), or null
   int n_col_tiles;
   // k split of the tail tiles (pipelined down kernels; max_parts <= 1: off).  Workgroup ids
   // below wg_upper are the tiles themselves, ids from wg_upper on the extra k ranges of the
@@ -136,10 +138,17 @@ __device__ inline bool tile_of_workgroup(const TiledParams& p, int wid, int& rt,
   // Row tiles are sorted by expert, so the expert owning this logical id is the expert of
   // row tile logical / nct; that tile's m0 tells where the expert's tiles start.
   const int rt_any = logical / nct;
-  const int e = p.tile_group[rt_any];
-  const int first = rt_any - p.tile_m0[rt_any] / TM;
-  const int cnt = p.g.offsets[e + 1] - p.g.offsets[e];
-  const int nt = (cnt + TM - 1) / TM;
+  int first, nt;
+  if (p.tile_li) {  // tiles of uneven height: the list says where the expert's tiles start
+    const int li = p.tile_li[rt_any];
+    first = rt_any - (li & 0xffff);
+    nt = li >> 16;
+  } else {
+    const int e = p.tile_group[rt_any];
+    const int cnt = p.g.offsets[e + 1] - p.g.offsets[e];
+    first = rt_any - p.tile_m0[rt_any] / TM;
+    nt = (cnt + TM - 1) / TM;
+  }
   int local = logical - first * nct;
   const int full = nct / kColGroup;
   const int patch = nt * kColGroup;
@@ -415,12 +424,16 @@ __device__ inline void wait_vm_lgkm0() {
   __builtin_amdgcn_s_waitcnt(0x0070 | (N & 15) | ((N >> 4) << 14));
 }
 constexpr int kRingA = 3;  // A stages of 64 k (32 KiB each)
-constexpr int kRingB = 4;  // B stages of 32 k (16 KiB each)
+constexpr int kRingB = 3;  // B stages of 32 k (16 KiB each); a fourth measured no faster
+// Rows 256..287 of a nine-group tile: their own ring of 64-k stages (4 KiB each = four chunks of
+// 8 rows x 128 bytes, swizzled like the A chunks), one stage per A stage.
+constexpr int kXaStage = 256;  // uint4 per stage
 
 template <bool UP>
 __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p) {
   constexpr int NA = kRingA, NB = kRingB;
-  __shared__ uint4 S[NA * 2048 + NB * 1024];  // A ring, then B ring
+  constexpr int XA0 = NA * 2048 + NB * 1024;            // first uint4 of the extra-rows ring
+  __shared__ uint4 S[XA0 + NA * kXaStage];              // A ring, B ring, extra-rows ring
   int wid, n_parts, part;  // k range `part` of `n_parts` (1 unless this is a split tail tile)
   if (!split_of_workgroup(p, p.k_pad / 64, wid, n_parts, part)) return;
   int rt, ct;
@@ -430,7 +443,10 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p)
   const int tm0 = p.tile_m0[rt];
   const int base = p.g.offsets[e];
   const int cnt = p.g.offsets[e + 1] - base;
-  const int rows_here = min(TM, cnt - tm0);
+  const int rows_here = p.tile_rows ? p.tile_rows[rt] : min(TM, cnt - tm0);
+  // A tile of nine 32-row groups: rows 256.. ride along as a ninth group whose 32 x 256 results
+  // are shared out over the four waves (two 32 x 32 blocks each).
+  const bool tall = rows_here > TM;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -488,6 +504,17 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p)
       arow[q] = p.a + (size_t)src * p.a_stride + (pslot ^ r8 ^ (q & 1)) * 8;
     }
   }
+  // extra rows (tall tiles): wave w fills chunk w of a stage, rows 256 + 8 w ..
+  const uint16_t* xrow = nullptr;
+  if (tall) {
+    const int r8 = lane >> 3, pslot = lane & 7;
+    int m = TM + wave * 8 + r8;
+    if (m >= rows_here) m = 0;
+    int src;
+    if (UP) src = p.g.perm[base + tm0 + m] / p.g.pair_div;
+    else src = base + tm0 + m;
+    xrow = p.a + (size_t)src * p.a_stride + (pslot ^ r8 ^ (wave & 1)) * 8;
+  }
   // fragment read offsets (uint4 units inside a stage): A row group i adds 256, k16 unit u of
   // the 64-k stage selects the swizzled segment; B row group j of this wave, unit u adds 64.
   int aoff[4];
@@ -497,6 +524,8 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p)
 #pragma unroll
     for (int u = 0; u < 4; ++u) aoff[u] = rowbase + ((2 * u + kh) ^ r8 ^ cpar);
   }
+  // the ninth group's fragment of unit u sits at aoff[u] of row group 0 in its own ring
+  const int xoff0 = XA0 - wm * 16 * 64;
   const int boff0 = NA * 2048 + (UP ? 2 * wn : 4 * wn) * 128 + lane;
   constexpr int kBJ1 = 128, kBJ2 = UP ? 512 : 256, kBJ3 = UP ? 640 : 384;
 
@@ -513,6 +542,11 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p)
   auto dma_a = [&](int buf, int q, int t) {  // chunk q of this wave, 64-k stage t
     dma16(arow[q] + (size_t)(ks0 / 2 + t) * 64, sa_fill + buf * 32768 + q * kChunk);
   };
+  const uint32_t xa_fill = (uint32_t)(uintptr_t)(lptr_t)S + XA0 * 16 + wave * kChunk;
+  auto dma_xa = [&](int buf, int t) {  // this wave's chunk of the extra rows, 64-k stage t
+    dma16(xrow + (size_t)(ks0 / 2 + t) * 64, xa_fill + buf * (kXaStage * 16));
+  };
+
   // the 8 fragment reads of one k16 unit, in the order the MFMAs consume them
   auto read_frag = [&](int n, uint4 (&FA)[4], uint4 (&FB)[4], int a0, int b0) {
     switch (n) {
@@ -569,11 +603,15 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p)
         for (int q = 0; q < 8; ++q) dma_a(t, q, min(t, nst - 1));
       }
     };
-    // issued so far: B0 B1 B2 B3; now A0 A1, then per step: half of A(s/2 + 2), B(s + 4).
+    // issued so far: B0 .. B(NB-1); now A0 A1, then per step: half of A(s/2 + 2), B(s + NB).
     // A wave that loads A rows waits for everything (A1 lands right behind A0), one that
     // does not only for B0.
+    // In the middle of step s the wave needs its loads of B(s + 1); issued after them are
+    // (NB - 1) halves of A stages and (NB - 2) B stages, of which the A half of step s - 2 must
+    // have landed as well (the next A stage's first rows): at most 4 groups of 4 may stay out.
+    constexpr int kMidWait = LA ? (4 * (2 * NB - 3) < 16 ? 4 * (2 * NB - 3) : 16) : 4 * (NB - 2);
     fill_a(0); fill_a(1);
-    wait_vm_lgkm0<LA ? 0 : 12>();
+    wait_vm_lgkm0<LA ? 0 : 4 * (NB - 1)>();
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
@@ -589,7 +627,7 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p)
         const int bbuf_n = bbuf + 1 == NB ? 0 : bbuf + 1;
         half(mul_c, la_c, yes{}, fa0, fb0, fa1, fb1, aoff[1] + abuf * 2048, boff0 + bbuf * 1024 + 64,
              abuf_i, ta, q0{});
-        wait_vm_lgkm0<LA ? 16 : 8>();
+        wait_vm_lgkm0<kMidWait>();
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
@@ -602,7 +640,7 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p)
         const int bbuf_n = bbuf + 1 == NB ? 0 : bbuf + 1;
         half(mul_c, la_c, yes{}, fa0, fb0, fa1, fb1, aoff[3] + abuf * 2048, boff0 + bbuf * 1024 + 64,
              abuf_i, ta, q4{});
-        wait_vm_lgkm0<LA ? 16 : 8>();
+        wait_vm_lgkm0<kMidWait>();
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
@@ -614,8 +652,146 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p)
     }
     wait_vm_lgkm0<0>();
   };
+  // ---- tiles of nine groups ------------------------------------------------------------------
+  // The same pipeline with 18 MFMAs per unit: behind the 16 of the main 256 rows come two on the
+  // ninth group's fragment FX and two of the B fragments the wave holds anyway (gate / up group
+  // wm of its half in the gate/up phase, groups 2 wm, 2 wm + 1 in the down phase).  FX of the
+  // next unit is read behind the first of them; the wave's one load per 64-k stage of the extra
+  // rows goes behind MFMA 9 of the step half that issues A chunks 0..3.  Every wave of such a
+  // tile loads A rows and all main row groups are full, so there is one form only.
+  auto half_tall = [&](f32x16 (&accx)[2], auto dma_is_a_c, auto xa_c, uint4 (&FA)[4], uint4 (&FB)[4], uint4 (&NA_)[4],
+                       uint4 (&NB_)[4], uint4& FX, uint4& NX, int a0, int b0, int x0, int dbuf,
+                       int dks, auto aq0_c) {
+#pragma unroll
+    for (int m = 0; m < 18; ++m) {
+      if (m < 16) {
+        const int i = m >> 2, j = m & 3;
+        acc[i][j] = mfma32(FA[i], FB[j], acc[i][j]);
+      } else {
+        const int jj = m - 16;
+        const uint4 b_lo = UP ? FB[jj == 0 ? 0 : 2] : FB[jj];       // wm == 0
+        const uint4 b_hi = UP ? FB[jj == 0 ? 1 : 3] : FB[2 + jj];   // wm == 1
+        uint4 bsel;
+        bsel.x = wm ? b_hi.x : b_lo.x;
+        bsel.y = wm ? b_hi.y : b_lo.y;
+        bsel.z = wm ? b_hi.z : b_lo.z;
+        bsel.w = wm ? b_hi.w : b_lo.w;
+        // The ninth group's accumulators live in ordinary VGPRs (the 256 accumulation registers
+        // are taken): the instruction is spelled out so that the allocator cannot move them.
+        // Nothing reads these registers before the same instruction of the next unit, sixteen
+        // matrix instructions later, so no wait states are owed there; the two owed between the
+        // selects that write the B operand and the instruction reading it are spelled out too
+        // (the compiler counts them for the matrix instructions it emits itself, not for this).
+        const bf16x8 fxv = *(const bf16x8*)&FX, bv = *(const bf16x8*)&bsel;
+        asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0"
+                     : "+v"(accx[jj])
+                     : "v"(fxv), "v"(bv));
+      }
+      if (m < 8) read_frag(m, NA_, NB_, a0, b0);
+      if (m == 16) NX = S[x0];
+      if (m >= 8 && m < 16 && (m & 1) == 0) {
+        if (decltype(dma_is_a_c)::value) dma_a(dbuf, decltype(aq0_c)::value + ((m - 8) >> 1), dks);
+        else dma_b(dbuf, (m - 8) >> 1, dks);
+      }
+      if (decltype(xa_c)::value && m == 9) dma_xa(dbuf, dks);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto run_tall = [&](f32x16 (&accx)[2]) {
+    typedef integral_constant<int, 0> q0;
+    typedef integral_constant<int, 4> q4;
+    uint4 fa0[4], fb0[4], fa1[4], fb1[4], fx0, fx1;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) accx[0][r] = accx[1][r] = 0.f;
+    const int nst = nks / 2;  // 64-k stages
+    // issued so far: B0 .. B(NB-1); now A0 X0 A1 X1.  Per pair of steps a wave then issues
+    // A-half, X, B | A-half, B; in the middle of step s it needs B(s + 1), behind which went
+    // (NB - 1) A halves, (NB - 2) B stages and (NB - 1) / 2 rounded either way X loads.  With
+    // NB = 3: two A halves, one B stage and exactly one X load (one of steps s - 1, s is even).
+    static_assert(NB == 3, "the wait count below is worked out for a B ring of three stages");
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int q = 0; q < 8; ++q) dma_a(t, q, min(t, nst - 1));
+      dma_xa(t, min(t, nst - 1));
+    }
+    wait_vm_lgkm0<0>();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int n = 0; n < 8; ++n) read_frag(n, fa0, fb0, aoff[0], boff0);
+    fx0 = S[xoff0 + aoff[0]];
+    int abuf = 0, bbuf = 0;
+    for (int s = 0; s < nks; s += 2) {
+      const int abuf_n = abuf + 1 == NA ? 0 : abuf + 1;
+      const int abuf_i = abuf == 0 ? NA - 1 : abuf - 1;
+      const int ta = min(s / 2 + NA - 1, nst - 1);
+      const int xcur = xoff0 + abuf * kXaStage, xnext = xoff0 + abuf_n * kXaStage;
+      {
+        const int bbuf_n = bbuf + 1 == NB ? 0 : bbuf + 1;
+        half_tall(accx, yes{}, yes{}, fa0, fb0, fa1, fb1, fx0, fx1, aoff[1] + abuf * 2048,
+                  boff0 + bbuf * 1024 + 64, xcur + aoff[1], abuf_i, ta, q0{});
+        wait_vm_lgkm0<13>();
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        half_tall(accx, no{}, no{}, fa1, fb1, fa0, fb0, fx1, fx0, aoff[2] + abuf * 2048,
+                  boff0 + bbuf_n * 1024, xcur + aoff[2], bbuf, min(s + NB, nks - 1), q0{});
+        bbuf = bbuf_n;
+      }
+      {
+        const int bbuf_n = bbuf + 1 == NB ? 0 : bbuf + 1;
+        half_tall(accx, yes{}, no{}, fa0, fb0, fa1, fb1, fx0, fx1, aoff[3] + abuf * 2048,
+                  boff0 + bbuf * 1024 + 64, xcur + aoff[3], abuf_i, ta, q4{});
+        wait_vm_lgkm0<13>();
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        half_tall(accx, no{}, no{}, fa1, fb1, fa0, fb0, fx1, fx0, aoff[0] + abuf_n * 2048,
+                  boff0 + bbuf_n * 1024, xnext + aoff[0], bbuf, min(s + 1 + NB, nks - 1), q0{});
+        bbuf = bbuf_n;
+      }
+      abuf = abuf_n;
+    }
+    wait_vm_lgkm0<0>();
+  };
   const bool loads_a = wave * 64 < rows_here;
-  if (my_rows >= 97) run(integral_constant<int, 2>{}, yes{});
+  if (tall) {
+    f32x16 accx[2];  // rows 256.. x this wave's two column groups
+    run_tall(accx);
+    // a matrix instruction's results may be read by other instructions 18 passes-of-4 later
+    asm volatile("s_nop 15\n\ts_nop 15" : "+v"(accx[0]), "+v"(accx[1])::"memory");
+    if (UP) {  // gate in accx[0], up in accx[1], this wave's 32 x 32 block
+      uint16_t* h = (uint16_t*)p.out;
+      const int n = nb0 * 16 + (2 * wn + wm) * 32 + l32;
+      if (n < p.n_blocks * 16) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int mrow = TM + 8 * (r >> 2) + 4 * kh + (r & 3);
+          if (mrow < rows_here)
+            h[(size_t)(base + tm0 + mrow) * p.out_stride + n] =
+                (uint16_t)bf16_rne_pair(swiglu_fast(accx[0][r], accx[1][r]), 0.f);
+        }
+      }
+    } else {  // column groups 4 wn + 2 wm, + 1 of this wave
+      float* y = (float*)p.out + (size_t)part * p.out_part_stride;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = TM + 8 * (r >> 2) + 4 * kh + (r & 3);
+        if (m >= rows_here) continue;
+        const int pair = p.g.perm[base + tm0 + m];
+        if (p.part_flags && part == 0 && wn == 0 && wm == 0 && l32 == 0)
+          p.part_flags[(size_t)pair * p.n_col_tiles + ct] = (uint8_t)n_parts;
+        float* yr = y + (size_t)pair * p.out_stride;
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj) {
+          const int n = nb0 * 16 + (4 * wn + 2 * wm + jj) * 32 + l32;
+          if (n < p.n_rows) yr[n] = accx[jj][r];
+        }
+      }
+    }
+  } else if (my_rows >= 97) run(integral_constant<int, 2>{}, yes{});
   else if (my_rows > 0) {
     if (loads_a) run(integral_constant<int, 1>{}, yes{});
     else run(integral_constant<int, 1>{}, no{});
@@ -1032,6 +1208,8 @@ hipError_t launch_ffn_up_tiled(const FfnArgs& a, hipStream_t s) {
   p.tile_group = a.tile_group;
   p.tile_m0 = a.tile_m0;
   p.n_tiles = a.n_tiles;
+  p.tile_rows = a.tile_rows;
+  p.tile_li = a.tile_li;
   p.n_col_tiles = (a.gate.n_pad + 127) / 128;
   p.max_parts = 1;
   if (!int8 && p.k_pad % 64 == 0 && p.k_pad >= 128) return launch_tiled_dma<true>(p, a.max_row_tiles, s);
@@ -1060,6 +1238,8 @@ hipError_t launch_ffn_down_tiled(const FfnArgs& a, hipStream_t s) {
   p.tile_group = a.tile_group;
   p.tile_m0 = a.tile_m0;
   p.n_tiles = a.n_tiles;
+  p.tile_rows = a.tile_rows;
+  p.tile_li = a.tile_li;
   p.n_col_tiles = (a.down.n_pad + 255) / 256;
   p.max_parts = 1;
   const bool pipelined = int8 ? p.k_pad >= 128 : (p.k_pad % 64 == 0 && p.k_pad >= 128);

@@ -118,6 +118,7 @@ struct WsView {
   int32_t *idx = nullptr, *counts = nullptr, *offsets = nullptr, *active = nullptr,
           *n_active = nullptr, *perm = nullptr, *inv = nullptr, *blk_counts = nullptr,
           *shared_desc = nullptr, *ident = nullptr, *tile_group = nullptr, *tile_m0 = nullptr,
+          *tile_rows = nullptr, *tile_li = nullptr,
           *s_tile_group = nullptr, *s_tile_m0 = nullptr;
   float *w = nullptr, *sgate = nullptr, *y = nullptr, *ys = nullptr, *logits = nullptr;
   void *h = nullptr, *hs = nullptr;
@@ -342,6 +343,8 @@ size_t ws_layout(const AteniaMoeLayer* L, int T, int y_parts, uint8_t* base, WsV
   const size_t max_tiles = (P + kTileM - 1) / kTileM + L->E;
   t.tile_group = (int32_t*)take(max_tiles * 4);
   t.tile_m0 = (int32_t*)take(max_tiles * 4);
+  t.tile_rows = (int32_t*)take(max_tiles * 4);
+  t.tile_li = (int32_t*)take(max_tiles * 4);
   t.s_tile_group = (int32_t*)take(((size_t)T / kTileM + 1) * 4);
   t.s_tile_m0 = (int32_t*)take(((size_t)T / kTileM + 1) * 4);
   t.ident = (int32_t*)take((size_t)T * 4);
@@ -453,13 +456,26 @@ int ensure_pg_copy(AteniaMoeLayer* L) {
 struct BatchPlan {
   bool routed_streams;  // weight-streaming kernels (decode) instead of the tiled ones
   bool pg_prefill;      // per-group int8 layer running the tiled kernels on its bf16 copy
+  bool tall_tiles;      // row tiles of up to nine 32-row groups (bf16 pipelined kernels only)
 };
+// Tiles of uneven height can be switched off (tuning knob ATENIA_MOE_TALL_TILES=0, read once).
+bool tall_tiles_enabled() {
+  static const bool v = [] {
+    const char* e = getenv("ATENIA_MOE_TALL_TILES");
+    return !(e && atoi(e) == 0);
+  }();
+  return v;
+}
 BatchPlan plan_batch(const AteniaMoeLayer* L, int T) {
   const bool int8w = L->wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
   BatchPlan p;
   p.routed_streams = batch_streams(T, (long long)T * L->k, L->E, int8w ? 32 : 16);
   p.pg_prefill = L->group_size > 0 && !p.routed_streams && L->d_kpad % 64 == 0 &&
                  L->f_kpad % 64 == 0 && (L->fs == 0 || L->fs_kpad % 64 == 0);
+  // both phases of the routed experts on the bf16 pipelined kernel (K a multiple of 64, >= 128)
+  const bool bf16_tiles = L->wdtype == ATENIA_MOE_WEIGHT_BF16 || p.pg_prefill;
+  p.tall_tiles = tall_tiles_enabled() && !p.routed_streams && bf16_tiles && L->d_kpad % 64 == 0 &&
+                 L->d_kpad >= 128 && L->f_kpad % 64 == 0 && L->f_kpad >= 128;
   return p;
 }
 
@@ -557,6 +573,9 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   pa.tile_m0 = V.tile_m0;
   pa.n_tiles = V.shared_desc + 4;
   pa.shared_n_tiles = V.shared_desc + 5;
+  pa.tile_rows = V.tile_rows;
+  pa.tile_li = V.tile_li;
+  pa.max_tile_groups = plan_batch(L, T).tall_tiles ? 9 : 8;
   ra.fuse_permute = last >= kStagePermute ? &pa : nullptr;
   const bool v3 = L->v3_n_group > 0;
   if (v3 || L->E > 31) ra.logits_tmp = V.logits;
@@ -647,6 +666,8 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   fa.tile_group = V.tile_group;
   fa.tile_m0 = V.tile_m0;
   fa.n_tiles = V.shared_desc + 4;
+  fa.tile_rows = V.tile_rows;
+  fa.tile_li = V.tile_li;
   fa.max_row_tiles = (int)(((size_t)T * L->k + kTileM - 1) / kTileM +
                            std::min<long long>(L->E, (long long)T * L->k));
   const bool split_tail = tiled && tiled_down_splits_tail(fa.down, ffn_dtype);
@@ -683,6 +704,8 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
     fsd.tile_group = V.s_tile_group;
     fsd.tile_m0 = V.s_tile_m0;
     fsd.n_tiles = V.shared_desc + 5;
+    fsd.tile_rows = nullptr;  // the shared expert's rows are cut into whole 256-row tiles
+    fsd.tile_li = nullptr;
     fsd.max_row_tiles = (T + kTileM - 1) / kTileM;
   }
 
@@ -1279,6 +1302,9 @@ int atenia_moe_hip_layer_permute(AteniaMoeLayer* L, const int32_t* idx_host, int
   pa.tile_m0 = nullptr;
   pa.n_tiles = nullptr;
   pa.shared_n_tiles = nullptr;
+  pa.tile_rows = nullptr;
+  pa.tile_li = nullptr;
+  pa.max_tile_groups = 8;
   HIP_TRY(launch_permute(pa, L->stream, nullptr));
   if (hipStreamSynchronize(L->stream) != hipSuccess)
     return fail(ATENIA_MOE_ERR_SYNC, "stream synchronisation failed");

@@ -106,6 +106,11 @@ struct PermuteArgs {
   int32_t* tile_m0;
   int32_t* n_tiles;         // [1]
   int32_t* shared_n_tiles;  // [1] = ceil(T / kTileM) (may be null)
+  // Tiles of uneven height (max_tile_groups == 9, see permute.hip): rows of each tile and its
+  // index inside its expert | (tiles of the expert << 16); may be null when max_tile_groups <= 8.
+  int32_t* tile_rows;
+  int32_t* tile_li;
+  int max_tile_groups;      // 0 / 8: 256-row tiles; 9: tiles of up to 288 rows
 };
 hipError_t launch_permute(const PermuteArgs& a, hipStream_t s, int* n_launches);
 
@@ -138,6 +143,8 @@ struct FfnArgs {
   const int32_t* tile_group;
   const int32_t* tile_m0;
   const int32_t* n_tiles;
+  const int32_t* tile_rows;  // null: every tile is min(kTileM, rows left) high
+  const int32_t* tile_li;    // null: tile i of an expert starts at row i * kTileM
   int max_row_tiles;   // upper bound of *n_tiles (grid sizing)
   // Single-token decode (see launch_ffn_down_decode1): routing weights [k], layer output [d]
   // and optional residual [d] of the one token; the down launch then also does the combine.

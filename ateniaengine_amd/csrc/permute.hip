@@ -61,7 +61,32 @@ struct TileOut {
   int32_t* tile_m0;
   int32_t* n_tiles;
   int32_t* shared_n_tiles;
+  int32_t* tile_rows;  // rows of each tile (may be null)
+  int32_t* tile_li;    // index of the tile inside its expert | (tiles of the expert << 16) (may be null)
+  int max_groups;      // 32-row groups a tile may hold: 8 (256-row tiles) or 9
 };
+
+// Row tiles of an expert with c rows.  max_groups == 8: whole 256-row tiles and one tile with
+// the rest.  max_groups == 9: the expert's 32-row groups are dealt evenly over as few tiles as
+// hold them, so that a rest of up to 32 rows per tile rides in a tile of nine groups instead of
+// becoming a tile of its own (which would stream a whole weight panel for a handful of rows).
+__device__ inline int expert_tiles(int c, int max_groups) {
+  if (max_groups <= 8) return (c + kTileM - 1) / kTileM;
+  const int G = (c + 31) >> 5;
+  return (G + max_groups - 1) / max_groups;
+}
+__device__ inline void expert_tile(int c, int max_groups, int nt, int i, int& m0, int& rows) {
+  if (max_groups <= 8) {
+    m0 = i * kTileM;
+    rows = min(kTileM, c - m0);
+    return;
+  }
+  const int G = (c + 31) >> 5;
+  const int q = G / nt, r = G - q * nt;          // the first r tiles hold q + 1 groups
+  const int g0 = i * q + min(i, r);
+  m0 = g0 * 32;
+  rows = min((q + (i < r ? 1 : 0)) * 32, c - m0);
+}
 
 // counts -> offsets / active list / row-tile list.  Block-cooperative: every thread of the
 // block calls it (barriers inside), thread e owns expert e.  Three prefix sums over the experts
@@ -74,7 +99,7 @@ __device__ void finish_offsets(int E, const int32_t* counts, int32_t* offsets, i
   const bool mine = tid < E;
   const int c = mine ? counts[tid] : 0;
   const int a = c > 0 ? 1 : 0;
-  const int nt = to.tile_group ? (c + kTileM - 1) / kTileM : 0;
+  const int nt = to.tile_group ? expert_tiles(c, to.max_groups) : 0;
   if (tid < kMaxRouterRows) {
     sRows[tid] = c;
     sAct[tid] = a;
@@ -101,8 +126,12 @@ __device__ void finish_offsets(int E, const int32_t* counts, int32_t* offsets, i
     if (a) active[sAct[tid] - 1] = tid;
     const int t0 = sTiles[tid] - nt;
     for (int i = 0; i < nt; ++i) {
+      int m0, rows;
+      expert_tile(c, to.max_groups, nt, i, m0, rows);
       to.tile_group[t0 + i] = tid;
-      to.tile_m0[t0 + i] = i * kTileM;
+      to.tile_m0[t0 + i] = m0;
+      if (to.tile_rows) to.tile_rows[t0 + i] = rows;
+      if (to.tile_li) to.tile_li[t0 + i] = i | (nt << 16);
     }
   }
   if (tid == 0) {
@@ -242,7 +271,8 @@ __global__ void fill_i32_kernel(int32_t* p, int n, int32_t v, int32_t step) {
 hipError_t launch_permute(const PermuteArgs& a, hipStream_t s, int* n_launches) {
   const int P = a.T * a.k, E = a.E;
   if (P <= 0) return hipErrorInvalidValue;
-  TileOut to{a.tile_group, a.tile_m0, a.n_tiles, a.shared_n_tiles};
+  TileOut to{a.tile_group, a.tile_m0, a.n_tiles, a.shared_n_tiles, a.tile_rows, a.tile_li,
+             a.max_tile_groups > 0 ? a.max_tile_groups : 8};
   if (P <= kPermuteBlock) {
     size_t sm = ((size_t)kWaves * E + E + E + 1) * sizeof(int32_t);
     permute_single_kernel<<<1, kPermuteBlock, sm, s>>>(a.idx, P, E, a.T, a.counts, a.offsets,

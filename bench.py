@@ -356,7 +356,8 @@ def main():
     if a.tokens <= 0:
         a.tokens = max(cfg["sweep"])
     decode_ts = [int(t) for t in a.decode_tokens.split(",") if t]
-    decode_ts = [t for t in decode_ts if t != a.tokens and (t in cfg["sweep"] or a.decode_tokens != "1,16")]
+    decode_ts = [t for t in decode_ts if t > 0 and t != a.tokens and
+                 (t in cfg["sweep"] or a.decode_tokens != "1,16")]
     if a.sweep == "all":
         a.sweep = ",".join(str(t) for t in cfg["sweep"] if t != a.tokens and t not in decode_ts)
     router, gate, up, down, shared = make_weights(torch, np, a.seed, f32=f32w)
@@ -447,9 +448,23 @@ def main():
         for _ in range(a.host_steps):
             layer.forward(xh)
         host_ms = (time.perf_counter() - t0) * 1e3 / a.host_steps
-        host = dict(tokens=a.tokens, forward_host_ms=host_ms, tokens_per_s=a.tokens / (host_ms * 1e-3),
+        # the same entry point when the caller's buffers are page-locked (hipHostMalloc /
+        # torch pin_memory): the copies then run as direct DMA
+        xp = torch.empty((a.tokens, D_MODEL), dtype=torch.float32, pin_memory=True)
+        op = torch.empty((a.tokens, D_MODEL), dtype=torch.float32, pin_memory=True)
+        xp.copy_(torch.from_numpy(xh))
+        call = lambda: capi._check(capi.lib().atenia_moe_hip_layer_forward(
+            layer._h, xp.data_ptr(), a.tokens, op.data_ptr()))
+        call()
+        t0 = time.perf_counter()
+        for _ in range(a.host_steps):
+            call()
+        pinned_ms = (time.perf_counter() - t0) * 1e3 / a.host_steps
+        host = dict(tokens=a.tokens, forward_host_ms=host_ms, forward_host_pinned_ms=pinned_ms,
+                    tokens_per_s=a.tokens / (host_ms * 1e-3),
                     host_bytes_moved=2.0 * a.tokens * D_MODEL * 4,
-                    note="atenia_moe_hip_layer_forward: pageable host buffers in and out, synchronous")
+                    note="atenia_moe_hip_layer_forward, synchronous, [T*d] f32 in and out: "
+                         "pageable caller buffers / page-locked caller buffers")
 
     cpu = None
     parity = None

@@ -88,25 +88,28 @@ def traffic(fetch_db, write_db, config, maps, copy_bytes):
     w_rows, w_unit = per_kernel(write_db, "WRITE_SIZE")
     print(f"# calibration: a {copy_bytes} byte device copy reads FETCH_SIZE x {f_unit:.1f} B and "
           f"WRITE_SIZE x {w_unit:.1f} B per unit")
-    for m in maps:
-        tokens, rest = m.split(":", 1)
-        stage, pattern = rest.split("=", 1)
+    def pick(rows, pattern):
         grid = None
         if "@" in pattern:  # <substring>@gx,gy,gz picks one launch shape of the kernel
             pattern, g = pattern.rsplit("@", 1)
             grid = tuple(int(v) for v in g.split(","))
-        fr = [r for r in f_rows if pattern in short(r[0]) and (grid is None or r[1:4] == grid)]
-        wr = [r for r in w_rows if pattern in short(r[0]) and (grid is None or r[1:4] == grid)]
-        if not fr or not wr:
-            sys.exit(f"no dispatch matches {pattern!r}")
-        # the launch with the most fetched bytes among the matches (a pattern may match the
-        # same kernel at several batch sizes; give a tighter pattern or grid to separate them)
-        f = max(fr, key=lambda r: r[6])
-        w = [r for r in wr if r[1:4] == f[1:4]] or wr
-        w = max(w, key=lambda r: r[6])
-        print(f"# {short(f[0])[:70]} grid {f[1:4]}: read {f[6] * f_unit / 1e9:.3f} GB, "
-              f"written {w[6] * w_unit / 1e9:.3f} GB per launch")
-        print(f"traffic {config} {int(tokens)} {stage} {f[6] * f_unit + w[6] * w_unit:.1f}")
+        pattern = pattern.replace(",_", ", ")  # "<1,_false>" may be written for "<1, false>"
+        hit = [r for r in rows if pattern in short(r[0]) and (grid is None or r[1:4] == grid)]
+        if not hit:
+            sys.exit(f"no dispatch matches {pattern!r} {grid or ''}")
+        # several launch shapes of one kernel match a bare substring: the largest one is meant
+        return max(hit, key=lambda r: r[6])
+
+    for m in maps:
+        tokens, rest = m.split(":", 1)
+        stage, patterns = rest.split("=", 1)
+        total = 0.0
+        for pattern in patterns.split("+"):  # a stage of several launches: their sum
+            f, w = pick(f_rows, pattern), pick(w_rows, pattern)
+            print(f"# {short(f[0])[:70]} grid {f[1:4]}: read {f[6] * f_unit / 1e9:.3f} GB, "
+                  f"written {w[6] * w_unit / 1e9:.3f} GB per launch")
+            total += f[6] * f_unit + w[6] * w_unit
+        print(f"traffic {config} {int(tokens)} {stage} {total:.1f}")
 
 
 def main():
@@ -123,7 +126,7 @@ def main():
     t.add_argument("write_db")
     t.add_argument("--config", required=True)
     t.add_argument("--map", action="append", default=[], required=True,
-                   help="<tokens>:<stage>=<substring of the kernel name>[@gx,gy,gz]")
+                   help="<tokens>:<stage>=<substring of the kernel name>[@gx,gy,gz][+<another launch>...]")
     t.add_argument("--copy-bytes", type=float, default=float(1 << 30))
     a = ap.parse_args()
     if a.cmd == "kernels":

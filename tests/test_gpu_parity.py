@@ -288,6 +288,35 @@ def test_layer_forward_skewed_load(ora, wd):
         assert counts.max() > 600 and (counts < 40).any()
 
 
+def _tiles(c, max_groups):
+    g = -(-c // 32)
+    return -(-c // 256) if max_groups == 8 else -(-g // max_groups)
+
+
+@pytest.mark.parametrize("T", [540, 1100, 2130])
+@pytest.mark.parametrize("wd", [capi.WEIGHT_BF16, capi.WEIGHT_INT8_W8A16])
+def test_row_tiles_of_nine_groups(ora, wd, T):
+    """Expert loads just above a multiple of 256 rows: the bf16 kernels then cut an expert's rows
+    into tiles of up to nine 32-row groups (257..288 rows ride in one tile) instead of a full tile
+    plus a tile of a few rows; the int8 kernels keep 256-row tiles on the same lists.  Loads of
+    about T / 2 per expert: 270 (one tile of nine groups), 550 (two), 1065 (9 + 8 + 8 + 9 ...)."""
+    E, k, d, f = 4, 2, 128, 256
+    W = S.make_weights(500 + T, E, d, f, router_std=0.05 / np.sqrt(d))
+    oL, gL = S.build_pair(ora, W, k, capi.CONVENTION_ATENIA, wd)
+    with gL:
+        x = S.make_tokens(600 + T, T, d)
+        check_layer(ora, oL, gL, x, TOL_BF16, sample=range(0, T, 7))
+        _, _, counts, _, _ = gL.last_routing(T)
+        assert any(_tiles(int(c), 9) < _tiles(int(c), 8) for c in counts), counts
+        # per-expert outputs of the rows that ride in the ninth group, against the f64 reference
+        y, _ = gL.last_expert_outputs(T)
+        idx, *_ = gL.last_routing(T)
+        for t in (T - 1, T - 3, T - 40):
+            for s_, e in enumerate(idx[t]):
+                ref = ora.expert_forward_f64(oL.w_gate[e], oL.w_up[e], oL.w_down[e], x[t])
+                assert S.rel_err(y[t, s_], ref) <= TOL_BF16_TOY
+
+
 def test_f32_path_matches_certified_cpu_path_closely(ora):
     """f32 weights: the GPU keeps the reference's cast sequence, so outputs sit within a few
     f32 ulps of the certified CPU path, far inside the 1e-5 bar."""
