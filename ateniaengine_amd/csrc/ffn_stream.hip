@@ -41,6 +41,7 @@ struct StreamParams {
   void* out;            // up: h bf16 [rows, out_stride]; down: y f32 [pairs, out_stride]
   int out_stride;
   GroupDesc g;
+  InlineSelect sel;     // gate/up launch of a single token that routes it itself (logits != null)
 };
 
 __device__ inline uint16_t bf16_rne(float f) {
@@ -98,7 +99,9 @@ __device__ inline f32x4 mfma(bf16x8 a, bf16x8 b, f32x4 c) {
 // S  : adjacent 16-row strips per workgroup (1 or 2).  With two, a wave multiplies the token
 //      rows it loaded with the blocks of both strips, which halves the activation traffic from
 //      L2 per weight byte -- what the streaming rate falls with once an expert has more than 16 rows.
-template <int MT, bool INT8, bool UP, int WAVES, bool PG, int S = 1>
+// SEL : single-token gate/up launch that also routes the token (p.sel); a form of its own
+//       because the f64 softmax doubles the register count of the whole kernel
+template <int MT, bool INT8, bool UP, int WAVES, bool PG, int S = 1, bool SEL = false>
 __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p_routed,
                                                                 StreamParams p_shared,
                                                                 int shared_y) {
@@ -107,10 +110,30 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p_r
   const StreamParams& p = sh ? p_shared : p_routed;
   if ((int)blockIdx.x * 16 * S >= p.n_pad) return;  // the grid spans the wider of the two
   const int u = sh ? 0 : blockIdx.y;
-  if (u >= *p.g.n_active) return;
-  const int e = p.g.active[u];
-  const int base = p.g.offsets[e];
-  const int cnt = p.g.offsets[e + 1] - base;
+  int e, base, cnt;
+  if (SEL && !sh) {
+    // One token whose routing is still open: every wave derives it from the logits (the same
+    // bits in all of them), group u is the u-th selected expert, and one wave of the launch
+    // writes routing and grouping down for the launches that follow.
+    const int ln = threadIdx.x & 63;
+    const WaveRouting wr = wave_softmax_topk(p.sel.logits, p.sel.E, p.sel.k, p.sel.renorm, ln);
+    if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x < 64)
+      wave_write_routing(p.sel, wr, ln);
+    e = wave_selected_expert(wr.mask, u);
+    if (e < 0 || u >= p.sel.k) return;
+    base = u;
+    cnt = 1;
+  } else if (p.g.idx1) {  // one token: group u is its u-th expert, row u
+    if (u >= p.g.pair_div) return;
+    e = p.g.idx1[u];
+    base = u;
+    cnt = 1;
+  } else {
+    if (u >= *p.g.n_active) return;
+    e = p.g.active[u];
+    base = p.g.offsets[e];
+    cnt = p.g.offsets[e + 1] - base;
+  }
   const int m0 = blockIdx.z * 16 * MT;
   if (m0 >= cnt) return;
   // 16-row tiles of this slice that hold rows.  The others are not loaded: their A registers
@@ -187,7 +210,7 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p_r
     int pos = m0 + 16 * i + mm;
     if (pos >= cnt) pos = m0;
     if (UP) {
-      int pair = p.g.perm[base + pos];
+      int pair = p.g.idx1 ? base + pos : p.g.perm[base + pos];
       arow[i] = p.a + (size_t)(pair / p.g.pair_div) * p.a_stride + (KB / 4) * kq;
     } else {
       arow[i] = p.a + (size_t)(base + pos) * p.a_stride + (KB / 4) * kq;
@@ -327,7 +350,7 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p_r
           float h = (g / (1.f + __expf(-g))) * uu;
           ((uint16_t*)p.out)[(size_t)(base + pos) * p.out_stride + n] = bf16_rne(h);
         } else if (n < p.n_rows) {
-          int pair = p.g.perm[base + pos];
+          int pair = p.g.idx1 ? base + pos : p.g.perm[base + pos];
           ((float*)p.out)[(size_t)pair * p.out_stride + n] = acc[0][t][i][r] * sa;
         }
       }
@@ -357,9 +380,9 @@ __global__ __launch_bounds__(1024) void ffn_down_decode1_kernel(StreamParams p, 
   constexpr int KB = INT8 ? kKbInt8 : kKbBf16;
   __shared__ float red[16][16];
   float partial = 0.f;
-  if (j < k && j < *p.g.n_active) {  // uniform per wave
-    const int e = p.g.active[j];
-    const int base = p.g.offsets[e];
+  if (j < k && (p.g.idx1 || j < *p.g.n_active)) {  // uniform per wave
+    const int e = p.g.idx1 ? p.g.idx1[j] : p.g.active[j];
+    const int base = p.g.idx1 ? j : p.g.offsets[e];
     const int kb_per = (p.nkb + KS - 1) / KS;
     const int kb0 = slice * kb_per;
     const int kb1 = min(p.nkb, kb0 + kb_per);
@@ -419,19 +442,147 @@ __global__ __launch_bounds__(1024) void ffn_down_decode1_kernel(StreamParams p, 
   const int n = nb * 16 + mm;
   if (n >= p.n_rows) return;
   float o = 0.f;
-  const int n_active = *p.g.n_active;
+  const int n_active = p.g.idx1 ? k : *p.g.n_active;
   for (int jj = 0; jj < k && jj < n_active; ++jj) {
     float y = red[jj * KS][mm];
 #pragma unroll
     for (int sl = 1; sl < KS; ++sl) y += red[jj * KS + sl][mm];
-    const int e = p.g.active[jj];
+    const int e = p.g.idx1 ? p.g.idx1[jj] : p.g.active[jj];
     if (INT8) y = y * p.sa[(size_t)e * p.n_rows + n];
-    const int pair = p.g.perm[p.g.offsets[e]];
+    const int pair = p.g.idx1 ? jj : p.g.perm[p.g.offsets[e]];
     ((float*)p.out)[(size_t)pair * p.out_stride + n] = y;
     // The product must be rounded before it is added: an opaque multiply keeps the compiler
     // (-ffp-contract=fast in this file) from fusing it into an FMA.
     float prod;
     asm volatile("v_mul_f32 %0, %1, %2" : "=v"(prod) : "v"(w[pair]), "v"(y));
+    o = o + prod;
+  }
+  if (residual) o = residual[n] + o;
+  out[n] = o;
+}
+
+// Down projection + combine for ONE token, any k with a shared expert or without: the general
+// form of the kernel above.  A workgroup owns a 16-row strip of W_d of every expert of the
+// token and of the shared expert; its waves are dealt out as sr K slices per routed expert and
+// ss slices of the shared one (k sr + ss <= 16, chosen by the host so that the slices are about
+// equally long: the shared expert is usually several times as wide).  Partial sums meet in LDS
+// in slice order, lanes 0..15 finish out[n] = sum_j w_j y_j[n] + s y_shared[n] (+ residual) with
+// the combine kernel's arithmetic and order (src/moe/sparse.rs:226-233; shared expert and
+// residual as in combine.hip), and y / y_shared are stored as the separate launches store them.
+// One launch instead of three (routed down, shared down, combine).  With fewer strips than
+// compute units (d = 2048: 128) every strip is shared by two workgroups of eight rows each.
+//
+// A slice is short here (22 blocks on the Qwen1.5-MoE and DeepSeek-MoE shapes), so the launch
+// is a chain of memory round trips rather than a stream: a wave therefore requests up to kChunk
+// weight blocks at once (all of its slice, usually) and the h rows are staged in LDS by the whole
+// workgroup meanwhile (stage_h; needs idx1), instead of two small batches in turn with the h
+// pieces fetched per lane.
+template <bool INT8>
+__global__ __launch_bounds__(1024) void ffn_down_combine1_kernel(
+    StreamParams p, StreamParams ps, int k, int sr, int ss, int halves, int stage_h,
+    const float* __restrict__ w, const float* __restrict__ sgate, const float* residual,
+    float* out) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t sH[];  // [k][K routed] [K shared]
+  const int nb = blockIdx.x / halves;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int kq = lane >> 4, mm = lane & 15;
+  // halves == 2: the workgroup computes rows 8 h .. 8 h + 7 of the strip only and its lanes load
+  // just those rows of every weight block (four full 128-byte lines of the block's eight).
+  const bool lane_on = halves == 1 || (mm >> 3) == (int)(blockIdx.x - nb * halves);
+  constexpr int KB = INT8 ? kKbInt8 : kKbBf16;
+  constexpr int AV = INT8 ? 2 : 1;
+  constexpr int kChunk = INT8 ? 11 : 22;  // weight blocks a wave requests at once
+  __shared__ float red[16][16];
+  const int routed_waves = k * sr;
+  const bool is_shared = wave >= routed_waves;
+  const int j = is_shared ? 0 : wave / sr;
+  const int slice = is_shared ? wave - routed_waves : wave - j * sr;
+  const int n_slices = is_shared ? ss : sr;
+  const bool live = is_shared || p.g.idx1 || j < *p.g.n_active;  // uniform per wave
+  const StreamParams& q = is_shared ? ps : p;
+  const int kb_per = (q.nkb + n_slices - 1) / n_slices;
+  const int kb0 = slice * kb_per;
+  const int kb1 = live ? min(q.nkb, kb0 + kb_per) : kb0;
+  int e = 0, base = 0;
+  if (live && !is_shared) {
+    e = p.g.idx1 ? p.g.idx1[j] : p.g.active[j];
+    base = p.g.idx1 ? j : p.g.offsets[e];
+  }
+  const uint4* pa = q.wa + (size_t)e * q.w_stride_u4 + (size_t)nb * q.nkb * 64 + lane;
+  uint4 wreg[kChunk];
+  auto load_w = [&](int kb) {
+#pragma unroll
+    for (int u = 0; u < kChunk; ++u)
+      wreg[u] = (lane_on && kb + u < kb1) ? load_stream(pa + (size_t)(kb + u) * 64)
+                                          : uint4{0u, 0u, 0u, 0u};
+  };
+  load_w(kb0);
+  // h rows into LDS: row j of the routed experts (K = p.nkb * KB each), then the shared one.
+  const int kr = p.nkb * KB, ksh = ss > 0 ? ps.nkb * KB : 0;
+  if (stage_h) {
+    const int cr = kr / 8, total = k * cr + ksh / 8;  // 16-byte pieces
+    for (int c = threadIdx.x; c < total; c += blockDim.x) {
+      const uint4* src;
+      if (c < k * cr) {
+        const int row = c / cr;
+        src = (const uint4*)(p.a + (size_t)row * p.a_stride) + (c - row * cr);
+      } else {
+        src = (const uint4*)ps.a + (c - k * cr);
+      }
+      ((uint4*)sH)[c] = *src;
+    }
+    __syncthreads();
+  }
+  const uint16_t* xrow = stage_h ? sH + (is_shared ? k * kr : j * kr) + (KB / 4) * kq
+                                 : q.a + (size_t)base * q.a_stride + (KB / 4) * kq;
+  f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int kb = kb0; kb < kb1; kb += kChunk) {
+    if (kb > kb0) load_w(kb);
+#pragma unroll
+    for (int u = 0; u < kChunk; ++u) {
+      if (kb + u < kb1) {
+        const uint4* xp = (const uint4*)(xrow + (size_t)(kb + u) * KB);
+        if (INT8) {
+          bf16x8 al, ah;
+          widen_i8x16(wreg[u], al, ah);
+          uint4 x0 = xp[0], x1 = xp[AV - 1];
+          acc = mfma(*(bf16x8*)&x0, al, acc);
+          acc = mfma(*(bf16x8*)&x1, ah, acc);
+        } else {
+          acc = mfma(xp[0], wreg[u], acc);
+        }
+      }
+    }
+  }
+  // D layout: lanes 0..15 (kq == 0), element 0 = row 0, column mm
+  if (kq == 0) red[wave][mm] = live ? acc[0] : 0.f;
+  __syncthreads();
+  if (threadIdx.x >= 16 || !lane_on) return;
+  const int n = nb * 16 + mm;
+  if (n >= p.n_rows) return;
+  float o = 0.f;
+  const int n_active = p.g.idx1 ? k : *p.g.n_active;
+  for (int jj = 0; jj < k && jj < n_active; ++jj) {
+    float y = red[jj * sr][mm];
+    for (int sl = 1; sl < sr; ++sl) y += red[jj * sr + sl][mm];
+    const int ee = p.g.idx1 ? p.g.idx1[jj] : p.g.active[jj];
+    if (INT8) y = y * p.sa[(size_t)ee * p.n_rows + n];
+    const int pair = p.g.idx1 ? jj : p.g.perm[p.g.offsets[ee]];
+    ((float*)p.out)[(size_t)pair * p.out_stride + n] = y;
+    // The product must be rounded before it is added: an opaque multiply keeps the compiler
+    // (-ffp-contract=fast in this file) from fusing it into an FMA.
+    float prod;
+    asm volatile("v_mul_f32 %0, %1, %2" : "=v"(prod) : "v"(w[pair]), "v"(y));
+    o = o + prod;
+  }
+  if (ss > 0) {
+    float y = red[routed_waves][mm];
+    for (int sl = 1; sl < ss; ++sl) y += red[routed_waves + sl][mm];
+    if (INT8) y = y * ps.sa[n];
+    ((float*)ps.out)[n] = y;
+    const float sc = sgate ? sgate[0] : 1.0f;
+    float prod;
+    asm volatile("v_mul_f32 %0, %1, %2" : "=v"(prod) : "v"(sc), "v"(y));
     o = o + prod;
   }
   if (residual) o = residual[n] + o;
@@ -461,6 +612,8 @@ hipError_t launch_stream(const StreamParams& p, int n_groups, int rows_max, hipS
   if (INT8 && p.group_blocks > 0) {
     if (mt == 1 && two)
       ffn_stream_kernel<1, INT8, UP, W, INT8, 2><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
+    else if (mt == 1 && UP && p.sel.logits)
+      ffn_stream_kernel<1, INT8, UP, W, INT8, 1, UP><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
     else if (mt == 1)
       ffn_stream_kernel<1, INT8, UP, W, INT8><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
     else if (two)
@@ -471,6 +624,8 @@ hipError_t launch_stream(const StreamParams& p, int n_groups, int rows_max, hipS
   }
   if (mt == 1 && two)
     ffn_stream_kernel<1, INT8, UP, W, false, 2><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
+  else if (mt == 1 && UP && p.sel.logits)
+    ffn_stream_kernel<1, INT8, UP, W, false, 1, UP><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
   else if (mt == 1)
     ffn_stream_kernel<1, INT8, UP, W, false><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
   else if (two)
@@ -504,6 +659,7 @@ StreamParams stream_params_up(const FfnArgs& a) {
   p.out = a.h;
   p.out_stride = a.h_stride;
   p.g = a.g;
+  p.sel = a.sel;
   return p;
 }
 StreamParams stream_params_down(const FfnArgs& a) {
@@ -524,6 +680,7 @@ StreamParams stream_params_down(const FfnArgs& a) {
   p.out = a.y;
   p.out_stride = a.y_stride;
   p.g = a.g;
+  p.sel = InlineSelect{};
   return p;
 }
 // The shared expert can ride in the routed experts' launch when both stream (no tiles, no f32
@@ -568,21 +725,73 @@ hipError_t launch_ffn_down(const FfnArgs& a, hipStream_t s, const FfnArgs* share
               : launch_stream<false, false>(p, a.n_groups_max, a.rows_max, s, fuse ? &ps : nullptr);
 }
 
-bool ffn_down_decode1_supported(int T, int k, int wdtype, bool tiled, bool shared) {
-  return T == 1 && k >= 1 && k <= 2 && wdtype != ATENIA_MOE_WEIGHT_F32 && !tiled && !shared;
+// Slices per routed expert (sr) and of the shared expert (ss) for the single-token down +
+// combine launch: k sr + ss <= 16 waves, the longest slice as short as possible, then as many
+// waves as possible.  False when the token's experts do not fit 16 waves.
+static bool decode1_slices(int k, int nkb_r, int nkb_s, int* sr_out, int* ss_out) {
+  long best = -1;
+  for (int sr = 1; sr <= 8; ++sr) {
+    for (int ss = nkb_s > 0 ? 1 : 0; ss <= (nkb_s > 0 ? 8 : 0); ++ss) {
+      if (k * sr + ss > 16) continue;
+      const int lr = (nkb_r + sr - 1) / sr, ls = ss ? (nkb_s + ss - 1) / ss : 0;
+      const long cost = (long)(lr > ls ? lr : ls) * 64 - (k * sr + ss);
+      if (best < 0 || cost < best) {
+        best = cost;
+        *sr_out = sr;
+        *ss_out = ss;
+      }
+    }
+  }
+  return best >= 0;
 }
 
-hipError_t launch_ffn_down_decode1(const FfnArgs& a, hipStream_t s) {
+bool ffn_down_decode1_supported(int T, const FfnArgs& a, int k, bool tiled, const FfnArgs* shared) {
+  if (!(T == 1 && k >= 1 && a.wdtype != ATENIA_MOE_WEIGHT_F32 && !tiled &&
+        a.down.group_blocks == 0))
+    return false;
+  if (!shared) return k <= 15;
+  if (shared->wdtype != a.wdtype || shared->use_tiled || shared->down.group_blocks != 0 ||
+      shared->down.n_rows != a.down.n_rows || shared->down.n_pad != a.down.n_pad)
+    return false;
+  int sr, ss;
+  const int kb = a.wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16 ? kKbInt8 : kKbBf16;
+  return decode1_slices(k, a.down.k_pad / kb, shared->down.k_pad / kb, &sr, &ss);
+}
+
+hipError_t launch_ffn_down_decode1(const FfnArgs& a, hipStream_t s, const FfnArgs* shared) {
   const bool int8 = a.wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
   const StreamParams p = stream_params_down(a);
   const dim3 grid(a.down.n_pad / 16);
-  const int threads = 64 * 8 * a.fuse_k;
+  if (!shared && a.fuse_k <= 2) {
+    const int threads = 64 * 8 * a.fuse_k;
+    if (int8)
+      ffn_down_decode1_kernel<true><<<grid, threads, 0, s>>>(p, a.fuse_k, a.fuse_w,
+                                                             a.fuse_residual, a.fuse_out);
+    else
+      ffn_down_decode1_kernel<false><<<grid, threads, 0, s>>>(p, a.fuse_k, a.fuse_w,
+                                                              a.fuse_residual, a.fuse_out);
+    return hipGetLastError();
+  }
+  const StreamParams ps = shared ? stream_params_down(*shared) : p;
+  int sr = 1, ss = 0;
+  if (!decode1_slices(a.fuse_k, p.nkb, shared ? ps.nkb : 0, &sr, &ss)) return hipErrorInvalidValue;
+  const int threads = 64 * (a.fuse_k * sr + ss);
+  const int halves = (int)grid.x * 2 <= (a.n_cus > 0 ? a.n_cus : 256) ? 2 : 1;
+  const dim3 g2(grid.x * halves);
+  // h rows in LDS when the router left the token's experts in idx1 (row j = expert j's h) and
+  // they fit next to the reduction buffer
+  const size_t kb_elems = int8 ? kKbInt8 : kKbBf16;
+  const size_t h_bytes = ((size_t)a.fuse_k * p.nkb + (shared ? ps.nkb : 0)) * kb_elems * 2;
+  const int stage_h = a.g.idx1 != nullptr && h_bytes <= 48 * 1024;
+  const size_t smem = stage_h ? h_bytes : 0;
   if (int8)
-    ffn_down_decode1_kernel<true><<<grid, threads, 0, s>>>(p, a.fuse_k, a.fuse_w, a.fuse_residual,
-                                                           a.fuse_out);
+    ffn_down_combine1_kernel<true><<<g2, threads, smem, s>>>(p, ps, a.fuse_k, sr, ss, halves, stage_h,
+                                                             a.fuse_w, a.fuse_sgate,
+                                                             a.fuse_residual, a.fuse_out);
   else
-    ffn_down_decode1_kernel<false><<<grid, threads, 0, s>>>(p, a.fuse_k, a.fuse_w, a.fuse_residual,
-                                                            a.fuse_out);
+    ffn_down_combine1_kernel<false><<<g2, threads, smem, s>>>(p, ps, a.fuse_k, sr, ss, halves, stage_h,
+                                                              a.fuse_w, a.fuse_sgate,
+                                                              a.fuse_residual, a.fuse_out);
   return hipGetLastError();
 }
 

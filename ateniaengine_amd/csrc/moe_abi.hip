@@ -583,6 +583,11 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
     ra.logits_out = V.logits;
     ra.shared_gate = nullptr;  // the V3 block adds its shared experts ungated
   }
+  // One token through the streaming gate/up launch: that launch can route the token itself from
+  // the logits, so a router launch that spreads its rows need not be followed by a launch that
+  // only selects.
+  ra.defer_select = T == 1 && last >= kStageFfn && !v3 && !f32w && L->E <= 64 &&
+                    plan_batch(L, T).routed_streams;
   int fused = 0;
   if (first <= kStageRouter) {
     HIP_TRY(launch_router(ra, s, &fused));
@@ -647,6 +652,19 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   fa.g.n_active = V.n_active;
   fa.g.perm = V.perm;
   fa.g.pair_div = L->k;
+  fa.g.idx1 = T == 1 && fused ? V.idx : nullptr;
+  if (fused == 2) {  // the router left the logits: the gate/up launch selects and groups
+    fa.sel.logits = V.logits;
+    fa.sel.E = L->E;
+    fa.sel.k = L->k;
+    fa.sel.renorm = ra.renorm;
+    fa.sel.idx = V.idx;
+    fa.sel.w = V.w;
+    fa.sel.status = L->status.as<int32_t>();
+    fa.sel.fg = FusedGrouping{pa.counts, pa.offsets, pa.perm, pa.inv, pa.active, pa.n_active,
+                              pa.shared_offsets, pa.tile_group, pa.tile_m0, pa.n_tiles,
+                              pa.shared_n_tiles};
+  }
   fa.n_groups_max = (int)std::min<long long>(L->E, (long long)T * L->k);
   fa.rows_max = T;
   fa.gate = pg_prefill ? L->gate_b : L->gate;
@@ -680,12 +698,14 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   FfnArgs fsd{};
   if (L->fs > 0) {
     fsd = fa;
+    fsd.sel = InlineSelect{};
     const int32_t* sd = V.shared_desc;
     fsd.g.offsets = sd;
     fsd.g.active = sd + 2;
     fsd.g.n_active = sd + 3;
     fsd.g.perm = V.ident;
     fsd.g.pair_div = 1;
+    fsd.g.idx1 = T == 1 ? sd : nullptr;  // sd[0] = 0: the one group, its one row
     fsd.n_groups_max = 1;
     fsd.rows_max = T;
     fsd.gate = pg_prefill ? L->s_gate_b : L->s_gate;
@@ -721,23 +741,23 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
     }
   }
   tm.mark();  // ev[3]: gate/up done
-  // One token, up to two experts, no shared expert, whole pipeline requested: the down launch
-  // finishes the combine as well (same bits as the two launches, one launch less).
-  const bool fuse1 = first <= kStageFfn && last >= kStageCombine &&
-                     L->group_size == 0 &&
-                     ffn_down_decode1_supported(T, L->k, L->wdtype, tiled, L->fs > 0);
+  // One token, whole pipeline requested: the down launch covers the routed experts and the
+  // shared one and finishes the combine as well (one launch instead of two or three).
+  const bool fuse1 = first <= kStageFfn && last >= kStageCombine && L->group_size == 0 &&
+                     ffn_down_decode1_supported(T, fa, L->k, tiled, L->fs > 0 ? &fsd : nullptr);
   if (first <= kStageFfn) {
     if (fuse1) {
       fa.fuse_w = V.w;
       fa.fuse_out = d_out;
       fa.fuse_residual = d_residual;
+      fa.fuse_sgate = gated ? V.sgate : nullptr;
       fa.fuse_k = L->k;
-      HIP_TRY(launch_ffn_down_decode1(fa, s));
+      HIP_TRY(launch_ffn_down_decode1(fa, s, L->fs > 0 ? &fsd : nullptr));
     } else {
       HIP_TRY(launch_ffn_down(fa, s, fuse_shared_down ? &fsd : nullptr));
     }
     L->launches[3] = 1;
-    if (L->fs > 0 && !fuse_shared_down) {
+    if (L->fs > 0 && !fuse_shared_down && !fuse1) {
       HIP_TRY(launch_ffn_down(fsd, s));
       L->launches[3] = 2;
     }

@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "select_wave.h"
+
 namespace atenia_moe {
 
 // ---- limits ------------------------------------------------------------------------------
@@ -33,6 +35,11 @@ struct GroupDesc {
   const int32_t* n_active;  // [1]
   const int32_t* perm;      // [rows] pair id (token*pair_div + slot) of each grouped row
   int pair_div;             // token = pair id / pair_div
+  // One-token launches whose router also wrote the grouping: the token's experts in ascending
+  // order, [pair_div] entries; group j is then expert idx1[j] with the single row j = pair j.
+  // A kernel that sees it reads one value where the lists above cost three dependent loads.
+  // Null otherwise.
+  const int32_t* idx1;
 };
 
 // One expert projection family as stored on the device.
@@ -73,8 +80,13 @@ struct RouterArgs {
   // scratch [T, E] the launcher may use to split the work of few tokens over more workgroups
   // (null = none)
   float* logits_tmp;
+  // T == 1 only: when the launcher spreads the rows over workgroups (logits to logits_tmp), it
+  // may leave the selection and the grouping to the caller's next launch instead of a small
+  // launch of its own; *fused_permute is then 2.
+  int defer_select;
 };
-// *fused_permute is set to 1 when the launch also produced the expert grouping.
+// *fused_permute is set to 1 when the launch also produced the expert grouping, to 2 when the
+// logits are in logits_tmp and the caller's next launch has to route the token (defer_select).
 hipError_t launch_router(const RouterArgs& a, hipStream_t s, int* fused_permute);
 
 // DeepSeek-V3 routing from raw logits (src/moe/v3_router.rs:206-309).
@@ -151,7 +163,11 @@ struct FfnArgs {
   const float* fuse_w;
   float* fuse_out;
   const float* fuse_residual;
+  const float* fuse_sgate;  // [1] sigmoid gate of the shared expert, or null (weight 1)
   int fuse_k;
+  // Single token whose routing the router launch left undone (RouterArgs::defer_select): the
+  // gate/up launch routes it from the logits; sel.logits == null otherwise.
+  InlineSelect sel;
 };
 bool tiled_supported(const WeightSet& w, int wdtype);
 // True when the tiled down launch for these weights can split the k range of tail tiles.
@@ -165,8 +181,8 @@ hipError_t launch_ffn_down(const FfnArgs& a, hipStream_t s, const FfnArgs* share
 bool ffn_stream_fuses_shared(const FfnArgs& a, const FfnArgs& shared, bool down_phase);
 // One token, at most two experts per token, blocked (bf16 / int8) weights: the down projection
 // of all the token's experts and the weighted combine in one launch.
-bool ffn_down_decode1_supported(int T, int k, int wdtype, bool tiled, bool shared);
-hipError_t launch_ffn_down_decode1(const FfnArgs& a, hipStream_t s);
+bool ffn_down_decode1_supported(int T, const FfnArgs& a, int k, bool tiled, const FfnArgs* shared);
+hipError_t launch_ffn_down_decode1(const FfnArgs& a, hipStream_t s, const FfnArgs* shared);
 
 struct CombineArgs {
   int T, k, d;

@@ -39,7 +39,6 @@ constexpr int kRouterThreads = 256;
 constexpr int kKc = 32;            // columns staged per step
 constexpr int kLd = kKc + 1;       // padded LDS row stride (words)
 constexpr int kTokenThreads = 1024;
-constexpr int kNoLsb = 32767;      // lsb exponent marker of a zero
 
 __device__ inline float load_x(const float* x, size_t i) { return x[i]; }
 __device__ inline float load_x(const uint16_t* x, size_t i) {
@@ -56,6 +55,7 @@ __device__ inline uint16_t f32_to_bf16_rne(float f) {
 
 // Exponent of the lowest set bit of a finite f32 (v = odd * 2^result); kNoLsb for zero,
 // and a hugely negative value for inf/NaN so that no exactness claim survives them.
+constexpr int kNoLsb = 32767;
 __device__ inline int lsb_exponent(float v) {
   uint32_t b = __float_as_uint(v);
   int e = (b >> 23) & 0xff;
@@ -528,12 +528,6 @@ hipError_t dispatch_router_batch(const RouterArgs& a, int R, hipStream_t s) {
   return launch_router_batch<XT, 4, 1, 64>(a, s);
 }
 
-// Outputs of the expert grouping for the single-token case (see permute.hip for the contract).
-struct FusedGrouping {
-  int32_t *counts, *offsets, *perm, *inv, *active, *n_active, *shared_offsets;
-  int32_t *tile_group, *tile_m0, *n_tiles, *shared_n_tiles;
-};
-
 // The expert grouping of ONE token from its selection flags (what kernel 2 would produce).
 // Called by the threads e = 0..E-1 of the workgroup (sel in LDS, already synchronised): thread e
 // counts the selected experts before it and writes its own entries.
@@ -620,47 +614,67 @@ __global__ __launch_bounds__(kTokenThreads) void router_token_kernel(
   float* sLogit = sX + d;                      // [E]
   float* sWt = sLogit + E;                     // [E]
   int32_t* sSel = (int32_t*)(sWt + E);         // [E]
-  int32_t* sBad = sSel + E;                    // [1]
-  int32_t* sPartQ = sBad + 1;                  // [max(R, NW)]
-  int16_t* sLx = (int16_t*)(sPartQ + (R > NW ? R : NW));  // [d]
+  int32_t* sBad = sSel + E;                    // [2]: second look wanted, sequential order wanted
+  int32_t* sNeed = sBad + 2;                   // [R]
+  int32_t* sPartQ = sNeed + R;                 // [max(R, NW)]
 
-  if (tid == 0) *sBad = 0;
+  if (tid < 2) sBad[tid] = 0;
+  // Work items: (row, k slice).  With few rows each row is split over several waves so that
+  // all 16 waves stream the router matrix.  Partial results meet in LDS; under the interval
+  // certificate below their order of addition cannot change what the sum rounds to.
+  const int KS = R >= NW ? 1 : NW / R;              // k slices per row
+  const int slice = ((d + KS - 1) / KS + 3) & ~3;   // multiple of 4 for float4 loads
+  const bool vec_ok = (d & 3) == 0;
+  // The weights of the wave's first item are requested before the token is staged: they do not
+  // depend on it, and at one token per launch the two round trips to memory would otherwise
+  // follow each other.
+  constexpr int kPre = 8;
+  float4 wpre[kPre];
+  const bool pre = vec_ok && wave < R * KS;
+  if (pre) {
+    const int r = wave / KS, ksl = wave - r * KS;
+    const float* wr = row_lo + r < E ? w_router + (size_t)(row_lo + r) * d : gate_vec;
+    const int c_lo = ksl * slice, c_hi = min(d, c_lo + slice);
+#pragma unroll
+    for (int i = 0; i < kPre; ++i) {
+      const int c = c_lo + lane * 4 + i * 256;
+      wpre[i] = c < c_hi ? *(const float4*)(wr + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+  }
   const int c_end = xb ? (d_pad > d ? d_pad : d) : d;
   for (int c = tid; c < c_end; c += kTokenThreads) {
     float v = c < d ? load_x(x, (size_t)t * d + c) : 0.f;
-    if (c < d) {
-      sX[c] = v;
-      sLx[c] = (int16_t)max(lsb_exponent(v), -32000);
-    }
+    if (c < d) sX[c] = v;
     if (xb && blockIdx.y == 0 && c < d_pad) xb[(size_t)t * d_pad + c] = f32_to_bf16_rne(v);
   }
   __syncthreads();
 
-  // Work items: (row, k slice).  With few rows each row is split over several waves so that
-  // all 16 waves stream the router matrix.  Partial results meet in LDS; under the exactness
-  // certificate their order of addition cannot change the sum (or, under the interval
-  // certificate below, cannot change what the sum rounds to).
-  const int KS = R >= NW ? 1 : NW / R;              // k slices per row
-  const int slice = ((d + KS - 1) / KS + 3) & ~3;   // multiple of 4 for float4 loads
-  const bool vec_ok = (d & 3) == 0;
   for (int item = wave; item < R * KS; item += NW) {
     const int r = item / KS, ksl = item - r * KS;
     const float* wr = row_lo + r < E ? w_router + (size_t)(row_lo + r) * d : gate_vec;
     const int c_lo = ksl * slice, c_hi = min(d, c_lo + slice);
     double acc = 0.0, asum = 0.0;
-    int qmin = kNoLsb;
     auto one = [&](float wv, int c) {
       float xv = sX[c];
       double wd = (double)wv, xd = (double)xv;
       acc = fma(wd, xd, acc);
       asum = fma(fabs(wd), fabs(xd), asum);
-      int lx = sLx[c];
-      int lw = lsb_exponent(wv);
-      if (lx != kNoLsb && lw != kNoLsb) qmin = min(qmin, lx + lw);
     };
     if (vec_ok) {
+      int c = c_lo + lane * 4;
+      if (item == wave) {  // the first item: its first kPre steps are in registers already
+#pragma unroll
+        for (int i = 0; i < kPre; ++i, c += 256) {
+          if (c < c_hi) {
+            one(wpre[i].x, c);
+            one(wpre[i].y, c + 1);
+            one(wpre[i].z, c + 2);
+            one(wpre[i].w, c + 3);
+          }
+        }
+      }
 #pragma unroll 4
-      for (int c = c_lo + lane * 4; c < c_hi; c += 256) {
+      for (; c < c_hi; c += 256) {
         float4 w4 = *(const float4*)(wr + c);
         one(w4.x, c);
         one(w4.y, c + 1);
@@ -674,34 +688,29 @@ __global__ __launch_bounds__(kTokenThreads) void router_token_kernel(
     for (int off = 32; off >= 1; off >>= 1) {
       acc += __shfl_xor(acc, off);
       asum += __shfl_xor(asum, off);
-      qmin = min(qmin, __shfl_xor(qmin, off));
     }
     if (lane == 0) {
       sPart[item] = acc;
       sPartA[item] = asum;
-      sPartQ[item] = qmin;
     }
   }
   __syncthreads();
   if (tid < R) {
     double acc = 0.0, asum = 0.0;
-    int qmin = kNoLsb;
     for (int ksl = 0; ksl < KS; ++ksl) {
       acc += sPart[tid * KS + ksl];
       asum += sPartA[tid * KS + ksl];
-      qmin = min(qmin, sPartQ[tid * KS + ksl]);
     }
-    // Exact in every order iff sum|p| < 2^(q+53); asum itself carries a relative error of
-    // at most d * 2^-53, covered by the margin.
-    bool exact = qmin == kNoLsb || (qmin > -2000 && asum * 1.000001 < ldexp(1.0, qmin + 53));
-    if (!exact) {
-      // Second certificate, for operands that are not exact in every order (f32-valued rows):
-      // any order of d exact products summed in f64 lands within g = d * 2^-53 * sum|p| of the
-      // true sum (standard bound, 1 / (1 - d u) absorbed by the margin), so this sum and the
+    bool exact;
+    {
+      // The certificate: any order of d exact products summed in f64 lands within
+      // g = d * 2^-53 * sum|p| of the true sum (standard bound, 1 / (1 - d u) absorbed by the
+      // margin; asum's own relative error of d * 2^-53 likewise), so this sum and the
       // reference's sequential one differ by at most 2 g.  If both ends of [acc - 2g, acc + 2g]
       // round to the same f32 (the same f32 sigmoid for the gate row), the reference's result is
       // that value, whatever its order.  Rounding is monotone; the two extra units of 2^-53
-      // cover the roundings of acc -/+ e themselves.
+      // cover the roundings of acc -/+ e themselves.  About one sum in a thousand sits close
+      // enough to an f32 rounding boundary to fail this; those rows get the second look below.
       const double e = asum * ((double)(2 * d + 4) * 1.1102230246251565e-16) * 1.0001;
       const double lo = acc - e, hi = acc + e;
       if (row_lo + tid < E) {
@@ -713,10 +722,44 @@ __global__ __launch_bounds__(kTokenThreads) void router_token_kernel(
       }
     }
     sAcc[tid] = acc;
-    if (!exact) *sBad = 1;
+    sNeed[tid] = exact ? 0 : 1;
+    if (!exact) {
+      sPartA[tid * KS] = asum;  // this thread's own entries: nobody else reads them
+      sBad[0] = 1;
+    }
   }
   __syncthreads();
-  if (*sBad) {
+  if (sBad[0]) {
+    // Second look, for the flagged rows only: when every product of a row is a multiple of 2^q
+    // and sum|p| < 2^(q+53), every partial sum of every order is exact in f64, so the sum
+    // above IS the reference's sequential one (bf16-valued operands satisfy this).  asum carries
+    // a relative error of at most d * 2^-53, covered by the margin.
+    for (int item = wave; item < R * KS; item += NW) {
+      const int r = item / KS, ksl = item - r * KS;
+      int qmin = kNoLsb;
+      if (sNeed[r]) {
+        const float* wr = row_lo + r < E ? w_router + (size_t)(row_lo + r) * d : gate_vec;
+        const int c_lo = ksl * slice, c_hi = min(d, c_lo + slice);
+        for (int c = c_lo + lane; c < c_hi; c += 64) {
+          const int lx = lsb_exponent(sX[c]), lw = lsb_exponent(wr[c]);
+          if (lx != kNoLsb && lw != kNoLsb) qmin = min(qmin, lx + lw);
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) qmin = min(qmin, __shfl_xor(qmin, off));
+      }
+      if (lane == 0) sPartQ[item] = qmin;
+    }
+    __syncthreads();
+    if (tid < R && sNeed[tid]) {
+      int qmin = kNoLsb;
+      for (int ksl = 0; ksl < KS; ++ksl) qmin = min(qmin, sPartQ[tid * KS + ksl]);
+      const double asum = sPartA[tid * KS];
+      const bool exact = qmin == kNoLsb || (qmin > -2000 && asum * 1.000001 < ldexp(1.0, qmin + 53));
+      if (!exact) sBad[1] = 1;
+    }
+    __syncthreads();
+  }
+  if (sBad[1]) {
     // The reference's own order: one sequential c-ascending f64 sum per row.
     for (int r = tid; r < R; r += kTokenThreads) {
       const float* wr = row_lo + r < E ? w_router + (size_t)(row_lo + r) * d : gate_vec;
@@ -759,8 +802,8 @@ hipError_t launch_router(const RouterArgs& a, hipStream_t s, int* fused_permute)
                         (R <= 64 || (long long)a.T * R * a.d <= (16ll << 20));
   if (token_ok) {
     const size_t np = R > kTokenThreads / 64 ? R : kTokenThreads / 64;
-    size_t smem = ((size_t)R + a.E + 2 * np) * 8 + (size_t)a.d * 4 + (size_t)a.E * 12 + 4 +
-                  np * 4 + (size_t)a.d * 2 + 16;
+    size_t smem = ((size_t)R + a.E + 2 * np) * 8 + (size_t)a.d * 4 + (size_t)a.E * 12 + 8 +
+                  ((size_t)R + np) * 4 + 16;
     if (smem <= 64 * 1024) {
       // Many rows, few tokens: one workgroup per token would stream the whole stacked matrix
       // through a single CU.  The rows are spread over workgroups instead (four rows each, a
@@ -790,6 +833,11 @@ hipError_t launch_router(const RouterArgs& a, hipStream_t s, int* fused_permute)
         router_token_kernel<float><<<grid, kTokenThreads, smem, s>>>(
             (const float*)a.x, a.T, a.d, a.E, a.k, a.renorm, a.w_router, a.router_bias,
             a.shared_gate, a.idx, a.w, a.sgate, a.xb, a.d_pad, a.status, lg, fg_token);
+      if (spread && !a.logits_out && a.defer_select && a.T == 1 && a.E <= 64 && fg.counts) {
+        // the caller's next launch routes the token itself from the logits (select_wave.h)
+        if (fused_permute) *fused_permute = 2;
+        return hipGetLastError();
+      }
       if (spread && !a.logits_out) {
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;

@@ -65,6 +65,7 @@ fn main() {
         .unwrap_or_else(|_| manifest.join("../../ateniaengine_amd/csrc"));
     let header = csrc.join("../../include/atenia_moe_hip.h");
     println!("cargo::rerun-if-changed={}", header.display());
+    println!("cargo::rerun-if-changed={}", csrc.join("select_wave.h").display());
     println!("cargo::rerun-if-changed={}", csrc.join("moe_internal.h").display());
 
     let out = PathBuf::from(env::var("OUT_DIR").unwrap());

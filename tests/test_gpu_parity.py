@@ -410,8 +410,8 @@ def test_packed_gate_up_layout(ora):
         assert a.forward(x).tobytes() == b.forward(x).tobytes()
 
 
-@pytest.mark.parametrize("wd", [capi.WEIGHT_F32, capi.WEIGHT_BF16])
-@pytest.mark.parametrize("T,shared", [(1, False), (37, True), (700, False)])
+@pytest.mark.parametrize("wd", [capi.WEIGHT_F32, capi.WEIGHT_BF16, capi.WEIGHT_INT8_W8A16])
+@pytest.mark.parametrize("T,shared", [(1, False), (1, True), (37, True), (700, False)])
 def test_combine_is_bit_exact_given_expert_outputs(ora, wd, T, shared):
     """src/moe/sparse.rs:87-116, 226-233: out = sum over slots of w * y with the product and the
     sum rounded separately in f32 (an FMA gives other bits), then += the shared expert's row.
