@@ -54,8 +54,9 @@ __device__ inline uint16_t bf16_rne(float f) {
 __device__ inline uint32_t pack_i8_pair(uint32_t w, int sh) {
   float f0 = (float)(int8_t)((w >> sh) & 0xff);
   float f1 = (float)(int8_t)((w >> (sh + 8)) & 0xff);
-  // |q| <= 127 is exact in bf16, so dropping the low 16 bits loses nothing.
-  return (__float_as_uint(f0) >> 16) | (__float_as_uint(f1) & 0xffff0000u);
+  // |q| <= 128 is exact in bf16, so dropping the low 16 bits loses nothing: one byte permute
+  // takes the high halves of both floats (bytes 2, 3 of f0 below bytes 2, 3 of f1).
+  return __builtin_amdgcn_perm(__float_as_uint(f1), __float_as_uint(f0), 0x07060302u);
 }
 __device__ inline void widen_i8x16(uint4 q, bf16x8& lo, bf16x8& hi) {
   uint4 l, h;
@@ -492,7 +493,10 @@ __global__ __launch_bounds__(1024) void ffn_down_combine1_kernel(
   constexpr int KB = INT8 ? kKbInt8 : kKbBf16;
   constexpr int AV = INT8 ? 2 : 1;
   constexpr int kChunk = INT8 ? 11 : 22;  // weight blocks a wave requests at once
-  __shared__ float red[16][16];
+  // Every expert's K range is cut into the same eight slices as in the separate down launch
+  // (eight waves per strip there) and the eight partial sums are added in the same order, so y
+  // has the bits of that launch; a wave here takes 8 / sr (8 / ss) consecutive slices.
+  __shared__ float red[16 * 8][16];
   const int routed_waves = k * sr;
   const bool is_shared = wave >= routed_waves;
   const int j = is_shared ? 0 : wave / sr;
@@ -500,9 +504,11 @@ __global__ __launch_bounds__(1024) void ffn_down_combine1_kernel(
   const int n_slices = is_shared ? ss : sr;
   const bool live = is_shared || p.g.idx1 || j < *p.g.n_active;  // uniform per wave
   const StreamParams& q = is_shared ? ps : p;
-  const int kb_per = (q.nkb + n_slices - 1) / n_slices;
-  const int kb0 = slice * kb_per;
-  const int kb1 = live ? min(q.nkb, kb0 + kb_per) : kb0;
+  const int subs = 8 / n_slices;
+  const int kb8 = (q.nkb + 7) / 8;
+  const int sub0 = slice * subs;
+  const int kb0 = min(q.nkb, sub0 * kb8);
+  const int kb1 = live ? min(q.nkb, (sub0 + subs) * kb8) : kb0;
   int e = 0, base = 0;
   if (live && !is_shared) {
     e = p.g.idx1 ? p.g.idx1[j] : p.g.active[j];
@@ -536,11 +542,21 @@ __global__ __launch_bounds__(1024) void ffn_down_combine1_kernel(
   const uint16_t* xrow = stage_h ? sH + (is_shared ? k * kr : j * kr) + (KB / 4) * kq
                                  : q.a + (size_t)base * q.a_stride + (KB / 4) * kq;
   f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int unit = is_shared ? k : j;
+  int sub = sub0;
+  int bound = min(q.nkb, (sub0 + 1) * kb8);  // first block of the next slice
+  auto flush = [&] {  // D layout: lanes 0..15 (kq == 0), element 0 = row 0, column mm
+    if (kq == 0) red[unit * 8 + sub][mm] = acc[0];
+    acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    ++sub;
+    bound = min(q.nkb, bound + kb8);
+  };
   for (int kb = kb0; kb < kb1; kb += kChunk) {
     if (kb > kb0) load_w(kb);
 #pragma unroll
     for (int u = 0; u < kChunk; ++u) {
       if (kb + u < kb1) {
+        if (kb + u == bound) flush();
         const uint4* xp = (const uint4*)(xrow + (size_t)(kb + u) * KB);
         if (INT8) {
           bf16x8 al, ah;
@@ -554,8 +570,8 @@ __global__ __launch_bounds__(1024) void ffn_down_combine1_kernel(
       }
     }
   }
-  // D layout: lanes 0..15 (kq == 0), element 0 = row 0, column mm
-  if (kq == 0) red[wave][mm] = live ? acc[0] : 0.f;
+  if (live)
+    while (sub < sub0 + subs) flush();  // the last slice, and empty ones (a short K) as zeros
   __syncthreads();
   if (threadIdx.x >= 16 || !lane_on) return;
   const int n = nb * 16 + mm;
@@ -563,8 +579,9 @@ __global__ __launch_bounds__(1024) void ffn_down_combine1_kernel(
   float o = 0.f;
   const int n_active = p.g.idx1 ? k : *p.g.n_active;
   for (int jj = 0; jj < k && jj < n_active; ++jj) {
-    float y = red[jj * sr][mm];
-    for (int sl = 1; sl < sr; ++sl) y += red[jj * sr + sl][mm];
+    float y = red[jj * 8][mm];
+#pragma unroll
+    for (int sl = 1; sl < 8; ++sl) y += red[jj * 8 + sl][mm];
     const int ee = p.g.idx1 ? p.g.idx1[jj] : p.g.active[jj];
     if (INT8) y = y * p.sa[(size_t)ee * p.n_rows + n];
     const int pair = p.g.idx1 ? jj : p.g.perm[p.g.offsets[ee]];
@@ -576,8 +593,9 @@ __global__ __launch_bounds__(1024) void ffn_down_combine1_kernel(
     o = o + prod;
   }
   if (ss > 0) {
-    float y = red[routed_waves][mm];
-    for (int sl = 1; sl < ss; ++sl) y += red[routed_waves + sl][mm];
+    float y = red[k * 8][mm];
+#pragma unroll
+    for (int sl = 1; sl < 8; ++sl) y += red[k * 8 + sl][mm];
     if (INT8) y = y * ps.sa[n];
     ((float*)ps.out)[n] = y;
     const float sc = sgate ? sgate[0] : 1.0f;
@@ -725,13 +743,14 @@ hipError_t launch_ffn_down(const FfnArgs& a, hipStream_t s, const FfnArgs* share
               : launch_stream<false, false>(p, a.n_groups_max, a.rows_max, s, fuse ? &ps : nullptr);
 }
 
-// Slices per routed expert (sr) and of the shared expert (ss) for the single-token down +
-// combine launch: k sr + ss <= 16 waves, the longest slice as short as possible, then as many
-// waves as possible.  False when the token's experts do not fit 16 waves.
+// Waves per routed expert (sr) and of the shared expert (ss) for the single-token down +
+// combine launch: powers of two up to 8 (a wave takes 8 / sr of the eight K slices),
+// k sr + ss <= 16 waves, the longest share as short as possible, then as many waves as
+// possible.  False when the token's experts do not fit 16 waves.
 static bool decode1_slices(int k, int nkb_r, int nkb_s, int* sr_out, int* ss_out) {
   long best = -1;
-  for (int sr = 1; sr <= 8; ++sr) {
-    for (int ss = nkb_s > 0 ? 1 : 0; ss <= (nkb_s > 0 ? 8 : 0); ++ss) {
+  for (int sr = 1; sr <= 8; sr *= 2) {
+    for (int ss = nkb_s > 0 ? 1 : 0; ss <= (nkb_s > 0 ? 8 : 0); ss = ss ? ss * 2 : 9) {
       if (k * sr + ss > 16) continue;
       const int lr = (nkb_r + sr - 1) / sr, ls = ss ? (nkb_s + ss - 1) / ss : 0;
       const long cost = (long)(lr > ls ? lr : ls) * 64 - (k * sr + ss);

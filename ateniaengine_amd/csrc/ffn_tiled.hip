@@ -102,7 +102,9 @@ __device__ inline float swiglu_fast(float g, float u) {
 __device__ inline uint32_t pack_i8_pair(uint32_t w, int sh) {
   float f0 = (float)(int8_t)((w >> sh) & 0xff);
   float f1 = (float)(int8_t)((w >> (sh + 8)) & 0xff);
-  return (__float_as_uint(f0) >> 16) | (__float_as_uint(f1) & 0xffff0000u);
+  // |q| <= 128 is exact in bf16, so dropping the low 16 bits loses nothing: one byte permute
+  // takes the high halves of both floats (bytes 2, 3 of f0 below bytes 2, 3 of f1).
+  return __builtin_amdgcn_perm(__float_as_uint(f1), __float_as_uint(f0), 0x07060302u);
 }
 __device__ inline void widen_i8x16(uint4 q, uint4& lo, uint4& hi) {
   lo.x = pack_i8_pair(q.x, 0);

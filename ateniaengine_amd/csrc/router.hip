@@ -625,22 +625,6 @@ __global__ __launch_bounds__(kTokenThreads) void router_token_kernel(
   const int KS = R >= NW ? 1 : NW / R;              // k slices per row
   const int slice = ((d + KS - 1) / KS + 3) & ~3;   // multiple of 4 for float4 loads
   const bool vec_ok = (d & 3) == 0;
-  // The weights of the wave's first item are requested before the token is staged: they do not
-  // depend on it, and at one token per launch the two round trips to memory would otherwise
-  // follow each other.
-  constexpr int kPre = 8;
-  float4 wpre[kPre];
-  const bool pre = vec_ok && wave < R * KS;
-  if (pre) {
-    const int r = wave / KS, ksl = wave - r * KS;
-    const float* wr = row_lo + r < E ? w_router + (size_t)(row_lo + r) * d : gate_vec;
-    const int c_lo = ksl * slice, c_hi = min(d, c_lo + slice);
-#pragma unroll
-    for (int i = 0; i < kPre; ++i) {
-      const int c = c_lo + lane * 4 + i * 256;
-      wpre[i] = c < c_hi ? *(const float4*)(wr + c) : make_float4(0.f, 0.f, 0.f, 0.f);
-    }
-  }
   const int c_end = xb ? (d_pad > d ? d_pad : d) : d;
   for (int c = tid; c < c_end; c += kTokenThreads) {
     float v = c < d ? load_x(x, (size_t)t * d + c) : 0.f;
@@ -661,20 +645,8 @@ __global__ __launch_bounds__(kTokenThreads) void router_token_kernel(
       asum = fma(fabs(wd), fabs(xd), asum);
     };
     if (vec_ok) {
-      int c = c_lo + lane * 4;
-      if (item == wave) {  // the first item: its first kPre steps are in registers already
-#pragma unroll
-        for (int i = 0; i < kPre; ++i, c += 256) {
-          if (c < c_hi) {
-            one(wpre[i].x, c);
-            one(wpre[i].y, c + 1);
-            one(wpre[i].z, c + 2);
-            one(wpre[i].w, c + 3);
-          }
-        }
-      }
 #pragma unroll 4
-      for (; c < c_hi; c += 256) {
+      for (int c = c_lo + lane * 4; c < c_hi; c += 256) {
         float4 w4 = *(const float4*)(wr + c);
         one(w4.x, c);
         one(w4.y, c + 1);

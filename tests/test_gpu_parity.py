@@ -154,6 +154,27 @@ def test_router_token_kernel_inexact_rows_fall_back(ora):
         assert (idx == o_idx).all() and ulp_diff(w, o_w).max() <= 1
 
 
+def test_router_batched_kernel_with_wide_exponent_spread(ora):
+    """More than 512 tokens on a bf16 layer leave the per-token kernel for the batched one, which
+    keeps the reference's summation order outright: f32-valued activations with a wide exponent
+    spread (huge sum|p| against a small result) and bf16-valued tokens must both route as the
+    oracle does."""
+    E, k, d, T = 12, 3, 512, 600
+    W = S.make_weights(17, E, d, 16, router_std=1.0)
+    oL, gL = S.build_pair(ora, W, k, 0, capi.WEIGHT_BF16)
+    rng = np.random.default_rng(18)
+    x = (rng.standard_normal((T, d)) * np.exp2(rng.integers(-30, 30, size=(T, d)))).astype(
+        np.float32)
+    with gL:
+        idx, w = gL.route(x)
+        o_idx, o_w = oL.route_tokens(x)
+        assert (idx == o_idx).all() and ulp_diff(w, o_w).max() <= 1
+        xb = S.make_tokens(19, T, d)
+        idx, w = gL.route(xb)
+        o_idx, o_w = oL.route_tokens(xb)
+        assert (idx == o_idx).all() and ulp_diff(w, o_w).max() <= 1
+
+
 def test_router_engineered_ties(ora):
     """Duplicate router rows give exactly equal weights; the lower index must win."""
     E, k, d, T = 8, 2, 64, 40
@@ -439,7 +460,10 @@ def test_combine_is_bit_exact_given_expert_outputs(ora, wd, T, shared):
 
 
 @pytest.mark.parametrize("E,k,d,T,gated", [(8, 2, 4096, 512, False), (60, 4, 2048, 300, True),
-                                           (64, 6, 1024, 97, False)])
+                                           (64, 6, 1024, 97, False),
+                                           # above 512 tokens: the batched sequential kernel
+                                           (8, 2, 4096, 1000, False), (60, 4, 2048, 700, True),
+                                           (64, 6, 1024, 1037, False), (20, 3, 72, 530, True)])
 def test_router_f32_valued_rows_on_blocked_layers(ora, E, k, d, T, gated):
     """f32-valued activations on a bf16 layer (what a reference caller hands over): sums of such
     products are not exact in every order, so the per-token kernel either proves that its sum and
