@@ -278,11 +278,13 @@ class Layer:
         self.close()
 
     # -- the op ---------------------------------------------------------------------------
-    def forward(self, x) -> np.ndarray:
-        """[T, d] (or [T*d]) f32 host -> same shape f32 host."""
+    def forward(self, x, out=None) -> np.ndarray:
+        """[T, d] (or [T*d]) f32 host -> same shape f32 host (into `out` when given)."""
         x = np.ascontiguousarray(x, dtype=np.float32)
         assert x.size % self.d == 0
-        out = np.empty_like(x)
+        if out is None:
+            out = np.empty_like(x)
+        assert out.dtype == np.float32 and out.size == x.size and out.flags.c_contiguous
         _check(lib().atenia_moe_hip_layer_forward(self._h, _ptr(x), x.size // self.d, _ptr(out)))
         return out
 

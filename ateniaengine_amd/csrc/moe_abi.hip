@@ -161,6 +161,13 @@ struct AteniaMoeLayer {
   bool last_split = false;  // the last forward's down phase may have split tail tiles
 
   hipStream_t stream = nullptr;
+  // Host-buffer entry point, large batches: page-locked staging (two slots each way) and two
+  // copy streams, so that the copies of one chunk of tokens run beside the kernels of another.
+  hipStream_t h2d_stream = nullptr, d2h_stream = nullptr;
+  void *pin_in = nullptr, *pin_out = nullptr;
+  size_t pin_bytes = 0;  // per slot
+  hipEvent_t ev_h2d[2] = {}, ev_comp[2] = {}, ev_d2h[2] = {};
+  bool staging_ready = false;
   std::mutex mu;
   // Ordering of asynchronous forwards on one handle: a forward on another stream than the
   // previous one (`done_stream`) first waits for that stream's work, so two streams never use
@@ -813,6 +820,90 @@ int read_status(AteniaMoeLayer* L, hipStream_t s, int32_t* token, int32_t* exper
               ex);
 }
 
+// ---- host-buffer entry point, large batches -----------------------------------------------------
+// Tokens are independent, so a batch from pageable host memory is processed in chunks of
+// kHostChunkTokens: the calling thread copies chunk c + 1 into page-locked staging while the
+// copy engine moves chunk c to the device, the kernels of chunk c - 1 run, and the output of
+// chunk c - 2 travels back -- three streams at the default priority tied together by events.
+// The caller's pages cannot be registered on the fly (hipHostRegister is not available on every
+// host), hence the staging copy; it runs at memcpy speed and hides behind the kernels.
+constexpr int kHostChunkTokens = 1024;
+
+// Page-locked caller memory (hipHostMalloc and the like) is copied by the DMA engines directly;
+// staging it would only add a copy.
+bool is_page_locked(const void* p) {
+  hipPointerAttribute_t at{};
+  if (hipPointerGetAttributes(&at, p) != hipSuccess) {
+    (void)hipGetLastError();  // ordinary memory: the query fails and leaves its error behind
+    return false;
+  }
+  return at.type == hipMemoryTypeHost;
+}
+
+int ensure_host_staging(AteniaMoeLayer* L) {
+  const size_t need = (size_t)kHostChunkTokens * L->d * 4;
+  if (!L->staging_ready) {
+    HIP_TRY(hipStreamCreateWithFlags(&L->h2d_stream, hipStreamNonBlocking));
+    HIP_TRY(hipStreamCreateWithFlags(&L->d2h_stream, hipStreamNonBlocking));
+    for (int i = 0; i < 2; ++i) {
+      HIP_TRY(hipEventCreateWithFlags(&L->ev_h2d[i], hipEventDisableTiming));
+      HIP_TRY(hipEventCreateWithFlags(&L->ev_comp[i], hipEventDisableTiming));
+      HIP_TRY(hipEventCreateWithFlags(&L->ev_d2h[i], hipEventDisableTiming));
+    }
+    L->staging_ready = true;
+  }
+  if (L->pin_bytes < need) {
+    if (L->pin_in) (void)hipHostFree(L->pin_in);
+    if (L->pin_out) (void)hipHostFree(L->pin_out);
+    L->pin_in = L->pin_out = nullptr;
+    L->pin_bytes = 0;
+    HIP_TRY(hipHostMalloc(&L->pin_in, 2 * need, hipHostMallocDefault));
+    HIP_TRY(hipHostMalloc(&L->pin_out, 2 * need, hipHostMallocDefault));
+    L->pin_bytes = need;
+  }
+  return ATENIA_MOE_OK;
+}
+
+int forward_host_chunked(AteniaMoeLayer* L, const float* x_host, int T, float* out_host) {
+  int rc = ensure_host_staging(L);
+  if (rc) return rc;
+  const size_t row = (size_t)L->d * 4;
+  const int n_chunks = (T + kHostChunkTokens - 1) / kHostChunkTokens;
+  auto tokens_of = [&](int c) { return std::min(kHostChunkTokens, T - c * kHostChunkTokens); };
+  auto drain = [&](int c) -> int {  // chunk c's output: staging -> caller
+    const int slot = c & 1;
+    HIP_TRY(hipEventSynchronize(L->ev_d2h[slot]));
+    memcpy((char*)out_host + (size_t)c * kHostChunkTokens * row,
+           (char*)L->pin_out + slot * L->pin_bytes, (size_t)tokens_of(c) * row);
+    return ATENIA_MOE_OK;
+  };
+  for (int c = 0; c < n_chunks; ++c) {
+    const int slot = c & 1, n = tokens_of(c);
+    const size_t off = (size_t)c * kHostChunkTokens * row, bytes = (size_t)n * row;
+    // the in-slot is free once the copy of chunk c - 2 has left it
+    if (c >= 2) HIP_TRY(hipEventSynchronize(L->ev_h2d[slot]));
+    memcpy((char*)L->pin_in + slot * L->pin_bytes, (const char*)x_host + off, bytes);
+    HIP_TRY(hipMemcpyAsync((char*)L->x_in.p + off, (char*)L->pin_in + slot * L->pin_bytes, bytes,
+                           hipMemcpyHostToDevice, L->h2d_stream));
+    HIP_TRY(hipEventRecord(L->ev_h2d[slot], L->h2d_stream));
+    HIP_TRY(hipStreamWaitEvent(L->stream, L->ev_h2d[slot], 0));
+    rc = run_forward(L, (char*)L->x_in.p + off, ATENIA_MOE_ACT_F32, n,
+                     (float*)((char*)L->out.p + off), L->stream, kStageRouter, kStageCombine);
+    if (rc) return rc;
+    HIP_TRY(hipEventRecord(L->ev_comp[slot], L->stream));
+    // the out-slot is free once the caller has chunk c - 2's rows
+    if (c >= 2 && (rc = drain(c - 2))) return rc;
+    HIP_TRY(hipStreamWaitEvent(L->d2h_stream, L->ev_comp[slot], 0));
+    HIP_TRY(hipMemcpyAsync((char*)L->pin_out + slot * L->pin_bytes, (char*)L->out.p + off, bytes,
+                           hipMemcpyDeviceToHost, L->d2h_stream));
+    HIP_TRY(hipEventRecord(L->ev_d2h[slot], L->d2h_stream));
+  }
+  for (int c = std::max(0, n_chunks - 2); c < n_chunks; ++c)
+    if ((rc = drain(c))) return rc;
+  // the taps read the most recent forward: that is the last chunk
+  return read_status(L, L->stream, nullptr, nullptr);
+}
+
 }  // namespace
 
 extern "C" {
@@ -980,6 +1071,17 @@ int atenia_moe_hip_layer_destroy(AteniaMoeLayer* L) {
     if (L->ev_valid)
       for (auto& e : L->ev) (void)hipEventDestroy(e);
     if (L->done) (void)hipEventDestroy(L->done);
+    if (L->staging_ready) {
+      for (int i = 0; i < 2; ++i) {
+        (void)hipEventDestroy(L->ev_h2d[i]);
+        (void)hipEventDestroy(L->ev_comp[i]);
+        (void)hipEventDestroy(L->ev_d2h[i]);
+      }
+      (void)hipStreamDestroy(L->h2d_stream);
+      (void)hipStreamDestroy(L->d2h_stream);
+    }
+    if (L->pin_in) (void)hipHostFree(L->pin_in);
+    if (L->pin_out) (void)hipHostFree(L->pin_out);
     if (L->stream) (void)hipStreamDestroy(L->stream);
     L->magic = 0;
   }
@@ -1045,6 +1147,10 @@ int atenia_moe_hip_layer_forward(AteniaMoeLayer* L, const float* x_host, int n_t
   std::lock_guard<std::mutex> lock(L->mu);
   int rc = ensure_workspace(L, n_tokens);
   if (rc) return rc;
+  // From four chunks on the overlap pays; the taps (last routing, expert outputs, stage times)
+  // then describe the last chunk, as after that many separate calls.
+  if (n_tokens >= 4 * kHostChunkTokens && !(is_page_locked(x_host) && is_page_locked(out_host)))
+    return forward_host_chunked(L, x_host, n_tokens, out_host);
   const size_t bytes = (size_t)n_tokens * L->d * 4;
   HIP_TRY(hipMemcpyAsync(L->x_in.p, x_host, bytes, hipMemcpyHostToDevice, L->stream));
   rc = run_forward(L, L->x_in.p, ATENIA_MOE_ACT_F32, n_tokens, L->out.as<float>(), L->stream,
