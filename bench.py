@@ -406,6 +406,7 @@ def main():
     if shared is not None:
         kw.update(s_gate=shared[0], s_up=shared[1], s_down=shared[2])
     layer = capi.Layer(w_gate=gate, w_up=up, w_down=down, weight_dtype=wdt, **kw)
+    e_bias = None
     if cfg.get("v3"):
         v3 = cfg["v3"]
         e_bias = (0.05 * np.random.default_rng(a.seed + 2).standard_normal(N_EXPERTS)).astype(np.float32)
@@ -474,6 +475,8 @@ def main():
         flops_tok = 2.0 * D_MODEL * N_EXPERTS + 6.0 * TOP_K * D_MODEL * D_FF + 6.0 * D_MODEL * D_FF_SHARED
         n = a.cpu_tokens if a.cpu_tokens > 0 else int(1024 * 704.7e6 / flops_tok)
         n = max(1, min(n, a.tokens))
+        if cfg.get("v3") and a.cpu_tokens < 0:
+            n = min(n, 512)  # that path runs token by token on one core
         # the headline batch, recomputed once so `out_head` matches `x_head`
         layer.forward_device(x_head.data_ptr(), ACT, a.tokens, out_head.data_ptr(),
                              torch.cuda.current_stream().cuda_stream)
@@ -486,17 +489,28 @@ def main():
                        **stored)
         cores = ora.hw_threads()
         ora.set_threads(cores)
-        oL.execute(xs[:1])  # warm the pages
+        if cfg.get("v3"):  # the DeepSeek-V3 router in front of the same experts (one thread)
+            v3 = cfg["v3"]
+            cores = 1
+            run = lambda rows: oL.v3_forward(rows, e_bias, v3["n_group"], v3["topk_group"],
+                                             v3["scale"], v3["norm"])[:2]
+        else:
+            run = lambda rows: oL.execute(rows)[:2]
+        run(xs[:1])  # warm the pages
         t0 = time.perf_counter()
-        ref, o_idx, _ = oL.execute(xs)
+        ref, o_idx = run(xs)
         dt = time.perf_counter() - t0
         cpu = dict(value=n / dt, unit="tokens/s", cores=cores, kind="port",
                    sample=f"{n} tokens of the T={a.tokens} batch, certified policy "
-                          "(f32 weights, f64 accumulation), rows parallel over all cores")
-        o_all, _ = oL.route_tokens(x_head.to(torch.float32).cpu().numpy())
+                          "(f32 weights, f64 accumulation), rows parallel over the cores used")
+        if cfg.get("v3"):  # routing checked on the sample the CPU path ran
+            o_all, idx_gpu, n_routed = o_idx, idx_gpu[:n], n
+        else:
+            o_all, _ = oL.route_tokens(x_head.to(torch.float32).cpu().numpy())
+            n_routed = int(a.tokens)
         parity = dict(
             routing_mismatched_tokens=int((idx_gpu != o_all).any(axis=1).sum()),
-            tokens_routed=int(a.tokens),
+            tokens_routed=n_routed,
             max_rel_err_vs_cpu_path=float(np.abs(got - ref).max() / np.abs(ref).max()),
             sample_tokens=n)
 
