@@ -135,6 +135,7 @@ struct AteniaMoeLayer {
   int group_size = 0;  // per-group int8: input elements per scale (0 = per-row scales)
 
   DevBuf w_router, router_bias, shared_gate;
+  bool router_fits_bf16 = false;  // every router / gate value is exactly a bf16 value
   DevBuf wg, wu, wd, sg, su, sd;        // routed experts
   DevBuf swg, swu, swd, ssg, ssu, ssd;  // shared expert
   WeightSet gate{}, up{}, down{}, s_gate{}, s_up{}, s_down{};
@@ -161,12 +162,11 @@ struct AteniaMoeLayer {
   bool last_split = false;  // the last forward's down phase may have split tail tiles
 
   hipStream_t stream = nullptr;
-  // Host-buffer entry point, large batches: page-locked staging (two slots each way) and two
-  // copy streams, so that the copies of one chunk of tokens run beside the kernels of another.
-  hipStream_t h2d_stream = nullptr, d2h_stream = nullptr;
+  // Host-buffer entry point, large batches: page-locked staging (two slots each way); the
+  // events tell the host when the copy engine has emptied / filled a slot.
   void *pin_in = nullptr, *pin_out = nullptr;
   size_t pin_bytes = 0;  // per slot
-  hipEvent_t ev_h2d[2] = {}, ev_comp[2] = {}, ev_d2h[2] = {};
+  hipEvent_t ev_h2d[2] = {}, ev_d2h[2] = {};
   bool staging_ready = false;
   std::mutex mu;
   // Ordering of asynchronous forwards on one handle: a forward on another stream than the
@@ -550,6 +550,7 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   ra.k = L->k;
   ra.renorm = L->conv == ATENIA_MOE_CONVENTION_ATENIA;
   ra.w_router = L->w_router.as<float>();
+  ra.w_fits_bf16 = L->router_fits_bf16;
   ra.router_bias = L->router_bias.as<float>();
   const bool gated = L->fs > 0 && L->conv == ATENIA_MOE_CONVENTION_HUGGINGFACE_QWEN &&
                      L->shared_gate.p != nullptr && L->v3_n_group == 0;
@@ -821,12 +822,14 @@ int read_status(AteniaMoeLayer* L, hipStream_t s, int32_t* token, int32_t* exper
 }
 
 // ---- host-buffer entry point, large batches -----------------------------------------------------
-// Tokens are independent, so a batch from pageable host memory is processed in chunks of
-// kHostChunkTokens: the calling thread copies chunk c + 1 into page-locked staging while the
-// copy engine moves chunk c to the device, the kernels of chunk c - 1 run, and the output of
-// chunk c - 2 travels back -- three streams at the default priority tied together by events.
-// The caller's pages cannot be registered on the fly (hipHostRegister is not available on every
-// host), hence the staging copy; it runs at memcpy speed and hides behind the kernels.
+// A batch from pageable host memory travels through page-locked staging in chunks of
+// kHostChunkTokens: the calling thread copies chunk c + 1 into a staging slot while the copy
+// engine moves chunk c to the device; after the one forward over the whole batch the output comes
+// back the same way (the copy engine fills one slot while the thread empties the other).  The
+// caller's pages cannot be registered on the fly (hipHostRegister is not available on every
+// host), hence the staging copy; it runs at memcpy speed, about twice what the runtime's own
+// pageable copies reach.  Everything is ordered on the handle's stream; the events only tell the
+// host when a slot is free or full.
 constexpr int kHostChunkTokens = 1024;
 
 // Page-locked caller memory (hipHostMalloc and the like) is copied by the DMA engines directly;
@@ -843,11 +846,8 @@ bool is_page_locked(const void* p) {
 int ensure_host_staging(AteniaMoeLayer* L) {
   const size_t need = (size_t)kHostChunkTokens * L->d * 4;
   if (!L->staging_ready) {
-    HIP_TRY(hipStreamCreateWithFlags(&L->h2d_stream, hipStreamNonBlocking));
-    HIP_TRY(hipStreamCreateWithFlags(&L->d2h_stream, hipStreamNonBlocking));
     for (int i = 0; i < 2; ++i) {
       HIP_TRY(hipEventCreateWithFlags(&L->ev_h2d[i], hipEventDisableTiming));
-      HIP_TRY(hipEventCreateWithFlags(&L->ev_comp[i], hipEventDisableTiming));
       HIP_TRY(hipEventCreateWithFlags(&L->ev_d2h[i], hipEventDisableTiming));
     }
     L->staging_ready = true;
@@ -864,12 +864,25 @@ int ensure_host_staging(AteniaMoeLayer* L) {
   return ATENIA_MOE_OK;
 }
 
-int forward_host_chunked(AteniaMoeLayer* L, const float* x_host, int T, float* out_host) {
+int forward_host_staged(AteniaMoeLayer* L, const float* x_host, int T, float* out_host) {
   int rc = ensure_host_staging(L);
   if (rc) return rc;
   const size_t row = (size_t)L->d * 4;
   const int n_chunks = (T + kHostChunkTokens - 1) / kHostChunkTokens;
   auto tokens_of = [&](int c) { return std::min(kHostChunkTokens, T - c * kHostChunkTokens); };
+  for (int c = 0; c < n_chunks; ++c) {
+    const int slot = c & 1;
+    const size_t off = (size_t)c * kHostChunkTokens * row, bytes = (size_t)tokens_of(c) * row;
+    // the slot is free once the copy of chunk c - 2 has left it
+    if (c >= 2) HIP_TRY(hipEventSynchronize(L->ev_h2d[slot]));
+    memcpy((char*)L->pin_in + slot * L->pin_bytes, (const char*)x_host + off, bytes);
+    HIP_TRY(hipMemcpyAsync((char*)L->x_in.p + off, (char*)L->pin_in + slot * L->pin_bytes, bytes,
+                           hipMemcpyHostToDevice, L->stream));
+    HIP_TRY(hipEventRecord(L->ev_h2d[slot], L->stream));
+  }
+  rc = run_forward(L, L->x_in.p, ATENIA_MOE_ACT_F32, T, L->out.as<float>(), L->stream,
+                   kStageRouter, kStageCombine);
+  if (rc) return rc;
   auto drain = [&](int c) -> int {  // chunk c's output: staging -> caller
     const int slot = c & 1;
     HIP_TRY(hipEventSynchronize(L->ev_d2h[slot]));
@@ -878,29 +891,16 @@ int forward_host_chunked(AteniaMoeLayer* L, const float* x_host, int T, float* o
     return ATENIA_MOE_OK;
   };
   for (int c = 0; c < n_chunks; ++c) {
-    const int slot = c & 1, n = tokens_of(c);
-    const size_t off = (size_t)c * kHostChunkTokens * row, bytes = (size_t)n * row;
-    // the in-slot is free once the copy of chunk c - 2 has left it
-    if (c >= 2) HIP_TRY(hipEventSynchronize(L->ev_h2d[slot]));
-    memcpy((char*)L->pin_in + slot * L->pin_bytes, (const char*)x_host + off, bytes);
-    HIP_TRY(hipMemcpyAsync((char*)L->x_in.p + off, (char*)L->pin_in + slot * L->pin_bytes, bytes,
-                           hipMemcpyHostToDevice, L->h2d_stream));
-    HIP_TRY(hipEventRecord(L->ev_h2d[slot], L->h2d_stream));
-    HIP_TRY(hipStreamWaitEvent(L->stream, L->ev_h2d[slot], 0));
-    rc = run_forward(L, (char*)L->x_in.p + off, ATENIA_MOE_ACT_F32, n,
-                     (float*)((char*)L->out.p + off), L->stream, kStageRouter, kStageCombine);
-    if (rc) return rc;
-    HIP_TRY(hipEventRecord(L->ev_comp[slot], L->stream));
-    // the out-slot is free once the caller has chunk c - 2's rows
+    const int slot = c & 1;
+    const size_t off = (size_t)c * kHostChunkTokens * row, bytes = (size_t)tokens_of(c) * row;
+    // the slot is free once the caller has chunk c - 2's rows
     if (c >= 2 && (rc = drain(c - 2))) return rc;
-    HIP_TRY(hipStreamWaitEvent(L->d2h_stream, L->ev_comp[slot], 0));
     HIP_TRY(hipMemcpyAsync((char*)L->pin_out + slot * L->pin_bytes, (char*)L->out.p + off, bytes,
-                           hipMemcpyDeviceToHost, L->d2h_stream));
-    HIP_TRY(hipEventRecord(L->ev_d2h[slot], L->d2h_stream));
+                           hipMemcpyDeviceToHost, L->stream));
+    HIP_TRY(hipEventRecord(L->ev_d2h[slot], L->stream));
   }
   for (int c = std::max(0, n_chunks - 2); c < n_chunks; ++c)
     if ((rc = drain(c))) return rc;
-  // the taps read the most recent forward: that is the last chunk
   return read_status(L, L->stream, nullptr, nullptr);
 }
 
@@ -984,6 +984,23 @@ int atenia_moe_hip_layer_create(const AteniaMoeLayerDesc* D, AteniaMoeLayer** ou
   if ((rc = upload_f32(D->w_router, E * d, L->w_router))) return bail(rc);
   if (D->router_bias && (rc = upload_f32(D->router_bias, E, L->router_bias))) return bail(rc);
   if (D->shared_gate && (rc = upload_f32(D->shared_gate, d, L->shared_gate))) return bail(rc);
+  {
+    // Router rows (and the gate vector) whose f32 values all fit bf16, as they do when the
+    // checkpoint was bf16: with bf16 activations every product then has few enough significant
+    // bits that a sum in any order is exact in f64, which is what lets the router use the
+    // matrix cores without a slow path (router.hip).
+    auto fits_bf16 = [](const float* p, size_t n) {
+      uint32_t low = 0;
+      for (size_t i = 0; i < n; ++i) {
+        uint32_t u;
+        memcpy(&u, p + i, 4);
+        low |= u;
+      }
+      return (low & 0xffffu) == 0;
+    };
+    L->router_fits_bf16 = fits_bf16(D->w_router, E * d) &&
+                          (!D->shared_gate || fits_bf16(D->shared_gate, d));
+  }
 
   DevBuf staging;
   const size_t eb = elem_bytes_of(L->wdtype);
@@ -1074,11 +1091,8 @@ int atenia_moe_hip_layer_destroy(AteniaMoeLayer* L) {
     if (L->staging_ready) {
       for (int i = 0; i < 2; ++i) {
         (void)hipEventDestroy(L->ev_h2d[i]);
-        (void)hipEventDestroy(L->ev_comp[i]);
         (void)hipEventDestroy(L->ev_d2h[i]);
       }
-      (void)hipStreamDestroy(L->h2d_stream);
-      (void)hipStreamDestroy(L->d2h_stream);
     }
     if (L->pin_in) (void)hipHostFree(L->pin_in);
     if (L->pin_out) (void)hipHostFree(L->pin_out);
@@ -1147,10 +1161,8 @@ int atenia_moe_hip_layer_forward(AteniaMoeLayer* L, const float* x_host, int n_t
   std::lock_guard<std::mutex> lock(L->mu);
   int rc = ensure_workspace(L, n_tokens);
   if (rc) return rc;
-  // From four chunks on the overlap pays; the taps (last routing, expert outputs, stage times)
-  // then describe the last chunk, as after that many separate calls.
-  if (n_tokens >= 4 * kHostChunkTokens && !(is_page_locked(x_host) && is_page_locked(out_host)))
-    return forward_host_chunked(L, x_host, n_tokens, out_host);
+  if (n_tokens >= 2 * kHostChunkTokens && !(is_page_locked(x_host) && is_page_locked(out_host)))
+    return forward_host_staged(L, x_host, n_tokens, out_host);
   const size_t bytes = (size_t)n_tokens * L->d * 4;
   HIP_TRY(hipMemcpyAsync(L->x_in.p, x_host, bytes, hipMemcpyHostToDevice, L->stream));
   rc = run_forward(L, L->x_in.p, ATENIA_MOE_ACT_F32, n_tokens, L->out.as<float>(), L->stream,

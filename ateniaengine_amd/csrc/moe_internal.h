@@ -63,6 +63,7 @@ struct RouterArgs {
   int x_is_bf16;
   int T, d, E, k, renorm;
   const float* w_router;     // [E, d]
+  int w_fits_bf16;           // every value of w_router and shared_gate is exactly a bf16 value
   const float* router_bias;  // [E] or null
   const float* shared_gate;  // [d] or null
   int32_t* idx;              // [T, k]

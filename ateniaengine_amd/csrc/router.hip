@@ -56,17 +56,14 @@ __device__ inline uint16_t f32_to_bf16_rne(float f) {
 // Exponent of the lowest set bit of a finite f32 (v = odd * 2^result); kNoLsb for zero,
 // and a hugely negative value for inf/NaN so that no exactness claim survives them.
 constexpr int kNoLsb = 32767;
-__device__ inline int lsb_exponent(float v) {
-  uint32_t b = __float_as_uint(v);
-  int e = (b >> 23) & 0xff;
-  uint32_t m = b & 0x7fffffu;
-  if (e == 0xff) return -100000;
-  if (e == 0) {
-    if (m == 0) return kNoLsb;
-    return -149 + (__ffs((int)m) - 1);
-  }
-  m |= 0x800000u;
-  return e - 150 + (__ffs((int)m) - 1);
+__device__ inline int lsb_exponent(float v) {  // selects only: it sits in unrolled loops
+  const uint32_t b = __float_as_uint(v);
+  const int e = (b >> 23) & 0xff;
+  const uint32_t m = b & 0x7fffffu;
+  const uint32_t mm = e ? (m | 0x800000u) : m;  // normal numbers carry the implicit one
+  int r = (e ? e - 150 : -149) + (__ffs((int)mm) - 1);
+  r = mm == 0 ? kNoLsb : r;
+  return e == 0xff ? -100000 : r;
 }
 
 // Softmax + top-k + renormalisation of ONE token by the threads r = 0..E-1 that call with
@@ -510,6 +507,332 @@ hipError_t launch_router_batch(const RouterArgs& a, hipStream_t s) {
   return hipGetLastError();
 }
 
+// ---- batches on the f64 matrix cores, any summation order made safe by a certificate ---------
+// v_mfma_f64_16x16x4_f64 (operand layout: see ffn_f32.hip): A = 16 rows of [W_r ; gate], B = 16
+// tokens, so lane l holds D[4 r + l / 16][l % 16] = rows 4 r + l / 16 of token l % 16.  A
+// workgroup owns 16 tokens and all rows (RB blocks of 16); its four waves split k and add their
+// partial sums in wave order.  f32 operands widen exactly and their products are exact in f64,
+// so the result differs from the reference's c-ascending sum only by the order of the f64
+// additions.  That is accepted only under the same two certificates as in router_token_kernel:
+//   interval : any order lands within g = d 2^-53 sum|p| of the true sum, and sum|p| is bounded
+//              here by |w_r| |x_t| (Cauchy-Schwarz; both norms are accumulated next to the
+//              matrix instructions); if [acc - 2g, acc + 2g] rounds to one f32 (one f32 sigmoid
+//              for the gate row) that value is the reference's;
+//   exactness: for the few sums that fail it, one wave checks that every product is a multiple
+//              of 2^q and sum|p| < 2^(q+53), which makes every order exact (bf16-valued
+//              operands pass);
+// and a sum that fails both is recomputed in the reference's order by one lane.
+// Against one sequential chain per (token, row) this is 3-4x faster at 4096 tokens.
+typedef __attribute__((__vector_size__(4 * sizeof(double)))) double f64x4_t;
+
+template <typename XT> struct XChunk;
+template <> struct XChunk<float> {
+  float4 lo, hi;
+  __device__ inline void load(const float* p) { lo = *(const float4*)p; hi = *(const float4*)(p + 4); }
+  __device__ inline void keep(bool k) {  // selects, no branch
+    lo.x = k ? lo.x : 0.f; lo.y = k ? lo.y : 0.f; lo.z = k ? lo.z : 0.f; lo.w = k ? lo.w : 0.f;
+    hi.x = k ? hi.x : 0.f; hi.y = k ? hi.y : 0.f; hi.z = k ? hi.z : 0.f; hi.w = k ? hi.w : 0.f;
+  }
+  __device__ inline void get(float (&f)[8]) const {
+    f[0] = lo.x; f[1] = lo.y; f[2] = lo.z; f[3] = lo.w; f[4] = hi.x; f[5] = hi.y; f[6] = hi.z; f[7] = hi.w;
+  }
+};
+template <> struct XChunk<uint16_t> {
+  uint4 v;
+  __device__ inline void load(const uint16_t* p) { v = *(const uint4*)p; }
+  __device__ inline void keep(bool k) {
+    v.x = k ? v.x : 0u; v.y = k ? v.y : 0u; v.z = k ? v.z : 0u; v.w = k ? v.w : 0u;
+  }
+  __device__ inline void get(float (&f)[8]) const {
+    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = __uint_as_float(u[i] << 16);
+      f[2 * i + 1] = __uint_as_float(u[i] & 0xffff0000u);
+    }
+  }
+};
+
+template <typename XT, int RB, int NBUF, int NWV>
+__global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
+    const XT* __restrict__ x, int T, int d, int E, int k, int renorm,
+    const float* __restrict__ w_router, const float* __restrict__ bias,
+    const float* __restrict__ gate_vec, int32_t* __restrict__ idx_out,
+    float* __restrict__ w_out, float* __restrict__ sgate_out, int32_t* __restrict__ status) {
+  constexpr int TT = 16;
+  const int R = E + (gate_vec ? 1 : 0);
+  const int t0 = blockIdx.x * TT;
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int r16 = lane & 15, q = lane >> 4;
+
+  extern __shared__ double smem_m[];
+  constexpr int NT = 64 * NWV;                    // NWV waves split k
+  double* sPart = smem_m;                         // [NWV][RB][4][64] partial sums
+  double* sXsq = sPart + NWV * RB * 4 * 64;       // [NWV][16]  partial |x_t|^2
+  double* sWsq = sXsq + NWV * 16;                 // [NWV][RB][16] partial |w_r|^2
+  double* sAcc = sWsq + NWV * RB * 16;            // [16][R]
+  double* sXn2 = sAcc + 16 * R;                   // [16]
+  double* sWn2 = sXn2 + 16;                       // [R]
+  float* sLogit = (float*)(sWn2 + R);             // [16][R]
+  uint8_t* sFlag = (uint8_t*)(sLogit + 16 * R);   // [16][R] 1 = the interval certificate failed
+
+  const int tok = min(t0 + r16, T - 1);  // rows past T repeat the last token; never written out
+  const XT* px = x + (size_t)tok * d + 8 * q;
+  const float* pw[RB];
+#pragma unroll
+  for (int b = 0; b < RB; ++b) {
+    const int r = min(16 * b + r16, R - 1);
+    pw[b] = (r < E ? w_router + (size_t)r * d : gate_vec) + 8 * q;
+  }
+  // k in steps of 32 (8 per lane), the steps dealt to the four waves in contiguous runs
+  const int nsteps = (d + 31) / 32;
+  const int per = (nsteps + NWV - 1) / NWV;
+  const int s0 = wave * per, s1 = min(nsteps, s0 + per);
+
+  // One row block: two accumulators in turn, so that consecutive matrix instructions do not
+  // wait for each other's result (summed once at the end; any order is as good).  With more
+  // blocks their instructions interleave anyway and the registers are better spent on a second
+  // workgroup per compute unit.
+  constexpr int NACC = RB == 1 ? 2 : 1;
+  f64x4_t acc[RB][NACC];
+#pragma unroll
+  for (int b = 0; b < RB; ++b)
+#pragma unroll
+    for (int n = 0; n < NACC; ++n) acc[b][n] = f64x4_t{0.0, 0.0, 0.0, 0.0};
+  double xsq = 0.0, wsq[RB];
+#pragma unroll
+  for (int b = 0; b < RB; ++b) wsq[b] = 0.0;
+
+  XChunk<XT> xc[NBUF];
+  XChunk<float> wc[NBUF][RB];
+  // Every step issues the same loads whatever the lane or the step: a chunk past d is fetched
+  // from the row's first columns and zeroed with selects, a step past the wave's range repeats
+  // its last one.  With a branch around a load the compiler can no longer count the loads in
+  // flight and waits for all of them (s_waitcnt vmcnt(0)) before every use -- the first cut of
+  // this kernel did, and ran one memory round trip per step.
+  auto load_step = [&](int buf, int st) {
+    st = min(st, s1 - 1);
+    const bool in = st * 32 + 8 * q < d;  // d is a multiple of 8: a chunk is whole or absent
+    const size_t off = in ? (size_t)st * 32 : 0;
+    xc[buf].load(px + off);
+    xc[buf].keep(in);
+#pragma unroll
+    for (int b = 0; b < RB; ++b) {
+      wc[buf][b].load(pw[b] + off);
+      wc[buf][b].keep(in);
+    }
+  };
+  auto multiply = [&](int buf) {
+    float xf[8];
+    xc[buf].get(xf);
+    double xd[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      xd[t] = (double)xf[t];
+      xsq = fma(xd[t], xd[t], xsq);
+    }
+#pragma unroll
+    for (int b = 0; b < RB; ++b) {
+      float wf[8];
+      wc[buf][b].get(wf);
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        const double wd = (double)wf[t];
+        wsq[b] = fma(wd, wd, wsq[b]);
+        acc[b][t % NACC] = __builtin_amdgcn_mfma_f64_16x16x4f64(wd, xd[t], acc[b][t % NACC], 0, 0, 0);
+      }
+    }
+  };
+  if (s0 < s1) {
+#pragma unroll
+    for (int i = 0; i < NBUF - 1; ++i) load_step(i, s0 + i);
+    for (int st = s0; st < s1; st += NBUF) {
+#pragma unroll
+      for (int i = 0; i < NBUF; ++i) {
+        load_step((i + NBUF - 1) % NBUF, st + i + NBUF - 1);
+        if (st + i < s1) multiply(i);  // scalar branch around matrix instructions only
+      }
+    }
+  }
+
+  // partial sums and norms of this wave -> LDS
+#pragma unroll
+  for (int b = 0; b < RB; ++b) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      sPart[((wave * RB + b) * 4 + r) * 64 + lane] = NACC == 2 ? acc[b][0][r] + acc[b][NACC - 1][r] : acc[b][0][r];
+    double v = wsq[b];
+    v += __shfl_xor(v, 16);
+    v += __shfl_xor(v, 32);
+    if (q == 0) sWsq[(wave * RB + b) * 16 + r16] = v;
+  }
+  {
+    double v = xsq;
+    v += __shfl_xor(v, 16);
+    v += __shfl_xor(v, 32);
+    if (q == 0) sXsq[wave * 16 + r16] = v;
+  }
+  __syncthreads();
+
+  // thread (token t, row class rr) finishes rows rr, rr + 16, ...
+  const int t = tid & 15, rr = tid >> 4;
+  double xn2 = 0.0;
+#pragma unroll
+  for (int w = 0; w < NWV; ++w) xn2 += sXsq[w * 16 + t];
+  if (rr == 0) sXn2[t] = xn2;
+  const double gfac = (double)(2 * d + 4) * 1.1102230246251565e-16 * 1.001;
+  for (int r = rr; r < R; r += NT / 16) {
+    const int b = r >> 4, rho = r & 15, reg = rho >> 2, qq = rho & 3;
+    double a = 0.0, wn2 = 0.0;
+#pragma unroll
+    for (int w = 0; w < NWV; ++w) {
+      a += sPart[((w * RB + b) * 4 + reg) * 64 + qq * 16 + t];
+      wn2 += sWsq[(w * RB + b) * 16 + rho];
+    }
+    if (t == 0) sWn2[r] = wn2;
+    // sum|p| <= |w_r| |x_t|; the factor 1.001 covers the roundings of the norms and the root
+    const double e = sqrt(xn2 * wn2) * gfac;
+    const double lo = a - e, hi = a + e;
+    bool ok;
+    if (r < E) {
+      const float flo = (float)lo, fhi = (float)hi;
+      ok = flo == fhi && isfinite(flo);
+    } else {
+      const float glo = (float)(1.0 / (1.0 + exp(-lo))), ghi = (float)(1.0 / (1.0 + exp(-hi)));
+      ok = glo == ghi;
+    }
+    sAcc[t * R + r] = a;
+    sFlag[t * R + r] = ok ? 0 : 1;
+  }
+  __syncthreads();
+
+  // Second look at the flagged sums (about one in a thousand), the whole workgroup on one sum
+  // at a time: the partial-sum area is free now and holds their list.
+  int* sList = (int*)sPart;      // [<= 16 R] flagged entries
+  int* sCount = sList + 16 * R;  // [1] how many, [2 ..] the waves' minima
+  if (tid == 0) *sCount = 0;
+  __syncthreads();
+  for (int ent = tid; ent < 16 * R; ent += NT)
+    if (sFlag[ent]) sList[atomicAdd(sCount, 1)] = ent;
+  __syncthreads();
+  const int n_flagged = *sCount;
+  for (int i = 0; i < n_flagged; ++i) {
+    const int ei = sList[i];
+    const int ft = ei / R, fr = ei - ft * R;
+    const XT* xr = x + (size_t)min(t0 + ft, T - 1) * d;
+    const float* wr = fr < E ? w_router + (size_t)fr * d : gate_vec;
+    int qmin = kNoLsb;
+#pragma unroll 2
+    for (int c = tid * 8; c < d; c += NT * 8) {  // eight columns per thread and trip
+      XChunk<XT> xn;
+      XChunk<float> wn;
+      xn.load(xr + c);
+      wn.load(wr + c);
+      float xf[8], wf[8];
+      xn.get(xf);
+      wn.get(wf);
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int lx = lsb_exponent(xf[u]), lw = lsb_exponent(wf[u]);
+        qmin = min(qmin, (lx != kNoLsb && lw != kNoLsb) ? lx + lw : kNoLsb);
+      }
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) qmin = min(qmin, __shfl_xor(qmin, off));
+    if (lane == 0) sCount[2 + wave] = qmin;
+    __syncthreads();
+    if (tid == 0) {
+      for (int w = 0; w < NWV; ++w) qmin = min(qmin, sCount[2 + w]);
+      const double bound = sqrt(sXn2[ft] * sWn2[fr]) * 1.001;
+      const bool exact = qmin == kNoLsb || (qmin > -2000 && bound < ldexp(1.0, qmin + 53));
+      if (!exact) {
+        // the reference's own order: one sequential c-ascending f64 sum
+        double a = 0.0;
+        for (int c = 0; c < d; ++c) a = fma((double)wr[c], (double)load_x(xr, c), a);
+        sAcc[ei] = a;
+      }
+    }
+    __syncthreads();
+  }
+
+  for (int ent = tid; ent < 16 * R; ent += NT) {
+    const int ft = ent / R, fr = ent - ft * R;
+    const double a = sAcc[ent];
+    if (fr < E) {
+      float logit = (float)a;
+      if (bias) logit = logit + bias[fr];
+      sLogit[ent] = logit;
+    } else if (t0 + ft < T) {
+      sgate_out[t0 + ft] = (float)(1.0 / (1.0 + exp(-a)));
+    }
+  }
+  __syncthreads();
+  if (E <= 64) {
+    // one wavefront per token (lane r = expert r, select_wave.h): the reference's sequential
+    // folds run over v_readlane values instead of one thread per token walking LDS
+    for (int tk = wave; tk < TT && t0 + tk < T; tk += NWV) {
+      const WaveRouting wr = wave_softmax_topk(sLogit + tk * R, E, k, renorm, lane);
+      if (wr.bad) {
+        atomicMin(&status[0], -3);
+        atomicMin(&status[1], ((t0 + tk) << 10) | lane);
+      }
+      if (wr.selected && wr.slot < k) {
+        const size_t o = (size_t)(t0 + tk) * k + wr.slot;
+        idx_out[o] = lane;
+        w_out[o] = wr.w;
+      }
+    }
+    return;
+  }
+  // the partial-sum area is free now: softmax scratch
+  double* sExp = smem_m;                          // [16][E]
+  double* sTok = sExp + 16 * E;                   // [16]
+  float* sWt = (float*)(sTok + 16);               // [16][E]
+  uint8_t* sSel = (uint8_t*)(sWt + 16 * E);       // [16][E]
+  softmax_topk_block(TT, R, E, k, renorm, t0, T, sLogit, sExp, sWt, sSel, sTok, idx_out, w_out,
+                     status);
+}
+
+template <typename XT, int RB, int NBUF, int NWV>
+hipError_t launch_router_mfma_rb(const RouterArgs& a, int R, hipStream_t s) {
+  const size_t smem = ((size_t)NWV * RB * 4 * 64 + NWV * 16 + (size_t)NWV * RB * 16 + (size_t)16 * R + 16 + R) * 8 +
+                      (size_t)16 * R * 4 + (size_t)16 * R + 16;
+  if (smem > 64 * 1024) return hipErrorInvalidValue;
+  router_mfma_kernel<XT, RB, NBUF, NWV><<<(a.T + 15) / 16, 64 * NWV, smem, s>>>(
+      (const XT*)a.x, a.T, a.d, a.E, a.k, a.renorm, a.w_router, a.router_bias, a.shared_gate,
+      a.idx, a.w, a.sgate, a.status);
+  return hipGetLastError();
+}
+
+// Up to 80 rows, d a multiple of 8, routing decided in the same launch, no bf16 copy of x to
+// write (bf16 activations of unpadded width: the store would sit in the loop).
+bool router_mfma_ok(const RouterArgs& a, int R) {
+  static const bool off = [] {
+    const char* e = getenv("ATENIA_MOE_ROUTER_MFMA");  // tuning knob: 0 = sequential chains
+    return e && atoi(e) == 0;
+  }();
+  // Up to 4096 tokens: measured 31-42 us against 57-75 us (8 rows, d = 4096) and about 70 us
+  // against 92-97 us (61-64 rows, d = 2048); larger batches are left to the sequential kernel,
+  // which then catches up (two tokens per thread) and has no slow path.
+  // Only with operands that make the exactness test pass -- bf16 activations and router rows whose
+  // f32 values fit bf16: otherwise every sum the interval test flags (one in a thousand) costs a
+  // sequential chain in its workgroup, and the launch lasts as long as the slowest of them.
+  return !off && R <= 80 && a.T <= 4096 && a.d % 8 == 0 && !a.logits_out && !a.xb &&
+         a.x_is_bf16 && a.w_fits_bf16 && a.E >= a.k;
+}
+
+template <typename XT>
+hipError_t launch_router_mfma(const RouterArgs& a, int R, hipStream_t s) {
+  // few rows: eight waves split k, so that a batch of 4096 tokens (256 workgroups, one per
+  // compute unit) still puts two waves on every SIMD
+  if (R <= 16) return launch_router_mfma_rb<XT, 1, 4, 8>(a, R, s);
+  if (R <= 32) return launch_router_mfma_rb<XT, 2, 3, 8>(a, R, s);
+  if (R <= 48) return launch_router_mfma_rb<XT, 3, 2, 4>(a, R, s);
+  if (R <= 64) return launch_router_mfma_rb<XT, 4, 2, 4>(a, R, s);
+  return launch_router_mfma_rb<XT, 5, 2, 4>(a, R, s);
+}
+
 template <typename XT>
 hipError_t dispatch_router_batch(const RouterArgs& a, int R, hipStream_t s) {
   if (R <= 16) return launch_router_batch<XT, 1, 1, 128>(a, s);
@@ -820,6 +1143,8 @@ hipError_t launch_router(const RouterArgs& a, hipStream_t s, int* fused_permute)
       return hipGetLastError();
     }
   }
+  if (router_mfma_ok(a, R))
+    return a.x_is_bf16 ? launch_router_mfma<uint16_t>(a, R, s) : launch_router_mfma<float>(a, R, s);
   // Up to 64 rows per workgroup; more rows only when the logits leave the kernel (row blocks).
   if ((R <= 64 || a.logits_out) && a.d % 4 == 0 && (!a.xb || a.d_pad % 4 == 0)) {
     return a.x_is_bf16 ? dispatch_router_batch<uint16_t>(a, R, s)

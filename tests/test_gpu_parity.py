@@ -176,6 +176,46 @@ def test_router_batched_kernel_with_wide_exponent_spread(ora):
         assert (idx == o_idx).all() and ulp_diff(w, o_w).max() <= 1
 
 
+@pytest.mark.parametrize("E,k,d,T,gated,bias,bf16_router,wide", [
+    (8, 2, 4096, 1000, False, False, True, False), (8, 2, 4096, 4096, False, False, True, False),
+    (60, 4, 2048, 700, True, False, True, False), (64, 6, 1024, 1037, False, True, True, True),
+    (20, 3, 96, 530, True, False, True, True), (33, 2, 160, 2000, False, False, True, False),
+    (79, 5, 256, 600, True, False, True, True), (48, 8, 512, 513, False, True, True, False),
+    (8, 2, 1024, 900, False, False, False, False)])
+def test_router_matrix_core_kernel(ora, E, k, d, T, gated, bias, bf16_router, wide):
+    """bf16 activations on the device, 513 to 4096 tokens, up to 80 rows, router rows whose values
+    fit bf16: the router runs on the f64 matrix cores in whatever order they add, and must still
+    give the reference's routing for every token -- through the interval certificate, the
+    exactness test, or the sequential recomputation (`wide`: activations spread over 60 binades
+    fail both tests for many sums).  Covers one to five row blocks, the gate row, a router bias
+    and more than 64 experts; the last case (f32-valued router rows) must take the sequential
+    kernel and agree as well."""
+    b = -1.2 * np.log(np.random.default_rng(2).permutation(E) + 1.0) if bias else None
+    W = S.make_weights(40 + E, E, d, 32, f_s=32 if gated else 0, gated=gated,
+                       router_std=1.0 / np.sqrt(d), bias=b)
+    if bf16_router:
+        W["w_router"] = S.bf16_round_trip(W["w_router"])[1]
+        if gated:
+            W["shared_gate"] = S.bf16_round_trip(W["shared_gate"])[1]
+    conv = capi.CONVENTION_HUGGINGFACE_QWEN if gated else capi.CONVENTION_ATENIA
+    oL, gL = S.build_pair(ora, W, k, conv, capi.WEIGHT_BF16)
+    if wide:
+        rng = np.random.default_rng(60 + T)
+        x = rng.standard_normal((T, d)) * np.exp2(rng.integers(-30, 30, size=(T, d)))
+        x = S.bf16_round_trip(x.astype(np.float32))[1]
+    else:
+        x = S.make_tokens(50 + T, T, d, bf16=True)
+    bits = (x.view(np.uint32) >> 16).astype(np.uint16)
+    with gL:
+        dx = DeviceArray.from_host(bits)
+        out = DeviceArray((T, d), np.float32, fill=0)
+        gL.forward_device(dx.ptr, capi.ACT_BF16, T, out.ptr)
+        idx, w, *_ = gL.last_routing(T)
+        o_idx, o_w = oL.route_tokens(x)
+        assert (idx == o_idx).all(), f"{(idx != o_idx).any(axis=1).sum()} tokens routed differently"
+        assert ulp_diff(w, o_w).max() <= 1
+
+
 def test_router_engineered_ties(ora):
     """Duplicate router rows give exactly equal weights; the lower index must win."""
     E, k, d, T = 8, 2, 64, 40
@@ -484,31 +524,32 @@ def test_router_f32_valued_rows_on_blocked_layers(ora, E, k, d, T, gated):
         assert ulp_diff(w, o_w).max() <= 1
 
 
-def test_host_entry_in_chunks_equals_the_device_entry(ora):
-    """From 4096 tokens on the host-buffer entry point stages the batch through page-locked
-    memory in chunks of 1024 tokens whose copies overlap the kernels of other chunks.  Tokens
-    are independent, so every row must equal what the device entry point gives for the same
-    chunk of tokens bit for bit, a ragged last chunk included, and sampled rows must sit within
-    the layer bar of the f64 reference."""
+def test_host_entry_staged_copies_equal_the_device_entry(ora):
+    """From 2048 tokens on the host-buffer entry point moves the batch through page-locked
+    staging in chunks of 1024 tokens (copy engine and calling thread work on alternate slots) and
+    runs one forward over the whole batch: the result must equal the device entry point's bit
+    for bit, a ragged last chunk included, the taps must describe the whole batch, and sampled
+    rows must sit within the layer bar of the f64 reference."""
     E, k, d, f = 8, 2, 128, 256
     W = S.make_weights(31, E, d, f, f_s=64)
     oL, gL = S.build_pair(ora, W, k, capi.CONVENTION_ATENIA, capi.WEIGHT_BF16)
-    T = 4 * 1024 + 333
-    x = S.make_tokens(32, T, d, bf16=True)
-    with gL:
-        out = gL.forward(x).reshape(T, d)
-        assert gL.status()[0] == 0
-        for c0 in (0, 1024, 3072, 4096):
-            n = min(1024, T - c0)
-            dx = DeviceArray.from_host(x[c0:c0 + n])
-            dy = DeviceArray((n, d), np.float32, fill=0)
-            gL.forward_device(dx.ptr, capi.ACT_F32, n, dy.ptr)
-            assert dy.to_host().tobytes() == out[c0:c0 + n].tobytes(), f"chunk at {c0}"
-        o_idx, _ = oL.route_tokens(x[::509])
-        for i, t in enumerate(range(0, T, 509)):
-            ref = oL.forward_f64(x[t], fixed_idx=o_idx[i])
-            assert S.rel_err(out[t], ref) <= TOL_BF16
-        # a second call reuses the staging; a small batch afterwards takes the direct path
-        assert gL.forward(x).reshape(T, d).tobytes() == out.tobytes()
-        small = gL.forward(x[:7]).reshape(7, d)  # other kernels: close, not the same bits
-        assert max(S.rel_err(small[i], out[i]) for i in range(7)) <= 2 * TOL_BF16
+    for T in (2048, 4 * 1024 + 333):
+        x = S.make_tokens(32 + T, T, d, bf16=True)
+        with S.build_pair(ora, W, k, capi.CONVENTION_ATENIA, capi.WEIGHT_BF16)[1] as g2:
+            out = g2.forward(x).reshape(T, d)
+            assert g2.status()[0] == 0
+            idx, *_ = g2.last_routing(T)
+            o_idx, _ = oL.route_tokens(x)
+            assert (idx == o_idx).all()
+            dx = DeviceArray.from_host(x)
+            dy = DeviceArray((T, d), np.float32, fill=0)
+            g2.forward_device(dx.ptr, capi.ACT_F32, T, dy.ptr)
+            assert dy.to_host().tobytes() == out.tobytes()
+            for t in range(0, T, 509):
+                ref = oL.forward_f64(x[t], fixed_idx=o_idx[t])
+                assert S.rel_err(out[t], ref) <= TOL_BF16
+            # a second call reuses the staging; a small batch afterwards takes the direct path
+            assert g2.forward(x).reshape(T, d).tobytes() == out.tobytes()
+            small = g2.forward(x[:7]).reshape(7, d)  # other kernels: close, not the same bits
+            assert max(S.rel_err(small[i], out[i]) for i in range(7)) <= 2 * TOL_BF16
+    gL.close() if hasattr(gL, "close") else None
