@@ -185,14 +185,18 @@ __global__ __launch_bounds__(256) void ffn_f32_mfma_kernel(
   struct Chunk {
     float4 lo, hi;
   };
+  // No branch around a load: with one the compiler cannot count the loads in flight any more
+  // and waits for all of them before every use (one memory round trip per step).  A chunk past
+  // the end of a row (k_cols is a multiple of 8: a chunk is whole or absent) is fetched from the
+  // row's first columns and zeroed with selects; a step past the wave's range repeats its last.
   auto load8 = [&](const float* p, int st) {
     Chunk c;
-    if (st * 32 + 8 * q < k_cols) {  // k_cols is a multiple of 8: a chunk is whole or absent
-      c.lo = *(const float4*)(p + (size_t)st * 32);
-      c.hi = *(const float4*)(p + (size_t)st * 32 + 4);
-    } else {
-      c.lo = c.hi = make_float4(0.f, 0.f, 0.f, 0.f);
-    }
+    const bool in = st * 32 + 8 * q < k_cols;
+    const size_t off = in ? (size_t)st * 32 : 0;
+    c.lo = *(const float4*)(p + off);
+    c.hi = *(const float4*)(p + off + 4);
+    c.lo.x = in ? c.lo.x : 0.f; c.lo.y = in ? c.lo.y : 0.f; c.lo.z = in ? c.lo.z : 0.f; c.lo.w = in ? c.lo.w : 0.f;
+    c.hi.x = in ? c.hi.x : 0.f; c.hi.y = in ? c.hi.y : 0.f; c.hi.z = in ? c.hi.z : 0.f; c.hi.w = in ? c.hi.w : 0.f;
     return c;
   };
   auto elem = [](const Chunk& c, int t) {
@@ -201,11 +205,11 @@ __global__ __launch_bounds__(256) void ffn_f32_mfma_kernel(
   };
   Chunk wA[2], wB[2], xs[2][MT] = {};
   auto load_step = [&](int buf, int st) {
+    st = min(st, s1 - 1);
     wA[buf] = load8(pa, st);
     if (UP) wB[buf] = load8(pb, st);
 #pragma unroll
-    for (int i = 0; i < MT; ++i)
-      if (i < mt_live) xs[buf][i] = load8(px[i], st);
+    for (int i = 0; i < MT; ++i) xs[buf][i] = load8(px[i], st);  // rows past the end: clamped
   };
   auto multiply = [&](int buf) {
 #pragma unroll
@@ -221,12 +225,14 @@ __global__ __launch_bounds__(256) void ffn_f32_mfma_kernel(
       }
     }
   };
-  if (s0 < s1) load_step(0, s0);
-  for (int st = s0; st < s1; st += 2) {
-    if (st + 1 < s1) load_step(1, st + 1);
-    multiply(0);
-    if (st + 2 < s1) load_step(0, st + 2);
-    if (st + 1 < s1) multiply(1);
+  if (s0 < s1) {
+    load_step(0, s0);
+    for (int st = s0; st < s1; st += 2) {
+      load_step(1, st + 1);
+      multiply(0);
+      load_step(0, st + 2);
+      if (st + 1 < s1) multiply(1);  // a scalar branch around matrix instructions only
+    }
   }
 
   if (KS > 1) {  // partial sums of waves 1..3 to LDS, wave 0 adds them in wave order
