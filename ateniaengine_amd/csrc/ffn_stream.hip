@@ -13,6 +13,11 @@
 // loads in flight.  A workgroup owns one or two adjacent 16-row strips of W_g and W_u (four
 // waves) or of W_d (eight waves); its waves split K and reduce through LDS.  Token rows (A
 // operand) come from L2.
+//
+// Kernels: ffn_stream_kernel (any small batch, either phase; its SEL form also routes a single
+// token from the router's logits), ffn_down_decode1_kernel and ffn_down_combine1_kernel (one
+// token: the down projections of all its experts, of the shared expert, and the combine in one
+// launch), repack_blocks_kernel (load-time repack into the block layout).
 #include "moe_internal.h"
 
 #include "../../include/atenia_moe_hip.h"

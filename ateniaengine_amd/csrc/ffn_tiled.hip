@@ -13,8 +13,9 @@
 //   ffn_tiled_pipe_kernel     bf16 weights, K a multiple of 64 and >= 128: 4 x 4 tiles of
 //                             v_mfma_f32_32x32x16_bf16 per wave, operands go global -> LDS
 //                             directly (global_load_lds_dwordx4) into a ring of three 64-k A
-//                             stages and four 32-k B stages, software-pipelined in units of 16
-//                             MFMAs with one barrier per 32-k step
+//                             stages and three 32-k B stages, software-pipelined in units of 16
+//                             MFMAs with one barrier per 32-k step; row tiles of up to nine
+//                             32-row groups (the ninth in a ring and registers of its own)
 //   ffn_tiled_pipe_i8_kernel  INT8 W8A16, K >= 128: same pipeline, weights stay int8 into LDS and
 //                             are widened to bf16 in registers, row scale applied to the
 //                             accumulator
@@ -387,9 +388,10 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_kernel(TiledParams p) {
 
 // ---- bf16 form: direct global->LDS loads, multi-stage rings, software-pipelined k loop ------
 // Same 256 x 256 tiling on v_mfma_f32_32x32x16_bf16 (each wave 128 x 128 = 4 x 4 MFMA tiles).
-// LDS holds a ring of three 64-k A stages (32 KiB each) and a ring of four 32-k B stages
-// (16 KiB each).  A wave fills a 1 KiB chunk with one global_load_lds_dwordx4 (lane l's 16
-// bytes land at chunk + 16*l), so no operand passes through registers on its way to LDS.
+// LDS holds a ring of three 64-k A stages (32 KiB each), a ring of three 32-k B stages
+// (16 KiB each) and a ring of three 4 KiB stages for the ninth row group of a tall tile.  A
+// wave fills a 1 KiB chunk with one global_load_lds_dwordx4 (lane l's 16 bytes land at
+// chunk + 16*l), so no operand passes through registers on its way to LDS.
 // The k loop works in k16 units of 16 MFMAs: while one unit multiplies, the 8 fragment reads
 // of the next unit and 4 loads of a stage several steps ahead are issued between its MFMAs
 // (pinned with sched_barrier), and the single barrier per 32-k step sits between the two
@@ -474,7 +476,7 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p)
     if (nb >= p.n_blocks) nb = p.n_blocks - 1;
     bptr[q] = wbase + (size_t)e * p.w_stride_u4 + (size_t)nb * p.nkb * 64 + kh * 16 + (brow & 15);
   }
-  // The first four B stages are requested before anything that depends on the row list:
+  // The first B stages are requested before anything that depends on the row list:
   // weight tiles come from HBM (the longest latency of the prologue) and need nothing but
   // the tile coordinates, so they fly while the pair ids of the A rows are looked up.
   const int st_lo = (p.k_pad / 64) * part / n_parts, st_hi = (p.k_pad / 64) * (part + 1) / n_parts;
