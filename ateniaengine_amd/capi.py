@@ -21,6 +21,7 @@ CONVENTION_HUGGINGFACE_QWEN = 1
 WEIGHT_F32, WEIGHT_BF16, WEIGHT_INT8_W8A16, WEIGHT_INT8_PER_GROUP = 0, 1, 2, 3
 ACT_F32, ACT_BF16 = 0, 1
 POLICY_CERTIFIED, POLICY_STRICT, POLICY_FAST = 0, 1, 2
+KERNELS_STREAM, KERNELS_MID, KERNELS_TILED, KERNELS_F32 = 0, 1, 2, 3
 NORM_GRAPH_F32, NORM_F64 = 0, 1
 OK, ERR_SYNC, ERR_LAUNCH = 0, 1, 2
 ERR_DIM, ERR_K, ERR_NON_FINITE, ERR_OOM, ERR_HANDLE, ERR_UNSUPPORTED = -1, -2, -3, -4, -5, -6
@@ -36,7 +37,7 @@ EXPORTS = (
     "atenia_moe_hip_layer_permute", "atenia_moe_hip_layer_last_routing",
     "atenia_moe_hip_layer_last_expert_outputs", "atenia_moe_hip_layer_set_profiling",
     "atenia_moe_hip_layer_stage_ms", "atenia_moe_hip_layer_stage_launches",
-    "atenia_moe_hip_layer_info", "atenia_moe_quantize_per_row_i8",
+    "atenia_moe_hip_layer_info", "atenia_moe_hip_layer_expert_kernels", "atenia_moe_quantize_per_row_i8",
     "atenia_moe_f32_to_bf16_trunc",
     "atenia_moe_hip_layer_last_non_finite", "atenia_moe_router_launch_device", "atenia_moe_permute_launch_device",
     "atenia_moe_expert_ffn_launch_device", "atenia_moe_combine_launch_device",
@@ -109,6 +110,7 @@ def lib():
         L.atenia_moe_hip_layer_stage_ms.argtypes = [P, P]
         L.atenia_moe_hip_layer_stage_launches.argtypes = [P, P]
         L.atenia_moe_hip_layer_info.argtypes = [P, P]
+        L.atenia_moe_hip_layer_expert_kernels.argtypes = [P, C.c_int64, P]
         L.atenia_moe_quantize_per_row_i8.argtypes = [P, C.c_size_t, C.c_size_t, P, P]
         L.atenia_moe_f32_to_bf16_trunc.argtypes = [P, C.c_size_t, P]
         L.atenia_moe_hip_layer_last_non_finite.argtypes = [P, P, P]
@@ -409,6 +411,13 @@ class Layer:
         n = np.zeros(N_STAGES, dtype=np.int32)
         _check(lib().atenia_moe_hip_layer_stage_launches(self._h, _ptr(n)))
         return n
+
+    def expert_kernels(self, T: int):
+        """(routed, shared) kernel family a batch of T tokens takes: KERNELS_STREAM / _MID /
+        _TILED / _F32; shared is -1 for a layer without a shared expert."""
+        v = np.zeros(2, dtype=np.int32)
+        _check(lib().atenia_moe_hip_layer_expert_kernels(self._h, T, _ptr(v)))
+        return int(v[0]), int(v[1])
 
     def info(self) -> dict:
         v = np.zeros(8, dtype=np.int64)

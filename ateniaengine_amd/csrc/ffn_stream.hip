@@ -15,10 +15,14 @@
 // operand) come from L2.
 //
 // Kernels: ffn_stream_kernel (any small batch, either phase; its SEL form also routes a single
-// token from the router's logits), ffn_down_decode1_kernel and ffn_down_combine1_kernel (one
+// token from the router's logits), ffn_mid_kernel (batches whose experts see a few dozen rows
+// each: the token rows of a workgroup's eight or four waves go through LDS, up to 128 rows of an
+// expert per pass over its weights), ffn_down_decode1_kernel and ffn_down_combine1_kernel (one
 // token: the down projections of all its experts, of the shared expert, and the combine in one
 // launch), repack_blocks_kernel (load-time repack into the block layout).
 #include "moe_internal.h"
+
+#include <type_traits>
 
 #include "../../include/atenia_moe_hip.h"
 
@@ -47,6 +51,7 @@ struct StreamParams {
   int out_stride;
   GroupDesc g;
   InlineSelect sel;     // gate/up launch of a single token that routes it itself (logits != null)
+  int mid_rot;          // mid-batch kernel: workgroups start their walk over K at different stages
 };
 
 __device__ inline uint16_t bf16_rne(float f) {
@@ -612,6 +617,231 @@ __global__ __launch_bounds__(1024) void ffn_down_combine1_kernel(
   out[n] = o;
 }
 
+// Mid-batch form: experts that see a few dozen rows each.  Still bound by HBM (every weight
+// byte is read once per 128 rows of its expert, straight into B-operand registers), but with
+// that many rows the token rows can no longer come from L2 per wave: the NWV waves of a
+// workgroup share them through LDS.  A wave owns its B strips over the whole K -- W_g and W_u
+// of one strip in the gate/up phase, NBD adjacent strips of W_d in the down phase -- so there
+// is no reduction across waves.  The workgroup's up to 128 token rows (eight 16-row tiles, A
+// operand) pass through a ring of three LDS stages of JB weight blocks of k each (64 k with
+// bf16 pairs or single int8 blocks, 128 k with int8 pairs), written from registers that were
+// loaded one step earlier, one barrier per stage.  Only the row tiles that hold rows are staged
+// and multiplied: ML (2, 4, 6 or 8) is the number of row tiles of the main loop, and a
+// workgroup picks the smallest form that covers its rows (staging all 128 rows whatever the
+// group held doubled the traffic of the launch at 32 rows per expert).  Weight blocks are
+// requested NWB - 1 stages ahead into a ring of NWB register buffers.  Every load of the loop
+// is issued unconditionally with a clamped stage index: a branch around a load makes the
+// compiler wait for all loads in flight before every use.  16-byte chunk c of LDS row r sits
+// at c ^ swz(r), which spreads the rows a fragment read touches over all banks.
+template <bool INT8, bool UP, int NWV, int JB, int NWB, int NBD = 2>
+__global__ __launch_bounds__(64 * NWV, 8 / NWV) void ffn_mid_kernel(StreamParams p) {
+  constexpr int MT = 8, NB = UP ? 2 : NBD, NST = 3;
+  constexpr int KB = INT8 ? kKbInt8 : kKbBf16;
+  constexpr int CH = KB * JB / 8;  // 16-byte chunks per row and stage
+  constexpr int ROWS = 16 * MT;
+  __shared__ u32x4 lds_a[NST * ROWS * CH];
+
+  const int u = blockIdx.y;
+  if (u >= *p.g.n_active) return;
+  const int e = p.g.active[u];
+  const int base = p.g.offsets[e];
+  const int cnt = p.g.offsets[e + 1] - base;
+  const int m0 = blockIdx.z * ROWS;
+  if (m0 >= cnt) return;
+  const int mt_live = __builtin_amdgcn_readfirstlane(min(MT, (cnt - m0 + 15) >> 4));
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int kq = lane >> 4, mm = lane & 15;
+  const int n_strips = p.n_pad >> 4;
+  const int ns = p.nkb / JB;  // stages; the launcher admits K of whole stages only
+
+  // The wave's two B strips.  A strip past the end is clamped to the last one: loaded and
+  // multiplied like any other (the barriers need every wave), never stored.
+  int strip[NB];
+  const uint4* pw[NB];
+  if (UP) {
+    strip[0] = strip[1] = blockIdx.x * NWV + wave;
+    const size_t off = (size_t)e * p.w_stride_u4 + (size_t)min(strip[0], n_strips - 1) * p.nkb * 64 + lane;
+    pw[0] = p.wa + off;
+    pw[1] = p.wb + off;
+  } else {
+#pragma unroll
+    for (int t = 0; t < NB; ++t) {
+      strip[t] = (blockIdx.x * NWV + wave) * NB + t;
+      pw[t] = p.wa + (size_t)e * p.w_stride_u4 + (size_t)min(strip[t], n_strips - 1) * p.nkb * 64 + lane;
+    }
+  }
+  // Ring of NWB register buffers of weight blocks: stage st lives in buffer st % NWB and is
+  // requested NWB - 1 steps before it is multiplied.
+  u32x4 wr[NWB][NB][JB];
+  // Workgroups walk K from different first stages (and wrap around): launched together and
+  // paced by the same memory system, they would otherwise all read the same offset of their
+  // 2^n-byte-spaced strips at the same time, i.e. the same few memory channels.
+  const int rot = p.mid_rot ? (int)((blockIdx.x * 13u + blockIdx.y * 29u + blockIdx.z * 7u) % (unsigned)ns) : 0;
+  auto stage_of = [&](int st) {
+    const int sc = min(st, ns - 1) + rot;
+    return sc >= ns ? sc - ns : sc;
+  };
+  auto load_w = [&](u32x4 (&w)[NB][JB], int st) {
+    const int sc = stage_of(st);
+#pragma unroll
+    for (int t = 0; t < NB; ++t)
+#pragma unroll
+      for (int j = 0; j < JB; ++j)
+        w[t][j] = __builtin_nontemporal_load((const u32x4*)(pw[t] + (size_t)(sc * JB + j) * 64));
+  };
+#pragma unroll
+  for (int b = 0; b < NWB - 1; ++b) load_w(wr[b], b);
+
+  // Chunk c of row r is stored at c ^ swz(r): eight consecutive rows then cover all banks
+  // (rows of 128 bytes or more: r & 7; rows of 64 bytes pair up: (r >> 1) & 3).
+  auto swz = [](int r) { return CH >= 8 ? (r & 7) : ((r >> 1) & 3); };
+
+  f32x4 acc[NB][MT];
+#pragma unroll
+  for (int t = 0; t < NB; ++t)
+#pragma unroll
+    for (int i = 0; i < MT; ++i) acc[t][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const u32x4* frag = lds_a + mm * CH;
+  const int sw = swz(mm);  // = swz(16 i + mm)
+
+  auto run = [&](auto ml_c) {
+    constexpr int ML = decltype(ml_c)::value;
+    // Token rows of the 16 ML rows this form multiplies: the workgroup's threads share the
+    // chunks of a stage, CPT (a power of two) consecutive chunks of one row each; surplus
+    // threads repeat the first ones.  Rows past the end of the group repeat
+    // its first row (an MFMA output row depends on its own input row only, and those rows are
+    // never stored).
+    constexpr int NT = 64 * NWV, NCH = 16 * ML * CH;
+    constexpr int CPT = NCH <= NT ? 1 : NCH <= 2 * NT ? 2 : NCH <= 4 * NT ? 4 : 8;
+    static_assert(CH % CPT == 0 && CPT * NT >= NCH, "mid-kernel staging");
+    const int q0 = ((int)threadIdx.x * CPT) % NCH;
+    const int ar = q0 / CH, ac = q0 % CH;
+    int apos = m0 + ar;
+    if (apos >= cnt) apos = m0;
+    const size_t arow = UP ? (size_t)(p.g.perm[base + apos] / p.g.pair_div) : (size_t)(base + apos);
+    const u32x4* ag = (const u32x4*)(p.a + arow * p.a_stride) + ac;
+    auto load_a = [&](u32x4 (&ga)[CPT], int st) {
+      const int sc = stage_of(st);
+#pragma unroll
+      for (int c = 0; c < CPT; ++c) ga[c] = ag[(size_t)sc * CH + c];
+    };
+    auto store_a = [&](const u32x4 (&ga)[CPT], int slot) {
+#pragma unroll
+      for (int c = 0; c < CPT; ++c)
+        lds_a[(slot * ROWS + ar) * CH + ((ac + c) ^ swz(ar))] = ga[c];
+    };
+    auto compute = [&](const u32x4 (&w)[NB][JB], int slot) {
+      const u32x4* fs = frag + slot * ROWS * CH;
+#pragma unroll
+      for (int j = 0; j < JB; ++j) {
+        if (INT8) {
+          bf16x8 bl[NB], bh[NB];
+#pragma unroll
+          for (int t = 0; t < NB; ++t)
+            widen_i8x16(make_uint4(w[t][j].x, w[t][j].y, w[t][j].z, w[t][j].w), bl[t], bh[t]);
+#pragma unroll
+          for (int i = 0; i < ML; ++i) {
+            const u32x4 x0 = fs[16 * i * CH + ((j * 8 + 2 * kq) ^ sw)];
+            const u32x4 x1 = fs[16 * i * CH + ((j * 8 + 2 * kq + 1) ^ sw)];
+#pragma unroll
+            for (int t = 0; t < NB; ++t) {
+              acc[t][i] = mfma(*(const bf16x8*)&x0, bl[t], acc[t][i]);
+              acc[t][i] = mfma(*(const bf16x8*)&x1, bh[t], acc[t][i]);
+            }
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < ML; ++i) {
+            const u32x4 x = fs[16 * i * CH + ((j * 4 + kq) ^ sw)];
+#pragma unroll
+            for (int t = 0; t < NB; ++t) acc[t][i] = mfma(*(const bf16x8*)&x, *(const bf16x8*)&w[t][j], acc[t][i]);
+          }
+        }
+      }
+    };
+    // Step st: the registers hold the rows of stage st + 2, whose slot was read last in step
+    // st - 1 (every wave is past that step's barrier); the rows of stage st + 3 and the weights
+    // of stage st + NWB - 1 are requested, then stage st is multiplied.
+    u32x4 ga[CPT];
+    auto step = [&](const u32x4 (&wc)[NB][JB], u32x4 (&wl)[NB][JB], int st) {
+      store_a(ga, (st + 2) % NST);
+      load_a(ga, st + 3);
+      load_w(wl, st + NWB - 1);
+      if (st < ns) compute(wc, st % NST);
+      __syncthreads();
+    };
+    load_a(ga, 0);
+    store_a(ga, 0);
+    load_a(ga, 1);
+    store_a(ga, 1);
+    load_a(ga, 2);
+    __syncthreads();
+    for (int st = 0; st < ns; st += NWB) {
+#pragma unroll
+      for (int b = 0; b < NWB; ++b) step(wr[b], wr[(b + NWB - 1) % NWB], st + b);
+    }
+  };
+  if (mt_live <= 2)
+    run(std::integral_constant<int, 2>{});
+  else if (mt_live <= 4)
+    run(std::integral_constant<int, 4>{});
+  else if (mt_live <= 6)
+    run(std::integral_constant<int, 6>{});
+  else
+    run(std::integral_constant<int, 8>{});
+
+  // D layout: lane holds rows 4*kq + r (r = 0..3) of column mm.
+#pragma unroll
+  for (int t = 0; t < (UP ? 1 : NB); ++t) {
+    const int n = strip[t] * 16 + mm;
+    const bool n_ok = strip[t] < n_strips && n < p.n_rows;
+    float sa = 1.f, sb = 1.f;
+    if (INT8) {
+      sa = n_ok ? p.sa[(size_t)e * p.n_rows + n] : 0.f;
+      if (UP) sb = n_ok ? p.sb[(size_t)e * p.n_rows + n] : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      if (i < mt_live) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int pos = m0 + 16 * i + 4 * kq + r;
+          if (pos < cnt && strip[t] < n_strips) {
+            if (UP) {
+              const float g = acc[0][i][r] * sa;
+              const float uu = acc[1][i][r] * sb;
+              const float h = (g / (1.f + __expf(-g))) * uu;
+              ((uint16_t*)p.out)[(size_t)(base + pos) * p.out_stride + n] = bf16_rne(h);
+            } else if (n_ok) {
+              const int pair = p.g.perm[base + pos];
+              ((float*)p.out)[(size_t)pair * p.out_stride + n] = acc[t][i][r] * sa;
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+// Mid-batch launch.  Measured on the Mixtral shape (T = 64 ... 384): gate/up runs best as two
+// workgroups of four waves per compute unit (the prologue of one overlaps the stream of the
+// other) with 64-k stages and a weight ring of four (bf16) or six (int8) buffers; the down
+// projection has few strips (d / 16) and a long K, so it takes one strip per wave and eight
+// waves per workgroup: d / 128 workgroups per expert instead of d / 256.
+template <bool INT8, bool UP>
+hipError_t launch_mid(const StreamParams& p_in, int n_groups, int rows_max, hipStream_t s) {
+  StreamParams p = p_in;
+  p.mid_rot = 1;
+  const int n_strips = p.n_pad / 16;
+  const int per_wg = UP ? 4 : 8;
+  dim3 grid((n_strips + per_wg - 1) / per_wg, n_groups, (rows_max + 127) / 128);
+  if (UP)
+    ffn_mid_kernel<INT8, true, 4, INT8 ? 1 : 2, INT8 ? 6 : 4><<<grid, 256, 0, s>>>(p);
+  else
+    ffn_mid_kernel<INT8, false, 8, 2, 3, 1><<<grid, 512, 0, s>>>(p);
+  return hipGetLastError();
+}
+
 template <bool INT8, bool UP>
 hipError_t launch_stream(const StreamParams& p, int n_groups, int rows_max, hipStream_t s,
                          const StreamParams* shared) {
@@ -683,6 +913,7 @@ StreamParams stream_params_up(const FfnArgs& a) {
   p.out_stride = a.h_stride;
   p.g = a.g;
   p.sel = a.sel;
+  p.mid_rot = 0;
   return p;
 }
 StreamParams stream_params_down(const FfnArgs& a) {
@@ -704,6 +935,7 @@ StreamParams stream_params_down(const FfnArgs& a) {
   p.out_stride = a.y_stride;
   p.g = a.g;
   p.sel = InlineSelect{};
+  p.mid_rot = 0;
   return p;
 }
 // The shared expert can ride in the routed experts' launch when both stream (no tiles, no f32
@@ -716,9 +948,17 @@ bool can_fuse_shared(const FfnArgs& a, const FfnArgs* sh, bool down_phase) {
         !sh->use_tiled && sh->rows_max == a.rows_max &&
         (sh->gate.group_blocks > 0) == (a.gate.group_blocks > 0)))
     return false;
+  if (a.use_mid || sh->use_mid) return false;
   return !down_phase || sh->down.k_pad <= 2 * a.down.k_pad;
 }
 }  // namespace
+
+// K of whole stages (64 k for bf16 blocks, 128 k for int8 blocks), per-row scales.
+bool ffn_mid_supported(const WeightSet& w, int wdtype) {
+  if (wdtype == ATENIA_MOE_WEIGHT_F32 || w.group_blocks != 0) return false;
+  const int kb = wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16 ? kKbInt8 : kKbBf16;
+  return w.k_pad % (2 * kb) == 0 && w.k_pad >= 2 * kb && w.n_pad >= 16;
+}
 
 bool ffn_stream_fuses_shared(const FfnArgs& a, const FfnArgs& shared, bool down_phase) {
   return can_fuse_shared(a, &shared, down_phase);
@@ -729,6 +969,13 @@ hipError_t launch_ffn_up(const FfnArgs& a, hipStream_t s, const FfnArgs* shared)
   if (a.use_tiled) return launch_ffn_up_tiled(a, s);
   const bool int8 = a.wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
   const StreamParams p = stream_params_up(a);
+  if (a.use_mid) {
+    if (!ffn_mid_supported(a.gate, a.wdtype) || !ffn_mid_supported(a.up, a.wdtype) || p.g.idx1 ||
+        p.sel.logits)
+      return hipErrorInvalidValue;
+    return int8 ? launch_mid<true, true>(p, a.n_groups_max, a.rows_max, s)
+                : launch_mid<false, true>(p, a.n_groups_max, a.rows_max, s);
+  }
   StreamParams ps;
   const bool fuse = can_fuse_shared(a, shared, false);
   if (fuse) ps = stream_params_up(*shared);
@@ -741,6 +988,11 @@ hipError_t launch_ffn_down(const FfnArgs& a, hipStream_t s, const FfnArgs* share
   if (a.use_tiled) return launch_ffn_down_tiled(a, s);
   const bool int8 = a.wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
   const StreamParams p = stream_params_down(a);
+  if (a.use_mid) {
+    if (!ffn_mid_supported(a.down, a.wdtype) || p.g.idx1) return hipErrorInvalidValue;
+    return int8 ? launch_mid<true, false>(p, a.n_groups_max, a.rows_max, s)
+                : launch_mid<false, false>(p, a.n_groups_max, a.rows_max, s);
+  }
   StreamParams ps;
   const bool fuse = can_fuse_shared(a, shared, true);
   if (fuse) ps = stream_params_down(*shared);

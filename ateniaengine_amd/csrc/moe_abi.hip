@@ -462,6 +462,7 @@ int ensure_pg_copy(AteniaMoeLayer* L) {
 // Which expert kernels a batch of T tokens takes (a pure function of the layer and T).
 struct BatchPlan {
   bool routed_streams;  // weight-streaming kernels (decode) instead of the tiled ones
+  bool routed_mid;      // ... in their mid-batch form (token rows shared through LDS)
   bool pg_prefill;      // per-group int8 layer running the tiled kernels on its bf16 copy
   bool tall_tiles;      // row tiles of up to nine 32-row groups (bf16 pipelined kernels only)
 };
@@ -473,10 +474,38 @@ bool tall_tiles_enabled() {
   }();
   return v;
 }
+// Average rows per expert (T k / E) between which the mid-batch streaming kernel serves the
+// routed experts (and the shared one with them).  Measured cross-overs on MI355X, whole forward:
+// against the register-resident streaming kernel at 12-16 rows (Mixtral shape bf16 T = 64
+// 0.481 / 0.487 ms, int8 T = 48 0.262 / 0.274; Qwen1.5-MoE shape T = 128 0.304 / 0.302;
+// DeepSeek-V2-Lite shape T = 128 0.259 / 0.280), against the tiled kernels at 48-68 rows for
+// bf16 (Mixtral T = 192 0.522 / 0.540, T = 224 equal; Qwen T = 1024 0.467 / 0.482; DeepSeek
+// T = 512 0.386 / 0.411, T = 1024 0.579 / 0.534) and at about 110 rows for int8, whose tiled
+// kernel widens every weight in the VALU (Mixtral int8 T = 192 0.346 / 0.526, T = 320
+// 0.467 / 0.535, T = 448 0.562 / 0.572).  Tuning knobs ATENIA_MOE_MID_MIN_AVG /
+// ATENIA_MOE_MID_MAX_AVG (read once; a maximum of 0 switches the kernel off).
+double mid_avg_bound(bool upper, bool int8w) {
+  static const double lo = [] {
+    const char* e = getenv("ATENIA_MOE_MID_MIN_AVG");
+    return e ? atof(e) : 12.0;
+  }();
+  static const double hi = [] {
+    const char* e = getenv("ATENIA_MOE_MID_MAX_AVG");
+    return e ? atof(e) : -1.0;
+  }();
+  if (!upper) return lo;
+  return hi >= 0.0 ? hi : int8w ? 104.0 : 52.0;
+}
 BatchPlan plan_batch(const AteniaMoeLayer* L, int T) {
   const bool int8w = L->wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
   BatchPlan p;
   p.routed_streams = batch_streams(T, (long long)T * L->k, L->E, int8w ? 32 : 16);
+  const double avg = (double)T * L->k / L->E;
+  p.routed_mid = T > kStreamMaxTokens && L->group_size == 0 &&
+                 stream_max_tokens_override() == 0 && avg >= mid_avg_bound(false, int8w) &&
+                 avg <= mid_avg_bound(true, int8w) && ffn_mid_supported(L->gate, L->wdtype) &&
+                 ffn_mid_supported(L->up, L->wdtype) && ffn_mid_supported(L->down, L->wdtype);
+  if (p.routed_mid) p.routed_streams = true;
   p.pg_prefill = L->group_size > 0 && !p.routed_streams && L->d_kpad % 64 == 0 &&
                  L->f_kpad % 64 == 0 && (L->fs == 0 || L->fs_kpad % 64 == 0);
   // both phases of the routed experts on the bf16 pipelined kernel (K a multiple of 64, >= 128)
@@ -689,6 +718,7 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   const bool tiled = !routed_streams && tiled_supported(fa.gate, ffn_dtype) &&
                      tiled_supported(fa.down, ffn_dtype);
   fa.use_tiled = tiled;
+  fa.use_mid = plan.routed_mid;
   fa.tile_group = V.tile_group;
   fa.tile_m0 = V.tile_m0;
   fa.n_tiles = V.shared_desc + 4;
@@ -727,8 +757,12 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
     // The shared expert follows the routed ones (it then rides in their launches): it is small
     // next to E routed experts, so its extra passes (one per 32 tokens) cost less than the
     // launches of its own that the tiled form would need.
-    fsd.use_tiled = !routed_streams && tiled_supported(fsd.gate, ffn_dtype) &&
-                    tiled_supported(fsd.down, ffn_dtype);
+    // (With the routed experts on the mid-batch kernel it takes that kernel too, one pass over
+    // its weights per 128 tokens; if its widths do not fit that kernel, the tiled ones.)
+    fsd.use_mid = plan.routed_mid && ffn_mid_supported(fsd.gate, ffn_dtype) &&
+                  ffn_mid_supported(fsd.up, ffn_dtype) && ffn_mid_supported(fsd.down, ffn_dtype);
+    fsd.use_tiled = (!routed_streams || (plan.routed_mid && !fsd.use_mid)) &&
+                    tiled_supported(fsd.gate, ffn_dtype) && tiled_supported(fsd.down, ffn_dtype);
     fsd.tile_group = V.s_tile_group;
     fsd.tile_m0 = V.s_tile_m0;
     fsd.n_tiles = V.shared_desc + 5;
@@ -1547,6 +1581,42 @@ int atenia_moe_hip_layer_stage_launches(AteniaMoeLayer* L, int32_t n[ATENIA_MOE_
   if (!n) return fail(ATENIA_MOE_ERR_DIM, "null pointer");
   std::lock_guard<std::mutex> lock(L->mu);
   for (int i = 0; i < ATENIA_MOE_N_STAGES; ++i) n[i] = L->launches[i];
+  return ATENIA_MOE_OK;
+}
+
+int atenia_moe_hip_layer_expert_kernels(const AteniaMoeLayer* L, int64_t n_tokens,
+                                        int32_t family[2]) {
+  if (!valid_handle(L)) return fail(ATENIA_MOE_ERR_HANDLE, "invalid layer handle");
+  if (!family) return fail(ATENIA_MOE_ERR_DIM, "null pointer");
+  if (n_tokens <= 0 || n_tokens > INT32_MAX) return fail(ATENIA_MOE_ERR_DIM, "n_tokens = %lld", (long long)n_tokens);
+  const int T = (int)n_tokens;
+  if (L->wdtype == ATENIA_MOE_WEIGHT_F32) {
+    family[0] = ATENIA_MOE_KERNELS_F32;
+    family[1] = L->fs > 0 ? ATENIA_MOE_KERNELS_F32 : -1;
+    return ATENIA_MOE_OK;
+  }
+  // the same decisions run_forward takes
+  const BatchPlan plan = plan_batch(L, T);
+  const int dt = plan.pg_prefill ? ATENIA_MOE_WEIGHT_BF16 : L->wdtype;
+  const WeightSet& g = plan.pg_prefill ? L->gate_b : L->gate;
+  const WeightSet& dn = plan.pg_prefill ? L->down_b : L->down;
+  const bool tiled = !plan.routed_streams && tiled_supported(g, dt) && tiled_supported(dn, dt);
+  family[0] = plan.routed_mid ? ATENIA_MOE_KERNELS_MID
+              : tiled         ? ATENIA_MOE_KERNELS_TILED
+                              : ATENIA_MOE_KERNELS_STREAM;
+  family[1] = -1;
+  if (L->fs > 0) {
+    const WeightSet& sg = plan.pg_prefill ? L->s_gate_b : L->s_gate;
+    const WeightSet& su = plan.pg_prefill ? L->s_up_b : L->s_up;
+    const WeightSet& sd = plan.pg_prefill ? L->s_down_b : L->s_down;
+    const bool s_mid = plan.routed_mid && ffn_mid_supported(sg, dt) && ffn_mid_supported(su, dt) &&
+                       ffn_mid_supported(sd, dt);
+    const bool s_tiled = (!plan.routed_streams || (plan.routed_mid && !s_mid)) &&
+                         tiled_supported(sg, dt) && tiled_supported(sd, dt);
+    family[1] = s_mid ? ATENIA_MOE_KERNELS_MID
+                : s_tiled ? ATENIA_MOE_KERNELS_TILED
+                          : ATENIA_MOE_KERNELS_STREAM;
+  }
   return ATENIA_MOE_OK;
 }
 

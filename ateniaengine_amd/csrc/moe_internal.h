@@ -151,6 +151,9 @@ struct FfnArgs {
   size_t y_part_stride;  // elements
   uint8_t* part_flags;
   int n_cus;             // compute units of the device
+  // Streaming family only: the mid-batch kernel (token rows shared through LDS, up to 128 rows
+  // of an expert per pass) instead of the register-resident one; needs ffn_mid_supported().
+  int use_mid;
   // tiled kernels only
   int use_tiled;
   const int32_t* tile_group;
@@ -171,6 +174,8 @@ struct FfnArgs {
   InlineSelect sel;
 };
 bool tiled_supported(const WeightSet& w, int wdtype);
+// Whether these weights (one projection family) can go through the mid-batch streaming kernel.
+bool ffn_mid_supported(const WeightSet& w, int wdtype);
 // True when the tiled down launch for these weights can split the k range of tail tiles.
 bool tiled_down_splits_tail(const WeightSet& down, int wdtype);
 hipError_t launch_ffn_up_tiled(const FfnArgs& a, hipStream_t s);

@@ -29,6 +29,10 @@ pub const ATENIA_MOE_POLICY_CERTIFIED: c_int = 0;
 pub const ATENIA_MOE_POLICY_STRICT: c_int = 1;
 pub const ATENIA_MOE_POLICY_FAST: c_int = 2;
 pub const ATENIA_MOE_N_STAGES: usize = 6;
+pub const ATENIA_MOE_KERNELS_STREAM: i32 = 0;
+pub const ATENIA_MOE_KERNELS_MID: i32 = 1;
+pub const ATENIA_MOE_KERNELS_TILED: i32 = 2;
+pub const ATENIA_MOE_KERNELS_F32: i32 = 3;
 
 pub const ATENIA_MOE_OK: c_int = 0;
 pub const ATENIA_MOE_ERR_SYNC: c_int = 1;
@@ -221,6 +225,11 @@ unsafe extern "C" {
         policy: c_int,
     ) -> c_int;
     pub fn atenia_moe_hip_layer_info(layer: *const AteniaMoeLayer, info: *mut i64) -> c_int;
+    pub fn atenia_moe_hip_layer_expert_kernels(
+        layer: *const AteniaMoeLayer,
+        n_tokens: i64,
+        family: *mut i32,
+    ) -> c_int;
     pub fn atenia_moe_quantize_per_row_i8(
         w: *const f32,
         rows: usize,
@@ -563,6 +572,16 @@ pub unsafe fn atenia_moe_hip_layer_set_numeric_policy(
 #[allow(unused_variables, clippy::missing_safety_doc)]
 pub unsafe fn atenia_moe_hip_layer_info(layer: *const AteniaMoeLayer, info: *mut i64) -> c_int {
     unreachable!("HIP symbol atenia_moe_hip_layer_info called in a build without atenia_hip")
+}
+
+#[cfg(not(atenia_hip))]
+#[allow(unused_variables, clippy::missing_safety_doc)]
+pub unsafe fn atenia_moe_hip_layer_expert_kernels(
+    layer: *const AteniaMoeLayer,
+    n_tokens: i64,
+    family: *mut i32,
+) -> c_int {
+    unreachable!("HIP symbol atenia_moe_hip_layer_expert_kernels called in a build without atenia_hip")
 }
 
 #[cfg(not(atenia_hip))]

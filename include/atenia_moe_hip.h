@@ -318,6 +318,18 @@ int atenia_moe_hip_layer_set_numeric_policy(AteniaMoeLayer* layer, int policy);
  * weight_dtype, bytes of expert weights per routed expert as stored in HBM. */
 int atenia_moe_hip_layer_info(const AteniaMoeLayer* layer, int64_t info[8]);
 
+/* Which expert kernels a batch of `n_tokens` tokens takes on this layer (a pure function of the
+ * layer and the batch size, nothing is launched): family[0] for the routed experts, family[1]
+ * for the shared expert (-1 without one).  No counterpart in the reference, whose CPU path has
+ * one expert loop (src/moe/layer.rs:405-443); a host uses it to see where its batch sizes fall
+ * and tests use it to know which kernel they exercised. */
+#define ATENIA_MOE_KERNELS_STREAM 0 /* weights streamed once, token rows in registers (decode) */
+#define ATENIA_MOE_KERNELS_MID 1    /* weights streamed once per 128 rows, token rows through LDS */
+#define ATENIA_MOE_KERNELS_TILED 2  /* 256-row tiles, matrix-core bound (prefill) */
+#define ATENIA_MOE_KERNELS_F32 3    /* f32 weights, f64 or f32 accumulation */
+int atenia_moe_hip_layer_expert_kernels(const AteniaMoeLayer* layer, int64_t n_tokens,
+                                        int32_t family[2]);
+
 /* Host-side weight preparation (load time, no GPU involved) ------------------------------ */
 
 /* Per-output-row symmetric int8 quantisation, bit-identical to `quantize_per_row_i8`

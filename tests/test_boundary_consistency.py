@@ -17,7 +17,7 @@ CRATE = os.path.join(ROOT, "ffi", "atenia-moe-hip-sys")
 MAKEFILE = os.path.join(ROOT, "ateniaengine_amd", "csrc", "Makefile")
 
 C_TO_RUST = {
-    "int": "c_int", "float": "f32", "double": "f64", "size_t": "usize",
+    "int": "c_int", "float": "f32", "double": "f64", "size_t": "usize", "int64_t": "i64",
     "const char*": "*const c_char", "const float*": "*const f32", "float*": "*mut f32",
     "const void*": "*const c_void", "void*": "*mut c_void", "int32_t*": "*mut i32",
     "const int32_t*": "*const i32", "int8_t*": "*mut i8", "uint16_t*": "*mut u16",
@@ -72,7 +72,7 @@ def rust_bindings():
 
 def test_header_prototypes_parse():
     protos = header_prototypes()
-    assert len(protos) == 35
+    assert len(protos) == 36
     assert protos["atenia_moe_hip_layer_forward"] == (
         "c_int", ["*mut AteniaMoeLayer", "*const f32", "c_int", "*mut f32"])
 
