@@ -634,14 +634,22 @@ __global__ __launch_bounds__(1024) void ffn_down_combine1_kernel(
 // compiler wait for all loads in flight before every use.  16-byte chunk c of LDS row r sits
 // at c ^ swz(r), which spreads the rows a fragment read touches over all banks.
 template <bool INT8, bool UP, int NWV, int JB, int NWB, int NBD = 2>
-__global__ __launch_bounds__(64 * NWV, 8 / NWV) void ffn_mid_kernel(StreamParams p) {
+__global__ __launch_bounds__(64 * NWV, 8 / NWV) void ffn_mid_kernel(StreamParams p_routed,
+                                                                    StreamParams p_shared,
+                                                                    int with_shared) {
   constexpr int MT = 8, NB = UP ? 2 : NBD, NST = 3;
   constexpr int KB = INT8 ? kKbInt8 : kKbBf16;
   constexpr int CH = KB * JB / 8;  // 16-byte chunks per row and stage
   constexpr int ROWS = 16 * MT;
   __shared__ u32x4 lds_a[NST * ROWS * CH];
 
-  const int u = blockIdx.y;
+  // A shared expert rides in the same launch as blockIdx.y == 0 (its own weights, widths and
+  // rows: one group of all T tokens).  First in the grid, because its K can be twice the
+  // routed experts' and its workgroups should not be the ones that start last.
+  const bool sh = with_shared && blockIdx.y == 0;
+  const StreamParams& p = sh ? p_shared : p_routed;
+  if ((int)blockIdx.x * (UP ? NWV : NWV * NB) * 16 >= p.n_pad) return;  // grid spans the wider
+  const int u = sh ? 0 : (int)blockIdx.y - (with_shared ? 1 : 0);
   if (u >= *p.g.n_active) return;
   const int e = p.g.active[u];
   const int base = p.g.offsets[e];
@@ -829,16 +837,18 @@ __global__ __launch_bounds__(64 * NWV, 8 / NWV) void ffn_mid_kernel(StreamParams
 // projection has few strips (d / 16) and a long K, so it takes one strip per wave and eight
 // waves per workgroup: d / 128 workgroups per expert instead of d / 256.
 template <bool INT8, bool UP>
-hipError_t launch_mid(const StreamParams& p_in, int n_groups, int rows_max, hipStream_t s) {
-  StreamParams p = p_in;
-  p.mid_rot = 1;
-  const int n_strips = p.n_pad / 16;
+hipError_t launch_mid(const StreamParams& p_in, int n_groups, int rows_max, hipStream_t s,
+                      const StreamParams* shared) {
+  StreamParams p = p_in, ps = shared ? *shared : p_in;
+  p.mid_rot = ps.mid_rot = 1;
+  const int n_pad = shared && shared->n_pad > p.n_pad ? shared->n_pad : p.n_pad;
+  const int n_strips = n_pad / 16;
   const int per_wg = UP ? 4 : 8;
-  dim3 grid((n_strips + per_wg - 1) / per_wg, n_groups, (rows_max + 127) / 128);
+  dim3 grid((n_strips + per_wg - 1) / per_wg, n_groups + (shared ? 1 : 0), (rows_max + 127) / 128);
   if (UP)
-    ffn_mid_kernel<INT8, true, 4, INT8 ? 1 : 2, INT8 ? 6 : 4><<<grid, 256, 0, s>>>(p);
+    ffn_mid_kernel<INT8, true, 4, INT8 ? 1 : 2, INT8 ? 6 : 4><<<grid, 256, 0, s>>>(p, ps, shared != nullptr);
   else
-    ffn_mid_kernel<INT8, false, 8, 2, 3, 1><<<grid, 512, 0, s>>>(p);
+    ffn_mid_kernel<INT8, false, 8, 2, 3, 1><<<grid, 512, 0, s>>>(p, ps, shared != nullptr);
   return hipGetLastError();
 }
 
@@ -938,8 +948,8 @@ StreamParams stream_params_down(const FfnArgs& a) {
   p.mid_rot = 0;
   return p;
 }
-// The shared expert can ride in the routed experts' launch when both stream (no tiles, no f32
-// weights), are stored alike and see the same rows bound.
+// The shared expert can ride in the routed experts' launch when both stream with the same
+// kernel (no tiles, no f32 weights), are stored alike and see the same rows bound.
 // In the down phase a strip's K is the expert's width: a shared expert much wider than the
 // routed ones would make its strips the launch's critical path (measured: Qwen1.5-MoE, shared
 // 4x as wide, 20 us fused against 18 us as two launches), so it keeps its own launch then.
@@ -948,7 +958,7 @@ bool can_fuse_shared(const FfnArgs& a, const FfnArgs* sh, bool down_phase) {
         !sh->use_tiled && sh->rows_max == a.rows_max &&
         (sh->gate.group_blocks > 0) == (a.gate.group_blocks > 0)))
     return false;
-  if (a.use_mid || sh->use_mid) return false;
+  if (a.use_mid != sh->use_mid) return false;
   return !down_phase || sh->down.k_pad <= 2 * a.down.k_pad;
 }
 }  // namespace
@@ -973,8 +983,11 @@ hipError_t launch_ffn_up(const FfnArgs& a, hipStream_t s, const FfnArgs* shared)
     if (!ffn_mid_supported(a.gate, a.wdtype) || !ffn_mid_supported(a.up, a.wdtype) || p.g.idx1 ||
         p.sel.logits)
       return hipErrorInvalidValue;
-    return int8 ? launch_mid<true, true>(p, a.n_groups_max, a.rows_max, s)
-                : launch_mid<false, true>(p, a.n_groups_max, a.rows_max, s);
+    StreamParams pm;
+    const bool fuse_mid = can_fuse_shared(a, shared, false);
+    if (fuse_mid) pm = stream_params_up(*shared);
+    return int8 ? launch_mid<true, true>(p, a.n_groups_max, a.rows_max, s, fuse_mid ? &pm : nullptr)
+                : launch_mid<false, true>(p, a.n_groups_max, a.rows_max, s, fuse_mid ? &pm : nullptr);
   }
   StreamParams ps;
   const bool fuse = can_fuse_shared(a, shared, false);
@@ -990,8 +1003,11 @@ hipError_t launch_ffn_down(const FfnArgs& a, hipStream_t s, const FfnArgs* share
   const StreamParams p = stream_params_down(a);
   if (a.use_mid) {
     if (!ffn_mid_supported(a.down, a.wdtype) || p.g.idx1) return hipErrorInvalidValue;
-    return int8 ? launch_mid<true, false>(p, a.n_groups_max, a.rows_max, s)
-                : launch_mid<false, false>(p, a.n_groups_max, a.rows_max, s);
+    StreamParams pm;
+    const bool fuse_mid = can_fuse_shared(a, shared, true);
+    if (fuse_mid) pm = stream_params_down(*shared);
+    return int8 ? launch_mid<true, false>(p, a.n_groups_max, a.rows_max, s, fuse_mid ? &pm : nullptr)
+                : launch_mid<false, false>(p, a.n_groups_max, a.rows_max, s, fuse_mid ? &pm : nullptr);
   }
   StreamParams ps;
   const bool fuse = can_fuse_shared(a, shared, true);
