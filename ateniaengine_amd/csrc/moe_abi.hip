@@ -474,46 +474,61 @@ bool tall_tiles_enabled() {
   }();
   return v;
 }
-// Average rows per expert (T k / E) between which the mid-batch streaming kernel serves the
-// routed experts (and the shared one in the same launches).  Measured cross-overs on MI355X,
-// whole forward, mid-batch kernel / the other one:
-//  * against the register-resident streaming kernel at 12-16 rows without a shared expert
-//    (Mixtral shape bf16 T = 64 0.481 / 0.487 ms, int8 T = 48 0.262 / 0.274) and at about 6 rows
-//    with one, whose T rows cost the streaming kernel a pass per 32 tokens (DeepSeek-V2-Lite
-//    shape T = 64 0.168 / 0.198, T = 128 0.206 / 0.281; Qwen1.5-MoE shape T = 96 0.288 / 0.285,
-//    T = 128 0.289 / 0.302);
+// Batch sizes served by the mid-batch streaming kernel (routed experts, and the shared one in
+// the same launches): from `min_tokens` tokens and `lo` rows per expert on average (T k / E) up
+// to `hi` rows.  Measured cross-overs on MI355X, whole forward, mid-batch kernel / the other one:
+//  * against the register-resident streaming kernel, without a shared expert: bf16 at 14-16 rows
+//    (Mixtral shape T = 48 0.476 / 0.465 ms, T = 64 0.481 / 0.487, T = 96 0.491 / 0.529), int8 at
+//    8-10 rows (T = 32 0.281 / 0.274, T = 40 0.258 / 0.267, T = 56 0.262 / 0.287);
+//  * with a shared expert that rides in both phases, its T rows cost the streaming kernel a pass
+//    per 32 tokens: from 40 tokens whatever the routed experts see (DeepSeek-V2-Lite shape
+//    T = 32 0.139 / 0.143, T = 40 0.147 / 0.157, T = 64 0.168 / 0.198, T = 128 0.206 / 0.281);
+//    one that keeps its own down launch (Qwen1.5-MoE shape, 4x as wide as the routed experts)
+//    from about 8 rows (T = 56 0.269 / 0.258, T = 96 0.288 / 0.285, T = 128 0.289 / 0.302);
 //  * against the tiled kernels at 52-72 rows for bf16 (Mixtral T = 192 0.522 / 0.540, T = 224
 //    equal; Qwen T = 1024 0.468 / 0.479, T = 1536 0.555 / 0.541; DeepSeek T = 640 0.415 / 0.437,
 //    T = 768 equal) and at about 110 rows for int8, whose tiled kernel widens every weight in the
 //    VALU (Mixtral int8 T = 192 0.346 / 0.526, T = 320 0.467 / 0.535, T = 448 0.562 / 0.572).
-// Tuning knobs ATENIA_MOE_MID_MIN_AVG / ATENIA_MOE_MID_MAX_AVG (read once; a maximum of 0
-// switches the kernel off).
-double mid_avg_bound(bool upper, bool int8w, bool has_shared) {
-  static const double lo = [] {
+// Tuning knobs ATENIA_MOE_MID_MIN_AVG / ATENIA_MOE_MID_MAX_AVG (read once) replace lo and hi;
+// a maximum of 0 switches the kernel off.
+struct MidBounds {
+  int min_tokens;
+  double lo, hi;
+};
+MidBounds mid_bounds(const AteniaMoeLayer* L) {
+  static const double env_lo = [] {
     const char* e = getenv("ATENIA_MOE_MID_MIN_AVG");
     return e ? atof(e) : -1.0;
   }();
-  static const double hi = [] {
+  static const double env_hi = [] {
     const char* e = getenv("ATENIA_MOE_MID_MAX_AVG");
     return e ? atof(e) : -1.0;
   }();
-  if (!upper) return lo >= 0.0 ? lo : has_shared ? 6.0 : 12.0;
-  return hi >= 0.0 ? hi : int8w ? 104.0 : has_shared ? 68.0 : 52.0;
+  const bool int8w = L->wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
+  // a shared expert that the mid-batch kernel can take along, in the down phase too
+  const bool rides = L->fs > 0 && ffn_mid_supported(L->s_gate, L->wdtype) &&
+                     ffn_mid_supported(L->s_up, L->wdtype) && ffn_mid_supported(L->s_down, L->wdtype);
+  const bool rides_down = rides && L->s_down.k_pad <= 2 * L->down.k_pad;
+  MidBounds b;
+  b.min_tokens = rides_down || int8w ? 40 : kStreamMaxTokens + 1;
+  b.lo = rides_down ? 0.0 : rides ? 8.0 : int8w ? 10.0 : 14.0;
+  b.hi = int8w ? 104.0 : rides ? 68.0 : 52.0;
+  if (env_lo >= 0.0) b.lo = env_lo;
+  if (env_hi >= 0.0) b.hi = env_hi;
+  return b;
 }
 BatchPlan plan_batch(const AteniaMoeLayer* L, int T) {
   const bool int8w = L->wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
   BatchPlan p;
   p.routed_streams = batch_streams(T, (long long)T * L->k, L->E, int8w ? 32 : 16);
   const double avg = (double)T * L->k / L->E;
-  // a shared expert that the mid-batch kernel can take along
-  const bool shared_rides = L->fs > 0 && ffn_mid_supported(L->s_gate, L->wdtype) &&
-                            ffn_mid_supported(L->s_up, L->wdtype) &&
-                            ffn_mid_supported(L->s_down, L->wdtype);
-  p.routed_mid = T > kStreamMaxTokens && L->group_size == 0 &&
-                 stream_max_tokens_override() == 0 &&
-                 avg >= mid_avg_bound(false, int8w, shared_rides) &&
-                 avg <= mid_avg_bound(true, int8w, shared_rides) && ffn_mid_supported(L->gate, L->wdtype) &&
-                 ffn_mid_supported(L->up, L->wdtype) && ffn_mid_supported(L->down, L->wdtype);
+  p.routed_mid = false;
+  if (L->group_size == 0 && stream_max_tokens_override() == 0 &&
+      ffn_mid_supported(L->gate, L->wdtype) && ffn_mid_supported(L->up, L->wdtype) &&
+      ffn_mid_supported(L->down, L->wdtype)) {
+    const MidBounds b = mid_bounds(L);
+    p.routed_mid = T >= b.min_tokens && avg >= b.lo && avg <= b.hi;
+  }
   if (p.routed_mid) p.routed_streams = true;
   p.pg_prefill = L->group_size > 0 && !p.routed_streams && L->d_kpad % 64 == 0 &&
                  L->f_kpad % 64 == 0 && (L->fs == 0 || L->fs_kpad % 64 == 0);
