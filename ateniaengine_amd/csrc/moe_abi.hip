@@ -480,17 +480,17 @@ bool tall_tiles_enabled() {
 //  * against the register-resident streaming kernel, without a shared expert: bf16 at 14-16 rows
 //    (Mixtral shape T = 48 0.476 / 0.465 ms, T = 64 0.481 / 0.487, T = 96 0.491 / 0.529), int8 at
 //    8-10 rows (T = 32 0.281 / 0.274, T = 40 0.258 / 0.267, T = 56 0.262 / 0.287);
-//  * with a shared expert that rides in both phases, its T rows cost the streaming kernel a pass
-//    per 32 tokens: from 40 tokens whatever the routed experts see (DeepSeek-V2-Lite shape
-//    T = 32 0.139 / 0.143, T = 40 0.147 / 0.157, T = 64 0.168 / 0.198, T = 128 0.206 / 0.281);
-//    one that keeps its own down launch (Qwen1.5-MoE shape, 4x as wide as the routed experts)
-//    from about 8 rows (T = 56 0.269 / 0.258, T = 96 0.288 / 0.285, T = 128 0.289 / 0.302);
+//  * with a shared expert that the kernel takes along, whose T rows cost the streaming kernel
+//    a pass per 32 tokens: from 32 tokens whatever the routed experts see (DeepSeek-V2-Lite
+//    shape T = 24 0.133 / 0.132, T = 32 0.139 / 0.143, T = 64 0.168 / 0.198, T = 128
+//    0.206 / 0.281; Qwen1.5-MoE shape T = 24 0.200 / 0.203, T = 32 0.222 / 0.231, T = 56
+//    0.240 / 0.259, T = 128 0.268 / 0.302);
 //  * against the tiled kernels at 52-72 rows for bf16 (Mixtral T = 192 0.522 / 0.540, T = 224
 //    equal; Qwen T = 1024 0.468 / 0.479, T = 1536 0.555 / 0.541; DeepSeek T = 640 0.415 / 0.437,
 //    T = 768 equal) and at about 110 rows for int8, whose tiled kernel widens every weight in the
 //    VALU (Mixtral int8 T = 192 0.346 / 0.526, T = 320 0.467 / 0.535, T = 448 0.562 / 0.572).
-// Tuning knobs ATENIA_MOE_MID_MIN_AVG / ATENIA_MOE_MID_MAX_AVG (read once) replace lo and hi;
-// a maximum of 0 switches the kernel off.
+// Tuning knobs ATENIA_MOE_MID_MIN_TOKENS / ATENIA_MOE_MID_MIN_AVG / ATENIA_MOE_MID_MAX_AVG (read
+// once) replace the three bounds; a maximum of 0 switches the kernel off.
 struct MidBounds {
   int min_tokens;
   double lo, hi;
@@ -504,17 +504,21 @@ MidBounds mid_bounds(const AteniaMoeLayer* L) {
     const char* e = getenv("ATENIA_MOE_MID_MAX_AVG");
     return e ? atof(e) : -1.0;
   }();
+  static const int env_min_tokens = [] {
+    const char* e = getenv("ATENIA_MOE_MID_MIN_TOKENS");
+    return e ? atoi(e) : 0;
+  }();
   const bool int8w = L->wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
-  // a shared expert that the mid-batch kernel can take along, in the down phase too
+  // a shared expert that the mid-batch kernel can take along
   const bool rides = L->fs > 0 && ffn_mid_supported(L->s_gate, L->wdtype) &&
                      ffn_mid_supported(L->s_up, L->wdtype) && ffn_mid_supported(L->s_down, L->wdtype);
-  const bool rides_down = rides && L->s_down.k_pad <= 2 * L->down.k_pad;
   MidBounds b;
-  b.min_tokens = rides_down || int8w ? 40 : kStreamMaxTokens + 1;
-  b.lo = rides_down ? 0.0 : rides ? 8.0 : int8w ? 10.0 : 14.0;
+  b.min_tokens = rides ? 32 : int8w ? 40 : kStreamMaxTokens + 1;
+  b.lo = rides ? 0.0 : int8w ? 10.0 : 14.0;
   b.hi = int8w ? 104.0 : rides ? 68.0 : 52.0;
   if (env_lo >= 0.0) b.lo = env_lo;
   if (env_hi >= 0.0) b.hi = env_hi;
+  if (env_min_tokens > 0) b.min_tokens = env_min_tokens;
   return b;
 }
 BatchPlan plan_batch(const AteniaMoeLayer* L, int T) {
