@@ -463,6 +463,7 @@ int ensure_pg_copy(AteniaMoeLayer* L) {
 struct BatchPlan {
   bool routed_streams;  // weight-streaming kernels (decode) instead of the tiled ones
   bool routed_mid;      // ... in their mid-batch form (token rows shared through LDS)
+  bool mid_down;        // the down phase alone takes the mid-batch form (gate/up streams from registers)
   bool pg_prefill;      // per-group int8 layer running the tiled kernels on its bf16 copy
   bool tall_tiles;      // row tiles of up to nine 32-row groups (bf16 pipelined kernels only)
 };
@@ -481,10 +482,11 @@ bool tall_tiles_enabled() {
 //    (Mixtral shape T = 48 0.476 / 0.465 ms, T = 64 0.481 / 0.487, T = 96 0.491 / 0.529), int8 at
 //    8-10 rows (T = 32 0.281 / 0.274, T = 40 0.258 / 0.267, T = 56 0.262 / 0.287);
 //  * with a shared expert that the kernel takes along, whose T rows cost the streaming kernel
-//    a pass per 32 tokens: from 32 tokens whatever the routed experts see (DeepSeek-V2-Lite
-//    shape T = 24 0.133 / 0.132, T = 32 0.139 / 0.143, T = 64 0.168 / 0.198, T = 128
-//    0.206 / 0.281; Qwen1.5-MoE shape T = 24 0.200 / 0.203, T = 32 0.222 / 0.231, T = 56
-//    0.240 / 0.259, T = 128 0.268 / 0.302);
+//    a pass per 32 tokens: from 40 tokens whatever the routed experts see (DeepSeek-V2-Lite
+//    shape T = 24 0.133 / 0.132, T = 40 0.147 / 0.157, T = 64 0.168 / 0.198, T = 128
+//    0.206 / 0.281; Qwen1.5-MoE shape T = 24 0.200 / 0.203, T = 40 0.230 / 0.247, T = 56
+//    0.240 / 0.259, T = 128 0.268 / 0.302; below 40 tokens the gate/up phase of the
+//    register-resident kernel is the faster one, Qwen T = 32 108 against 117 us);
 //  * against the tiled kernels at 52-72 rows for bf16 (Mixtral T = 192 0.522 / 0.540, T = 224
 //    equal; Qwen T = 1024 0.468 / 0.479, T = 1536 0.555 / 0.541; DeepSeek T = 640 0.415 / 0.437,
 //    T = 768 equal) and at about 110 rows for int8, whose tiled kernel widens every weight in the
@@ -513,7 +515,7 @@ MidBounds mid_bounds(const AteniaMoeLayer* L) {
   const bool rides = L->fs > 0 && ffn_mid_supported(L->s_gate, L->wdtype) &&
                      ffn_mid_supported(L->s_up, L->wdtype) && ffn_mid_supported(L->s_down, L->wdtype);
   MidBounds b;
-  b.min_tokens = rides ? 32 : int8w ? 40 : kStreamMaxTokens + 1;
+  b.min_tokens = rides || int8w ? 40 : kStreamMaxTokens + 1;
   b.lo = rides ? 0.0 : int8w ? 10.0 : 14.0;
   b.hi = int8w ? 104.0 : rides ? 68.0 : 52.0;
   if (env_lo >= 0.0) b.lo = env_lo;
@@ -527,11 +529,19 @@ BatchPlan plan_batch(const AteniaMoeLayer* L, int T) {
   p.routed_streams = batch_streams(T, (long long)T * L->k, L->E, int8w ? 32 : 16);
   const double avg = (double)T * L->k / L->E;
   p.routed_mid = false;
+  p.mid_down = false;
   if (L->group_size == 0 && stream_max_tokens_override() == 0 &&
       ffn_mid_supported(L->gate, L->wdtype) && ffn_mid_supported(L->up, L->wdtype) &&
       ffn_mid_supported(L->down, L->wdtype)) {
     const MidBounds b = mid_bounds(L);
     p.routed_mid = T >= b.min_tokens && avg >= b.lo && avg <= b.hi;
+    // Below those bounds the down phase still gains from the mid-batch form from 20 tokens on:
+    // it has d / 16 strips only, which that form spreads over d / 128 workgroups of eight waves
+    // that each own a strip over the whole K (no reduction through LDS), and a shared expert's
+    // down projection rides along.  Down launch, mid-batch / register-resident: Qwen1.5-MoE
+    // shape T = 20 65 / 75 us, T = 12 62 / 54; DeepSeek-V2-Lite T = 20 39 / 44, T = 12 37 / 36;
+    // Mixtral int8 T = 24 79 / 83, T = 48 80 / 97; Mixtral bf16 T = 24 142 / 144, T = 56 145 / 157.
+    p.mid_down = !p.routed_mid && p.routed_streams && T >= 20 && avg <= b.hi && b.hi > 0.0;
   }
   if (p.routed_mid) p.routed_streams = true;
   p.pg_prefill = L->group_size > 0 && !p.routed_streams && L->d_kpad % 64 == 0 &&
@@ -801,7 +811,6 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
 
   // Small batches stream both the routed experts and the shared one: one launch per phase.
   const bool fuse_shared_up = L->fs > 0 && ffn_stream_fuses_shared(fa, fsd, false);
-  const bool fuse_shared_down = L->fs > 0 && ffn_stream_fuses_shared(fa, fsd, true);
   if (first <= kStageFfn) {
     HIP_TRY(launch_ffn_up(fa, s, fuse_shared_up ? &fsd : nullptr));
     L->launches[2] = 1;
@@ -811,6 +820,12 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
     }
   }
   tm.mark();  // ev[3]: gate/up done
+  if (plan.mid_down) {  // the down phase alone in the mid-batch form
+    fa.use_mid = 1;
+    if (L->fs > 0)
+      fsd.use_mid = !fsd.use_tiled && ffn_mid_supported(fsd.down, ffn_dtype);
+  }
+  const bool fuse_shared_down = L->fs > 0 && ffn_stream_fuses_shared(fa, fsd, true);
   // One token, whole pipeline requested: the down launch covers the routed experts and the
   // shared one and finishes the combine as well (one launch instead of two or three).
   const bool fuse1 = first <= kStageFfn && last >= kStageCombine && L->group_size == 0 &&

@@ -320,7 +320,7 @@ int atenia_moe_hip_layer_info(const AteniaMoeLayer* layer, int64_t info[8]);
 
 /* Which expert kernels a batch of `n_tokens` tokens takes on this layer (a pure function of the
  * layer and the batch size, nothing is launched): family[0] for the routed experts, family[1]
- * for the shared expert (-1 without one).  No counterpart in the reference, whose CPU path has
+ * for the shared expert (-1 without one); where the two phases differ, that of the gate/up phase.  No counterpart in the reference, whose CPU path has
  * one expert loop (src/moe/layer.rs:405-443); a host uses it to see where its batch sizes fall
  * and tests use it to know which kernel they exercised. */
 #define ATENIA_MOE_KERNELS_STREAM 0 /* weights streamed once, token rows in registers (decode) */
