@@ -48,3 +48,50 @@ def test_random_layer(ora, E, k, d, f, fs, gated, conv, wd, T, seed):
         # a second, smaller batch on the same handle (grow-only workspace, stale state)
         T2 = max(1, T // 3)
         check_layer(ora, oL, gL, x[:T2], tol, sample=None if T2 <= 64 else range(0, T2, max(1, T2 // 40)))
+
+
+def _mid_cases(n, seed):
+    """Shapes the mid-batch kernel can take (K in whole 64-k / 128-k stages) at batch sizes inside
+    and on both sides of its bounds, with and without a shared expert it can take along."""
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(n):
+        wd = [capi.WEIGHT_BF16, capi.WEIGHT_INT8_W8A16][i % 2]
+        step = 128 if wd == capi.WEIGHT_INT8_W8A16 else 64
+        E = int(rng.choice([2, 4, 8, 16, 60]))
+        k = int(rng.integers(1, min(E, 6) + 1))
+        d = step * int(rng.integers(1, 4))
+        f = step * int(rng.integers(1, 6))
+        shared = bool(rng.integers(0, 2))
+        fs = (step * int(rng.integers(1, 9)) if rng.integers(0, 4) else 72) if shared else 0
+        gated = shared and bool(rng.integers(0, 2))
+        conv = int(rng.integers(0, 2)) if shared else 0
+        rows = float(rng.choice([3, 8, 14, 20, 35, 50, 70, 100, 130]))  # per expert on average
+        T = int(min(900, max(20, round(rows * E / k + rng.integers(-2, 3)))))
+        out.append(pytest.param(E, k, d, f, fs, gated, conv, wd, T, 3000 + i,
+                                id=f"{i}-E{E}k{k}d{d}f{f}s{fs}g{int(gated)}c{conv}w{wd}T{T}"))
+    return out
+
+
+_MID_SEEN = []
+
+
+@pytest.mark.parametrize("E,k,d,f,fs,gated,conv,wd,T,seed", _mid_cases(60, 20250311))
+def test_random_layer_mid_batch(ora, E, k, d, f, fs, gated, conv, wd, T, seed):
+    W = S.make_weights(seed, E, d, f, f_s=fs, gated=gated, router_std=1.0 / np.sqrt(d),
+                       outlier_frac=0.01 if wd == capi.WEIGHT_INT8_W8A16 else 0.0)
+    oL, gL = S.build_pair(ora, W, k, conv, wd)
+    with gL:
+        _MID_SEEN.append(gL.expert_kernels(T))
+        x = S.make_tokens(seed + 1, T, d)
+        sample = None if T <= 64 else sorted(set(np.linspace(0, T - 1, 48).astype(int).tolist()))
+        check_layer(ora, oL, gL, x, TOL_BF16_TOY, sample=sample)
+
+
+def test_random_layer_mid_batch_reached_the_kernel():
+    """The cases above must have exercised the mid-batch family, alone and with a shared expert
+    inside its launches (this runs after them: same module, defined later)."""
+    assert len(_MID_SEEN) == 60
+    routed_mid = sum(1 for r, s in _MID_SEEN if r == capi.KERNELS_MID)
+    shared_mid = sum(1 for r, s in _MID_SEEN if r == capi.KERNELS_MID and s == capi.KERNELS_MID)
+    assert routed_mid >= 20 and shared_mid >= 5, (routed_mid, shared_mid)
