@@ -13,7 +13,8 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("wd,T,k,shared", [(capi.WEIGHT_BF16, 1, 2, False), (capi.WEIGHT_BF16, 8, 3, True),
-                                           (capi.WEIGHT_INT8_W8A16, 1, 2, False), (capi.WEIGHT_BF16, 300, 2, False)])
+                                           (capi.WEIGHT_INT8_W8A16, 1, 2, False), (capi.WEIGHT_BF16, 300, 2, False),
+                                           (capi.WEIGHT_BF16, 100, 2, True), (capi.WEIGHT_INT8_W8A16, 150, 2, False)])
 def test_forward_replays_from_a_graph(ora, wd, T, k, shared):
     d = 256
     W = S.make_weights(40 + T, 8, d, 512, f_s=128 if shared else 0, gated=shared, router_std=1.0 / 16.0)

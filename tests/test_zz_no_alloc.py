@@ -53,7 +53,9 @@ def test_noalloc_equals_forward_device_twice_second_smaller(ora, name, E, k, d, 
     _, other = S.build_pair(ora, W2, 3, 0, capi.WEIGHT_BF16)
     bf16_rows = wd != capi.WEIGHT_F32
     with gL, other:
-        for T in (37, 9, 1, 300):  # 300 takes the tiled kernels (split tail buffers) where they exist
+        # 300 takes the tiled kernels (split tail buffers) where they exist, 120 the mid-batch
+        # kernel where the widths allow it, 37 that kernel for the down phase alone
+        for T in (37, 9, 1, 120, 300):
             x = S.make_tokens(1000 + T, T, d, bf16=bf16_rows)
             want = _run(gL, x, noalloc=False)
             got = _run(gL, x, noalloc=True)
