@@ -92,8 +92,11 @@ __device__ inline void expert_tile(int c, int max_groups, int nt, int i, int& m0
 // block calls it (barriers inside), thread e owns expert e.  Three prefix sums over the experts
 // (rows, active flags, row tiles) replace a serial walk whose stores and loads through generic
 // pointers waited for each other (12 us for 60 experts).  E <= kMaxRouterRows.
+// s_offsets (LDS, [E + 1], may be null) receives the offsets as well; valid after the caller's
+// next barrier.
 __device__ void finish_offsets(int E, const int32_t* counts, int32_t* offsets, int32_t* active,
-                               int32_t* n_active, int32_t* shared_offsets, int T, TileOut to) {
+                               int32_t* n_active, int32_t* shared_offsets, int T, TileOut to,
+                               int32_t* s_offsets = nullptr) {
   __shared__ int32_t sRows[kMaxRouterRows], sAct[kMaxRouterRows], sTiles[kMaxRouterRows];
   const int tid = threadIdx.x;
   const bool mine = tid < E;
@@ -123,6 +126,7 @@ __device__ void finish_offsets(int E, const int32_t* counts, int32_t* offsets, i
   }
   if (mine) {
     offsets[tid] = sRows[tid] - c;
+    if (s_offsets) s_offsets[tid] = sRows[tid] - c;
     if (a) active[sAct[tid] - 1] = tid;
     const int t0 = sTiles[tid] - nt;
     for (int i = 0; i < nt; ++i) {
@@ -136,6 +140,7 @@ __device__ void finish_offsets(int E, const int32_t* counts, int32_t* offsets, i
   }
   if (tid == 0) {
     offsets[E] = sRows[kMaxRouterRows - 1];
+    if (s_offsets) s_offsets[E] = sRows[kMaxRouterRows - 1];
     *n_active = sAct[kMaxRouterRows - 1];
     if (to.n_tiles) *to.n_tiles = sTiles[kMaxRouterRows - 1];
     if (to.shared_n_tiles) *to.shared_n_tiles = (T + kTileM - 1) / kTileM;
@@ -158,17 +163,11 @@ __global__ __launch_bounds__(kPermuteBlock) void permute_single_kernel(
   const bool valid = p < P;
   const int e = valid ? idx[p] : 0;
   int rank = block_stable_rank(e, valid, E, sWaveCnt, sBlkCnt);
-  if (threadIdx.x == 0) {
-    int run = 0;
-    for (int ee = 0; ee < E; ++ee) {
-      sOff[ee] = run;
-      run += sBlkCnt[ee];
-    }
-    sOff[E] = run;
-  }
-  __syncthreads();
   for (int ee = threadIdx.x; ee < E; ee += kPermuteBlock) counts[ee] = sBlkCnt[ee];
-  finish_offsets(E, sBlkCnt, offsets, active, n_active, shared_offsets, T, to);
+  // the exclusive scan of the counts comes out of finish_offsets' parallel prefix (one thread
+  // walking the experts in LDS took 3-4 us with 60 of them)
+  finish_offsets(E, sBlkCnt, offsets, active, n_active, shared_offsets, T, to, sOff);
+  __syncthreads();
   if (valid) {
     int pos = sOff[e] + rank;
     perm[pos] = p;
