@@ -633,7 +633,10 @@ __global__ __launch_bounds__(1024) void ffn_down_combine1_kernel(
 // is issued unconditionally with a clamped stage index: a branch around a load makes the
 // compiler wait for all loads in flight before every use.  16-byte chunk c of LDS row r sits
 // at c ^ swz(r), which spreads the rows a fragment read touches over all banks.
-template <bool INT8, bool UP, int NWV, int JB, int NWB, int NBD = 2>
+// PG: int8 with one scale per output row and k group (see ffn_stream_kernel): every 64-k block
+// is accumulated on its own and added to the running sum times the scale of its group; the
+// scales travel through the register ring with the blocks they belong to.
+template <bool INT8, bool UP, int NWV, int JB, int NWB, int NBD = 2, bool PG = false>
 __global__ __launch_bounds__(64 * NWV, 8 / NWV) void ffn_mid_kernel(StreamParams p_routed,
                                                                     StreamParams p_shared,
                                                                     int with_shared) {
@@ -678,9 +681,18 @@ __global__ __launch_bounds__(64 * NWV, 8 / NWV) void ffn_mid_kernel(StreamParams
       pw[t] = p.wa + (size_t)e * p.w_stride_u4 + (size_t)min(strip[t], n_strips - 1) * p.nkb * 64 + lane;
     }
   }
+  // per-group scales of this lane's output row (column mm of the D layout) in each strip
+  const float* psc[NB];
+  if (PG) {
+#pragma unroll
+    for (int t = 0; t < NB; ++t)
+      psc[t] = (UP && t == 1 ? p.sb : p.sa) + (size_t)e * p.n_kgroups * p.n_pad +
+               min(strip[t], n_strips - 1) * 16 + mm;
+  }
   // Ring of NWB register buffers of weight blocks: stage st lives in buffer st % NWB and is
   // requested NWB - 1 steps before it is multiplied.
   u32x4 wr[NWB][NB][JB];
+  float wsc[NWB][PG ? NB : 1][PG ? JB : 1];
   // Workgroups walk K from different first stages (and wrap around): launched together and
   // paced by the same memory system, they would otherwise all read the same offset of their
   // 2^n-byte-spaced strips at the same time, i.e. the same few memory channels.
@@ -689,16 +701,18 @@ __global__ __launch_bounds__(64 * NWV, 8 / NWV) void ffn_mid_kernel(StreamParams
     const int sc = min(st, ns - 1) + rot;
     return sc >= ns ? sc - ns : sc;
   };
-  auto load_w = [&](u32x4 (&w)[NB][JB], int st) {
+  auto load_w = [&](u32x4 (&w)[NB][JB], float (&sc_)[PG ? NB : 1][PG ? JB : 1], int st) {
     const int sc = stage_of(st);
 #pragma unroll
     for (int t = 0; t < NB; ++t)
 #pragma unroll
-      for (int j = 0; j < JB; ++j)
+      for (int j = 0; j < JB; ++j) {
         w[t][j] = __builtin_nontemporal_load((const u32x4*)(pw[t] + (size_t)(sc * JB + j) * 64));
+        if (PG) sc_[PG ? t : 0][PG ? j : 0] = psc[t][(size_t)((sc * JB + j) / p.group_blocks) * p.n_pad];
+      }
   };
 #pragma unroll
-  for (int b = 0; b < NWB - 1; ++b) load_w(wr[b], b);
+  for (int b = 0; b < NWB - 1; ++b) load_w(wr[b], wsc[b], b);
 
   // Chunk c of row r is stored at c ^ swz(r): eight consecutive rows then cover all banks
   // (rows of 128 bytes or more: r & 7; rows of 64 bytes pair up: (r >> 1) & 3).
@@ -738,7 +752,7 @@ __global__ __launch_bounds__(64 * NWV, 8 / NWV) void ffn_mid_kernel(StreamParams
       for (int c = 0; c < CPT; ++c)
         lds_a[(slot * ROWS + ar) * CH + ((ac + c) ^ swz(ar))] = ga[c];
     };
-    auto compute = [&](const u32x4 (&w)[NB][JB], int slot) {
+    auto compute = [&](const u32x4 (&w)[NB][JB], const float (&sc_)[PG ? NB : 1][PG ? JB : 1], int slot) {
       const u32x4* fs = frag + slot * ROWS * CH;
 #pragma unroll
       for (int j = 0; j < JB; ++j) {
@@ -753,8 +767,14 @@ __global__ __launch_bounds__(64 * NWV, 8 / NWV) void ffn_mid_kernel(StreamParams
             const u32x4 x1 = fs[16 * i * CH + ((j * 8 + 2 * kq + 1) ^ sw)];
 #pragma unroll
             for (int t = 0; t < NB; ++t) {
-              acc[t][i] = mfma(*(const bf16x8*)&x0, bl[t], acc[t][i]);
-              acc[t][i] = mfma(*(const bf16x8*)&x1, bh[t], acc[t][i]);
+              if (PG) {
+                f32x4 ta = mfma(*(const bf16x8*)&x0, bl[t], f32x4{0.f, 0.f, 0.f, 0.f});
+                ta = mfma(*(const bf16x8*)&x1, bh[t], ta);
+                acc[t][i] += ta * sc_[PG ? t : 0][PG ? j : 0];
+              } else {
+                acc[t][i] = mfma(*(const bf16x8*)&x0, bl[t], acc[t][i]);
+                acc[t][i] = mfma(*(const bf16x8*)&x1, bh[t], acc[t][i]);
+              }
             }
           }
         } else {
@@ -771,11 +791,11 @@ __global__ __launch_bounds__(64 * NWV, 8 / NWV) void ffn_mid_kernel(StreamParams
     // st - 1 (every wave is past that step's barrier); the rows of stage st + 3 and the weights
     // of stage st + NWB - 1 are requested, then stage st is multiplied.
     u32x4 ga[CPT];
-    auto step = [&](const u32x4 (&wc)[NB][JB], u32x4 (&wl)[NB][JB], int st) {
+    auto step = [&](int bc, int bl_, int st) {
       store_a(ga, (st + 2) % NST);
       load_a(ga, st + 3);
-      load_w(wl, st + NWB - 1);
-      if (st < ns) compute(wc, st % NST);
+      load_w(wr[bl_], wsc[bl_], st + NWB - 1);
+      if (st < ns) compute(wr[bc], wsc[bc], st % NST);
       __syncthreads();
     };
     load_a(ga, 0);
@@ -786,7 +806,7 @@ __global__ __launch_bounds__(64 * NWV, 8 / NWV) void ffn_mid_kernel(StreamParams
     __syncthreads();
     for (int st = 0; st < ns; st += NWB) {
 #pragma unroll
-      for (int b = 0; b < NWB; ++b) step(wr[b], wr[(b + NWB - 1) % NWB], st + b);
+      for (int b = 0; b < NWB; ++b) step(b, (b + NWB - 1) % NWB, st + b);
     }
   };
   if (mt_live <= 2)
@@ -804,7 +824,7 @@ __global__ __launch_bounds__(64 * NWV, 8 / NWV) void ffn_mid_kernel(StreamParams
     const int n = strip[t] * 16 + mm;
     const bool n_ok = strip[t] < n_strips && n < p.n_rows;
     float sa = 1.f, sb = 1.f;
-    if (INT8) {
+    if (INT8 && !PG) {
       sa = n_ok ? p.sa[(size_t)e * p.n_rows + n] : 0.f;
       if (UP) sb = n_ok ? p.sb[(size_t)e * p.n_rows + n] : 0.f;
     }
@@ -845,6 +865,15 @@ hipError_t launch_mid(const StreamParams& p_in, int n_groups, int rows_max, hipS
   const int n_strips = n_pad / 16;
   const int per_wg = UP ? 4 : 8;
   dim3 grid((n_strips + per_wg - 1) / per_wg, n_groups + (shared ? 1 : 0), (rows_max + 127) / 128);
+  if constexpr (INT8) {
+    if (p.group_blocks > 0) {  // per-group scales: a shorter ring leaves room for them
+      if (UP)
+        ffn_mid_kernel<true, true, 4, 1, 4, 2, true><<<grid, 256, 0, s>>>(p, ps, shared != nullptr);
+      else
+        ffn_mid_kernel<true, false, 8, 2, 3, 1, true><<<grid, 512, 0, s>>>(p, ps, shared != nullptr);
+      return hipGetLastError();
+    }
+  }
   if (UP)
     ffn_mid_kernel<INT8, true, 4, INT8 ? 1 : 2, INT8 ? 6 : 4><<<grid, 256, 0, s>>>(p, ps, shared != nullptr);
   else
@@ -967,9 +996,10 @@ bool can_fuse_shared(const FfnArgs& a, const FfnArgs* sh, bool down_phase) {
 }
 }  // namespace
 
-// K of whole stages (64 k for bf16 blocks, 128 k for int8 blocks), per-row scales.
+// K of whole stages (64 k for bf16 blocks, 128 k for int8 blocks).
 bool ffn_mid_supported(const WeightSet& w, int wdtype) {
-  if (wdtype == ATENIA_MOE_WEIGHT_F32 || w.group_blocks != 0) return false;
+  if (wdtype == ATENIA_MOE_WEIGHT_F32) return false;
+  if (w.group_blocks != 0 && wdtype != ATENIA_MOE_WEIGHT_INT8_W8A16) return false;
   const int kb = wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16 ? kKbInt8 : kKbBf16;
   return w.k_pad % (2 * kb) == 0 && w.k_pad >= 2 * kb && w.n_pad >= 16;
 }

@@ -530,7 +530,7 @@ BatchPlan plan_batch(const AteniaMoeLayer* L, int T) {
   const double avg = (double)T * L->k / L->E;
   p.routed_mid = false;
   p.mid_down = false;
-  if (L->group_size == 0 && stream_max_tokens_override() == 0 &&
+  if (stream_max_tokens_override() == 0 &&
       ffn_mid_supported(L->gate, L->wdtype) && ffn_mid_supported(L->up, L->wdtype) &&
       ffn_mid_supported(L->down, L->wdtype)) {
     const MidBounds b = mid_bounds(L);
