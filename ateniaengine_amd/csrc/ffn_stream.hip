@@ -120,7 +120,8 @@ __global__ __launch_bounds__(64 * WAVES) void ffn_stream_kernel(StreamParams p_r
   const bool sh = (int)blockIdx.y == shared_y;
   const StreamParams& p = sh ? p_shared : p_routed;
   if ((int)blockIdx.x * 16 * S >= p.n_pad) return;  // the grid spans the wider of the two
-  const int u = sh ? 0 : blockIdx.y;
+  // shared_y == 0: the shared expert comes first in the grid and the routed groups follow
+  const int u = sh ? 0 : (int)blockIdx.y - (shared_y == 0 ? 1 : 0);
   int e, base, cnt;
   if (SEL && !sh) {
     // One token whose routing is still open: every wave derives it from the logits (the same
@@ -887,7 +888,9 @@ hipError_t launch_stream(const StreamParams& p, int n_groups, int rows_max, hipS
   // Up to 32 rows per expert per workgroup; larger groups take more workgroups along z.
   int mt = rows_max <= 16 ? 1 : 2;
   const StreamParams ps = shared ? *shared : p;
-  const int shared_y = shared ? n_groups : -1;
+  // A shared expert rides as the last group of the grid, or as the first one when its K is much
+  // longer than the routed experts' (its strips would otherwise start last and end the launch).
+  const int shared_y = !shared ? -1 : (!UP && shared->nkb > p.nkb) ? 0 : n_groups;
   const int n_pad = shared && shared->n_pad > p.n_pad ? shared->n_pad : p.n_pad;
   // Two strips per workgroup once experts can have more than 16 rows:
   // int8 (per-row and per-group scales) in both phases, bf16 in the down phase.  Measured at T = 48 on the Mixtral shape:
@@ -979,9 +982,13 @@ StreamParams stream_params_down(const FfnArgs& a) {
 }
 // The shared expert can ride in the routed experts' launch when both stream with the same
 // kernel (no tiles, no f32 weights), are stored alike and see the same rows bound.
-// In the down phase a strip's K is the expert's width: a shared expert much wider than the
-// routed ones would make its strips the launch's critical path (measured: Qwen1.5-MoE, shared
-// 4x as wide, 20 us fused against 18 us as two launches), so it keeps its own launch then.
+// In the down phase a strip's K is the expert's width: last in the grid, the strips of a shared
+// expert much wider than the routed ones end the launch (measured: Qwen1.5-MoE, shared 4x as
+// wide, T = 1: 20 us fused against 18 us as two launches).  With up to 32 rows it rides as the
+// first group instead (launch_stream) and is hidden behind the routed experts: down stage
+// T = 2 18.5 against 22.9 us as two launches, T = 16 52.2 / 60.1; beyond 32 rows, where its T
+// rows take several passes over its weights, a shared expert more than twice as wide keeps its
+// own launch.
 bool can_fuse_shared(const FfnArgs& a, const FfnArgs* sh, bool down_phase) {
   if (!(sh && a.wdtype != ATENIA_MOE_WEIGHT_F32 && sh->wdtype == a.wdtype && !a.use_tiled &&
         !sh->use_tiled && sh->rows_max == a.rows_max &&
@@ -992,6 +999,7 @@ bool can_fuse_shared(const FfnArgs& a, const FfnArgs* sh, bool down_phase) {
   // as long as it makes few passes: measured on the Qwen1.5-MoE shape, down phase fused / two
   // launches: T = 192 110 / 128 us, T = 256 121 / 131, T = 384 131 / 134, T = 768 183 / 146)
   if (a.use_mid && a.rows_max <= 384) return true;
+  if (!a.use_mid && down_phase && a.rows_max > 1 && a.rows_max <= 32) return true;  // first in the grid
   return !down_phase || sh->down.k_pad <= 2 * a.down.k_pad;
 }
 }  // namespace
