@@ -917,6 +917,22 @@ hipError_t launch_stream(const StreamParams& p, int n_groups, int rows_max, hipS
       ffn_stream_kernel<2, INT8, UP, W, INT8><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
     return hipGetLastError();
   }
+  if constexpr (!UP) {
+    // Short K (a strip of fewer than 64 blocks): four K slices instead of eight, so that a wave
+    // still has a few batches of blocks to pipeline.  Measured (44 blocks per strip, 60-64
+    // experts): down stage T = 16 36.3 -> 28.4 us and 52.1 -> 40.6 us, T = 8 26.9 -> 21.7; two
+    // slices are slower again (T = 2 17.5 against 15.9 us).  A single token keeps eight: its
+    // fused down + combine launch adds the slices up in that order, and the two must agree bit
+    // for bit.  ATENIA_MOE_DOWN_W4_BELOW moves the bound (0 = never).
+    static const int w4_below = [] {
+      const char* e = getenv("ATENIA_MOE_DOWN_W4_BELOW");
+      return e ? atoi(e) : 64;
+    }();
+    if (p.nkb < w4_below && mt == 1 && !two && rows_max > 1) {
+      ffn_stream_kernel<1, INT8, false, 4, false><<<grid, 256, 0, s>>>(p, ps, shared_y);
+      return hipGetLastError();
+    }
+  }
   if (mt == 1 && two)
     ffn_stream_kernel<1, INT8, UP, W, false, 2><<<grid, 64 * W, 0, s>>>(p, ps, shared_y);
   else if (mt == 1 && UP && p.sel.logits)
