@@ -920,7 +920,8 @@ hipError_t launch_stream(const StreamParams& p, int n_groups, int rows_max, hipS
   if constexpr (!UP) {
     // Short K (a strip of fewer than 64 blocks): four K slices instead of eight, so that a wave
     // still has a few batches of blocks to pipeline.  Measured (44 blocks per strip, 60-64
-    // experts): down stage T = 16 36.3 -> 28.4 us and 52.1 -> 40.6 us, T = 8 26.9 -> 21.7; two
+    // experts): down stage T = 16 36.3 -> 28.4 us and 52.1 -> 40.6 us, T = 8 26.9 -> 21.7, T = 19
+    // (two row tiles, two strips per workgroup) 36.1 -> 29.6 and 59.0 -> 46.2; two
     // slices are slower again (T = 2 17.5 against 15.9 us).  A single token keeps eight: its
     // fused down + combine launch adds the slices up in that order, and the two must agree bit
     // for bit.  ATENIA_MOE_DOWN_W4_BELOW moves the bound (0 = never).
@@ -928,8 +929,15 @@ hipError_t launch_stream(const StreamParams& p, int n_groups, int rows_max, hipS
       const char* e = getenv("ATENIA_MOE_DOWN_W4_BELOW");
       return e ? atoi(e) : 64;
     }();
-    if (p.nkb < w4_below && mt == 1 && !two && rows_max > 1) {
-      ffn_stream_kernel<1, INT8, false, 4, false><<<grid, 256, 0, s>>>(p, ps, shared_y);
+    if (p.nkb < w4_below && rows_max > 1) {
+      if (mt == 1 && two)
+        ffn_stream_kernel<1, INT8, false, 4, false, 2><<<grid, 256, 0, s>>>(p, ps, shared_y);
+      else if (mt == 1)
+        ffn_stream_kernel<1, INT8, false, 4, false><<<grid, 256, 0, s>>>(p, ps, shared_y);
+      else if (two)
+        ffn_stream_kernel<2, INT8, false, 4, false, 2><<<grid, 256, 0, s>>>(p, ps, shared_y);
+      else
+        ffn_stream_kernel<2, INT8, false, 4, false><<<grid, 256, 0, s>>>(p, ps, shared_y);
       return hipGetLastError();
     }
   }
