@@ -460,10 +460,11 @@ int ensure_pg_copy(AteniaMoeLayer* L) {
 }
 
 // Which expert kernels a batch of T tokens takes (a pure function of the layer and T).
+enum { kFamStream = 0, kFamMid = 1, kFamTiled = 2 };
 struct BatchPlan {
-  bool routed_streams;  // weight-streaming kernels (decode) instead of the tiled ones
-  bool routed_mid;      // ... in their mid-batch form (token rows shared through LDS)
-  bool mid_down;        // the down phase alone takes the mid-batch form (gate/up streams from registers)
+  int up, down;         // kernel family of the gate/up phase and of the down phase (kFam*)
+  bool routed_streams;  // gate/up phase: weight-streaming kernels (either form), not the tiled ones
+  bool routed_mid;      // gate/up phase in the mid-batch form (token rows shared through LDS)
   bool pg_prefill;      // per-group int8 layer running the tiled kernels on its bf16 copy
   bool tall_tiles;      // row tiles of up to nine 32-row groups (bf16 pipelined kernels only)
 };
@@ -494,8 +495,10 @@ bool tall_tiles_enabled() {
 // Tuning knobs ATENIA_MOE_MID_MIN_TOKENS / ATENIA_MOE_MID_MIN_AVG / ATENIA_MOE_MID_MAX_AVG (read
 // once) replace the three bounds; a maximum of 0 switches the kernel off.
 struct MidBounds {
-  int min_tokens;
-  double lo, hi;
+  int min_tokens, max_tokens;  // gate/up phase: batch sizes
+  double lo, hi;               // gate/up phase: rows per expert on average
+  int down_min_tokens;         // down phase: from this batch size ...
+  double down_hi;              // ... up to this many rows per expert on average
 };
 MidBounds mid_bounds(const AteniaMoeLayer* L) {
   static const double env_lo = [] {
@@ -516,47 +519,79 @@ MidBounds mid_bounds(const AteniaMoeLayer* L) {
                      ffn_mid_supported(L->s_up, L->wdtype) && ffn_mid_supported(L->s_down, L->wdtype);
   MidBounds b;
   b.min_tokens = rides || int8w ? 40 : kStreamMaxTokens + 1;
+  b.max_tokens = INT_MAX;
   b.lo = rides ? 0.0 : int8w ? 10.0 : 14.0;
   b.hi = int8w ? 104.0 : rides ? 68.0 : 52.0;
+  // The down phase alone gains from the mid-batch form from 20 tokens on when its K is long: it
+  // has d / 16 strips only, which that form spreads over d / 128 workgroups of eight waves that
+  // each own a strip over the whole K (no reduction through LDS).  Down launch, mid-batch /
+  // register-resident: Mixtral int8 T = 24 79 / 83 us, T = 48 80 / 97; Mixtral bf16 T = 24
+  // 142 / 144, T = 56 145 / 157.
+  b.down_min_tokens = 20;
+  b.down_hi = b.hi;
+  // Narrow experts (a down strip of fewer than 64 blocks, which the register-resident launch
+  // cuts into four K slices): that launch is the better one for longer, and the mid-batch form
+  // then stays ahead of the tiled kernels for longer, phase by phase (us, DeepSeek-V2-Lite /
+  // Qwen1.5-MoE shapes, stream | mid | tiled):
+  //   gate/up  T = 32 64 | 67, 110 | 117;  T = 48 77 | 74, 125 | 123;  T = 128 137 | 106 | 136,
+  //            158 | 132 | 175;  T = 512 181 | 186 (mid | tiled), 178 | 184;  T = 640 202 | 187,
+  //            186 | 183;  T = 768 223 | 195, 196 | 186
+  //   down     T = 32 35 | 43, 56 | 72;  T = 48 48 | 47, 77 | 80;  T = 64 57 | 52, 78 | 84;
+  //            T = 128 84 | 65, 85 | 101;  T = 256 132 | 90, 122 | 122;  T = 384 179 | 109 | 154,
+  //            159 | 132 | 188;  T = 1024 168 | 181 (mid | tiled), 156 | 199;  T = 1536 224 | 198,
+  //            186 | 206;  T = 2048 278 | 220, 272 | 215
+  // (the Qwen shape's shared expert is 4x as wide as a routed one and keeps a down launch of its
+  // own beside the register-resident kernel, which is why that kernel holds out to 256 tokens.)
+  const int kb = int8w ? kKbInt8 : kKbBf16;
+  if (L->down.k_pad / kb < 64 && L->group_size == 0) {
+    const bool wide_shared = L->fs > 0 && L->s_down.k_pad > 2 * L->down.k_pad;
+    if (rides) {
+      b.min_tokens = 48;
+      b.max_tokens = 640;
+      b.hi = 52.0;
+    }
+    b.down_min_tokens = wide_shared ? 256 : 56;
+    b.down_hi = 100.0;
+  }
   if (env_lo >= 0.0) b.lo = env_lo;
-  if (env_hi >= 0.0) b.hi = env_hi;
-  if (env_min_tokens > 0) b.min_tokens = env_min_tokens;
+  if (env_hi >= 0.0) b.hi = b.down_hi = env_hi;
+  if (env_min_tokens > 0) b.min_tokens = b.down_min_tokens = env_min_tokens;
   return b;
 }
 BatchPlan plan_batch(const AteniaMoeLayer* L, int T) {
   const bool int8w = L->wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
   BatchPlan p;
-  p.routed_streams = batch_streams(T, (long long)T * L->k, L->E, int8w ? 32 : 16);
+  const bool base_streams = batch_streams(T, (long long)T * L->k, L->E, int8w ? 32 : 16);
   const double avg = (double)T * L->k / L->E;
-  p.routed_mid = false;
-  p.mid_down = false;
+  p.up = p.down = base_streams ? kFamStream : kFamTiled;
   if (stream_max_tokens_override() == 0 &&
       ffn_mid_supported(L->gate, L->wdtype) && ffn_mid_supported(L->up, L->wdtype) &&
       ffn_mid_supported(L->down, L->wdtype)) {
     const MidBounds b = mid_bounds(L);
-    p.routed_mid = T >= b.min_tokens && avg >= b.lo && avg <= b.hi;
-    // Below those bounds the down phase still gains from the mid-batch form from 20 tokens on:
-    // it has d / 16 strips only, which that form spreads over d / 128 workgroups of eight waves
-    // that each own a strip over the whole K (no reduction through LDS), and a shared expert's
-    // down projection rides along.  Down launch, mid-batch / register-resident: Qwen1.5-MoE
-    // shape T = 20 65 / 75 us, T = 12 62 / 54; DeepSeek-V2-Lite T = 20 39 / 44, T = 12 37 / 36;
-    // Mixtral int8 T = 24 79 / 83, T = 48 80 / 97; Mixtral bf16 T = 24 142 / 144, T = 56 145 / 157.
-    p.mid_down = !p.routed_mid && p.routed_streams && T >= 20 && avg <= b.hi && b.hi > 0.0;
+    if (T >= b.min_tokens && T <= b.max_tokens && avg >= b.lo && avg <= b.hi) p.up = kFamMid;
+    if (b.hi > 0.0 && T >= b.down_min_tokens && avg <= b.down_hi)
+      p.down = kFamMid;
+    else if (p.up == kFamMid && T < b.down_min_tokens)
+      p.down = kFamStream;  // narrow experts: the register-resident down launch holds out longer
+    // a per-group layer runs the tiled kernels on a bf16 copy: both phases or neither
+    if (L->group_size > 0 && (p.up == kFamTiled) != (p.down == kFamTiled))
+      p.up = p.down = kFamTiled;
   }
-  if (p.routed_mid) p.routed_streams = true;
-  p.pg_prefill = L->group_size > 0 && !p.routed_streams && L->d_kpad % 64 == 0 &&
+  p.routed_streams = p.up != kFamTiled;
+  p.routed_mid = p.up == kFamMid;
+  p.pg_prefill = L->group_size > 0 && p.up == kFamTiled && L->d_kpad % 64 == 0 &&
                  L->f_kpad % 64 == 0 && (L->fs == 0 || L->fs_kpad % 64 == 0);
-  // both phases of the routed experts on the bf16 pipelined kernel (K a multiple of 64, >= 128)
+  // the routed experts on the bf16 pipelined kernel (K a multiple of 64, >= 128)
   const bool bf16_tiles = L->wdtype == ATENIA_MOE_WEIGHT_BF16 || p.pg_prefill;
-  p.tall_tiles = tall_tiles_enabled() && !p.routed_streams && bf16_tiles && L->d_kpad % 64 == 0 &&
-                 L->d_kpad >= 128 && L->f_kpad % 64 == 0 && L->f_kpad >= 128;
+  p.tall_tiles = tall_tiles_enabled() && (p.up == kFamTiled || p.down == kFamTiled) && bf16_tiles &&
+                 L->d_kpad % 64 == 0 && L->d_kpad >= 128 && L->f_kpad % 64 == 0 && L->f_kpad >= 128;
   return p;
 }
 
 // Partial output buffers the no-alloc workspace of a T-token batch needs (the tiled down phase
 // may split tail tiles over k; the streaming kernels write one buffer).
 int noalloc_y_parts(const AteniaMoeLayer* L, int T) {
-  return plan_batch(L, T).routed_streams || L->wdtype == ATENIA_MOE_WEIGHT_F32 ? 1 : kMaxYParts;
+  return plan_batch(L, T).down != kFamTiled || L->wdtype == ATENIA_MOE_WEIGHT_F32 ? 1 : kMaxYParts;
 }
 
 bool stream_is_capturing(hipStream_t s) {
@@ -566,6 +601,16 @@ bool stream_is_capturing(hipStream_t s) {
     return false;
   }
   return st != hipStreamCaptureStatusNone;
+}
+
+// Family of the shared expert in a phase where the routed experts take `fam`: the same one where
+// its widths allow it; beside the mid-batch kernel, if they do not, the tiled ones.
+void shared_family(FfnArgs& fsd, int fam, int ffn_dtype) {
+  const bool mid_ok = ffn_mid_supported(fsd.gate, ffn_dtype) && ffn_mid_supported(fsd.up, ffn_dtype) &&
+                      ffn_mid_supported(fsd.down, ffn_dtype);
+  const bool tiles_ok = tiled_supported(fsd.gate, ffn_dtype) && tiled_supported(fsd.down, ffn_dtype);
+  fsd.use_mid = fam == kFamMid && mid_ok;
+  fsd.use_tiled = (fam == kFamTiled || (fam == kFamMid && !mid_ok)) && tiles_ok;
 }
 
 // `view`: the workspace to run on (nullptr = the handle's own).  no_alloc: fail instead of
@@ -708,7 +753,7 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   // src/cuda/int8_to_bf16.cu:91-110; rounding halves the error against the q * scale the
   // reference's CPU path multiplies with).  Decode batches stream the int8 weights themselves.
   const BatchPlan plan = plan_batch(L, T);
-  const bool routed_streams = plan.routed_streams, pg_prefill = plan.pg_prefill;
+  const bool pg_prefill = plan.pg_prefill;
   if (pg_prefill && !L->pg_ready && no_alloc)
     return fail(ATENIA_MOE_ERR_UNSUPPORTED,
                 "per-group int8: a batch of %d tokens needs the layer's bf16 copy, which is made by "
@@ -753,10 +798,14 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   fa.y_stride = L->d;
   // Tiled (MFMA-bound) kernels once an expert can see more rows than the streaming kernel
   // keeps in registers; below that the weights are streamed once (HBM-bound).
-  const bool tiled = !routed_streams && tiled_supported(fa.gate, ffn_dtype) &&
-                     tiled_supported(fa.down, ffn_dtype);
-  fa.use_tiled = tiled;
-  fa.use_mid = plan.routed_mid;
+  // (each phase has its own family; a tiled phase whose widths the tiled kernels do not take
+  // falls back to the register-resident streaming kernel)
+  const bool tiles_ok = tiled_supported(fa.gate, ffn_dtype) && tiled_supported(fa.down, ffn_dtype);
+  const int fam_up = plan.up == kFamTiled && !tiles_ok ? kFamStream : plan.up;
+  const int fam_down = plan.down == kFamTiled && !tiles_ok ? kFamStream : plan.down;
+  const bool tiled = fam_up == kFamTiled;  // gate/up phase
+  fa.use_tiled = fam_up == kFamTiled;
+  fa.use_mid = fam_up == kFamMid;
   fa.tile_group = V.tile_group;
   fa.tile_m0 = V.tile_m0;
   fa.n_tiles = V.shared_desc + 4;
@@ -764,7 +813,7 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   fa.tile_li = V.tile_li;
   fa.max_row_tiles = (int)(((size_t)T * L->k + kTileM - 1) / kTileM +
                            std::min<long long>(L->E, (long long)T * L->k));
-  const bool split_tail = tiled && tiled_down_splits_tail(fa.down, ffn_dtype);
+  const bool split_tail = fam_down == kFamTiled && tiled_down_splits_tail(fa.down, ffn_dtype);
   fa.y_parts = split_tail ? std::min(kMaxYParts, V.y_parts) : 1;
   fa.y_part_stride = (size_t)T * L->k * L->d;
   fa.part_flags = split_tail ? V.part_flags : nullptr;
@@ -797,10 +846,7 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
     // launches of its own that the tiled form would need.
     // (With the routed experts on the mid-batch kernel it takes that kernel too, one pass over
     // its weights per 128 tokens; if its widths do not fit that kernel, the tiled ones.)
-    fsd.use_mid = plan.routed_mid && ffn_mid_supported(fsd.gate, ffn_dtype) &&
-                  ffn_mid_supported(fsd.up, ffn_dtype) && ffn_mid_supported(fsd.down, ffn_dtype);
-    fsd.use_tiled = (!routed_streams || (plan.routed_mid && !fsd.use_mid)) &&
-                    tiled_supported(fsd.gate, ffn_dtype) && tiled_supported(fsd.down, ffn_dtype);
+    shared_family(fsd, fam_up, ffn_dtype);
     fsd.tile_group = V.s_tile_group;
     fsd.tile_m0 = V.s_tile_m0;
     fsd.n_tiles = V.shared_desc + 5;
@@ -820,11 +866,10 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
     }
   }
   tm.mark();  // ev[3]: gate/up done
-  if (plan.mid_down) {  // the down phase alone in the mid-batch form
-    fa.use_mid = 1;
-    if (L->fs > 0)
-      fsd.use_mid = !fsd.use_tiled && ffn_mid_supported(fsd.down, ffn_dtype);
-  }
+  // the down phase may take another family than gate/up did
+  fa.use_tiled = fam_down == kFamTiled;
+  fa.use_mid = fam_down == kFamMid;
+  if (L->fs > 0) shared_family(fsd, fam_down, ffn_dtype);
   const bool fuse_shared_down = L->fs > 0 && ffn_stream_fuses_shared(fa, fsd, true);
   // One token, whole pipeline requested: the down launch covers the routed experts and the
   // shared one and finishes the combine as well (one launch instead of two or three).
@@ -1638,27 +1683,26 @@ int atenia_moe_hip_layer_expert_kernels(const AteniaMoeLayer* L, int64_t n_token
     family[1] = L->fs > 0 ? ATENIA_MOE_KERNELS_F32 : -1;
     return ATENIA_MOE_OK;
   }
-  // the same decisions run_forward takes
+  // the same decisions run_forward takes for the gate/up phase
   const BatchPlan plan = plan_batch(L, T);
   const int dt = plan.pg_prefill ? ATENIA_MOE_WEIGHT_BF16 : L->wdtype;
   const WeightSet& g = plan.pg_prefill ? L->gate_b : L->gate;
   const WeightSet& dn = plan.pg_prefill ? L->down_b : L->down;
-  const bool tiled = !plan.routed_streams && tiled_supported(g, dt) && tiled_supported(dn, dt);
-  family[0] = plan.routed_mid ? ATENIA_MOE_KERNELS_MID
-              : tiled         ? ATENIA_MOE_KERNELS_TILED
-                              : ATENIA_MOE_KERNELS_STREAM;
+  const bool tiles_ok = tiled_supported(g, dt) && tiled_supported(dn, dt);
+  const int fam = plan.up == kFamTiled && !tiles_ok ? kFamStream : plan.up;
+  auto name = [](int f) {
+    return f == kFamMid ? ATENIA_MOE_KERNELS_MID
+           : f == kFamTiled ? ATENIA_MOE_KERNELS_TILED : ATENIA_MOE_KERNELS_STREAM;
+  };
+  family[0] = name(fam);
   family[1] = -1;
   if (L->fs > 0) {
-    const WeightSet& sg = plan.pg_prefill ? L->s_gate_b : L->s_gate;
-    const WeightSet& su = plan.pg_prefill ? L->s_up_b : L->s_up;
-    const WeightSet& sd = plan.pg_prefill ? L->s_down_b : L->s_down;
-    const bool s_mid = plan.routed_mid && ffn_mid_supported(sg, dt) && ffn_mid_supported(su, dt) &&
-                       ffn_mid_supported(sd, dt);
-    const bool s_tiled = (!plan.routed_streams || (plan.routed_mid && !s_mid)) &&
-                         tiled_supported(sg, dt) && tiled_supported(sd, dt);
-    family[1] = s_mid ? ATENIA_MOE_KERNELS_MID
-                : s_tiled ? ATENIA_MOE_KERNELS_TILED
-                          : ATENIA_MOE_KERNELS_STREAM;
+    FfnArgs fsd{};
+    fsd.gate = plan.pg_prefill ? L->s_gate_b : L->s_gate;
+    fsd.up = plan.pg_prefill ? L->s_up_b : L->s_up;
+    fsd.down = plan.pg_prefill ? L->s_down_b : L->s_down;
+    shared_family(fsd, fam, dt);
+    family[1] = name(fsd.use_mid ? kFamMid : fsd.use_tiled ? kFamTiled : kFamStream);
   }
   return ATENIA_MOE_OK;
 }
