@@ -1010,9 +1010,10 @@ StreamParams stream_params_down(const FfnArgs& a) {
 // expert much wider than the routed ones end the launch (measured: Qwen1.5-MoE, shared 4x as
 // wide, T = 1: 20 us fused against 18 us as two launches).  With up to 32 rows it rides as the
 // first group instead (launch_stream) and is hidden behind the routed experts: down stage
-// T = 2 18.5 against 22.9 us as two launches, T = 16 52.2 / 60.1; beyond 32 rows, where its T
-// rows take several passes over its weights, a shared expert more than twice as wide keeps its
-// own launch.
+// T = 2 18.5 against 22.9 us as two launches, T = 16 52.2 / 60.1, T = 48 72.8 / 77.5; from
+// 64 rows on, where its T rows take several passes over its weights, a shared expert more than
+// twice as wide is faster in a launch of its own (T = 64 81.3 / 79.0, T = 128 100.9 / 85.5).
+// ATENIA_MOE_WIDE_SHARED_ROWS moves the bound (default 48).
 bool can_fuse_shared(const FfnArgs& a, const FfnArgs* sh, bool down_phase) {
   if (!(sh && a.wdtype != ATENIA_MOE_WEIGHT_F32 && sh->wdtype == a.wdtype && !a.use_tiled &&
         !sh->use_tiled && sh->rows_max == a.rows_max &&
@@ -1023,7 +1024,11 @@ bool can_fuse_shared(const FfnArgs& a, const FfnArgs* sh, bool down_phase) {
   // as long as it makes few passes: measured on the Qwen1.5-MoE shape, down phase fused / two
   // launches: T = 192 110 / 128 us, T = 256 121 / 131, T = 384 131 / 134, T = 768 183 / 146)
   if (a.use_mid && a.rows_max <= 384) return true;
-  if (!a.use_mid && down_phase && a.rows_max > 1 && a.rows_max <= 32) return true;  // first in the grid
+  static const int wide_rows = [] {
+    const char* e = getenv("ATENIA_MOE_WIDE_SHARED_ROWS");
+    return e ? atoi(e) : 48;
+  }();
+  if (!a.use_mid && down_phase && a.rows_max > 1 && a.rows_max <= wide_rows) return true;  // first in the grid
   return !down_phase || sh->down.k_pad <= 2 * a.down.k_pad;
 }
 }  // namespace
