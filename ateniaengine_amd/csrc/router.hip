@@ -707,24 +707,32 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
   }
   __syncthreads();
 
-  // Second look at the flagged sums (about one in a thousand), the whole workgroup on one sum
-  // at a time: the partial-sum area is free now and holds their list.
-  int* sList = (int*)sPart;      // [<= 16 R] flagged entries
-  int* sCount = sList + 16 * R;  // [1] how many, [2 ..] the waves' minima
-  if (tid == 0) *sCount = 0;
+  // Second look at the flagged sums (about one in a thousand, so about one per workgroup and
+  // five in the unluckiest): the partial-sum area is free now and holds their list.  Every wave
+  // takes one flagged sum at a time and runs the exactness test on it by itself -- no barrier
+  // until all are through.  The sums that fail it too (a product with a very low last bit: a tiny
+  // activation is enough) go on a second list.
+  int* sList = (int*)sPart;          // [<= 16 R] flagged entries
+  int* sList2 = sList + 16 * R;      // [<= 16 R] entries that want the reference's own order
+  int* sCount = sList2 + 16 * R;     // [0] flagged, [1] for the chain
+  constexpr int kSeqChunk = 512;     // 8 KiB: with the lists it fits the smallest partial-sum area
+  double2* sSeq = (double2*)(((uintptr_t)(sCount + 2) + 15) & ~(uintptr_t)15);
+  static_assert(2 * 16 * 16 * RB * 4 + 8 + 16 + kSeqChunk * 16 <= NWV * RB * 4 * 64 * 8,
+                "lists and staging area must fit the partial-sum area");
+  if (tid < 2) sCount[tid] = 0;
   __syncthreads();
   for (int ent = tid; ent < 16 * R; ent += NT)
     if (sFlag[ent]) sList[atomicAdd(sCount, 1)] = ent;
   __syncthreads();
   const int n_flagged = *sCount;
-  for (int i = 0; i < n_flagged; ++i) {
+  for (int i = wave; i < n_flagged; i += NWV) {  // wave-uniform
     const int ei = sList[i];
     const int ft = ei / R, fr = ei - ft * R;
     const XT* xr = x + (size_t)min(t0 + ft, T - 1) * d;
     const float* wr = fr < E ? w_router + (size_t)fr * d : gate_vec;
     int qmin = kNoLsb;
 #pragma unroll 2
-    for (int c = tid * 8; c < d; c += NT * 8) {  // eight columns per thread and trip
+    for (int c = lane * 8; c < d; c += 64 * 8) {  // eight columns per lane and trip
       XChunk<XT> xn;
       XChunk<float> wn;
       xn.load(xr + c);
@@ -740,21 +748,37 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
     }
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) qmin = min(qmin, __shfl_xor(qmin, off));
-    if (lane == 0) sCount[2 + wave] = qmin;
-    __syncthreads();
-    if (tid == 0) {
-      for (int w = 0; w < NWV; ++w) qmin = min(qmin, sCount[2 + w]);
+    if (lane == 0) {
       const double bound = sqrt(sXn2[ft] * sWn2[fr]) * 1.001;
       const bool exact = qmin == kNoLsb || (qmin > -2000 && bound < ldexp(1.0, qmin + 53));
-      if (!exact) {
-        // the reference's own order: one sequential c-ascending f64 sum
-        double a = 0.0;
-        for (int c = 0; c < d; ++c) a = fma((double)wr[c], (double)load_x(xr, c), a);
-        sAcc[ei] = a;
-      }
+      if (!exact) sList2[atomicAdd(sCount + 1, 1)] = ei;
     }
-    __syncthreads();
   }
+  __syncthreads();
+  // The reference's own order for those: one sequential c-ascending f64 sum.  The workgroup
+  // widens kSeqChunk columns at a time into LDS and one thread walks them, so each step of the
+  // chain waits for an LDS read instead of two trips to L2 (d = 2048: ~10 us instead of ~115).
+  const int n_chain = sCount[1];
+  for (int i = 0; i < n_chain; ++i) {
+    const int ei = sList2[i];
+    const int ft = ei / R, fr = ei - ft * R;
+    const XT* xr = x + (size_t)min(t0 + ft, T - 1) * d;
+    const float* wr = fr < E ? w_router + (size_t)fr * d : gate_vec;
+    double a = 0.0;
+    for (int c0 = 0; c0 < d; c0 += kSeqChunk) {
+      const int n = min(kSeqChunk, d - c0);
+      for (int c = tid; c < n; c += NT)
+        sSeq[c] = double2{(double)wr[c0 + c], (double)load_x(xr, c0 + c)};
+      __syncthreads();
+      if (tid == 0) {
+#pragma unroll 8
+        for (int c = 0; c < n; ++c) a = fma(sSeq[c].x, sSeq[c].y, a);
+      }
+      __syncthreads();
+    }
+    if (tid == 0) sAcc[ei] = a;
+  }
+  if (n_chain) __syncthreads();
 
   for (int ent = tid; ent < 16 * R; ent += NT) {
     const int ft = ent / R, fr = ent - ft * R;
@@ -769,18 +793,67 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
   }
   __syncthreads();
   if (E <= 64) {
-    // one wavefront per token (lane r = expert r, select_wave.h): the reference's sequential
-    // folds run over v_readlane values instead of one thread per token walking LDS
-    for (int tk = wave; tk < TT && t0 + tk < T; tk += NWV) {
-      const WaveRouting wr = wave_softmax_topk(sLogit + tk * R, E, k, renorm, lane);
-      if (wr.bad) {
+    // Softmax and top-k with lane r = expert r, a wave taking the tokens wave, wave + NWV, ...
+    // Same arithmetic, casts and order as softmax_topk (and wave_softmax_topk in select_wave.h);
+    // what is laid out for speed is the two loops of 64 steps: the reference's sequential fold
+    // of the exponentials is run for all 16 tokens at once by 16 lanes reading LDS, and the
+    // ranking loop is unrolled in eights (experts past E hold weight 0 and an index above every
+    // real one, so they never sort before a real expert).
+    constexpr int TPW = TT / NWV;
+    double* sExp = smem_m;            // [16][64]: the partial-sum area again
+    double* sInv = sExp + TT * 64;    // [16]
+    static_assert((TT * 64 + TT) * 8 <= NWV * RB * 4 * 64 * 8, "softmax scratch must fit");
+    const bool on = lane < E;
+    double ex[TPW];
+#pragma unroll
+    for (int j = 0; j < TPW; ++j) {
+      const int tk = wave + j * NWV;
+      const float my = on ? sLogit[tk * R + lane] : -INFINITY;
+      float mx = fmaxf(-INFINITY, my);  // a NaN logit is skipped, as f32::max skips it
+#pragma unroll
+      for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+      ex[j] = on ? exp((double)(my - mx)) : 0.0;  // f32 subtraction, then f64 exp
+      sExp[tk * 64 + lane] = ex[j];
+    }
+    __syncthreads();
+    if (tid < TT) {
+      const double* xe = sExp + tid * 64;
+      double sum = 0.0;
+      for (int e0 = 0; e0 < E; e0 += 8) {  // sequential fold, e ascending; the padding adds +0
+#pragma unroll
+        for (int u = 0; u < 8; ++u) sum += xe[e0 + u];
+      }
+      sInv[tid] = sum > 0.0 ? 1.0 / sum : 0.0;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < TPW; ++j) {
+      const int tk = wave + j * NWV;
+      if (t0 + tk >= T) break;  // wave-uniform
+      const float wt = (float)(ex[j] * sInv[tk]);
+      if (on && (!isfinite(wt) || wt < 0.f)) {
         atomicMin(&status[0], -3);
         atomicMin(&status[1], ((t0 + tk) << 10) | lane);
       }
-      if (wr.selected && wr.slot < k) {
-        const size_t o = (size_t)(t0 + tk) * k + wr.slot;
+      int rank = 0;  // experts that sort before this one under (weight desc, index asc)
+      for (int e0 = 0; e0 < E; e0 += 8) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const float we = readlane_f32(wt, e0 + u);
+          rank += (we > wt) || (we == wt && e0 + u < lane);
+        }
+      }
+      const bool selected = on && rank < k;
+      const unsigned long long mask = __ballot(selected);
+      const int slot = __popcll(mask & ((1ull << lane) - 1ull));
+      double ssum = 0.0;  // ascending e, as the reference sums the sorted selection
+      for (unsigned long long m = mask; m; m &= m - 1)
+        ssum += (double)readlane_f32(wt, __ffsll((long long)m) - 1);
+      const double scale = renorm ? 1.0 / ssum : 1.0;
+      if (selected && slot < k) {
+        const size_t o = (size_t)(t0 + tk) * k + slot;
         idx_out[o] = lane;
-        w_out[o] = wr.w;
+        w_out[o] = (float)((double)wt * scale);
       }
     }
     return;

@@ -181,7 +181,8 @@ def test_router_batched_kernel_with_wide_exponent_spread(ora):
     (60, 4, 2048, 700, True, False, True, False), (64, 6, 1024, 1037, False, True, True, True),
     (20, 3, 96, 530, True, False, True, True), (33, 2, 160, 2000, False, False, True, False),
     (79, 5, 256, 600, True, False, True, True), (48, 8, 512, 513, False, True, True, False),
-    (60, 4, 512, 8192, True, False, True, False), (8, 2, 1024, 900, False, False, False, False)])
+    (60, 4, 512, 8192, True, False, True, False), (8, 2, 1536, 600, False, False, True, True),
+    (40, 4, 640, 520, False, True, True, True), (8, 2, 1024, 900, False, False, False, False)])
 def test_router_matrix_core_kernel(ora, E, k, d, T, gated, bias, bf16_router, wide):
     """bf16 activations on the device, 513 to 8192 tokens, up to 80 rows, router rows whose values
     fit bf16: the router runs on the f64 matrix cores in whatever order they add, and must still
