@@ -553,14 +553,93 @@ template <> struct XChunk<uint16_t> {
   }
 };
 
+// Largest value over the 64 lanes of a wave, in every lane: four DPP steps make each row of 16
+// lanes uniform (swap neighbours, swap pairs, mirror the half row, mirror the row), the four row
+// values meet on the scalar side.
+__device__ inline int wave_max_i32(int v) {
+  v = max(v, __builtin_amdgcn_update_dpp(v, v, 0xB1, 0xf, 0xf, false));   // quad_perm [1,0,3,2]
+  v = max(v, __builtin_amdgcn_update_dpp(v, v, 0x4E, 0xf, 0xf, false));   // quad_perm [2,3,0,1]
+  v = max(v, __builtin_amdgcn_update_dpp(v, v, 0x141, 0xf, 0xf, false));  // row_half_mirror
+  v = max(v, __builtin_amdgcn_update_dpp(v, v, 0x140, 0xf, 0xf, false));  // row_mirror
+  return max(max(__builtin_amdgcn_readlane(v, 0), __builtin_amdgcn_readlane(v, 16)),
+             max(__builtin_amdgcn_readlane(v, 32), __builtin_amdgcn_readlane(v, 48)));
+}
+
+// Top-k of one token from its softmax weights (lane r = expert r) and the routing written out:
+// the k experts that sort first under (weight desc, index asc) are found as k times the largest
+// weight still available, the lowest lane among equals.  Weights are >= +0, so their bit
+// patterns order like integers (-1 = not available; a NaN weight is reported by the caller).
+// The weights of the selection are summed e ascending, as the reference sums its sorted
+// selection (dense.rs:172-187, sparse.rs:142-191).
+__device__ inline void wave_topk_write(float wt, bool on, int lane, int k, int renorm, int token,
+                                       int32_t* __restrict__ idx_out, float* __restrict__ w_out) {
+  const int wbits = on ? __float_as_int(wt) : -1;
+  unsigned long long avail = ~0ull, mask = 0ull;
+  for (int r = 0; r < k; ++r) {
+    const int v = (avail >> lane) & 1ull ? wbits : -1;
+    const int m = wave_max_i32(v);
+    const unsigned long long cand = __ballot(v == m && m >= 0);
+    if (!cand) break;  // wave-uniform; k <= E makes it unreachable
+    const unsigned long long win = cand & (~cand + 1ull);
+    mask |= win;
+    avail &= ~win;
+  }
+  const bool selected = (mask >> lane) & 1ull;
+  const int slot = __popcll(mask & ((1ull << lane) - 1ull));
+  double ssum = 0.0;
+  for (unsigned long long m = mask; m; m &= m - 1)
+    ssum += (double)readlane_f32(wt, __ffsll((long long)m) - 1);
+  const double scale = renorm ? 1.0 / ssum : 1.0;
+  if (selected && slot < k) {
+    const size_t o = (size_t)token * k + slot;
+    idx_out[o] = lane;
+    w_out[o] = (float)((double)wt * scale);
+  }
+}
+
+// Softmax + top-k from logits that another launch left in HBM, one wavefront per token (up to 64
+// experts).  Same arithmetic, casts and order as softmax_topk; the sequential fold of the
+// exponentials runs over v_readlane values.
+constexpr int kWaveSelectThreads = 256;
+__global__ __launch_bounds__(kWaveSelectThreads) void wave_select_kernel(
+    const float* __restrict__ logits, int T, int E, int k, int renorm,
+    int32_t* __restrict__ idx_out, float* __restrict__ w_out, int32_t* __restrict__ status) {
+  const int lane = threadIdx.x & 63;
+  const int t = blockIdx.x * (kWaveSelectThreads / 64) + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  if (t >= T) return;
+  const bool on = lane < E;
+  const float my = on ? logits[(size_t)t * E + lane] : -INFINITY;
+  float mx = fmaxf(-INFINITY, my);  // a NaN logit is skipped, as f32::max skips it
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+  const double ex = on ? exp((double)(my - mx)) : 0.0;  // f32 subtraction, then f64 exp
+  double sum = 0.0;
+  for (int e0 = 0; e0 < E; e0 += 8) {  // sequential fold, e ascending; lanes past E add +0
+#pragma unroll
+    for (int u = 0; u < 8; ++u) sum += readlane_f64(ex, e0 + u);
+  }
+  const double inv = sum > 0.0 ? 1.0 / sum : 0.0;
+  const float wt = (float)(ex * inv);
+  if (on && (!isfinite(wt) || wt < 0.f)) {
+    atomicMin(&status[0], -3);
+    atomicMin(&status[1], (t << 10) | lane);
+  }
+  wave_topk_write(wt, on, lane, k, renorm, t, idx_out, w_out);
+}
+
 template <typename XT, int RB, int NBUF, int NWV>
 __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
     const XT* __restrict__ x, int T, int d, int E, int k, int renorm,
     const float* __restrict__ w_router, const float* __restrict__ bias,
     const float* __restrict__ gate_vec, int32_t* __restrict__ idx_out,
-    float* __restrict__ w_out, float* __restrict__ sgate_out, int32_t* __restrict__ status) {
+    float* __restrict__ w_out, float* __restrict__ sgate_out, int32_t* __restrict__ status,
+    float* __restrict__ logits_out) {
+  // gridDim.y > 1 (only with logits_out): this workgroup owns the rows row0 .. row0 + R - 1 of
+  // the stacked matrix [W_r ; gate] and leaves the logits to another launch; otherwise all rows.
   constexpr int TT = 16;
-  const int R = E + (gate_vec ? 1 : 0);
+  const int R_all = E + (gate_vec ? 1 : 0);
+  const int row0 = blockIdx.y * 16 * RB;
+  const int R = min(16 * RB, R_all - row0);
   const int t0 = blockIdx.x * TT;
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -582,7 +661,7 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
   const float* pw[RB];
 #pragma unroll
   for (int b = 0; b < RB; ++b) {
-    const int r = min(16 * b + r16, R - 1);
+    const int r = row0 + min(16 * b + r16, R - 1);
     pw[b] = (r < E ? w_router + (size_t)r * d : gate_vec) + 8 * q;
   }
   // k in steps of 32 (8 per lane), the steps dealt to the four waves in contiguous runs
@@ -695,7 +774,7 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
     const double e = sqrt(xn2 * wn2) * gfac;
     const double lo = a - e, hi = a + e;
     bool ok;
-    if (r < E) {
+    if (row0 + r < E) {
       const float flo = (float)lo, fhi = (float)hi;
       ok = flo == fhi && isfinite(flo);
     } else {
@@ -708,51 +787,76 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
   __syncthreads();
 
   // Second look at the flagged sums (about one in a thousand, so about one per workgroup and
-  // five in the unluckiest): the partial-sum area is free now and holds their list.  Every wave
-  // takes one flagged sum at a time and runs the exactness test on it by itself -- no barrier
-  // until all are through.  The sums that fail it too (a product with a very low last bit: a tiny
-  // activation is enough) go on a second list.
+  // five in the unluckiest): the partial-sum area is free now and holds their list.  The
+  // exactness test reads both rows of a flagged sum once; those reads are dealt to the waves in
+  // pieces of 512 columns, whichever sum they belong to, so a workgroup with one flagged sum
+  // and one with five both keep all their waves busy.  The sums that fail this test too (a
+  // product with a very low last bit: one tiny activation is enough) go on a second list.
   int* sList = (int*)sPart;          // [<= 16 R] flagged entries
   int* sList2 = sList + 16 * R;      // [<= 16 R] entries that want the reference's own order
-  int* sCount = sList2 + 16 * R;     // [0] flagged, [1] for the chain
+  int* sQ = sList2 + 16 * R;         // [<= 16 R] lowest last-bit exponent of a flagged entry's products
+  int* sCount = sQ + 16 * R;         // [0] flagged, [1] for the chain
   constexpr int kSeqChunk = 512;     // 8 KiB: with the lists it fits the smallest partial-sum area
   double2* sSeq = (double2*)(((uintptr_t)(sCount + 2) + 15) & ~(uintptr_t)15);
-  static_assert(2 * 16 * 16 * RB * 4 + 8 + 16 + kSeqChunk * 16 <= NWV * RB * 4 * 64 * 8,
+  static_assert(3 * 16 * 16 * RB * 4 + 8 + 16 + kSeqChunk * 16 <= NWV * RB * 4 * 64 * 8,
                 "lists and staging area must fit the partial-sum area");
   if (tid < 2) sCount[tid] = 0;
   __syncthreads();
   for (int ent = tid; ent < 16 * R; ent += NT)
-    if (sFlag[ent]) sList[atomicAdd(sCount, 1)] = ent;
+    if (sFlag[ent]) {
+      const int at = atomicAdd(sCount, 1);
+      sList[at] = ent;
+      sQ[at] = kNoLsb;
+    }
   __syncthreads();
   const int n_flagged = *sCount;
-  for (int i = wave; i < n_flagged; i += NWV) {  // wave-uniform
-    const int ei = sList[i];
-    const int ft = ei / R, fr = ei - ft * R;
-    const XT* xr = x + (size_t)min(t0 + ft, T - 1) * d;
-    const float* wr = fr < E ? w_router + (size_t)fr * d : gate_vec;
-    int qmin = kNoLsb;
-#pragma unroll 2
-    for (int c = lane * 8; c < d; c += 64 * 8) {  // eight columns per lane and trip
-      XChunk<XT> xn;
-      XChunk<float> wn;
-      xn.load(xr + c);
-      wn.load(wr + c);
+  const int pieces = (d + 511) / 512;
+  const int n_items = n_flagged * pieces;
+  constexpr int NB = 4;  // pieces a wave has in flight: their loads leave together
+  for (int it0 = wave; it0 < n_items; it0 += NWV * NB) {  // wave-uniform
+    XChunk<XT> xn[NB];
+    XChunk<float> wn[NB];
+    int ent[NB];
+    bool in[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      const int it = it0 + b * NWV;
+      const bool valid = it < n_items;  // a piece past the end re-reads the first one
+      const int itc = valid ? it : it0;
+      const int i = itc / pieces, piece = itc - i * pieces;
+      const int ei = sList[i];
+      const int ft = ei / R, fr = ei - ft * R;
+      const XT* xr = x + (size_t)min(t0 + ft, T - 1) * d;
+      const float* wr = row0 + fr < E ? w_router + (size_t)(row0 + fr) * d : gate_vec;
+      const int c = piece * 512 + lane * 8;  // eight columns per lane
+      in[b] = valid && c < d;                // d is a multiple of 8: a chunk is whole or absent
+      ent[b] = i;
+      xn[b].load(xr + (c < d ? c : 0));
+      wn[b].load(wr + (c < d ? c : 0));
+    }
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
       float xf[8], wf[8];
-      xn.get(xf);
-      wn.get(wf);
+      xn[b].get(xf);
+      wn[b].get(wf);
+      int qmin = kNoLsb;
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         const int lx = lsb_exponent(xf[u]), lw = lsb_exponent(wf[u]);
-        qmin = min(qmin, (lx != kNoLsb && lw != kNoLsb) ? lx + lw : kNoLsb);
+        qmin = min(qmin, (in[b] && lx != kNoLsb && lw != kNoLsb) ? lx + lw : kNoLsb);
       }
-    }
 #pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) qmin = min(qmin, __shfl_xor(qmin, off));
-    if (lane == 0) {
-      const double bound = sqrt(sXn2[ft] * sWn2[fr]) * 1.001;
-      const bool exact = qmin == kNoLsb || (qmin > -2000 && bound < ldexp(1.0, qmin + 53));
-      if (!exact) sList2[atomicAdd(sCount + 1, 1)] = ei;
+      for (int off = 32; off >= 1; off >>= 1) qmin = min(qmin, __shfl_xor(qmin, off));
+      if (lane == 0 && qmin != kNoLsb) atomicMin(sQ + ent[b], qmin);
     }
+  }
+  __syncthreads();
+  for (int i = tid; i < n_flagged; i += NT) {
+    const int ei = sList[i], qmin = sQ[i];
+    const int ft = ei / R, fr = ei - ft * R;
+    const double bound = sqrt(sXn2[ft] * sWn2[fr]) * 1.001;
+    const bool exact = qmin == kNoLsb || (qmin > -2000 && bound < ldexp(1.0, qmin + 53));
+    if (!exact) sList2[atomicAdd(sCount + 1, 1)] = ei;
   }
   __syncthreads();
   // The reference's own order for those: one sequential c-ascending f64 sum.  The workgroup
@@ -763,7 +867,7 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
     const int ei = sList2[i];
     const int ft = ei / R, fr = ei - ft * R;
     const XT* xr = x + (size_t)min(t0 + ft, T - 1) * d;
-    const float* wr = fr < E ? w_router + (size_t)fr * d : gate_vec;
+    const float* wr = row0 + fr < E ? w_router + (size_t)(row0 + fr) * d : gate_vec;
     double a = 0.0;
     for (int c0 = 0; c0 < d; c0 += kSeqChunk) {
       const int n = min(kSeqChunk, d - c0);
@@ -783,22 +887,24 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
   for (int ent = tid; ent < 16 * R; ent += NT) {
     const int ft = ent / R, fr = ent - ft * R;
     const double a = sAcc[ent];
-    if (fr < E) {
+    if (row0 + fr < E) {
       float logit = (float)a;
-      if (bias) logit = logit + bias[fr];
+      if (bias) logit = logit + bias[row0 + fr];
       sLogit[ent] = logit;
+      if (logits_out && t0 + ft < T) logits_out[(size_t)(t0 + ft) * E + row0 + fr] = logit;
     } else if (t0 + ft < T) {
       sgate_out[t0 + ft] = (float)(1.0 / (1.0 + exp(-a)));
     }
   }
+  if (logits_out) return;  // routing is decided by another launch from the logits
   __syncthreads();
   if (E <= 64) {
     // Softmax and top-k with lane r = expert r, a wave taking the tokens wave, wave + NWV, ...
     // Same arithmetic, casts and order as softmax_topk (and wave_softmax_topk in select_wave.h);
     // what is laid out for speed is the two loops of 64 steps: the reference's sequential fold
     // of the exponentials is run for all 16 tokens at once by 16 lanes reading LDS, and the
-    // ranking loop is unrolled in eights (experts past E hold weight 0 and an index above every
-    // real one, so they never sort before a real expert).
+    // selection takes k maxima over the wave instead of ranking every expert against every
+    // other.
     constexpr int TPW = TT / NWV;
     double* sExp = smem_m;            // [16][64]: the partial-sum area again
     double* sInv = sExp + TT * 64;    // [16]
@@ -835,26 +941,7 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
         atomicMin(&status[0], -3);
         atomicMin(&status[1], ((t0 + tk) << 10) | lane);
       }
-      int rank = 0;  // experts that sort before this one under (weight desc, index asc)
-      for (int e0 = 0; e0 < E; e0 += 8) {
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const float we = readlane_f32(wt, e0 + u);
-          rank += (we > wt) || (we == wt && e0 + u < lane);
-        }
-      }
-      const bool selected = on && rank < k;
-      const unsigned long long mask = __ballot(selected);
-      const int slot = __popcll(mask & ((1ull << lane) - 1ull));
-      double ssum = 0.0;  // ascending e, as the reference sums the sorted selection
-      for (unsigned long long m = mask; m; m &= m - 1)
-        ssum += (double)readlane_f32(wt, __ffsll((long long)m) - 1);
-      const double scale = renorm ? 1.0 / ssum : 1.0;
-      if (selected && slot < k) {
-        const size_t o = (size_t)(t0 + tk) * k + slot;
-        idx_out[o] = lane;
-        w_out[o] = (float)((double)wt * scale);
-      }
+      wave_topk_write(wt, on, lane, k, renorm, t0 + tk, idx_out, w_out);
     }
     return;
   }
@@ -874,7 +961,27 @@ hipError_t launch_router_mfma_rb(const RouterArgs& a, int R, hipStream_t s) {
   if (smem > 64 * 1024) return hipErrorInvalidValue;
   router_mfma_kernel<XT, RB, NBUF, NWV><<<(a.T + 15) / 16, 64 * NWV, smem, s>>>(
       (const XT*)a.x, a.T, a.d, a.E, a.k, a.renorm, a.w_router, a.router_bias, a.shared_gate,
-      a.idx, a.w, a.sgate, a.status);
+      a.idx, a.w, a.sgate, a.status, nullptr);
+  return hipGetLastError();
+}
+
+// The same kernel with the rows dealt to workgroups in blocks of 16 (eight waves split k), the
+// logits left in HBM and the routing decided by a second launch, one wave per token: with many
+// rows and a batch that gives fewer workgroups of 16 tokens than the chip has compute units,
+// four times as many workgroups of a quarter of the length.
+template <typename XT>
+hipError_t launch_router_mfma_split(const RouterArgs& a, int R, hipStream_t s) {
+  constexpr int NWV = 8, RB = 1, RL = 16;
+  const size_t smem = ((size_t)NWV * RB * 4 * 64 + NWV * 16 + (size_t)NWV * RB * 16 + (size_t)16 * RL + 16 + RL) * 8 +
+                      (size_t)16 * RL * 4 + (size_t)16 * RL + 16;
+  router_mfma_kernel<XT, RB, 4, NWV><<<dim3((a.T + 15) / 16, (R + 15) / 16), 64 * NWV, smem, s>>>(
+      (const XT*)a.x, a.T, a.d, a.E, a.k, a.renorm, a.w_router, a.router_bias, a.shared_gate,
+      a.idx, a.w, a.sgate, a.status, a.logits_tmp);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  constexpr int per = kWaveSelectThreads / 64;
+  wave_select_kernel<<<(a.T + per - 1) / per, kWaveSelectThreads, 0, s>>>(
+      a.logits_tmp, a.T, a.E, a.k, a.renorm, a.idx, a.w, a.status);
   return hipGetLastError();
 }
 
@@ -904,15 +1011,36 @@ bool router_mfma_ok(const RouterArgs& a, int R) {
          a.x_is_bf16 && a.w_fits_bf16 && a.E >= a.k;
 }
 
+// When the rows are dealt to workgroups.  Measured on MI355X, d = 2048, route stage in us,
+// split / one workgroup per 16 tokens: 64 rows T = 600 26 / 54, 1024 25 / 54, 2048 36 / 57,
+// 3072 57 / 58, 4096 64 / 59, 8192 116 / 87; 32 rows T = 1024 24 / 29, 2048 25 / (29-32),
+// 4096 37 / 32; 48 rows, d = 4096, T = 2048 54 / 81.  Against the per-token kernel below 512
+// tokens (64 rows): T = 16 23 / 19, 32 24 / 23, 48 24 / 27, 64 24 / 32, 128 24 / 28, 256 24 / 32,
+// 384 25 / 47, 512 25 / 50; 32 rows: T = 128 23 / 20, 512 23 / 35.
+// ATENIA_MOE_ROUTER_SPLIT_MIN_T / _MAX_T move the bounds (a maximum of 0 switches it off).
+bool router_mfma_split_wanted(const RouterArgs& a, int R) {
+  static const int max_t = [] {
+    const char* e = getenv("ATENIA_MOE_ROUTER_SPLIT_MAX_T");
+    return e ? atoi(e) : 2048;
+  }();
+  static const int min_t = [] {
+    const char* e = getenv("ATENIA_MOE_ROUTER_SPLIT_MIN_T");
+    return e ? atoi(e) : -1;
+  }();
+  const int lo = min_t >= 0 ? min_t : R > 32 ? 40 : 192;
+  return R > 16 && a.E <= 64 && a.logits_tmp && a.T >= lo && a.T <= max_t;
+}
+
 template <typename XT>
 hipError_t launch_router_mfma(const RouterArgs& a, int R, hipStream_t s) {
+  if (router_mfma_split_wanted(a, R)) return launch_router_mfma_split<XT>(a, R, s);
   // few rows: eight waves split k, so that a batch of 4096 tokens (256 workgroups, one per
   // compute unit) still puts two waves on every SIMD
   if (R <= 16) return launch_router_mfma_rb<XT, 1, 4, 8>(a, R, s);
   if (R <= 32) return launch_router_mfma_rb<XT, 2, 3, 8>(a, R, s);
-  if (R <= 48) return launch_router_mfma_rb<XT, 3, 2, 4>(a, R, s);
-  if (R <= 64) return launch_router_mfma_rb<XT, 4, 2, 4>(a, R, s);
-  return launch_router_mfma_rb<XT, 5, 2, 4>(a, R, s);
+  if (R <= 48) return launch_router_mfma_rb<XT, 3, 3, 4>(a, R, s);
+  if (R <= 64) return launch_router_mfma_rb<XT, 4, 3, 4>(a, R, s);
+  return launch_router_mfma_rb<XT, 5, 3, 4>(a, R, s);
 }
 
 template <typename XT>
@@ -1175,7 +1303,8 @@ hipError_t launch_router(const RouterArgs& a, hipStream_t s, int* fused_permute)
   if (R > kMaxRouterRows || a.T <= 0) return hipErrorInvalidValue;
   // The per-token kernel re-reads the whole stacked matrix for every token; with many rows
   // (row blocks, logits mode) that only pays for a handful of tokens.
-  const bool token_ok = a.T <= a.token_kernel_max_tokens &&
+  const bool mfma = router_mfma_ok(a, R);
+  const bool token_ok = a.T <= a.token_kernel_max_tokens && !(mfma && router_mfma_split_wanted(a, R)) &&
                         (R <= 64 || (long long)a.T * R * a.d <= (16ll << 20));
   if (token_ok) {
     const size_t np = R > kTokenThreads / 64 ? R : kTokenThreads / 64;
@@ -1225,7 +1354,7 @@ hipError_t launch_router(const RouterArgs& a, hipStream_t s, int* fused_permute)
       return hipGetLastError();
     }
   }
-  if (router_mfma_ok(a, R))
+  if (mfma)
     return a.x_is_bf16 ? launch_router_mfma<uint16_t>(a, R, s) : launch_router_mfma<float>(a, R, s);
   // Up to 64 rows per workgroup; more rows only when the logits leave the kernel (row blocks).
   if ((R <= 64 || a.logits_out) && a.d % 4 == 0 && (!a.xb || a.d_pad % 4 == 0)) {

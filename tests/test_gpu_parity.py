@@ -182,9 +182,17 @@ def test_router_batched_kernel_with_wide_exponent_spread(ora):
     (20, 3, 96, 530, True, False, True, True), (33, 2, 160, 2000, False, False, True, False),
     (79, 5, 256, 600, True, False, True, True), (48, 8, 512, 513, False, True, True, False),
     (60, 4, 512, 8192, True, False, True, False), (8, 2, 1536, 600, False, False, True, True),
-    (40, 4, 640, 520, False, True, True, True), (8, 2, 1024, 900, False, False, False, False)])
+    (40, 4, 640, 520, False, True, True, True),
+    # the rows dealt to workgroups in blocks of 16, selection as a second launch: from 40 tokens
+    # (more than 32 rows) or 192 (17 to 32 rows) up to 2048
+    (60, 4, 2048, 40, True, False, True, False), (64, 6, 512, 200, False, True, True, True),
+    (32, 4, 256, 192, False, False, True, False), (61, 4, 128, 2048, False, False, True, True),
+    # beyond 2048 tokens one workgroup holds all rows again: two to four row blocks
+    (20, 3, 96, 2100, True, False, True, True), (40, 4, 640, 2500, False, True, True, True),
+    (64, 6, 1024, 2300, False, False, True, True),
+    (8, 2, 1024, 900, False, False, False, False)])
 def test_router_matrix_core_kernel(ora, E, k, d, T, gated, bias, bf16_router, wide):
-    """bf16 activations on the device, 513 to 8192 tokens, up to 80 rows, router rows whose values
+    """bf16 activations on the device, up to 8192 tokens, up to 80 rows, router rows whose values
     fit bf16: the router runs on the f64 matrix cores in whatever order they add, and must still
     give the reference's routing for every token -- through the interval certificate, the
     exactness test, or the sequential recomputation (`wide`: activations spread over 60 binades
