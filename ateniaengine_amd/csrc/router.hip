@@ -1015,8 +1015,8 @@ bool router_mfma_ok(const RouterArgs& a, int R) {
 // split / one workgroup per 16 tokens: 64 rows T = 600 26 / 54, 1024 25 / 54, 2048 36 / 57,
 // 3072 57 / 58, 4096 64 / 59, 8192 116 / 87; 32 rows T = 1024 24 / 29, 2048 25 / (29-32),
 // 4096 37 / 32; 48 rows, d = 4096, T = 2048 54 / 81.  Against the per-token kernel below 512
-// tokens (64 rows): T = 16 23 / 19, 32 24 / 23, 48 24 / 27, 64 24 / 32, 128 24 / 28, 256 24 / 32,
-// 384 25 / 47, 512 25 / 50; 32 rows: T = 128 23 / 20, 512 23 / 35.
+// tokens (64 rows): T = 16 23 / 15, 32 24 / 19, 48 24 / 23, 56 24 / 27, 64 24 / 29, 128 24 / 28,
+// 256 24 / 32, 384 25 / 47, 512 25 / 50; 32 rows: T = 128 23 / 20, 512 23 / 35.
 // ATENIA_MOE_ROUTER_SPLIT_MIN_T / _MAX_T move the bounds (a maximum of 0 switches it off).
 bool router_mfma_split_wanted(const RouterArgs& a, int R) {
   static const int max_t = [] {
@@ -1027,7 +1027,7 @@ bool router_mfma_split_wanted(const RouterArgs& a, int R) {
     const char* e = getenv("ATENIA_MOE_ROUTER_SPLIT_MIN_T");
     return e ? atoi(e) : -1;
   }();
-  const int lo = min_t >= 0 ? min_t : R > 32 ? 40 : 192;
+  const int lo = min_t >= 0 ? min_t : R > 32 ? 52 : 192;
   return R > 16 && a.E <= 64 && a.logits_tmp && a.T >= lo && a.T <= max_t;
 }
 
@@ -1347,6 +1347,12 @@ hipError_t launch_router(const RouterArgs& a, hipStream_t s, int* fused_permute)
       if (spread && !a.logits_out) {
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
+        if (a.E <= 64 && !fg.counts) {  // one wave per token
+          constexpr int per = kWaveSelectThreads / 64;
+          wave_select_kernel<<<(a.T + per - 1) / per, kWaveSelectThreads, 0, s>>>(
+              lg, a.T, a.E, a.k, a.renorm, a.idx, a.w, a.status);
+          return hipGetLastError();
+        }
         const int TT = kSelectThreads / a.E;
         softmax_select_kernel<<<(a.T + TT - 1) / TT, kSelectThreads, 0, s>>>(
             lg, a.T, a.E, a.k, a.renorm, a.idx, a.w, a.status, fg);

@@ -183,9 +183,9 @@ def test_router_batched_kernel_with_wide_exponent_spread(ora):
     (79, 5, 256, 600, True, False, True, True), (48, 8, 512, 513, False, True, True, False),
     (60, 4, 512, 8192, True, False, True, False), (8, 2, 1536, 600, False, False, True, True),
     (40, 4, 640, 520, False, True, True, True),
-    # the rows dealt to workgroups in blocks of 16, selection as a second launch: from 40 tokens
+    # the rows dealt to workgroups in blocks of 16, selection as a second launch: from 52 tokens
     # (more than 32 rows) or 192 (17 to 32 rows) up to 2048
-    (60, 4, 2048, 40, True, False, True, False), (64, 6, 512, 200, False, True, True, True),
+    (60, 4, 2048, 52, True, False, True, False), (64, 6, 512, 200, False, True, True, True),
     (32, 4, 256, 192, False, False, True, False), (61, 4, 128, 2048, False, False, True, True),
     # beyond 2048 tokens one workgroup holds all rows again: two to four row blocks
     (20, 3, 96, 2100, True, False, True, True), (40, 4, 640, 2500, False, True, True, True),
