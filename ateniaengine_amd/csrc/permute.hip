@@ -9,10 +9,12 @@
 // ascending in p inside each expert (a stable counting sort).  All integer work; results are
 // unique, so they must match the CPU oracle bit for bit.
 //
-// Small batches (P <= 1024 pairs) take one launch of one block.  Larger ones take three:
+// Small batches (P <= 1024 pairs) take one launch of one block; up to 16 blocks of 1024 pairs
+// still one launch, every block counting the whole list for itself.  Larger ones take three:
 // per-block histograms, one block that scans them, and a scatter pass that recomputes each
 // block's stable ranks.
 #include <algorithm>
+#include <cstdlib>
 
 #include "moe_internal.h"
 
@@ -30,17 +32,18 @@ __device__ int block_stable_rank(int e, bool valid, int E, int32_t* sWaveCnt,
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   for (int j = tid; j < kWaves * E; j += kPermuteBlock) sWaveCnt[j] = 0;
   __syncthreads();
-  int my_rank = 0;
-  unsigned long long todo = __ballot(valid);
+  // The lanes of this wave with the same expert: one ballot per bit of the expert index, each
+  // lane keeping the side its own bit is on (eight ballots for up to 256 experts, where a loop
+  // over the distinct experts of the wave took one round of ballot + shuffle per expert).
   const unsigned long long lt = lane == 0 ? 0ull : (~0ull >> (64 - lane));
-  while (todo) {
-    int leader = __ffsll((long long)todo) - 1;
-    int e0 = __shfl(e, leader);
-    unsigned long long m = __ballot(valid && e == e0);
-    if (valid && e == e0) my_rank = __popcll(m & lt);
-    if (lane == leader) sWaveCnt[wave * E + e0] = __popcll(m);
-    todo &= ~m;
+  unsigned long long m = __ballot(valid);
+  for (int b = 0; (1 << b) < E; ++b) {  // wave-uniform trip count
+    const bool bit = (e >> b) & 1;
+    const unsigned long long B = __ballot(bit);
+    m &= bit ? B : ~B;
   }
+  const int my_rank = __popcll(m & lt);
+  if (valid && (m & lt) == 0ull) sWaveCnt[wave * E + e] = __popcll(m);  // the first lane of its group
   __syncthreads();
   for (int ee = tid; ee < E; ee += kPermuteBlock) {
     int run = 0;
@@ -93,42 +96,65 @@ __device__ inline void expert_tile(int c, int max_groups, int nt, int i, int& m0
 // (rows, active flags, row tiles) replace a serial walk whose stores and loads through generic
 // pointers waited for each other (12 us for 60 experts).  E <= kMaxRouterRows.
 // s_offsets (LDS, [E + 1], may be null) receives the offsets as well; valid after the caller's
-// next barrier.
+// next barrier.  write_out = false: only s_offsets is wanted (another block writes the lists).
 __device__ void finish_offsets(int E, const int32_t* counts, int32_t* offsets, int32_t* active,
                                int32_t* n_active, int32_t* shared_offsets, int T, TileOut to,
-                               int32_t* s_offsets = nullptr) {
-  __shared__ int32_t sRows[kMaxRouterRows], sAct[kMaxRouterRows], sTiles[kMaxRouterRows];
+                               int32_t* s_offsets = nullptr, bool write_out = true) {
+  // exclusive prefixes over the experts, totals at [kMaxRouterRows]
+  __shared__ int32_t sRows[kMaxRouterRows + 1], sAct[kMaxRouterRows + 1], sTiles[kMaxRouterRows + 1];
   const int tid = threadIdx.x;
   const bool mine = tid < E;
   const int c = mine ? counts[tid] : 0;
   const int a = c > 0 ? 1 : 0;
   const int nt = to.tile_group ? expert_tiles(c, to.max_groups) : 0;
-  if (tid < kMaxRouterRows) {
-    sRows[tid] = c;
-    sAct[tid] = a;
-    sTiles[tid] = nt;
+  if (tid < 64) {
+    // One wave scans all three: a lane owns EPL consecutive experts, the lane totals are
+    // scanned with six shuffles each (barrier-free; sixteen barriers of 1024 threads for a
+    // step-by-step scan in LDS took longer than everything else in the launch).
+    constexpr int EPL = kMaxRouterRows / 64;
+    int cr[EPL], ca[EPL], ct[EPL];
+    int r = 0, q = 0, t = 0;
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) {
+      const int ee = EPL * tid + j;
+      const int cc = ee < E ? counts[ee] : 0;
+      cr[j] = r;
+      ca[j] = q;
+      ct[j] = t;
+      r += cc;
+      q += cc > 0 ? 1 : 0;
+      t += to.tile_group ? expert_tiles(cc, to.max_groups) : 0;
+    }
+    int ir = r, iq = q, it = t;  // inclusive over the lanes
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int ur = __shfl_up(ir, off), uq = __shfl_up(iq, off), ut = __shfl_up(it, off);
+      if (tid >= off) {
+        ir += ur;
+        iq += uq;
+        it += ut;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) {
+      sRows[EPL * tid + j] = ir - r + cr[j];
+      sAct[EPL * tid + j] = iq - q + ca[j];
+      sTiles[EPL * tid + j] = it - t + ct[j];
+    }
+    if (tid == 63) {
+      sRows[kMaxRouterRows] = ir;
+      sAct[kMaxRouterRows] = iq;
+      sTiles[kMaxRouterRows] = it;
+    }
   }
   __syncthreads();
-  for (int off = 1; off < kMaxRouterRows; off <<= 1) {  // inclusive scans, all three at once
-    int r = 0, q = 0, t = 0;
-    if (tid < kMaxRouterRows && tid >= off) {
-      r = sRows[tid - off];
-      q = sAct[tid - off];
-      t = sTiles[tid - off];
-    }
-    __syncthreads();
-    if (tid < kMaxRouterRows) {
-      sRows[tid] += r;
-      sAct[tid] += q;
-      sTiles[tid] += t;
-    }
-    __syncthreads();
-  }
+  if (mine && s_offsets) s_offsets[tid] = sRows[tid];
+  if (tid == 0 && s_offsets) s_offsets[E] = sRows[kMaxRouterRows];
+  if (!write_out) return;
   if (mine) {
-    offsets[tid] = sRows[tid] - c;
-    if (s_offsets) s_offsets[tid] = sRows[tid] - c;
-    if (a) active[sAct[tid] - 1] = tid;
-    const int t0 = sTiles[tid] - nt;
+    offsets[tid] = sRows[tid];
+    if (a) active[sAct[tid]] = tid;
+    const int t0 = sTiles[tid];
     for (int i = 0; i < nt; ++i) {
       int m0, rows;
       expert_tile(c, to.max_groups, nt, i, m0, rows);
@@ -139,10 +165,9 @@ __device__ void finish_offsets(int E, const int32_t* counts, int32_t* offsets, i
     }
   }
   if (tid == 0) {
-    offsets[E] = sRows[kMaxRouterRows - 1];
-    if (s_offsets) s_offsets[E] = sRows[kMaxRouterRows - 1];
-    *n_active = sAct[kMaxRouterRows - 1];
-    if (to.n_tiles) *to.n_tiles = sTiles[kMaxRouterRows - 1];
+    offsets[E] = sRows[kMaxRouterRows];
+    *n_active = sAct[kMaxRouterRows];
+    if (to.n_tiles) *to.n_tiles = sTiles[kMaxRouterRows];
     if (to.shared_n_tiles) *to.shared_n_tiles = (T + kTileM - 1) / kTileM;
     if (shared_offsets) {
       shared_offsets[0] = 0;
@@ -170,6 +195,51 @@ __global__ __launch_bounds__(kPermuteBlock) void permute_single_kernel(
   __syncthreads();
   if (valid) {
     int pos = sOff[e] + rank;
+    perm[pos] = p;
+    inv[p] = pos;
+  }
+}
+
+// A few thousand pairs in ONE launch: block b places the pairs b * 1024 .. of the list, and
+// counts for itself what the three-launch form below passes through HBM -- every block reads
+// the whole index list (at most kMultiBlocks * 1024 entries, from L2) and keeps, per expert,
+// the total and the number of pairs in the blocks before its own.  Block 0 writes the lists.
+constexpr int kMultiBlocks = 16;
+__global__ __launch_bounds__(kPermuteBlock) void permute_multi_kernel(
+    const int32_t* __restrict__ idx, int P, int E, int T, int32_t* counts, int32_t* offsets,
+    int32_t* perm, int32_t* inv, int32_t* active, int32_t* n_active, int32_t* shared_offsets,
+    TileOut to) {
+  extern __shared__ int32_t sm[];
+  int32_t* sWaveCnt = sm;               // [kWaves][E]
+  int32_t* sBlkCnt = sm + kWaves * E;   // [E]
+  int32_t* sOff = sBlkCnt + E;          // [E+1]
+  int32_t* sTot = sOff + E + 1;         // [E]
+  int32_t* sBefore = sTot + E;          // [E]
+  const int tid = threadIdx.x, blk = blockIdx.x, nblk = gridDim.x;
+  for (int j = tid; j < E; j += kPermuteBlock) {
+    sTot[j] = 0;
+    sBefore[j] = 0;
+  }
+  __syncthreads();
+  int e = 0;
+  for (int c = 0; c < nblk; ++c) {
+    const int q = c * kPermuteBlock + tid;
+    if (q < P) {
+      const int ee = idx[q];
+      atomicAdd(&sTot[ee], 1);
+      if (c < blk) atomicAdd(&sBefore[ee], 1);
+      if (c == blk) e = ee;
+    }
+  }
+  const int p = blk * kPermuteBlock + tid;
+  const bool valid = p < P;
+  int rank = block_stable_rank(e, valid, E, sWaveCnt, sBlkCnt);  // barriers inside: the counts are complete
+  if (blk == 0)
+    for (int ee = tid; ee < E; ee += kPermuteBlock) counts[ee] = sTot[ee];
+  finish_offsets(E, sTot, offsets, active, n_active, shared_offsets, T, to, sOff, blk == 0);
+  __syncthreads();
+  if (valid) {
+    int pos = sOff[e] + sBefore[e] + rank;
     perm[pos] = p;
     inv[p] = pos;
   }
@@ -281,6 +351,19 @@ hipError_t launch_permute(const PermuteArgs& a, hipStream_t s, int* n_launches) 
     return hipGetLastError();
   }
   const int nblk = (P + kPermuteBlock - 1) / kPermuteBlock;
+  static const int multi_max = [] {
+    const char* e = getenv("ATENIA_MOE_PERMUTE_MULTI_BLOCKS");  // tuning knob: 0 = three launches
+    const int n = e ? atoi(e) : kMultiBlocks;
+    return n < 0 ? 0 : n > 64 ? 64 : n;
+  }();
+  if (nblk <= multi_max) {
+    size_t sm = ((size_t)kWaves * E + 4 * (size_t)E + 1) * sizeof(int32_t);
+    permute_multi_kernel<<<nblk, kPermuteBlock, sm, s>>>(a.idx, P, E, a.T, a.counts, a.offsets,
+                                                         a.perm, a.inv, a.active, a.n_active,
+                                                         a.shared_offsets, to);
+    if (n_launches) *n_launches = 1;
+    return hipGetLastError();
+  }
   permute_hist_kernel<<<nblk, kPermuteBlock, (size_t)E * sizeof(int32_t), s>>>(a.idx, P, E,
                                                                                  a.blk_counts);
   const int nseg = std::max(1, std::min(nblk, kPermuteBlock / E));
