@@ -992,12 +992,10 @@ bool router_mfma_ok(const RouterArgs& a, int R) {
     const char* e = getenv("ATENIA_MOE_ROUTER_MFMA");  // tuning knob: 0 = sequential chains
     return e && atoi(e) == 0;
   }();
-  // Up to 8192 tokens (6144 with one block of rows): measured 31-42 us against 57-75 us (8 rows, d = 4096, T <= 4096) and, with
-  // 61-64 rows and d = 2048, about 70 us against 92-97 us up to T = 4096, 97-138 against 142 at
-  // T = 6144, 102-105 against 127 at T = 8192; at T = 12288 174-210 against 186-189 and at
-  // T = 16384 225 against 195: larger batches are left to the sequential kernel, which catches
-  // up there (two tokens per thread) and has no slow path.  ATENIA_MOE_ROUTER_MFMA_MAX_T moves
-  // the bound.
+  // Against the sequential kernel (route stage, us): 8 rows, d = 4096: T = 4096 32 / 57-75,
+  // 8192 48 / 89, 16384 89 / 160; 61-64 rows, d = 2048: T = 4096 59 / 92-97, 8192 86 / 87,
+  // 12288 127 / 178, 16384 155 / 180.  ATENIA_MOE_ROUTER_MFMA_MAX_T sets an upper bound on the
+  // batch (none by default).
   // Only with operands that make the exactness test pass -- bf16 activations and router rows whose
   // f32 values fit bf16: otherwise every sum the interval test flags (one in a thousand) costs a
   // sequential chain in its workgroup, and the launch lasts as long as the slowest of them.
@@ -1005,8 +1003,7 @@ bool router_mfma_ok(const RouterArgs& a, int R) {
     const char* e = getenv("ATENIA_MOE_ROUTER_MFMA_MAX_T");
     return e ? atoi(e) : 0;
   }();
-  // (8 rows, d = 4096: T = 6144 52 against 104 us, T = 8192 146 against 108)
-  const int t_max = max_t > 0 ? max_t : R <= 16 ? 6144 : 8192;
+  const int t_max = max_t > 0 ? max_t : 0x7fffffff;
   return !off && R <= 80 && a.T <= t_max && a.d % 8 == 0 && !a.logits_out && !a.xb &&
          a.x_is_bf16 && a.w_fits_bf16 && a.E >= a.k;
 }

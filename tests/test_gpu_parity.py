@@ -189,10 +189,10 @@ def test_router_batched_kernel_with_wide_exponent_spread(ora):
     (32, 4, 256, 192, False, False, True, False), (61, 4, 128, 2048, False, False, True, True),
     # beyond 2048 tokens one workgroup holds all rows again: two to four row blocks
     (20, 3, 96, 2100, True, False, True, True), (40, 4, 640, 2500, False, True, True, True),
-    (64, 6, 1024, 2300, False, False, True, True),
+    (64, 6, 1024, 2300, False, False, True, True), (8, 2, 256, 20000, False, False, True, False),
     (8, 2, 1024, 900, False, False, False, False)])
 def test_router_matrix_core_kernel(ora, E, k, d, T, gated, bias, bf16_router, wide):
-    """bf16 activations on the device, up to 8192 tokens, up to 80 rows, router rows whose values
+    """bf16 activations on the device, any batch size, up to 80 rows, router rows whose values
     fit bf16: the router runs on the f64 matrix cores in whatever order they add, and must still
     give the reference's routing for every token -- through the interval certificate, the
     exactness test, or the sequential recomputation (`wide`: activations spread over 60 binades
