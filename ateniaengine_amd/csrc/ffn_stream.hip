@@ -640,25 +640,29 @@ __global__ __launch_bounds__(1024) void ffn_down_combine1_kernel(
 template <bool INT8, bool UP, int NWV, int JB, int NWB, int NBD = 2, bool PG = false>
 __global__ __launch_bounds__(64 * NWV, 8 / NWV) void ffn_mid_kernel(StreamParams p_routed,
                                                                     StreamParams p_shared,
-                                                                    int with_shared) {
+                                                                    int shared_blocks) {
   constexpr int MT = 8, NB = UP ? 2 : NBD, NST = 3;
   constexpr int KB = INT8 ? kKbInt8 : kKbBf16;
   constexpr int CH = KB * JB / 8;  // 16-byte chunks per row and stage
   constexpr int ROWS = 16 * MT;
   __shared__ u32x4 lds_a[NST * ROWS * CH];
 
-  // A shared expert rides in the same launch as blockIdx.y == 0 (its own weights, widths and
-  // rows: one group of all T tokens).  First in the grid, because its K can be twice the
-  // routed experts' and its workgroups should not be the ones that start last.
-  const bool sh = with_shared && blockIdx.y == 0;
+  // A shared expert rides in the same launch (its own weights, widths and rows: one group of
+  // all T tokens): its row blocks are blockIdx.y = 0 .. shared_blocks - 1 (at z = 0), the routed
+  // experts follow along y with their row blocks along z.  All of the shared expert comes first
+  // in the grid that way, because its K can be several times the routed experts' and its
+  // workgroups should not be the ones that start last (with its row blocks along z as well, the
+  // later ones started behind every routed workgroup and ended the launch).
+  const bool sh = (int)blockIdx.y < shared_blocks;
   const StreamParams& p = sh ? p_shared : p_routed;
   if ((int)blockIdx.x * (UP ? NWV : NWV * NB) * 16 >= p.n_pad) return;  // grid spans the wider
-  const int u = sh ? 0 : (int)blockIdx.y - (with_shared ? 1 : 0);
+  const int u = sh ? 0 : (int)blockIdx.y - shared_blocks;
   if (u >= *p.g.n_active) return;
   const int e = p.g.active[u];
   const int base = p.g.offsets[e];
   const int cnt = p.g.offsets[e + 1] - base;
-  const int m0 = blockIdx.z * ROWS;
+  // (a shared row block at z > 0 does not exist: it gets a block number past every row count)
+  const int m0 = (sh ? (blockIdx.z ? 1 << 20 : (int)blockIdx.y) : (int)blockIdx.z) * ROWS;
   if (m0 >= cnt) return;
   const int mt_live = __builtin_amdgcn_readfirstlane(min(MT, (cnt - m0 + 15) >> 4));
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -865,20 +869,22 @@ hipError_t launch_mid(const StreamParams& p_in, int n_groups, int rows_max, hipS
   const int n_pad = shared && shared->n_pad > p.n_pad ? shared->n_pad : p.n_pad;
   const int n_strips = n_pad / 16;
   const int per_wg = UP ? 4 : 8;
-  dim3 grid((n_strips + per_wg - 1) / per_wg, n_groups + (shared ? 1 : 0), (rows_max + 127) / 128);
+  const int row_blocks = (rows_max + 127) / 128;
+  const int sb = shared ? row_blocks : 0;  // the shared expert has rows_max = T rows
+  dim3 grid((n_strips + per_wg - 1) / per_wg, n_groups + sb, row_blocks);
   if constexpr (INT8) {
     if (p.group_blocks > 0) {  // per-group scales: a shorter ring leaves room for them
       if (UP)
-        ffn_mid_kernel<true, true, 4, 1, 4, 2, true><<<grid, 256, 0, s>>>(p, ps, shared != nullptr);
+        ffn_mid_kernel<true, true, 4, 1, 4, 2, true><<<grid, 256, 0, s>>>(p, ps, sb);
       else
-        ffn_mid_kernel<true, false, 8, 2, 3, 1, true><<<grid, 512, 0, s>>>(p, ps, shared != nullptr);
+        ffn_mid_kernel<true, false, 8, 2, 3, 1, true><<<grid, 512, 0, s>>>(p, ps, sb);
       return hipGetLastError();
     }
   }
   if (UP)
-    ffn_mid_kernel<INT8, true, 4, INT8 ? 1 : 2, INT8 ? 6 : 4><<<grid, 256, 0, s>>>(p, ps, shared != nullptr);
+    ffn_mid_kernel<INT8, true, 4, INT8 ? 1 : 2, INT8 ? 6 : 4><<<grid, 256, 0, s>>>(p, ps, sb);
   else
-    ffn_mid_kernel<INT8, false, 8, 2, 3, 1><<<grid, 512, 0, s>>>(p, ps, shared != nullptr);
+    ffn_mid_kernel<INT8, false, 8, 2, 3, 1><<<grid, 512, 0, s>>>(p, ps, sb);
   return hipGetLastError();
 }
 
@@ -1020,10 +1026,15 @@ bool can_fuse_shared(const FfnArgs& a, const FfnArgs* sh, bool down_phase) {
         (sh->gate.group_blocks > 0) == (a.gate.group_blocks > 0)))
     return false;
   if (a.use_mid != sh->use_mid) return false;
-  // (the mid-batch launch starts the shared expert's workgroups first, which hides a wider one
-  // as long as it makes few passes: measured on the Qwen1.5-MoE shape, down phase fused / two
-  // launches: T = 192 110 / 128 us, T = 256 121 / 131, T = 384 131 / 134, T = 768 183 / 146)
-  if (a.use_mid && a.rows_max <= 384) return true;
+  // (the mid-batch launch starts all of the shared expert's workgroups first, which hides a
+  // wider one: measured on the Qwen1.5-MoE shape, whole forward fused / a launch of its own
+  // beyond 384 rows: T = 512 312 / 336 us, T = 768 339 / 365, T = 1024 363 / 386, T = 1280
+  // 420 / 430.  ATENIA_MOE_MID_SHARED_ROWS sets a bound.)
+  static const int mid_rows = [] {
+    const char* e = getenv("ATENIA_MOE_MID_SHARED_ROWS");
+    return e ? atoi(e) : 1 << 30;
+  }();
+  if (a.use_mid && a.rows_max <= mid_rows) return true;
   static const int wide_rows = [] {
     const char* e = getenv("ATENIA_MOE_WIDE_SHARED_ROWS");
     return e ? atoi(e) : 48;

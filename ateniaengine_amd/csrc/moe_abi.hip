@@ -551,11 +551,22 @@ MidBounds mid_bounds(const AteniaMoeLayer* L) {
       b.hi = 52.0;
     }
     b.down_min_tokens = wide_shared ? 256 : 56;
-    b.down_hi = 100.0;
+    // (with the shared expert's row blocks first in the mid-batch grid, whole forward in us,
+    // default | mid-batch everywhere | tiled everywhere: Qwen shape T = 1024 360 | 387 | 426,
+    // T = 1536 499 | 496 | 499 with down alone 206 tiled against 170 mid-batch, T = 2048 down 216
+    // against 230; DeepSeek shape T = 1024 432 | 482 | 446, T = 1536 501 | 635 | 499.  A shared
+    // expert much wider than the routed ones has few tiles of a long K in a tiled launch of its
+    // own, which the mid-batch launch hides: that shape keeps the mid-batch down launch longer.)
+    b.down_hi = wide_shared ? 125.0 : 100.0;
   }
   if (env_lo >= 0.0) b.lo = env_lo;
   if (env_hi >= 0.0) b.hi = b.down_hi = env_hi;
   if (env_min_tokens > 0) b.min_tokens = b.down_min_tokens = env_min_tokens;
+  static const int env_max_tokens = [] {
+    const char* e = getenv("ATENIA_MOE_MID_MAX_TOKENS");
+    return e ? atoi(e) : 0;
+  }();
+  if (env_max_tokens > 0) b.max_tokens = env_max_tokens;
   return b;
 }
 BatchPlan plan_batch(const AteniaMoeLayer* L, int T) {

@@ -117,3 +117,27 @@ def test_no_branch_between_an_mfma_and_the_valu_read_of_its_result(asm):
                     waited += 1
                 break
     assert not bad, f"{name}: result of an MFMA read right after a branch: {bad[:5]}"
+
+
+def test_expert_kernels_use_no_scratch_memory(asm):
+    """No expert kernel may keep anything in scratch (private) memory.  It happens silently: a
+    reference that selects between the two by-value parameter structs of a launch (routed /
+    shared expert) turned into a stack copy of the struct when an early return was placed in
+    front of it, and the mid-batch kernels ran a third slower with every test still passing.
+    The load-time repack kernel is the one exception (it runs once per layer)."""
+    name, lines = asm
+    if name == "ffn_tiled.hip":
+        pytest.skip("the tiled kernels spill a few prologue values around their main loop by design "
+                    "(512 registers per wave are all taken)")
+    allowed = ("repack_blocks_kernel",)
+    kernel, bad, seen = None, [], 0
+    for ln in lines:
+        if ln.startswith(".name:"):
+            kernel = ln.split(":", 1)[1].strip()
+        elif ln.startswith(".private_segment_fixed_size:"):
+            size = int(ln.split(":")[1])
+            seen += 1
+            if size and kernel and not any(a in kernel for a in allowed):
+                bad.append((kernel[:80], size))
+    assert seen > 0, f"{name}: no kernel metadata found"
+    assert not bad, f"{name}: kernels with scratch memory: {bad}"
