@@ -173,6 +173,9 @@ struct AteniaMoeLayer {
   // previous one (`done_stream`) first waits for that stream's work, so two streams never use
   // the workspace at the same time (skipped while a stream is being captured into a graph).
   hipEvent_t done = nullptr;
+  // a shared expert that takes launches of its own runs beside the routed experts (run_forward)
+  hipStream_t side = nullptr;
+  hipEvent_t ev_fork = nullptr, ev_join = nullptr;
   hipStream_t done_stream = nullptr;
   bool done_valid = false;
 
@@ -605,6 +608,14 @@ int noalloc_y_parts(const AteniaMoeLayer* L, int T) {
   return plan_batch(L, T).down != kFamTiled || L->wdtype == ATENIA_MOE_WEIGHT_F32 ? 1 : kMaxYParts;
 }
 
+bool side_stream_enabled() {
+  static const bool on = [] {
+    const char* e = getenv("ATENIA_MOE_SHARED_SIDE_STREAM");  // 0 = everything on the caller's stream
+    return !(e && atoi(e) == 0);
+  }();
+  return on;
+}
+
 bool stream_is_capturing(hipStream_t s) {
   hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
   if (hipStreamIsCapturing(s, &st) != hipSuccess) {
@@ -868,14 +879,45 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
 
   // Small batches stream both the routed experts and the shared one: one launch per phase.
   const bool fuse_shared_up = L->fs > 0 && ffn_stream_fuses_shared(fa, fsd, false);
+  // A shared expert with tiled launches of its own: its gate/up and down depend on nothing the
+  // routed experts compute, and each is a launch of few tiles (T / 256 row tiles; the down
+  // launch of a wide shared expert fills a quarter of the chip for the length of its long K).
+  // They go to a stream of the handle's own, between an event the caller's stream records after
+  // the grouping and one it waits for before the first launch that reads the shared expert's
+  // results, so that the hardware deals the tiles of both to the compute units as they free up.
+  // Not under stream capture (no cross-stream dependencies are recorded into a caller's graph)
+  // and not with stage profiling on (the stage events sit on the caller's stream only).  While
+  // the shared expert's down launch has fewer tiles than the chip has compute units; beyond,
+  // its launches fill the chip by themselves and two kernels at once only share L2 worse.
+  // Whole forward, one stream / two (us): Qwen1.5-MoE shape T = 1536 468 / 437, 2048 524 / 442,
+  // 3072 646 / 561, 4096 783 / 711, 8192 1249 / 1239, 16384 2313 / 2336; DeepSeek-V2-Lite shape
+  // T = 1024 436 / 409, 1536 497 / 442, 2048 561 / 514, 3072 717 / 658, 4096 834 / 813,
+  // 8192 1360 / 1379, 16384 2546 / 2592.
+  const long long shared_down_tiles =
+      (long long)((T + kTileM - 1) / kTileM) * ((L->d + 255) / 256);
+  const bool side_run = side_stream_enabled() && L->fs > 0 && !fuse_shared_up && tiled && L->side &&
+                        shared_down_tiles < fa.n_cus && first <= kStageFfn && !L->profiling &&
+                        !stream_is_capturing(s);
+  bool side_open = false;
   if (first <= kStageFfn) {
+    if (side_run) {
+      HIP_TRY(hipEventRecord(L->ev_fork, s));
+      HIP_TRY(hipStreamWaitEvent(L->side, L->ev_fork, 0));
+      side_open = true;
+    }
     HIP_TRY(launch_ffn_up(fa, s, fuse_shared_up ? &fsd : nullptr));
     L->launches[2] = 1;
     if (L->fs > 0 && !fuse_shared_up) {
-      HIP_TRY(launch_ffn_up(fsd, s));
+      HIP_TRY(launch_ffn_up(fsd, side_run ? L->side : s));
       L->launches[2] = 2;
     }
   }
+  auto side_join = [&]() -> hipError_t {  // the caller's stream waits for the side stream's work
+    if (!side_open) return hipSuccess;
+    side_open = false;
+    hipError_t e = hipEventRecord(L->ev_join, L->side);
+    return e != hipSuccess ? e : hipStreamWaitEvent(s, L->ev_join, 0);
+  };
   tm.mark();  // ev[3]: gate/up done
   // the down phase may take another family than gate/up did
   fa.use_tiled = fam_down == kFamTiled;
@@ -895,13 +937,15 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
       fa.fuse_k = L->k;
       HIP_TRY(launch_ffn_down_decode1(fa, s, L->fs > 0 ? &fsd : nullptr));
     } else {
+      if (fuse_shared_down) HIP_TRY(side_join());  // the fused launch reads the shared expert's h
       HIP_TRY(launch_ffn_down(fa, s, fuse_shared_down ? &fsd : nullptr));
     }
     L->launches[3] = 1;
     if (L->fs > 0 && !fuse_shared_down && !fuse1) {
-      HIP_TRY(launch_ffn_down(fsd, s));
+      HIP_TRY(launch_ffn_down(fsd, side_open ? L->side : s));
       L->launches[3] = 2;
     }
+    HIP_TRY(side_join());
     L->stage_T[kStageFfn] = T;
   }
   tm.mark();  // ev[4]: down done
@@ -1200,6 +1244,12 @@ int atenia_moe_hip_layer_create(const AteniaMoeLayerDesc* D, AteniaMoeLayer** ou
   }
   if (hipEventCreateWithFlags(&L->done, hipEventDisableTiming) != hipSuccess)
     return bail(fail(ATENIA_MOE_ERR_LAUNCH, "hipEventCreate failed"));
+  if (L->fs > 0 && side_stream_enabled()) {
+    if (hipStreamCreateWithFlags(&L->side, hipStreamNonBlocking) != hipSuccess ||
+        hipEventCreateWithFlags(&L->ev_fork, hipEventDisableTiming) != hipSuccess ||
+        hipEventCreateWithFlags(&L->ev_join, hipEventDisableTiming) != hipSuccess)
+      return bail(fail(ATENIA_MOE_ERR_LAUNCH, "stream / event creation failed"));
+  }
   if (hipGetDevice(&L->device) != hipSuccess)
     return bail(fail(ATENIA_MOE_ERR_LAUNCH, "hipGetDevice failed"));
   if ((rc = resolve_static_scratch(L->device, nullptr))) return bail(rc);
@@ -1221,6 +1271,9 @@ int atenia_moe_hip_layer_destroy(AteniaMoeLayer* L) {
     if (L->ev_valid)
       for (auto& e : L->ev) (void)hipEventDestroy(e);
     if (L->done) (void)hipEventDestroy(L->done);
+    if (L->ev_fork) (void)hipEventDestroy(L->ev_fork);
+    if (L->ev_join) (void)hipEventDestroy(L->ev_join);
+    if (L->side) (void)hipStreamDestroy(L->side);
     if (L->staging_ready) {
       for (int i = 0; i < 2; ++i) {
         (void)hipEventDestroy(L->ev_h2d[i]);

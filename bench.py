@@ -306,7 +306,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=20)  # 20 x 2.4 ms: the clocks are up by then
     ap.add_argument("--config", default="mixtral_bf16", choices=sorted(CONFIGS),
                     help="layer shape (the headline metric is quoted on mixtral_bf16)")
     ap.add_argument("--tokens", type=int, default=0,

@@ -36,7 +36,12 @@
  * two streams never use one workspace at the same time.  The one exception is a stream that is
  * being captured into a HIP graph: no cross-stream wait is recorded there, and replays of graphs
  * that hold calls on one handle must be ordered by the caller.  Different handles may run
- * concurrently.
+ * concurrently.  A layer with a shared expert owns a second stream (default priority): in
+ * batches where that expert takes launches of its own they run there, beside the routed
+ * experts' on the caller's stream, between an event recorded on the caller's stream and one it
+ * waits for before the call's last launch -- everything a call enqueues is complete when the
+ * caller's stream has passed the call (never under stream capture, where all launches stay on
+ * the captured stream).
  */
 #ifndef ATENIA_MOE_HIP_H
 #define ATENIA_MOE_HIP_H

@@ -403,6 +403,32 @@ def test_mid_batch_kernel(ora, wd, T, d, f_s, skew):
                 assert S.rel_err(ys[t], ref) <= TOL_BF16
 
 
+@pytest.mark.parametrize("wd", [capi.WEIGHT_BF16, capi.WEIGHT_INT8_W8A16])
+@pytest.mark.parametrize("T,f_s", [(700, 256), (1500, 128)])
+def test_shared_expert_on_its_own_stream(ora, wd, T, f_s):
+    """Tiled family with a shared expert: its two launches run on a stream of the handle's own
+    beside the routed experts' (forked after the grouping, joined before the combine).  The result
+    must be the oracle's, and bit for bit what the same kernels give one after the other on the
+    caller's stream (stage profiling on keeps everything there) -- on repeated calls, so that a
+    missing wait between the streams would show as a stale read."""
+    E, k, d, f = 8, 2, 256, 384
+    W = S.make_weights(900 + T, E, d, f, f_s=f_s, gated=True, router_std=0.05 / np.sqrt(d),
+                       outlier_frac=0.01 if wd != capi.WEIGHT_BF16 else 0.0)
+    oL, gL = S.build_pair(ora, W, k, capi.CONVENTION_HUGGINGFACE_QWEN, wd)
+    with gL:
+        routed, shared = gL.expert_kernels(T)
+        assert routed == capi.KERNELS_TILED and shared == capi.KERNELS_TILED, (routed, shared)
+        xs = [S.make_tokens(950 + T + i, T, d) for i in range(3)]
+        check_layer(ora, oL, gL, xs[0], TOL_BF16_TOY, sample=range(0, T, 29))
+        two = [gL.forward(x).copy() for x in xs]
+        two += [gL.forward(x).copy() for x in xs]  # again, back to back
+        gL.set_profiling(True)
+        one = [gL.forward(x).copy() for x in xs]
+        gL.set_profiling(False)
+        for i in range(6):
+            assert two[i].tobytes() == one[i % 3].tobytes(), f"call {i} differs from the one-stream result"
+
+
 def _tiles(c, max_groups):
     g = -(-c // 32)
     return -(-c // 256) if max_groups == 8 else -(-g // max_groups)
