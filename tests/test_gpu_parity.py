@@ -404,14 +404,16 @@ def test_mid_batch_kernel(ora, wd, T, d, f_s, skew):
 
 
 @pytest.mark.parametrize("wd", [capi.WEIGHT_BF16, capi.WEIGHT_INT8_W8A16])
-@pytest.mark.parametrize("T,f_s", [(700, 256), (1500, 128)])
-def test_shared_expert_on_its_own_stream(ora, wd, T, f_s):
+@pytest.mark.parametrize("E,T,f_s", [(8, 700, 256), (8, 1500, 128), (16, 700, 256)])
+def test_shared_expert_on_its_own_stream(ora, wd, E, T, f_s):
     """Tiled family with a shared expert: its two launches run on a stream of the handle's own
     beside the routed experts' (forked after the grouping, joined before the combine).  The result
     must be the oracle's, and bit for bit what the same kernels give one after the other on the
     caller's stream (stage profiling on keeps everything there) -- on repeated calls, so that a
-    missing wait between the streams would show as a stale read."""
-    E, k, d, f = 8, 2, 256, 384
+    missing wait between the streams would show as a stale read.  With 16 experts the down phase
+    is the mid-batch launch with the shared expert inside (87 rows per expert), which must wait
+    for the shared expert's gate/up on the other stream."""
+    k, d, f = 2, 256, 384
     W = S.make_weights(900 + T, E, d, f, f_s=f_s, gated=True, router_std=0.05 / np.sqrt(d),
                        outlier_frac=0.01 if wd != capi.WEIGHT_BF16 else 0.0)
     oL, gL = S.build_pair(ora, W, k, capi.CONVENTION_HUGGINGFACE_QWEN, wd)
