@@ -263,7 +263,10 @@ def test_non_finite_input_is_reported(ora):
 
 # ---- permute: bit-exact counts / offsets / perm ----------------------------------------
 @pytest.mark.parametrize("T,k,E", [(1, 2, 8), (16, 2, 8), (512, 2, 8), (513, 2, 8), (3000, 4, 60),
-                                   (16384, 6, 64), (700, 1, 3), (100, 8, 8)])
+                                   (16384, 6, 64), (700, 1, 3), (100, 8, 8),
+                                   # one launch up to 16 blocks of 1024 pairs, three beyond; expert
+                                   # counts that use all eight index bits
+                                   (2048, 8, 256), (2049, 8, 256), (4096, 4, 200), (300, 5, 129)])
 def test_permute_bit_exact(ora, T, k, E):
     rng = np.random.default_rng(T + E)
     p = rng.random(E) ** 3
