@@ -965,6 +965,13 @@ hipError_t launch_router_mfma_rb(const RouterArgs& a, int R, hipStream_t s) {
   return hipGetLastError();
 }
 
+// (defined further down: selection from logits in HBM with one thread per expert, up to 256 experts)
+constexpr int kSelectThreads = 256;
+__global__ __launch_bounds__(kSelectThreads) void softmax_select_kernel(
+    const float* __restrict__ logits, int T, int E, int k, int renorm,
+    int32_t* __restrict__ idx_out, float* __restrict__ w_out, int32_t* __restrict__ status,
+    FusedGrouping fg);
+
 // The same kernel with the rows dealt to workgroups in blocks of 16 (eight waves split k), the
 // logits left in HBM and the routing decided by a second launch, one wave per token: with many
 // rows and a batch that gives fewer workgroups of 16 tokens than the chip has compute units,
@@ -976,12 +983,18 @@ hipError_t launch_router_mfma_split(const RouterArgs& a, int R, hipStream_t s) {
                       (size_t)16 * RL * 4 + (size_t)16 * RL + 16;
   router_mfma_kernel<XT, RB, 4, NWV><<<dim3((a.T + 15) / 16, (R + 15) / 16), 64 * NWV, smem, s>>>(
       (const XT*)a.x, a.T, a.d, a.E, a.k, a.renorm, a.w_router, a.router_bias, a.shared_gate,
-      a.idx, a.w, a.sgate, a.status, a.logits_tmp);
+      a.idx, a.w, a.sgate, a.status, a.logits_out ? a.logits_out : a.logits_tmp);
   hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return e;
-  constexpr int per = kWaveSelectThreads / 64;
-  wave_select_kernel<<<(a.T + per - 1) / per, kWaveSelectThreads, 0, s>>>(
-      a.logits_tmp, a.T, a.E, a.k, a.renorm, a.idx, a.w, a.status);
+  if (e != hipSuccess || a.logits_out) return e;  // the caller's own launch routes from the logits
+  if (a.E <= 64) {
+    constexpr int per = kWaveSelectThreads / 64;
+    wave_select_kernel<<<(a.T + per - 1) / per, kWaveSelectThreads, 0, s>>>(
+        a.logits_tmp, a.T, a.E, a.k, a.renorm, a.idx, a.w, a.status);
+  } else {
+    const int TT = kSelectThreads / a.E;
+    softmax_select_kernel<<<(a.T + TT - 1) / TT, kSelectThreads, 0, s>>>(
+        a.logits_tmp, a.T, a.E, a.k, a.renorm, a.idx, a.w, a.status, FusedGrouping{});
+  }
   return hipGetLastError();
 }
 
@@ -1004,8 +1017,10 @@ bool router_mfma_ok(const RouterArgs& a, int R) {
     return e ? atoi(e) : 0;
   }();
   const int t_max = max_t > 0 ? max_t : 0x7fffffff;
-  return !off && R <= 80 && a.T <= t_max && a.d % 8 == 0 && !a.logits_out && !a.xb &&
-         a.x_is_bf16 && a.w_fits_bf16 && a.E >= a.k;
+  const bool operands = !off && a.T <= t_max && a.d % 8 == 0 && !a.xb && a.x_is_bf16 &&
+                        a.w_fits_bf16 && a.E >= a.k;
+  if (R < 0) return operands;  // the form that deals the rows to workgroups takes any row count
+  return operands && R <= 80 && !a.logits_out;
 }
 
 // When the rows are dealt to workgroups.  Measured on MI355X, d = 2048, route stage in us,
@@ -1025,12 +1040,22 @@ bool router_mfma_split_wanted(const RouterArgs& a, int R) {
     return e ? atoi(e) : -1;
   }();
   const int lo = min_t >= 0 ? min_t : R > 32 ? 52 : 192;
-  return R > 16 && a.E <= 64 && a.logits_tmp && a.T >= lo && a.T <= max_t;
+  if (R <= 16 || a.T < lo || !router_mfma_ok(a, -1)) return false;
+  // The raw logits are wanted (another launch routes), or more rows than one workgroup holds:
+  // no other form on the matrix cores, so at every batch size.  DeepSeek-V3 router shape (256
+  // rows, d = 7168, logits for the group-limited selection), route stage in us, this form /
+  // the per-token kernel up to 512 tokens and the sequential-order kernel beyond: T = 64
+  // 74 / 249, 256 130 / 249, 512 164 / 251, 1024 220 / 260, 2048 354 / 316, 4096 626 / 645,
+  // 8192 1172 / 1302 (30 GFLOP of f64 there: 25 TFLOP/s against 78.6 at the f64 matrix peak;
+  // several blocks of 16 tokens per workgroup, to read the 7 MB matrix less often, and two or
+  // four row blocks per workgroup, to read the tokens less often, both measured no faster).
+  if (a.logits_out) return true;
+  if (!a.logits_tmp || a.E > kSelectThreads) return false;
+  return R > 80 || a.T <= max_t;
 }
 
 template <typename XT>
 hipError_t launch_router_mfma(const RouterArgs& a, int R, hipStream_t s) {
-  if (router_mfma_split_wanted(a, R)) return launch_router_mfma_split<XT>(a, R, s);
   // few rows: eight waves split k, so that a batch of 4096 tokens (256 workgroups, one per
   // compute unit) still puts two waves on every SIMD
   if (R <= 16) return launch_router_mfma_rb<XT, 1, 4, 8>(a, R, s);
@@ -1094,7 +1119,6 @@ __device__ inline void write_single_token_grouping(const FusedGrouping& fg, cons
 // Softmax + top-k from logits that another launch left in HBM: used when the rows of the
 // router matrix were spread over several workgroups per token (many experts, few tokens), so
 // no single workgroup holds all logits of a token.  256 / E tokens per workgroup.
-constexpr int kSelectThreads = 256;
 __global__ __launch_bounds__(kSelectThreads) void softmax_select_kernel(
     const float* __restrict__ logits, int T, int E, int k, int renorm,
     int32_t* __restrict__ idx_out, float* __restrict__ w_out, int32_t* __restrict__ status,
@@ -1301,7 +1325,10 @@ hipError_t launch_router(const RouterArgs& a, hipStream_t s, int* fused_permute)
   // The per-token kernel re-reads the whole stacked matrix for every token; with many rows
   // (row blocks, logits mode) that only pays for a handful of tokens.
   const bool mfma = router_mfma_ok(a, R);
-  const bool token_ok = a.T <= a.token_kernel_max_tokens && !(mfma && router_mfma_split_wanted(a, R)) &&
+  if (router_mfma_split_wanted(a, R))
+    return a.x_is_bf16 ? launch_router_mfma_split<uint16_t>(a, R, s)
+                       : launch_router_mfma_split<float>(a, R, s);
+  const bool token_ok = a.T <= a.token_kernel_max_tokens &&
                         (R <= 64 || (long long)a.T * R * a.d <= (16ll << 20));
   if (token_ok) {
     const size_t np = R > kTokenThreads / 64 ? R : kTokenThreads / 64;

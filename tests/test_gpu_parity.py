@@ -190,6 +190,11 @@ def test_router_batched_kernel_with_wide_exponent_spread(ora):
     # beyond 2048 tokens one workgroup holds all rows again: two to four row blocks
     (20, 3, 96, 2100, True, False, True, True), (40, 4, 640, 2500, False, True, True, True),
     (64, 6, 1024, 2300, False, False, True, True), (8, 2, 256, 20000, False, False, True, False),
+    (79, 5, 256, 2100, True, False, True, True),
+    # more than 64 experts: rows dealt to workgroups at every batch size, selection with one thread
+    # per expert
+    (128, 8, 256, 300, False, False, True, False), (200, 6, 512, 1100, False, True, True, True),
+    (255, 4, 128, 2500, True, False, True, False),
     (8, 2, 1024, 900, False, False, False, False)])
 def test_router_matrix_core_kernel(ora, E, k, d, T, gated, bias, bf16_router, wide):
     """bf16 activations on the device, any batch size, up to 80 rows, router rows whose values
