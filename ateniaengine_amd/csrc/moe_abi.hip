@@ -885,8 +885,10 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   // They go to a stream of the handle's own, between an event the caller's stream records after
   // the grouping and one it waits for before the first launch that reads the shared expert's
   // results, so that the hardware deals the tiles of both to the compute units as they free up.
-  // Not under stream capture (no cross-stream dependencies are recorded into a caller's graph)
-  // and not with stage profiling on (the stage events sit on the caller's stream only).  While
+  // Not under stream capture (no cross-stream dependencies are recorded into a caller's graph),
+  // not from the entry point that allocates nothing (its callers get launches on their own
+  // stream and nothing else) and not with stage profiling on (the stage events sit on the
+  // caller's stream only).  While
   // the shared expert's down launch has fewer tiles than the chip has compute units; beyond,
   // its launches fill the chip by themselves and two kernels at once only share L2 worse.
   // Whole forward, one stream / two (us): Qwen1.5-MoE shape T = 1536 468 / 437, 2048 524 / 442,
@@ -897,7 +899,7 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
       (long long)((T + kTileM - 1) / kTileM) * ((L->d + 255) / 256);
   const bool side_run = side_stream_enabled() && L->fs > 0 && !fuse_shared_up && tiled && L->side &&
                         shared_down_tiles < fa.n_cus && first <= kStageFfn && !L->profiling &&
-                        !stream_is_capturing(s);
+                        !no_alloc && !stream_is_capturing(s);
   bool side_open = false;
   if (first <= kStageFfn) {
     if (side_run) {
