@@ -40,8 +40,8 @@
  * batches where that expert takes launches of its own they run there, beside the routed
  * experts' on the caller's stream, between an event recorded on the caller's stream and one it
  * waits for before the call's last launch -- everything a call enqueues is complete when the
- * caller's stream has passed the call (never under stream capture, where all launches stay on
- * the captured stream).
+ * caller's stream has passed the call (never under stream capture nor from the entry point that
+ * allocates nothing: there all launches stay on the caller's stream).
  */
 #ifndef ATENIA_MOE_HIP_H
 #define ATENIA_MOE_HIP_H
