@@ -40,7 +40,7 @@ CONFIGS = {
     "qwen_bf16": dict(d=2048, E=60, k=4, f=1408, fs=5632, gated=True, conv=1, wd="bf16",
                       zipf=False, sweep=(1, 16, 64, 128, 256, 8192)),
     "deepseek_bf16": dict(d=2048, E=64, k=6, f=1408, fs=2816, gated=False, conv=1, wd="bf16",
-                          zipf=True, sweep=(1, 16, 64, 1024, 16384)),
+                          zipf=True, sweep=(1, 16, 64, 128, 1024, 16384)),
     # DeepSeek-V3 router shape (256 experts in 8 groups, top-8 of the 4 best groups) in front of
     # narrow experts: times the sigmoid / group-limited routing path, not a checkpoint shape.
     "v3route_bf16": dict(d=7168, E=256, k=8, f=256, fs=256, gated=False, conv=1, wd="bf16",
@@ -314,7 +314,9 @@ def main():
     ap.add_argument("--decode-tokens", type=str, default="1,16",
                     help="decode batch sizes, comma separated (empty = skip); reported as "
                          "`decode` (the first) and `decode<T>` (the others)")
-    ap.add_argument("--sweep", type=str, default="", help="extra batch sizes, comma separated")
+    ap.add_argument("--sweep", type=str, default="128",
+                    help="extra batch sizes, comma separated (default: 128 tokens, where the "
+                         "mid-batch kernels serve the layer; \"all\": the configuration's own list)")
     ap.add_argument("--cpu-tokens", type=int, default=-1,
                     help="tokens of the CPU-baseline sample (0 = skip; default: about 12 s of "
                          "CPU work on 16 cores)")
@@ -360,6 +362,9 @@ def main():
                  (t in cfg["sweep"] or a.decode_tokens != "1,16")]
     if a.sweep == "all":
         a.sweep = ",".join(str(t) for t in cfg["sweep"] if t != a.tokens and t not in decode_ts)
+    elif a.sweep == "128":  # the default: only where the configuration lists that batch size
+        a.sweep = "128" if 128 in cfg["sweep"] and a.tokens != 128 and 128 not in decode_ts else ""
+    a.sweep = ",".join(t for t in a.sweep.split(",") if t and int(t) > 0)  # "0" = none
     router, gate, up, down, shared = make_weights(torch, np, a.seed, f32=f32w)
     router_f32 = upcast(np, router)
     if cfg["zipf"]:  # logits ~ N(0,1) plus a log-Zipf(1.2) bias: skewed expert load
