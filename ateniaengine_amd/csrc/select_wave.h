@@ -76,6 +76,76 @@ __device__ inline WaveRouting wave_softmax_topk(const float* lg, int E, int k, i
   return r;
 }
 
+// Largest value over the 64 lanes of a wave, in every lane: four DPP steps make each row of 16
+// lanes uniform (swap neighbours, swap pairs, mirror the half row, mirror the row), the four row
+// values meet on the scalar side.
+__device__ inline int wave_max_i32(int v) {
+  v = max(v, __builtin_amdgcn_update_dpp(v, v, 0xB1, 0xf, 0xf, false));   // quad_perm [1,0,3,2]
+  v = max(v, __builtin_amdgcn_update_dpp(v, v, 0x4E, 0xf, 0xf, false));   // quad_perm [2,3,0,1]
+  v = max(v, __builtin_amdgcn_update_dpp(v, v, 0x141, 0xf, 0xf, false));  // row_half_mirror
+  v = max(v, __builtin_amdgcn_update_dpp(v, v, 0x140, 0xf, 0xf, false));  // row_mirror
+  return max(max(__builtin_amdgcn_readlane(v, 0), __builtin_amdgcn_readlane(v, 16)),
+             max(__builtin_amdgcn_readlane(v, 32), __builtin_amdgcn_readlane(v, 48)));
+}
+
+// Top-k of one token from its softmax weights (lane r = expert r) and the routing written out:
+// the k experts that sort first under (weight desc, index asc) are found as k times the largest
+// weight still available, the lowest lane among equals.  Weights are >= +0, so their bit
+// patterns order like integers (-1 = not available; a NaN weight is reported by the caller).
+// The weights of the selection are summed e ascending, as the reference sums its sorted
+// selection (dense.rs:172-187, sparse.rs:142-191).
+__device__ inline void wave_topk_write(float wt, bool on, int lane, int k, int renorm, int token,
+                                       int32_t* __restrict__ idx_out, float* __restrict__ w_out) {
+  const int wbits = on ? __float_as_int(wt) : -1;
+  unsigned long long avail = ~0ull, mask = 0ull;
+  for (int r = 0; r < k; ++r) {
+    const int v = (avail >> lane) & 1ull ? wbits : -1;
+    const int m = wave_max_i32(v);
+    const unsigned long long cand = __ballot(v == m && m >= 0);
+    if (!cand) break;  // wave-uniform; k <= E makes it unreachable
+    const unsigned long long win = cand & (~cand + 1ull);
+    mask |= win;
+    avail &= ~win;
+  }
+  const bool selected = (mask >> lane) & 1ull;
+  const int slot = __popcll(mask & ((1ull << lane) - 1ull));
+  double ssum = 0.0;
+  for (unsigned long long m = mask; m; m &= m - 1)
+    ssum += (double)readlane_f32(wt, __ffsll((long long)m) - 1);
+  const double scale = renorm ? 1.0 / ssum : 1.0;
+  if (selected && slot < k) {
+    const size_t o = (size_t)token * k + slot;
+    idx_out[o] = lane;
+    w_out[o] = (float)((double)wt * scale);
+  }
+}
+
+// Softmax + top-k of token t from its logits row in memory, by one wavefront (up to 64 experts).
+// Same arithmetic, casts and order as softmax_topk in router.hip; the sequential fold of the
+// exponentials runs over v_readlane values.  Every lane of the wave must call.
+__device__ inline void wave_select_token(const float* __restrict__ lg, int E, int k, int renorm,
+                                         int t, int lane, int32_t* __restrict__ idx_out,
+                                         float* __restrict__ w_out, int32_t* __restrict__ status) {
+  const bool on = lane < E;
+  const float my = on ? lg[lane] : -INFINITY;
+  float mx = fmaxf(-INFINITY, my);  // a NaN logit is skipped, as f32::max skips it
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+  const double ex = on ? exp((double)(my - mx)) : 0.0;  // f32 subtraction, then f64 exp
+  double sum = 0.0;
+  for (int e0 = 0; e0 < E; e0 += 8) {  // sequential fold, e ascending; lanes past E add +0
+#pragma unroll
+    for (int u = 0; u < 8; ++u) sum += readlane_f64(ex, e0 + u);
+  }
+  const double inv = sum > 0.0 ? 1.0 / sum : 0.0;
+  const float wt = (float)(ex * inv);
+  if (on && (!isfinite(wt) || wt < 0.f)) {
+    atomicMin(&status[0], -3);
+    atomicMin(&status[1], (t << 10) | lane);
+  }
+  wave_topk_write(wt, on, lane, k, renorm, t, idx_out, w_out);
+}
+
 // Expert of group u (the u-th selected expert, ascending), or -1.
 __device__ inline int wave_selected_expert(unsigned long long mask, int u) {
   for (int i = 0; i < u && mask; ++i) mask &= mask - 1;
