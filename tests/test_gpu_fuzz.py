@@ -96,3 +96,53 @@ def test_random_layer_mid_batch_reached_the_kernel():
     routed_mid = sum(1 for r, s in _MID_SEEN if r == capi.KERNELS_MID)
     shared_mid = sum(1 for r, s in _MID_SEEN if r == capi.KERNELS_MID and s == capi.KERNELS_MID)
     assert routed_mid >= 20 and shared_mid >= 5, (routed_mid, shared_mid)
+
+
+def _router_cases(n, seed):
+    """bf16 activations on the device with router rows that fit bf16: every form of the router on
+    the f64 matrix cores (rows dealt to workgroups or not, one to five row blocks, more than 64
+    experts) and the per-token kernel below their batch sizes."""
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(n):
+        E = int(rng.choice([2, 8, 15, 16, 17, 31, 32, 33, 48, 60, 64, 65, 79, 80, 96, 128, 200, 255]))
+        k = int(rng.integers(1, min(E, 8) + 1))
+        d = int(rng.choice([8, 64, 96, 256, 520, 1024, 2048]))
+        T = int(rng.choice([2, 17, 51, 52, 53, 191, 192, 193, 300, 511, 513, 1000, 2048, 2049, 3000]))
+        gated = bool(rng.integers(0, 2)) and E < 255
+        bias = bool(rng.integers(0, 2))
+        wide = bool(rng.integers(0, 3) == 0)  # activations over 60 binades: sequential fallback
+        out.append(pytest.param(E, k, d, T, gated, bias, wide, 3000 + i,
+                                id=f"{i}-E{E}k{k}d{d}T{T}g{int(gated)}b{int(bias)}w{int(wide)}"))
+    return out
+
+
+@pytest.mark.parametrize("E,k,d,T,gated,bias,wide,seed", _router_cases(60, 20251125))
+def test_random_router_on_device_bf16(ora, E, k, d, T, gated, bias, wide, seed):
+    from tests.hipmem import DeviceArray
+    from tests.test_gpu_parity import ulp_diff
+    b = -1.2 * np.log(np.random.default_rng(seed).permutation(E) + 1.0) if bias else None
+    W = S.make_weights(seed, E, d, 16, f_s=16 if gated else 0, gated=gated,
+                       router_std=1.0 / np.sqrt(d), bias=b)
+    W["w_router"] = S.bf16_round_trip(W["w_router"])[1]
+    if gated:
+        W["shared_gate"] = S.bf16_round_trip(W["shared_gate"])[1]
+    conv = capi.CONVENTION_HUGGINGFACE_QWEN if gated else capi.CONVENTION_ATENIA
+    oL, gL = S.build_pair(ora, W, k, conv, capi.WEIGHT_BF16)
+    rng = np.random.default_rng(seed + 1)
+    if wide:
+        x = rng.standard_normal((T, d)) * np.exp2(rng.integers(-30, 30, size=(T, d)))
+    else:
+        x = rng.standard_normal((T, d))
+    x = S.bf16_round_trip(x.astype(np.float32))[1]
+    bits = (x.view(np.uint32) >> 16).astype(np.uint16)
+    with gL:
+        dx = DeviceArray.from_host(bits)
+        out = DeviceArray((T, d), np.float32, fill=0)
+        gL.forward_device(dx.ptr, capi.ACT_BF16, T, out.ptr)
+        idx, w, counts, offsets, perm = gL.last_routing(T)
+        o_idx, o_w = oL.route_tokens(x)
+        assert (idx == o_idx).all(), f"{(idx != o_idx).any(axis=1).sum()} tokens routed differently"
+        assert ulp_diff(w, o_w).max() <= 1
+        oc, oo, op = ora.permute(o_idx, E)
+        assert (counts == oc).all() and (offsets == oo).all() and (perm == op).all()
