@@ -136,6 +136,7 @@ struct AteniaMoeLayer {
 
   DevBuf w_router, router_bias, shared_gate;
   bool router_fits_bf16 = false;  // every router / gate value is exactly a bf16 value
+  DevBuf router_lsb;              // [E + 1] i32: lowest last-bit exponent of each router row / the gate
   DevBuf wg, wu, wd, sg, su, sd;        // routed experts
   DevBuf swg, swu, swd, ssg, ssu, ssd;  // shared expert
   WeightSet gate{}, up{}, down{}, s_gate{}, s_up{}, s_down{};
@@ -685,6 +686,7 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   ra.renorm = L->conv == ATENIA_MOE_CONVENTION_ATENIA;
   ra.w_router = L->w_router.as<float>();
   ra.w_fits_bf16 = L->router_fits_bf16;
+  ra.w_lsb_min = L->router_lsb.as<int32_t>();
   ra.router_bias = L->router_bias.as<float>();
   const bool gated = L->fs > 0 && L->conv == ATENIA_MOE_CONVENTION_HUGGINGFACE_QWEN &&
                      L->shared_gate.p != nullptr && L->v3_n_group == 0;
@@ -1179,6 +1181,29 @@ int atenia_moe_hip_layer_create(const AteniaMoeLayerDesc* D, AteniaMoeLayer** ou
     };
     L->router_fits_bf16 = fits_bf16(D->w_router, E * d) &&
                           (!D->shared_gate || fits_bf16(D->shared_gate, d));
+    // Lowest last-bit exponent over each row (v = odd * 2^q; 32767 = the row is all zeros, a
+    // hugely negative value = it holds an inf or a NaN): with the same minimum over a token's
+    // activations it bounds the last bit of every product of the pair from below, which settles
+    // most of the sums the router's interval test flags without reading either row again.
+    auto row_lsb = [](const float* p, size_t n) {
+      int q = 32767;
+      for (size_t i = 0; i < n; ++i) {
+        uint32_t u;
+        memcpy(&u, p + i, 4);
+        const int e = (u >> 23) & 0xff;
+        const uint32_t m = u & 0x7fffffu, mm = e ? (m | 0x800000u) : m;
+        if (e == 0xff) return -100000;
+        if (mm == 0) continue;
+        q = std::min(q, (e ? e - 150 : -149) + __builtin_ctz(mm));
+      }
+      return q;
+    };
+    std::vector<int32_t> lsb(E + 1, 32767);
+    for (size_t r = 0; r < E; ++r) lsb[r] = row_lsb(D->w_router + r * d, d);
+    if (D->shared_gate) lsb[E] = row_lsb(D->shared_gate, d);
+    if ((rc = L->router_lsb.ensure(lsb.size() * 4))) return bail(rc);
+    if (hipMemcpy(L->router_lsb.p, lsb.data(), lsb.size() * 4, hipMemcpyHostToDevice) != hipSuccess)
+      return bail(fail(ATENIA_MOE_ERR_LAUNCH, "upload of the router row table failed"));
   }
 
   DevBuf staging;

@@ -64,6 +64,7 @@ struct RouterArgs {
   int T, d, E, k, renorm;
   const float* w_router;     // [E, d]
   int w_fits_bf16;           // every value of w_router and shared_gate is exactly a bf16 value
+  const int32_t* w_lsb_min;  // [E + 1] lowest last-bit exponent of each router row / the gate (or null)
   const float* router_bias;  // [E] or null
   const float* shared_gate;  // [d] or null
   int32_t* idx;              // [T, k]

@@ -571,7 +571,7 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
     const float* __restrict__ w_router, const float* __restrict__ bias,
     const float* __restrict__ gate_vec, int32_t* __restrict__ idx_out,
     float* __restrict__ w_out, float* __restrict__ sgate_out, int32_t* __restrict__ status,
-    float* __restrict__ logits_out) {
+    float* __restrict__ logits_out, const int32_t* __restrict__ w_lsb) {
   // gridDim.y > 1 (only with logits_out): this workgroup owns the rows row0 .. row0 + R - 1 of
   // the stacked matrix [W_r ; gate] and leaves the logits to another launch; otherwise all rows.
   constexpr int TT = 16;
@@ -592,7 +592,12 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
   double* sXn2 = sAcc + 16 * R;                   // [16]
   double* sWn2 = sXn2 + 16;                       // [R]
   float* sLogit = (float*)(sWn2 + R);             // [16][R]
-  uint8_t* sFlag = (uint8_t*)(sLogit + 16 * R);   // [16][R] 1 = the interval certificate failed
+  int* sXq = (int*)(sLogit + 16 * R);             // [NWV][16] lowest last-bit exponent of x_t (partial)
+  uint8_t* sFlag = (uint8_t*)(sXq + NWV * 16);    // [16][R] 1 = the interval certificate failed
+  // Several row blocks: the matrix instructions of a step leave the VALU time to follow the
+  // lowest last-bit exponent of the token's activations as well (with one block they would not).
+  constexpr bool kTrackLsb = RB >= 2;
+  int xq = kNoLsb;
 
   const int tok = min(t0 + r16, T - 1);  // rows past T repeat the last token; never written out
   const XT* px = x + (size_t)tok * d + 8 * q;
@@ -648,6 +653,7 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
     for (int t = 0; t < 8; ++t) {
       xd[t] = (double)xf[t];
       xsq = fma(xd[t], xd[t], xsq);
+      if (kTrackLsb) xq = min(xq, lsb_exponent(xf[t]));
     }
 #pragma unroll
     for (int b = 0; b < RB; ++b) {
@@ -689,6 +695,11 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
     v += __shfl_xor(v, 16);
     v += __shfl_xor(v, 32);
     if (q == 0) sXsq[wave * 16 + r16] = v;
+    if (kTrackLsb) {
+      xq = min(xq, __shfl_xor(xq, 16));
+      xq = min(xq, __shfl_xor(xq, 32));
+      if (q == 0) sXq[wave * 16 + r16] = xq;
+    }
   }
   __syncthreads();
 
@@ -698,6 +709,11 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
 #pragma unroll
   for (int w = 0; w < NWV; ++w) xn2 += sXsq[w * 16 + t];
   if (rr == 0) sXn2[t] = xn2;
+  int xq_t = kNoLsb;
+  if (kTrackLsb) {
+#pragma unroll
+    for (int w = 0; w < NWV; ++w) xq_t = min(xq_t, sXq[w * 16 + t]);
+  }
   const double gfac = (double)(2 * d + 4) * 1.1102230246251565e-16 * 1.001;
   for (int r = rr; r < R; r += NT / 16) {
     const int b = r >> 4, rho = r & 15, reg = rho >> 2, qq = rho & 3;
@@ -718,6 +734,19 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
     } else {
       const float glo = (float)(1.0 / (1.0 + exp(-lo))), ghi = (float)(1.0 / (1.0 + exp(-hi)));
       ok = glo == ghi;
+    }
+    if (kTrackLsb && !ok && w_lsb) {
+      // Exactness from the two minima alone: every product of the pair is a multiple of
+      // 2^(q_x + q_w), so with sum|p| < 2^(q_x + q_w + 53) every partial sum of every order is
+      // exact -- the test of the second look with a lower bound for q, which most flagged sums
+      // pass without either row being read again (all zeros on one side: the sum is exactly 0).
+      const int wq = w_lsb[min(row0 + r, E)];
+      if (xq_t == kNoLsb || wq == kNoLsb) {
+        ok = true;
+      } else {
+        const int ql = xq_t + wq;
+        ok = ql > -2000 && sqrt(xn2 * wn2) * 1.001 < ldexp(1.0, ql + 53);
+      }
     }
     sAcc[t * R + r] = a;
     sFlag[t * R + r] = ok ? 0 : 1;
@@ -895,11 +924,11 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
 template <typename XT, int RB, int NBUF, int NWV>
 hipError_t launch_router_mfma_rb(const RouterArgs& a, int R, hipStream_t s) {
   const size_t smem = ((size_t)NWV * RB * 4 * 64 + NWV * 16 + (size_t)NWV * RB * 16 + (size_t)16 * R + 16 + R) * 8 +
-                      (size_t)16 * R * 4 + (size_t)16 * R + 16;
+                      (size_t)16 * R * 4 + (size_t)NWV * 16 * 4 + (size_t)16 * R + 16;
   if (smem > 64 * 1024) return hipErrorInvalidValue;
   router_mfma_kernel<XT, RB, NBUF, NWV><<<(a.T + 15) / 16, 64 * NWV, smem, s>>>(
       (const XT*)a.x, a.T, a.d, a.E, a.k, a.renorm, a.w_router, a.router_bias, a.shared_gate,
-      a.idx, a.w, a.sgate, a.status, nullptr);
+      a.idx, a.w, a.sgate, a.status, nullptr, a.w_lsb_min);
   return hipGetLastError();
 }
 
@@ -918,10 +947,10 @@ template <typename XT>
 hipError_t launch_router_mfma_split(const RouterArgs& a, int R, hipStream_t s) {
   constexpr int NWV = 8, RB = 1, RL = 16;
   const size_t smem = ((size_t)NWV * RB * 4 * 64 + NWV * 16 + (size_t)NWV * RB * 16 + (size_t)16 * RL + 16 + RL) * 8 +
-                      (size_t)16 * RL * 4 + (size_t)16 * RL + 16;
+                      (size_t)16 * RL * 4 + (size_t)NWV * 16 * 4 + (size_t)16 * RL + 16;
   router_mfma_kernel<XT, RB, 4, NWV><<<dim3((a.T + 15) / 16, (R + 15) / 16), 64 * NWV, smem, s>>>(
       (const XT*)a.x, a.T, a.d, a.E, a.k, a.renorm, a.w_router, a.router_bias, a.shared_gate,
-      a.idx, a.w, a.sgate, a.status, a.logits_out ? a.logits_out : a.logits_tmp);
+      a.idx, a.w, a.sgate, a.status, a.logits_out ? a.logits_out : a.logits_tmp, a.w_lsb_min);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || a.logits_out) return e;  // the caller's own launch routes from the logits
   if (a.E <= 64) {
