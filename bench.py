@@ -38,7 +38,7 @@ CONFIGS = {
     "mixtral_int8g": dict(d=4096, E=8, k=2, f=14336, fs=0, gated=False, conv=0, wd="int8g",
                           zipf=False, sweep=(1, 16, 32, 64, 128, 4096)),
     "qwen_bf16": dict(d=2048, E=60, k=4, f=1408, fs=5632, gated=True, conv=1, wd="bf16",
-                      zipf=False, sweep=(1, 16, 64, 128, 256, 8192)),
+                      zipf=False, unit_logits=True, sweep=(1, 16, 64, 128, 256, 8192)),
     "deepseek_bf16": dict(d=2048, E=64, k=6, f=1408, fs=2816, gated=False, conv=1, wd="bf16",
                           zipf=True, sweep=(1, 16, 64, 128, 1024, 16384)),
     # DeepSeek-V3 router shape (256 experts in 8 groups, top-8 of the 4 best groups) in front of
@@ -66,19 +66,41 @@ def measured_hbm_traffic():
     """HBM bytes per launch (read + written) of the expert kernels as rocprofv3 measured them:
     the `traffic <config> <tokens> <stage> <bytes>` lines that rocprof_summary.py writes into the
     counter summaries under profiles/ (FETCH_SIZE / WRITE_SIZE passes scaled by a plain device
-    copy of known size).  {(config, tokens): {stage: bytes}}; empty when no summary is there."""
+    copy of known size).  {(config, tokens): {stage: (bytes, file, kernels_sha)}}; empty when no
+    summary is there.  A summary carries the hash of the kernel sources it was taken with
+    (`kernels_sha <hash>`): its figures are quoted only while that hash equals the one of the
+    sources in this tree, otherwise `traffic` is null and `traffic_source` says why."""
     import glob
     out = {}
     for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*hbm_counters*.txt"))):
+        sha = None
         with open(path) as fh:
             for ln in fh:
                 f = ln.split()
+                if len(f) == 2 and f[0] == "kernels_sha":
+                    sha = f[1]
                 if len(f) == 5 and f[0] == "traffic":
-                    out.setdefault((f[1], int(f[2])), {})[f[3]] = float(f[4])
+                    out.setdefault((f[1], int(f[2])), {})[f[3]] = (float(f[4]), os.path.basename(path), sha)
     return out
 
 
 MEASURED_HBM_TRAFFIC = measured_hbm_traffic()
+try:
+    from rocprof_summary import kernels_sha
+    KERNELS_SHA = kernels_sha()
+except Exception:  # the sources do not travel with every deployment of the library
+    KERNELS_SHA = None
+
+
+def traffic_of(config, tokens, stage):
+    """(bytes or None, source description) for roofline.traffic."""
+    hit = MEASURED_HBM_TRAFFIC.get((config, tokens), {}).get(stage)
+    if hit is None:
+        return None, None
+    nbytes, path, sha = hit
+    src = {"file": "profiles/" + path, "kernels_sha": sha, "this_build": KERNELS_SHA,
+           "current": sha is not None and sha == KERNELS_SHA}
+    return (nbytes if src["current"] else None), src
 
 
 def make_weights(torch, np, seed, f32=False):
@@ -206,10 +228,10 @@ def measure(torch, np, capi, layer, T, steps, warmup, seed):
         algorithmic_bytes=bytes_fwd, algorithmic_flops=flops_fwd,
     )
     up_ms, down_ms = stage_ms[2], stage_ms[3]
-    traffic = MEASURED_HBM_TRAFFIC.get((CONFIG_NAME, T))
     dom, dom_ms, dom_bytes, dom_flops = (
         ("expert_gate_up", up_ms, bytes_up, flops_up) if up_ms >= down_ms
         else ("expert_down", down_ms, bytes_down, flops_down))
+    traffic, traffic_src = traffic_of(CONFIG_NAME, T, dom)
     # HBM-bound while the weights outweigh the arithmetic: below ~300 rows per expert.
     hbm_bound = W_BYTES == 4 or ((dom_flops / (PEAK_BF16_TFLOPS * 1e12)) <
                                  (dom_bytes / (PEAK_HBM_GBS * 1e9)))
@@ -217,13 +239,13 @@ def measure(torch, np, capi, layer, T, steps, warmup, seed):
         ach = dom_bytes / (dom_ms * 1e-3) / 1e9
         r["roofline"] = dict(bound="hbm", kernel=dom, achieved=ach, peak=PEAK_HBM_GBS,
                              unit="GB/s", frac=ach / PEAK_HBM_GBS,
-                             traffic=traffic.get(dom) if traffic else None,
+                             traffic=traffic, traffic_source=traffic_src,
                              kernel_ms=float(dom_ms), algorithmic_bytes=dom_bytes)
     else:
         ach = dom_flops / (dom_ms * 1e-3) / 1e12
         r["roofline"] = dict(bound="mfma", kernel=dom, achieved=ach, peak=PEAK_BF16_TFLOPS,
                              unit="TFLOP/s", frac=ach / PEAK_BF16_TFLOPS,
-                             traffic=traffic.get(dom) if traffic else None,
+                             traffic=traffic, traffic_source=traffic_src,
                              kernel_ms=float(dom_ms), algorithmic_flops=dom_flops)
     return r, xs[0], out
 
@@ -302,6 +324,158 @@ def measure_dequant(torch, capi, steps, warmup, seed):
     return res
 
 
+# Batch sizes the benchmark list names per configuration (decode and prefill points).
+BASELINE_SWEEPS = {
+    "tiny_f32": (64,),
+    "mixtral_bf16": (1, 16, 128, 512, 4096),
+    "mixtral_int8": (1, 16, 4096),
+    "qwen_bf16": (1, 256, 8192),
+    "deepseek_bf16": (1, 1024, 16384),
+}
+# Layer-output bar against the CPU path: max|a - ref| / max|ref|.
+PARITY_BAR = {"f32": 1e-5, "bf16": 1e-2, "int8": 1e-2, "int8g": 1e-2}
+
+
+def compact(config, r):
+    """One entry of the `configs` list: what a table row needs."""
+    hbm = r["roofline"]["bound"] == "hbm"
+    return dict(config=config, tokens=r["tokens"], ms_per_step=r["ms_per_step"],
+                tokens_per_s=r["tokens_per_s"], bound=r["roofline"]["bound"],
+                forward_frac=r["forward_hbm_frac"] if hbm else r["forward_mfma_frac"],
+                forward_hbm_frac=r["forward_hbm_frac"], forward_mfma_frac=r["forward_mfma_frac"],
+                active_experts=r["active_experts"], stage_ms=r["stage_ms"],
+                roofline=r["roofline"])
+
+
+def build_config(torch, np, capi, name, seed, tmax):
+    """Sets the module's shape globals to configuration `name`, generates its weights and builds
+    its layer (experts resident in HBM).  Returns what the measurements and the CPU check need."""
+    global D_MODEL, N_EXPERTS, TOP_K, D_FF, D_FF_SHARED, W_BYTES, CONFIG_NAME, GROUP, ACT
+    cfg = CONFIGS[name]
+    CONFIG_NAME = name
+    D_MODEL, N_EXPERTS, TOP_K, D_FF, D_FF_SHARED = cfg["d"], cfg["E"], cfg["k"], cfg["f"], cfg["fs"]
+    f32w = cfg["wd"] == "f32"
+    W_BYTES = 4 if f32w else 1 if cfg["wd"] in ("int8", "int8g") else 2
+    ACT = capi.ACT_F32 if f32w else capi.ACT_BF16
+    GROUP = 128 if cfg["wd"] == "int8g" else 0
+    router, gate, up, down, shared = make_weights(torch, np, seed, f32=f32w)
+    router_f32 = upcast(np, router)
+    if cfg["zipf"] or cfg.get("unit_logits"):  # router rows ~ N(0, 1/d): logits ~ N(0, 1)
+        router_f32 = router_f32 * np.float32(1.0 / (W_STD * np.sqrt(D_MODEL)))
+        router_f32 = upcast(np, capi.f32_to_bf16_trunc(router_f32))
+    kw = dict(w_router=router_f32, top_k=TOP_K, convention=cfg["conv"], max_tokens_hint=tmax)
+    if cfg["zipf"]:  # plus a log-Zipf(1.2) bias: skewed expert load
+        rank = np.random.default_rng(seed).permutation(N_EXPERTS) + 1.0
+        kw["router_bias"] = (-1.2 * np.log(rank)).astype(np.float32)
+    if shared is not None and cfg["gated"]:
+        kw["shared_gate"] = shared[3]
+    # what the CPU path computes with: the stored values, upcast / dequantised to f32
+    stored = dict(w_gate=upcast(np, gate), w_up=upcast(np, up), w_down=upcast(np, down))
+    if shared is not None:
+        stored.update(s_gate=upcast(np, shared[0]), s_up=upcast(np, shared[1]),
+                      s_down=upcast(np, shared[2]))
+    if cfg["wd"] in ("int8", "int8g"):
+        # int8 of the bf16-valued weights (per output row, or per row and 128-element group),
+        # 0.1 % of rows scaled x8 first
+        rng = np.random.default_rng(seed + 1)
+        per_group = cfg["wd"] == "int8g"
+        if per_group:
+            kw["group_size"] = 128
+
+        def q8(bits, name):
+            w = upcast(np, bits)
+            rows = w.reshape(-1, w.shape[-1])
+            rows[rng.choice(rows.shape[0], size=rows.shape[0] // 1000, replace=False)] *= 8.0
+            q, sc = capi.quantize_per_group_i8(w, 128) if per_group else capi.quantize_per_row_i8(w)
+            full = np.repeat(sc, 128, axis=-1)[..., :w.shape[-1]] if per_group else sc[..., None]
+            stored[name] = q.astype(np.float32) * full
+            return q, sc
+        (gate, sg), (up, su), (down, sd) = q8(gate, "w_gate"), q8(up, "w_up"), q8(down, "w_down")
+        kw.update(scale_gate=sg, scale_up=su, scale_down=sd)
+        if shared is not None:
+            (g_, a1), (u_, a2), (d_, a3) = (q8(shared[0], "s_gate"), q8(shared[1], "s_up"),
+                                            q8(shared[2], "s_down"))
+            shared = (g_, u_, d_, shared[3])
+            kw.update(s_scale_gate=a1, s_scale_up=a2, s_scale_down=a3)
+        wdt = capi.WEIGHT_INT8_PER_GROUP if per_group else capi.WEIGHT_INT8_W8A16
+    else:
+        wdt = capi.WEIGHT_F32 if f32w else capi.WEIGHT_BF16
+    if shared is not None:
+        kw.update(s_gate=shared[0], s_up=shared[1], s_down=shared[2])
+    layer = capi.Layer(w_gate=gate, w_up=up, w_down=down, weight_dtype=wdt, **kw)
+    e_bias = None
+    if cfg.get("v3"):
+        v3 = cfg["v3"]
+        e_bias = (0.05 * np.random.default_rng(seed + 2).standard_normal(N_EXPERTS)).astype(np.float32)
+        layer.set_v3_router(v3["n_group"], v3["topk_group"], v3["scale"], v3["norm"], e_bias)
+    return dict(name=name, cfg=cfg, layer=layer, router_f32=router_f32, kw=kw, stored=stored,
+                e_bias=e_bias)
+
+
+def cpu_and_parity(torch, np, capi, ctx, x_head, out_head, tokens, cpu_tokens):
+    """The CPU path (the oracle: checker and reported baseline, never part of what is timed on
+    the GPU) on the first n tokens of the batch, and the parity report of the batch: routing of
+    every token against the CPU path, the smallest routing margin of the batch (k-th minus
+    (k+1)-th largest logit: how close the batch comes to a tie, the reference's fragility signal,
+    tests/moe_cert2_qwen_decomposition_test.rs:79-86), and on the n sample tokens the layer-output
+    bar max|a - ref| / max|ref| plus the reference's own metric block (src/moe/numerical.rs:58-88)."""
+    from oracle import moe_oracle as ora
+    cfg, layer, kw = ctx["cfg"], ctx["layer"], ctx["kw"]
+    flops_tok = 2.0 * D_MODEL * N_EXPERTS + 6.0 * TOP_K * D_MODEL * D_FF + 6.0 * D_MODEL * D_FF_SHARED
+    n = cpu_tokens if cpu_tokens > 0 else int(1024 * 704.7e6 / flops_tok)
+    n = max(1, min(n, tokens))
+    if cfg.get("v3") and cpu_tokens < 0:
+        n = min(n, 512)  # that path runs token by token on one core
+    # the batch recomputed once so that `out_head` matches `x_head`
+    layer.forward_device(x_head.data_ptr(), ACT, tokens, out_head.data_ptr(),
+                         torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    idx_gpu, *_ = layer.last_routing(tokens)
+    xs = x_head[:n].to(torch.float32).cpu().numpy()
+    got = out_head[:n].cpu().numpy()
+    oL = ora.Layer(w_router=ctx["router_f32"], top_k=TOP_K, convention=cfg["conv"],
+                   shared_gate=kw.get("shared_gate"), router_bias=kw.get("router_bias"),
+                   **ctx["stored"])
+    cores = ora.hw_threads()
+    ora.set_threads(cores)
+    if cfg.get("v3"):  # the DeepSeek-V3 router in front of the same experts (one thread)
+        v3 = cfg["v3"]
+        cores = 1
+        run = lambda rows: oL.v3_forward(rows, ctx["e_bias"], v3["n_group"], v3["topk_group"],
+                                         v3["scale"], v3["norm"])[:2]
+    else:
+        run = lambda rows: oL.execute(rows)[:2]
+    run(xs[:1])  # warm the pages
+    t0 = time.perf_counter()
+    ref, o_idx = run(xs)
+    dt = time.perf_counter() - t0
+    cpu = dict(value=n / dt, unit="tokens/s", cores=cores, kind="port",
+               sample=f"{n} tokens of the T={tokens} batch, certified policy "
+                      "(f32 weights, f64 accumulation), rows parallel over the cores used")
+    margin = None
+    if cfg.get("v3"):  # routing checked on the sample the CPU path ran
+        o_all, idx_gpu, n_routed = o_idx, idx_gpu[:n], n
+    else:
+        o_all, _, logits = oL.route_tokens(x_head.to(torch.float32).cpu().numpy(), want_logits=True)
+        n_routed = int(tokens)
+        if TOP_K < N_EXPERTS:
+            srt = np.sort(logits.astype(np.float64), axis=1)[:, ::-1]
+            gaps = srt[:, TOP_K - 1] - srt[:, TOP_K]
+            margin = dict(min_routing_margin=float(gaps.min()), at_token=int(gaps.argmin()),
+                          median_routing_margin=float(np.median(gaps)))
+    bar = PARITY_BAR[cfg["wd"]]
+    rel = float(np.abs(got - ref).max() / np.abs(ref).max())
+    parity = dict(
+        routing_mismatched_tokens=int((idx_gpu != o_all).any(axis=1).sum()),
+        tokens_routed=n_routed,
+        max_rel_err_vs_cpu_path=rel, bar=bar, within_bar=bool(rel <= bar),
+        sample_tokens=n)
+    if margin:
+        parity.update(margin)
+    parity.update(ora.numerical_metrics(got, ref))  # max_abs_diff, mean_abs_diff, rmse, argmax_match
+    return cpu, parity
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -314,9 +488,13 @@ def main():
     ap.add_argument("--decode-tokens", type=str, default="1,16",
                     help="decode batch sizes, comma separated (empty = skip); reported as "
                          "`decode` (the first) and `decode<T>` (the others)")
-    ap.add_argument("--sweep", type=str, default="128",
-                    help="extra batch sizes, comma separated (default: 128 tokens, where the "
-                         "mid-batch kernels serve the layer; \"all\": the configuration's own list)")
+    ap.add_argument("--sweep", type=str, default="default",
+                    help="extra batch sizes, comma separated (default: 128 and 512 tokens where the "
+                         "configuration lists them; \"all\": the configuration's own list)")
+    ap.add_argument("--all-configs", choices=("auto", "yes", "no"), default="auto",
+                    help="after the headline block, time every configuration of the benchmark list "
+                         "at its own batch sizes (`configs`); auto = with the default configuration "
+                         "unless the CPU leg is switched off")
     ap.add_argument("--cpu-tokens", type=int, default=-1,
                     help="tokens of the CPU-baseline sample (0 = skip; default: about 12 s of "
                          "CPU work on 16 cores)")
@@ -346,15 +524,9 @@ def main():
         print("bench.py: no gfx950 device; the HIP path has no fallback", file=sys.stderr)
         sys.exit(3)
     torch.cuda.set_device(0)
-    global D_MODEL, N_EXPERTS, TOP_K, D_FF, D_FF_SHARED, W_BYTES, CONFIG_NAME, GROUP, GRAPH, ACT
+    global GRAPH
     GRAPH = a.graph
     cfg = CONFIGS[a.config]
-    CONFIG_NAME = a.config
-    D_MODEL, N_EXPERTS, TOP_K, D_FF, D_FF_SHARED = cfg["d"], cfg["E"], cfg["k"], cfg["f"], cfg["fs"]
-    f32w = cfg["wd"] == "f32"
-    W_BYTES = 4 if f32w else 1 if cfg["wd"] in ("int8", "int8g") else 2
-    ACT = capi.ACT_F32 if f32w else capi.ACT_BF16
-    GROUP = 128 if cfg["wd"] == "int8g" else 0
     if a.tokens <= 0:
         a.tokens = max(cfg["sweep"])
     decode_ts = [int(t) for t in a.decode_tokens.split(",") if t]
@@ -362,60 +534,12 @@ def main():
                  (t in cfg["sweep"] or a.decode_tokens != "1,16")]
     if a.sweep == "all":
         a.sweep = ",".join(str(t) for t in cfg["sweep"] if t != a.tokens and t not in decode_ts)
-    elif a.sweep == "128":  # the default: only where the configuration lists that batch size
-        a.sweep = "128" if 128 in cfg["sweep"] and a.tokens != 128 and 128 not in decode_ts else ""
-    a.sweep = ",".join(t for t in a.sweep.split(",") if t and int(t) > 0)  # "0" = none
-    router, gate, up, down, shared = make_weights(torch, np, a.seed, f32=f32w)
-    router_f32 = upcast(np, router)
-    if cfg["zipf"]:  # logits ~ N(0,1) plus a log-Zipf(1.2) bias: skewed expert load
-        router_f32 = router_f32 * np.float32(1.0 / (W_STD * np.sqrt(D_MODEL)))
-        router_f32 = upcast(np, capi.f32_to_bf16_trunc(router_f32))
-    tmax = max([a.tokens] + decode_ts + [int(t) for t in a.sweep.split(",") if t])
-    kw = dict(w_router=router_f32, top_k=TOP_K, convention=cfg["conv"], max_tokens_hint=tmax)
-    if cfg["zipf"]:
-        rank = np.random.default_rng(a.seed).permutation(N_EXPERTS) + 1.0
-        kw["router_bias"] = (-1.2 * np.log(rank)).astype(np.float32)
-    if shared is not None and cfg["gated"]:
-        kw["shared_gate"] = shared[3]
-    # what the CPU path computes with: the stored values, upcast / dequantised to f32
-    stored = dict(w_gate=upcast(np, gate), w_up=upcast(np, up), w_down=upcast(np, down))
-    if shared is not None:
-        stored.update(s_gate=upcast(np, shared[0]), s_up=upcast(np, shared[1]),
-                      s_down=upcast(np, shared[2]))
-    if cfg["wd"] in ("int8", "int8g"):
-        # int8 of the bf16-valued weights (per output row, or per row and 128-element group),
-        # 0.1 % of rows scaled x8 first
-        rng = np.random.default_rng(a.seed + 1)
-        per_group = cfg["wd"] == "int8g"
-        if per_group:
-            kw["group_size"] = 128
-
-        def q8(bits, name):
-            w = upcast(np, bits)
-            rows = w.reshape(-1, w.shape[-1])
-            rows[rng.choice(rows.shape[0], size=rows.shape[0] // 1000, replace=False)] *= 8.0
-            q, sc = capi.quantize_per_group_i8(w, 128) if per_group else capi.quantize_per_row_i8(w)
-            full = np.repeat(sc, 128, axis=-1)[..., :w.shape[-1]] if per_group else sc[..., None]
-            stored[name] = q.astype(np.float32) * full
-            return q, sc
-        (gate, sg), (up, su), (down, sd) = q8(gate, "w_gate"), q8(up, "w_up"), q8(down, "w_down")
-        kw.update(scale_gate=sg, scale_up=su, scale_down=sd)
-        if shared is not None:
-            (g_, a1), (u_, a2), (d_, a3) = (q8(shared[0], "s_gate"), q8(shared[1], "s_up"),
-                                            q8(shared[2], "s_down"))
-            shared = (g_, u_, d_, shared[3])
-            kw.update(s_scale_gate=a1, s_scale_up=a2, s_scale_down=a3)
-        wdt = capi.WEIGHT_INT8_PER_GROUP if per_group else capi.WEIGHT_INT8_W8A16
-    else:
-        wdt = capi.WEIGHT_F32 if f32w else capi.WEIGHT_BF16
-    if shared is not None:
-        kw.update(s_gate=shared[0], s_up=shared[1], s_down=shared[2])
-    layer = capi.Layer(w_gate=gate, w_up=up, w_down=down, weight_dtype=wdt, **kw)
-    e_bias = None
-    if cfg.get("v3"):
-        v3 = cfg["v3"]
-        e_bias = (0.05 * np.random.default_rng(a.seed + 2).standard_normal(N_EXPERTS)).astype(np.float32)
-        layer.set_v3_router(v3["n_group"], v3["topk_group"], v3["scale"], v3["norm"], e_bias)
+    elif a.sweep == "default":  # the batch sizes of the configuration's own list between the two
+        a.sweep = ",".join(str(t) for t in (128, 512)
+                           if t in cfg["sweep"] and t != a.tokens and t not in decode_ts)
+    sweep_ts = [int(t) for t in a.sweep.split(",") if t and int(t) > 0]  # "0" = none
+    ctx = build_config(torch, np, capi, a.config, a.seed, max([a.tokens] + decode_ts + sweep_ts))
+    layer = ctx["layer"]
 
     if a.calibrate_copy:
         src = torch.empty(1 << 28, device="cuda", dtype=torch.float32)  # 1 GiB
@@ -432,7 +556,7 @@ def main():
         decodes[t], _, _ = measure(torch, np, capi, layer, t, max(a.steps, 50), max(a.warmup, 10),
                                    a.seed)
     sweep = []
-    for t in [int(t) for t in a.sweep.split(",") if t]:
+    for t in sweep_ts:
         r, _, _ = measure(torch, np, capi, layer, t, a.steps if t >= 512 else max(a.steps, 50),
                           a.warmup, a.seed)
         sweep.append(r)
@@ -441,8 +565,7 @@ def main():
     if a.block:
         block = [measure_block(torch, np, capi, layer, t, a.steps if t >= 512 else max(a.steps, 50),
                                a.warmup, a.seed)
-                 for t in sorted({a.tokens} | set(decode_ts) | {int(t) for t in a.sweep.split(",") if t})
-                 if t > 0]
+                 for t in sorted({a.tokens} | set(decode_ts) | set(sweep_ts)) if t > 0]
 
     # The entry point a caller of the reference's op reaches: [T * d] f32 in host memory in and
     # out (src/amg/graph.rs:5572-5589 hands a Vec<f32> over).  PCIe-inclusive, never `value`.
@@ -472,53 +595,14 @@ def main():
                     host_bytes_moved=2.0 * a.tokens * D_MODEL * 4,
                     note="atenia_moe_hip_layer_forward, synchronous, [T*d] f32 in and out: "
                          "pageable caller buffers / page-locked caller buffers")
+        del xp, op, xh, oh
 
     cpu = None
     parity = None
     if a.cpu_tokens != 0:
-        from oracle import moe_oracle as ora  # checker + reported CPU baseline only
-        flops_tok = 2.0 * D_MODEL * N_EXPERTS + 6.0 * TOP_K * D_MODEL * D_FF + 6.0 * D_MODEL * D_FF_SHARED
-        n = a.cpu_tokens if a.cpu_tokens > 0 else int(1024 * 704.7e6 / flops_tok)
-        n = max(1, min(n, a.tokens))
-        if cfg.get("v3") and a.cpu_tokens < 0:
-            n = min(n, 512)  # that path runs token by token on one core
-        # the headline batch, recomputed once so `out_head` matches `x_head`
-        layer.forward_device(x_head.data_ptr(), ACT, a.tokens, out_head.data_ptr(),
-                             torch.cuda.current_stream().cuda_stream)
-        torch.cuda.synchronize()
-        idx_gpu, *_ = layer.last_routing(a.tokens)
-        xs = x_head[:n].to(torch.float32).cpu().numpy()
-        got = out_head[:n].cpu().numpy()
-        oL = ora.Layer(w_router=router_f32, top_k=TOP_K, convention=cfg["conv"],
-                       shared_gate=kw.get("shared_gate"), router_bias=kw.get("router_bias"),
-                       **stored)
-        cores = ora.hw_threads()
-        ora.set_threads(cores)
-        if cfg.get("v3"):  # the DeepSeek-V3 router in front of the same experts (one thread)
-            v3 = cfg["v3"]
-            cores = 1
-            run = lambda rows: oL.v3_forward(rows, e_bias, v3["n_group"], v3["topk_group"],
-                                             v3["scale"], v3["norm"])[:2]
-        else:
-            run = lambda rows: oL.execute(rows)[:2]
-        run(xs[:1])  # warm the pages
-        t0 = time.perf_counter()
-        ref, o_idx = run(xs)
-        dt = time.perf_counter() - t0
-        cpu = dict(value=n / dt, unit="tokens/s", cores=cores, kind="port",
-                   sample=f"{n} tokens of the T={a.tokens} batch, certified policy "
-                          "(f32 weights, f64 accumulation), rows parallel over the cores used")
-        if cfg.get("v3"):  # routing checked on the sample the CPU path ran
-            o_all, idx_gpu, n_routed = o_idx, idx_gpu[:n], n
-        else:
-            o_all, _ = oL.route_tokens(x_head.to(torch.float32).cpu().numpy())
-            n_routed = int(a.tokens)
-        parity = dict(
-            routing_mismatched_tokens=int((idx_gpu != o_all).any(axis=1).sum()),
-            tokens_routed=n_routed,
-            max_rel_err_vs_cpu_path=float(np.abs(got - ref).max() / np.abs(ref).max()),
-            sample_tokens=n)
+        cpu, parity = cpu_and_parity(torch, np, capi, ctx, x_head, out_head, a.tokens, a.cpu_tokens)
 
+    f32w = cfg["wd"] == "f32"
     line = {
         "metric": "Mixtral-shape MoE layer tok/s; decode HBM GB/s and prefill MFMA TFLOPS",
         "value": head["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": a.steps,
@@ -537,6 +621,7 @@ def main():
         "sweep": sweep,
         "parity": parity,
         "host_entry": host,
+        "kernels_sha": KERNELS_SHA,
     }
     for t in decode_ts[1:]:
         line[f"decode{t}"] = decodes[t]
@@ -544,6 +629,37 @@ def main():
         line["block"] = block
     if a.dequant:
         line["dequant"] = measure_dequant(torch, capi, max(a.steps, 50), a.warmup, a.seed)
+
+    # Every configuration of the benchmark list at its own batch sizes, one compact entry per
+    # (configuration, T) (the reference's own bench walks its three families in one run,
+    # tests/moe_perf_scale_bench.rs:70-75); the headline configuration's entries repeat the
+    # figures above.  Weights are generated on the device as for the headline; the CPU path is
+    # timed on the headline only, here it checks a small token sample per configuration.
+    if a.all_configs == "auto":
+        a.all_configs = "yes" if a.config == "mixtral_bf16" and a.cpu_tokens != 0 else "no"
+    if a.all_configs == "yes":
+        entries = [compact(a.config, r) for r in
+                   sorted([head] + list(decodes.values()) + sweep, key=lambda r: r["tokens"])]
+        parities = {a.config: parity}
+        layer.close()
+        del ctx, layer, x_head, out_head
+        for name in BASELINE_SWEEPS:
+            if name == a.config:
+                continue
+            ts = BASELINE_SWEEPS[name]
+            ctx = build_config(torch, np, capi, name, a.seed, max(ts))
+            xo = None
+            for t in ts:
+                r, x_t, out_t = measure(torch, np, capi, ctx["layer"], t,
+                                        a.steps if t >= 512 else max(a.steps, 50), a.warmup, a.seed)
+                entries.append(compact(name, r))
+                xo = (x_t, out_t, t)
+            _, parities[name] = cpu_and_parity(torch, np, capi, ctx, xo[0], xo[1], xo[2],
+                                               min(xo[2], 64))
+            ctx["layer"].close()
+            del ctx, xo
+        line["configs"] = entries
+        line["configs_parity"] = parities
     print(json.dumps(line))
 
 

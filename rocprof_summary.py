@@ -30,6 +30,21 @@ import sqlite3
 import sys
 
 COPY_KERNEL = "__amd_rocclr_copyBuffer"
+ROOT = os.path.dirname(os.path.abspath(__file__))
+
+
+def kernels_sha():
+    """Short hash of the kernel sources this tree builds (csrc/*.hip, *.h, Makefile).  A counter
+    summary records it, and bench.py quotes the summary's HBM traffic only while the hash still
+    matches the sources it runs: after a kernel change the line says that the figure is stale."""
+    import hashlib
+    h = hashlib.sha256()
+    src = os.path.join(ROOT, "ateniaengine_amd", "csrc")
+    for name in sorted(os.listdir(src)):
+        if name.endswith((".hip", ".h")) or name == "Makefile":
+            with open(os.path.join(src, name), "rb") as fh:
+                h.update(name.encode() + b"\0" + fh.read())
+    return h.hexdigest()[:16]
 
 
 def find_db(path):
@@ -86,6 +101,7 @@ def traffic(fetch_db, write_db, config, maps, copy_bytes):
 
     f_rows, f_unit = per_kernel(fetch_db, "FETCH_SIZE")
     w_rows, w_unit = per_kernel(write_db, "WRITE_SIZE")
+    print(f"kernels_sha {kernels_sha()}")
     print(f"# calibration: a {copy_bytes} byte device copy reads FETCH_SIZE x {f_unit:.1f} B and "
           f"WRITE_SIZE x {w_unit:.1f} B per unit")
     def pick(rows, pattern):
