@@ -37,7 +37,8 @@ EXPORTS = (
     "atenia_moe_hip_layer_permute", "atenia_moe_hip_layer_last_routing",
     "atenia_moe_hip_layer_last_expert_outputs", "atenia_moe_hip_layer_set_profiling",
     "atenia_moe_hip_layer_stage_ms", "atenia_moe_hip_layer_stage_launches",
-    "atenia_moe_hip_layer_info", "atenia_moe_hip_layer_expert_kernels", "atenia_moe_quantize_per_row_i8",
+    "atenia_moe_hip_layer_info", "atenia_moe_hip_layer_expert_kernels", "atenia_moe_hip_plan_batch", "atenia_moe_hip_layer_last_down_split",
+    "atenia_moe_quantize_per_row_i8",
     "atenia_moe_f32_to_bf16_trunc",
     "atenia_moe_hip_layer_last_non_finite", "atenia_moe_router_launch_device", "atenia_moe_permute_launch_device",
     "atenia_moe_expert_ffn_launch_device", "atenia_moe_combine_launch_device",
@@ -111,6 +112,8 @@ def lib():
         L.atenia_moe_hip_layer_stage_launches.argtypes = [P, P]
         L.atenia_moe_hip_layer_info.argtypes = [P, P]
         L.atenia_moe_hip_layer_expert_kernels.argtypes = [P, C.c_int64, P]
+        L.atenia_moe_hip_plan_batch.argtypes = [C.c_int] * 7 + [C.c_int64, P]
+        L.atenia_moe_hip_layer_last_down_split.argtypes = [P, P]
         L.atenia_moe_quantize_per_row_i8.argtypes = [P, C.c_size_t, C.c_size_t, P, P]
         L.atenia_moe_f32_to_bf16_trunc.argtypes = [P, C.c_size_t, P]
         L.atenia_moe_hip_layer_last_non_finite.argtypes = [P, P, P]
@@ -213,6 +216,19 @@ def int8_to_bf16_launch_device(d_int8, d_scales, d_bf16, k: int, n: int, group_s
     return L.atenia_moe_int8_to_bf16_per_channel_launch_device(d_int8, d_scales, d_bf16, k, n, stream)
 
 
+PLAN_KEYS = ("up", "down", "shared_up", "shared_down", "y_bf16", "ys_bf16", "tall_tiles", "duo")
+
+
+def plan_batch(E: int, k: int, d: int, f: int, f_s: int, weight_dtype: int, T: int,
+               group_size: int = 0) -> dict:
+    """Which kernels a T-token batch takes on a layer of these dimensions (no device needed):
+    kernel family per phase for the routed and the shared expert (KERNELS_*; -1 = none), whether
+    the expert outputs reach the combine as bf16, tall row tiles, two-workgroup form per phase."""
+    v = np.zeros(8, dtype=np.int32)
+    _check(lib().atenia_moe_hip_plan_batch(E, k, d, f, f_s, weight_dtype, group_size, T, _ptr(v)))
+    return dict(zip(PLAN_KEYS, (int(i) for i in v)))
+
+
 def f32_to_bf16_trunc(a) -> np.ndarray:
     a = np.ascontiguousarray(a, dtype=np.float32)
     out = np.empty(a.shape, dtype=np.uint16)
@@ -257,7 +273,7 @@ class Layer:
                              "scale_up", "scale_down", "s_gate", "s_up", "s_down", "s_scale_gate",
                              "s_scale_up", "s_scale_down", "shared_gate")], group_size)
         self.E, self.k, self.d, self.f, self.fs = E, top_k, d, f, fs
-        self.convention, self.weight_dtype = convention, weight_dtype
+        self.convention, self.weight_dtype, self.group_size = convention, weight_dtype, group_size
         self._h = C.c_void_p()
         _check(lib().atenia_moe_hip_layer_create(C.addressof(desc), C.addressof(self._h)))
         del keep  # host arrays are only borrowed for the call
@@ -398,6 +414,12 @@ class Layer:
         _check(lib().atenia_moe_hip_layer_last_expert_outputs(self._h, _ptr(y), _ptr(ys)))
         return y, ys
 
+    def last_down_split(self, T: int) -> np.ndarray:
+        """[T, k, ceil(d / 256)] k ranges of the down tile behind each expert-output block (1 = whole)."""
+        parts = np.empty((T, self.k, (self.d + 255) // 256), dtype=np.uint8)
+        _check(lib().atenia_moe_hip_layer_last_down_split(self._h, _ptr(parts)))
+        return parts
+
     # -- timing ---------------------------------------------------------------------------
     def set_profiling(self, on: bool):
         _check(lib().atenia_moe_hip_layer_set_profiling(self._h, int(on)))
@@ -418,6 +440,11 @@ class Layer:
         v = np.zeros(2, dtype=np.int32)
         _check(lib().atenia_moe_hip_layer_expert_kernels(self._h, T, _ptr(v)))
         return int(v[0]), int(v[1])
+
+    def plan(self, T: int) -> dict:
+        """plan_batch for this layer's dimensions."""
+        return plan_batch(self.E, self.k, self.d, self.f, self.fs, self.weight_dtype, T,
+                          self.group_size)
 
     def info(self) -> dict:
         v = np.zeros(8, dtype=np.int64)

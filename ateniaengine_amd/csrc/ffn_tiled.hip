@@ -24,9 +24,7 @@
 //                             the way into LDS)
 // Weights are stored in HBM as 1 KiB blocks already in MFMA register order (moe_internal.h), so
 // a B chunk is a straight 1 KiB copy and every B fragment read is one ds_read_b128.
-#include <type_traits>
-
-#include "moe_internal.h"
+#include "ffn_tiled_common.h"
 
 #include "../../include/atenia_moe_hip.h"
 
@@ -34,176 +32,7 @@ namespace atenia_moe {
 
 namespace {
 
-typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
-typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
-
-constexpr int kThreads = 256;
-constexpr int TM = kTileM;   // 256 token rows
-constexpr int TNB = 256;     // B rows per tile (gate/up: 128 + 128)
-constexpr int TK = 64;       // k per LDS stage
-constexpr int kChunk = 1024; // bytes
-constexpr int kAStage = (TM / 16) * (TK / 32) * kChunk;   // 32 KiB
-constexpr int kBStage = (TNB / 16) * (TK / 32) * kChunk;  // 32 KiB
-constexpr int kStage = kAStage + kBStage;
-constexpr int kLdsBytes = 2 * kStage;                     // 128 KiB
-
-struct TiledParams {
-  const uint4* wa;      // gate (up phase) or down blocks
-  const uint4* wb;      // up blocks
-  const float* sa;      // int8 row scales [G, n_rows]
-  const float* sb;
-  int64_t w_stride_u4;
-  int n_rows;           // unpadded N
-  int n_blocks;         // n_pad / 16
-  int nkb;              // K blocks per strip (32 k each for bf16, 64 k for int8)
-  int k_pad;
-  const uint16_t* a;    // bf16 rows
-  int a_stride;
-  void* out;
-  int out_stride;
-  GroupDesc g;
-  const int32_t* tile_group;  // [n_tiles] expert of each row tile
-  const int32_t* tile_m0;     // [n_tiles] first row (relative to the group) of each row tile
-  const int32_t* n_tiles;     // [1]
-  const int32_t* tile_rows;   // [n_tiles] rows of each tile, or null: min(TM, rows left)
-  const int32_t* tile_li;     // [n_tiles] index inside the expert | (its tiles << 16), or null
-  int n_col_tiles;
-  // k split of the tail tiles (pipelined down kernels; max_parts <= 1: off).  Workgroup ids
-  // below wg_upper are the tiles themselves, ids from wg_upper on the extra k ranges of the
-  // tiles in the last, partly filled round over the n_cus compute units.
-  int max_parts;
-  int wg_upper;
-  int n_cus;
-  size_t out_part_stride;     // elements between the partial output buffers
-  uint8_t* part_flags;        // [pairs, n_col_tiles] partial buffers written per (row, column tile)
-};
-
-__device__ inline uint16_t bf16_rne(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
-}
-
-// Two f32 -> two bf16 (round to nearest even) in one v_cvt_pk_bf16_f32; low half = a.
-typedef __attribute__((ext_vector_type(2))) float f32x2_t;
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
-__device__ inline uint32_t bf16_rne_pair(float a, float b) {
-  f32x2_t v = {a, b};
-  bf16x2_t h = __builtin_convertvector(v, bf16x2_t);
-  return *(uint32_t*)&h;
-}
-
-// silu(g) * u with the hardware exp2 / rcp (1 ulp each; the result is rounded to bf16 next).
-__device__ inline float swiglu_fast(float g, float u) {
-  const float t = __builtin_amdgcn_exp2f(g * -1.4426950408889634f);
-  return g * __builtin_amdgcn_rcpf(1.f + t) * u;
-}
-
-__device__ inline uint32_t pack_i8_pair(uint32_t w, int sh) {
-  float f0 = (float)(int8_t)((w >> sh) & 0xff);
-  float f1 = (float)(int8_t)((w >> (sh + 8)) & 0xff);
-  // |q| <= 128 is exact in bf16, so dropping the low 16 bits loses nothing: one byte permute
-  // takes the high halves of both floats (bytes 2, 3 of f0 below bytes 2, 3 of f1).
-  return __builtin_amdgcn_perm(__float_as_uint(f1), __float_as_uint(f0), 0x07060302u);
-}
-__device__ inline void widen_i8x16(uint4 q, uint4& lo, uint4& hi) {
-  lo.x = pack_i8_pair(q.x, 0);
-  lo.y = pack_i8_pair(q.x, 16);
-  lo.z = pack_i8_pair(q.y, 0);
-  lo.w = pack_i8_pair(q.y, 16);
-  hi.x = pack_i8_pair(q.z, 0);
-  hi.y = pack_i8_pair(q.z, 16);
-  hi.z = pack_i8_pair(q.w, 0);
-  hi.w = pack_i8_pair(q.w, 16);
-}
-
-__device__ inline f32x4 mfma(uint4 a, uint4 b, f32x4 c) {
-  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(bf16x8*)&a, *(bf16x8*)&b, c, 0, 0, 0);
-}
-
-// Which (row tile, column tile) a workgroup computes.
-//
-// XCD-aware order: hardware deals consecutive workgroup ids round-robin to the 8 XCDs, each
-// with its own L2, so XCD x is given the contiguous run [x*per_xcd, (x+1)*per_xcd) of the
-// logical tile order.  In that order an expert's tiles are contiguous and walked in patches of
-// (all row tiles of the expert) x (8 column tiles): the ~32 workgroups an XCD runs at a time
-// share ~4 activation tiles and 8 weight tiles instead of streaming 64 different ones.
-constexpr int kColGroup = 8;
-__device__ inline bool tile_of_workgroup(const TiledParams& p, int wid, int& rt, int& ct) {
-  const int n_row_tiles = *p.n_tiles;
-  const int nct = p.n_col_tiles;
-  const int total = n_row_tiles * nct;
-  const int per_xcd = (total + 7) / 8;
-  const int slot = wid / 8;
-  const int logical = (wid % 8) * per_xcd + slot;
-  if (slot >= per_xcd || logical >= total) return false;
-  // Row tiles are sorted by expert, so the expert owning this logical id is the expert of
-  // row tile logical / nct; that tile's m0 tells where the expert's tiles start.
-  const int rt_any = logical / nct;
-  int first, nt;
-  if (p.tile_li) {  // tiles of uneven height: the list says where the expert's tiles start
-    const int li = p.tile_li[rt_any];
-    first = rt_any - (li & 0xffff);
-    nt = li >> 16;
-  } else {
-    const int e = p.tile_group[rt_any];
-    const int cnt = p.g.offsets[e + 1] - p.g.offsets[e];
-    first = rt_any - p.tile_m0[rt_any] / TM;
-    nt = (cnt + TM - 1) / TM;
-  }
-  int local = logical - first * nct;
-  const int full = nct / kColGroup;
-  const int patch = nt * kColGroup;
-  int cg, gw;
-  if (local < full * patch) {
-    cg = local / patch;
-    local -= cg * patch;
-    gw = kColGroup;
-  } else {
-    local -= full * patch;
-    cg = full;
-    gw = nct - full * kColGroup;
-  }
-  const int rl = local / gw;
-  rt = first + rl;
-  ct = cg * kColGroup + (local - rl * gw);
-  return true;
-}
-
-// Tail split of the down phase.  With one workgroup per CU at a time, tiles run in rounds of
-// n_cus; when the last round is at most half full, each of its tiles is cut into S k ranges
-// (S <= max_parts) so that the round fills the chip and lasts 1/S as long.  Range 0 is
-// computed by the tile's own workgroup, ranges 1..S-1 by workgroups with ids from wg_upper on;
-// range i writes its partial sums to buffer i, and range 0 records S per (row, column tile) so
-// that the combine adds up exactly the buffers that were written.  Sets wid (the tile's
-// workgroup id for tile_of_workgroup), S and part; false = nothing to do.
-__device__ inline bool split_of_workgroup(const TiledParams& p, int n_stages, int& wid, int& S,
-                                          int& part) {
-  wid = blockIdx.x;
-  S = 1;
-  part = 0;
-  if (p.max_parts <= 1) return true;
-  const int total = *p.n_tiles * p.n_col_tiles;
-  const int per_xcd = (total + 7) / 8;
-  const int full_slots = (total / p.n_cus) * (p.n_cus / 8);  // slots per XCD in the full rounds
-  const int tail = 8 * (per_xcd - full_slots);               // tile slots of the last round
-  int s_tail = 1;
-  if (tail > 0 && 2 * tail <= p.n_cus) s_tail = min(min(p.max_parts, p.n_cus / tail), n_stages / 2);
-  if (s_tail < 1) s_tail = 1;
-  if ((int)blockIdx.x >= p.wg_upper) {
-    const int x = blockIdx.x - p.wg_upper;
-    if (s_tail == 1 || x >= tail * (s_tail - 1)) return false;
-    part = 1 + x / tail;
-    const int j = x - (part - 1) * tail;
-    wid = (full_slots + j / 8) * 8 + (j & 7);
-    S = s_tail;
-    return true;
-  }
-  if (wid / 8 >= full_slots) S = s_tail;
-  return true;
-}
-
+// (types, TiledParams, the tile order and the LDS-DMA helpers live in ffn_tiled_common.h)
 template <bool INT8, bool UP>
 __global__ __launch_bounds__(kThreads) void ffn_tiled_kernel(TiledParams p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -396,44 +225,14 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_kernel(TiledParams p) {
 // of the next unit and 4 loads of a stage several steps ahead are issued between its MFMAs
 // (pinned with sched_barrier), and the single barrier per 32-k step sits between the two
 // units of the step so that no wave waits for LDS right after it.
-typedef __attribute__((address_space(3))) void* lptr_t;
-
-// One wave-wide 16-byte-per-lane load from global memory straight into LDS: lane l's bytes
-// land at lds_addr + 16*l.  Written as inline assembly so that the compiler's wait-count
-// insertion does not tie later LDS reads to these loads (it would drain all stages); the
-// kernel waits for exactly the stage it needs with an explicit s_waitcnt before its barrier.
-__device__ inline void dma16(const void* gaddr, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off"
-               :
-               : "v"(gaddr), "s"(lds_addr)
-               : "memory", "m0");
-}
-
-typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
-
-// v_mfma_f32_32x32x16_bf16 operand layout: A lane l holds row l%32, k = 8*(l/32)..+7 of a
-// 32 x 16 fragment; B the same with columns; D register r of lane l is element
-// (row 8*(r/4) + 4*(l/32) + r%4, column l%32).  Measured on MI355X the 32x32x16 form sustains
-// about 1.35x the rate of 16x16x32 in this kind of loop, so the tiled kernel uses it: an LDS
-// chunk (1 KiB) is one 32 x 16 fragment.
-__device__ inline f32x16 mfma32(uint4 a, uint4 b, f32x16 c) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8*)&a, *(bf16x8*)&b, c, 0, 0, 0);
-}
-
-// s_waitcnt vmcnt(N) lgkmcnt(0): vmcnt[3:0] in bits 3:0, vmcnt[5:4] in bits 15:14, expcnt
-// (bits 6:4) left at "no wait".  lgkmcnt(0) makes sure the wave's own LDS reads have returned
-// before it passes the barrier behind which other waves refill the buffers it read.
-template <int N>
-__device__ inline void wait_vm_lgkm0() {
-  __builtin_amdgcn_s_waitcnt(0x0070 | (N & 15) | ((N >> 4) << 14));
-}
 constexpr int kRingA = 3;  // A stages of 64 k (32 KiB each)
 constexpr int kRingB = 3;  // B stages of 32 k (16 KiB each); a fourth measured no faster
 // Rows 256..287 of a nine-group tile: their own ring of 64-k stages (4 KiB each = four chunks of
 // 8 rows x 128 bytes, swizzled like the A chunks), one stage per A stage.
 constexpr int kXaStage = 256;  // uint4 per stage
 
-template <bool UP>
+// YB (down phase only): y leaves as bf16 (TiledParams::out_bf16), staged through LDS.
+template <bool UP, bool YB = false>
 __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p) {
   constexpr int NA = kRingA, NB = kRingB;
   constexpr int XA0 = NA * 2048 + NB * 1024;            // first uint4 of the extra-rows ring
@@ -780,6 +579,7 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p)
       }
     } else {  // column groups 4 wn + 2 wm, + 1 of this wave
       float* y = (float*)p.out + (size_t)part * p.out_part_stride;
+      uint16_t* yb = (uint16_t*)p.out + (size_t)part * p.out_part_stride;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int m = TM + 8 * (r >> 2) + 4 * kh + (r & 3);
@@ -788,10 +588,14 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p)
         if (p.part_flags && part == 0 && wn == 0 && wm == 0 && l32 == 0)
           p.part_flags[(size_t)pair * p.n_col_tiles + ct] = (uint8_t)n_parts;
         float* yr = y + (size_t)pair * p.out_stride;
+        uint16_t* ybr = yb + (size_t)pair * p.out_stride;
 #pragma unroll
         for (int jj = 0; jj < 2; ++jj) {
           const int n = nb0 * 16 + (4 * wn + 2 * wm + jj) * 32 + l32;
-          if (n < p.n_rows) yr[n] = accx[jj][r];
+          if (n < p.n_rows) {
+            if (YB) ybr[n] = (uint16_t)bf16_rne_pair(accx[jj][r], 0.f);
+            else yr[n] = accx[jj][r];
+          }
         }
       }
     }
@@ -840,6 +644,49 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p)
       const int n = n0 + c8 * 8;
       if (mrow < rows_here && n < p.n_blocks * 16)
         *(uint4*)(h + (size_t)(base + tm0 + mrow) * p.out_stride + n) = v;
+    }
+  } else if (YB) {
+    // y as bf16, staged through LDS like h above so that every global store is 16 bytes per lane
+    // and a row's 256 bytes leave as two full lines: the wave's 128 x 128 block goes to its own
+    // region with a row pitch of 272 bytes and is read back 16 lanes per row, 4 rows at a time.
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();  // every wave's loads have landed and its reads are done
+    asm volatile("" ::: "memory");
+    constexpr int kPitch = 272;
+    char* stage = (char*)S + wave * (128 * kPitch);
+    const int r4 = lane >> 4, c16 = lane & 15;
+    int pair_of[32];  // pair id of the rows this lane stores
+#pragma unroll
+    for (int it = 0; it < 32; ++it) {
+      const int m = wm * 128 + it * 4 + r4;
+      pair_of[it] = p.g.perm[base + tm0 + min(m, rows_here - 1)];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {  // rows m and m + 1
+          const int m = i * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
+          const uint32_t hh = bf16_rne_pair(acc[i][j][r], acc[i][j][r + 1]);
+          char* dst = stage + m * kPitch + (j * 32 + l32) * 2;
+          *(uint16_t*)dst = (uint16_t)hh;
+          *(uint16_t*)(dst + kPitch) = (uint16_t)(hh >> 16);
+        }
+      }
+    }
+    uint16_t* yb = (uint16_t*)p.out + (size_t)part * p.out_part_stride;
+    const int n = nb0 * 16 + wn * 128 + c16 * 8;
+#pragma unroll
+    for (int it = 0; it < 32; ++it) {
+      const int m = it * 4 + r4;
+      const uint4 v = *(const uint4*)(stage + m * kPitch + c16 * 16);
+      const int mrow = wm * 128 + m;
+      if (mrow >= rows_here) continue;
+      const int pair = pair_of[it];
+      if (p.part_flags && part == 0 && wn == 0 && c16 == 0)
+        p.part_flags[(size_t)pair * p.n_col_tiles + ct] = (uint8_t)n_parts;
+      if (n < p.n_rows) *(uint4*)(yb + (size_t)pair * p.out_stride + n) = v;
     }
   } else {
     float* y = (float*)p.out + (size_t)part * p.out_part_stride;
@@ -1161,7 +1008,12 @@ hipError_t launch_tiled_dma(TiledParams p, int max_row_tiles, hipStream_t s) {
   n_wg = (n_wg + 7) / 8 * 8;
   p.wg_upper = n_wg;
   const int extra = p.max_parts > 1 ? p.n_cus : 0;  // room for the extra k ranges of a tail round
-  ffn_tiled_pipe_kernel<UP><<<n_wg + extra, kThreads, 0, s>>>(p);
+  if (!UP && p.out_bf16) {
+    if (p.n_rows % 8) return hipErrorInvalidValue;  // a lane stores 8 columns at once
+    ffn_tiled_pipe_kernel<false, true><<<n_wg + extra, kThreads, 0, s>>>(p);
+  } else {
+    ffn_tiled_pipe_kernel<UP><<<n_wg + extra, kThreads, 0, s>>>(p);
+  }
   return hipGetLastError();
 }
 
@@ -1216,7 +1068,17 @@ hipError_t launch_ffn_up_tiled(const FfnArgs& a, hipStream_t s) {
   p.tile_li = a.tile_li;
   p.n_col_tiles = (a.gate.n_pad + 127) / 128;
   p.max_parts = 1;
-  if (!int8 && p.k_pad % 64 == 0 && p.k_pad >= 128) return launch_tiled_dma<true>(p, a.max_row_tiles, s);
+  const bool pipe_bf16 = !int8 && p.k_pad % 64 == 0 && p.k_pad >= 128;
+  // A list of nine-group tiles in any other kernel would lose the rows past 256 of such a tile.
+  if (a.tall_tiles && (!pipe_bf16 || a.use_duo || !p.tile_rows || !p.tile_li)) return hipErrorInvalidValue;
+  if (a.use_duo) {
+    if (!pipe_bf16) return hipErrorInvalidValue;
+    p.tile_rows = nullptr;
+    p.tile_li = nullptr;
+    p.n_cus = a.n_cus;
+    return launch_tiled_duo_up(p, a.max_row_tiles, s);
+  }
+  if (pipe_bf16) return launch_tiled_dma<true>(p, a.max_row_tiles, s);
   if (int8 && p.k_pad >= 128) return launch_tiled_pipe_i8<true>(p, a.max_row_tiles, s);
   return int8 ? launch_tiled<true, true>(p, a.max_row_tiles, s)
               : launch_tiled<false, true>(p, a.max_row_tiles, s);
@@ -1247,6 +1109,18 @@ hipError_t launch_ffn_down_tiled(const FfnArgs& a, hipStream_t s) {
   p.n_col_tiles = (a.down.n_pad + 255) / 256;
   p.max_parts = 1;
   const bool pipelined = int8 ? p.k_pad >= 128 : (p.k_pad % 64 == 0 && p.k_pad >= 128);
+  const bool pipe_bf16 = !int8 && pipelined;
+  if (a.tall_tiles && (!pipe_bf16 || a.use_duo || !p.tile_rows || !p.tile_li)) return hipErrorInvalidValue;
+  if (a.y_bf16 && !pipe_bf16) return hipErrorInvalidValue;  // only those kernels store bf16
+  p.out_bf16 = a.y_bf16;
+  if (a.use_duo) {
+    // no k split of tail tiles in this form: the caller passes y_parts <= 1
+    if (!pipe_bf16 || (a.y_parts > 1 && a.part_flags)) return hipErrorInvalidValue;
+    p.tile_rows = nullptr;
+    p.tile_li = nullptr;
+    p.n_cus = a.n_cus;
+    return launch_tiled_duo_down(p, a.max_row_tiles, s);
+  }
   if (pipelined && a.y_parts > 1 && a.part_flags && a.n_cus >= 8) {
     p.max_parts = a.y_parts;
     p.n_cus = a.n_cus / 8 * 8;

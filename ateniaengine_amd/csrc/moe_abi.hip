@@ -161,6 +161,7 @@ struct AteniaMoeLayer {
   int stage_T[4] = {-1, -1, -1, -1};  // token count each pipeline stage last completed for
   int nf_token = -1, nf_expert = -1;  // location of the last non-finite routing weight reported
   bool last_split = false;  // the last forward's down phase may have split tail tiles
+  bool last_y_bf16 = false, last_ys_bf16 = false;  // ... and may have left y / ys as bf16
 
   hipStream_t stream = nullptr;
   // Host-buffer entry point, large batches: page-locked staging (two slots each way); the
@@ -471,7 +472,17 @@ struct BatchPlan {
   bool routed_mid;      // gate/up phase in the mid-batch form (token rows shared through LDS)
   bool pg_prefill;      // per-group int8 layer running the tiled kernels on its bf16 copy
   bool tall_tiles;      // row tiles of up to nine 32-row groups (bf16 pipelined kernels only)
+  bool duo_up, duo_down;  // tiled phase on the two-workgroups-per-compute-unit form (short K)
 };
+// Longest K (padded) for which a tiled bf16 phase takes the form with two workgroups per compute
+// unit (tuning knob ATENIA_MOE_DUO_MAX_K, read once; 0 switches the form off).
+int duo_max_k() {
+  static const int v = [] {
+    const char* e = getenv("ATENIA_MOE_DUO_MAX_K");
+    return e ? atoi(e) : 0;
+  }();
+  return v;
+}
 // Tiles of uneven height can be switched off (tuning knob ATENIA_MOE_TALL_TILES=0, read once).
 bool tall_tiles_enabled() {
   static const bool v = [] {
@@ -598,8 +609,17 @@ BatchPlan plan_batch(const AteniaMoeLayer* L, int T) {
                  L->f_kpad % 64 == 0 && (L->fs == 0 || L->fs_kpad % 64 == 0);
   // the routed experts on the bf16 pipelined kernel (K a multiple of 64, >= 128)
   const bool bf16_tiles = L->wdtype == ATENIA_MOE_WEIGHT_BF16 || p.pg_prefill;
-  p.tall_tiles = tall_tiles_enabled() && (p.up == kFamTiled || p.down == kFamTiled) && bf16_tiles &&
-                 L->d_kpad % 64 == 0 && L->d_kpad >= 128 && L->f_kpad % 64 == 0 && L->f_kpad >= 128;
+  const bool pipe_ok = bf16_tiles && L->d_kpad % 64 == 0 && L->d_kpad >= 128 && L->f_kpad % 64 == 0 &&
+                       L->f_kpad >= 128;
+  static const int duo_phases = [] {
+    const char* e = getenv("ATENIA_MOE_DUO_PHASES");
+    return e ? atoi(e) : 3;
+  }();
+  p.duo_up = pipe_ok && p.up == kFamTiled && L->d_kpad <= duo_max_k() && (duo_phases & 1);
+  p.duo_down = pipe_ok && p.down == kFamTiled && L->f_kpad <= duo_max_k() && (duo_phases & 2);
+  // (the two-workgroup form cuts 256-row tiles in two, so a batch that uses it keeps those)
+  p.tall_tiles = tall_tiles_enabled() && (p.up == kFamTiled || p.down == kFamTiled) && pipe_ok &&
+                 !p.duo_up && !p.duo_down;
   return p;
 }
 
@@ -607,6 +627,16 @@ BatchPlan plan_batch(const AteniaMoeLayer* L, int T) {
 // may split tail tiles over k; the streaming kernels write one buffer).
 int noalloc_y_parts(const AteniaMoeLayer* L, int T) {
   return plan_batch(L, T).down != kFamTiled || L->wdtype == ATENIA_MOE_WEIGHT_F32 ? 1 : kMaxYParts;
+}
+
+// Expert outputs of bf16 layers as bf16 between the tiled down launch and the combine (tuning
+// knob ATENIA_MOE_Y_BF16=0 keeps them f32; read once).
+bool y_bf16_enabled() {
+  static const bool on = [] {
+    const char* e = getenv("ATENIA_MOE_Y_BF16");
+    return !(e && atoi(e) == 0);
+  }();
+  return on;
 }
 
 bool side_stream_enabled() {
@@ -634,6 +664,65 @@ void shared_family(FfnArgs& fsd, int fam, int ffn_dtype) {
   const bool tiles_ok = tiled_supported(fsd.gate, ffn_dtype) && tiled_supported(fsd.down, ffn_dtype);
   fsd.use_mid = fam == kFamMid && mid_ok;
   fsd.use_tiled = (fam == kFamTiled || (fam == kFamMid && !mid_ok)) && tiles_ok;
+}
+
+// Everything run_forward decides about the expert kernels of a T-token batch, from the layer's
+// dimensions alone (no device state): the same function answers atenia_moe_hip_plan_batch.
+int family_name(int f) {
+  return f == kFamMid ? ATENIA_MOE_KERNELS_MID : f == kFamTiled ? ATENIA_MOE_KERNELS_TILED : ATENIA_MOE_KERNELS_STREAM;
+}
+struct ResolvedPlan {
+  BatchPlan plan;
+  int ffn_dtype;         // element type the expert kernels see (bf16 for a per-group layer's copy)
+  int fam_up, fam_down;  // routed experts, per phase (kFam*)
+  bool duo_up, duo_down; // tiled phase on the two-workgroup form
+  bool split_tail;       // tiled down launch may split the k range of tail tiles
+  bool y_bf16, ys_bf16;  // expert outputs left as bf16 for the combine (routed / shared)
+  int s_fam_up, s_fam_down;  // shared expert (-1: none)
+};
+// A per-group layer's bf16 copy has the dimensions of the int8 blocks and no group scales.
+WeightSet dims_of(const AteniaMoeLayer* L, const WeightSet& w, bool pg_prefill) {
+  WeightSet o = w;
+  if (pg_prefill) {
+    o.scale = nullptr;
+    o.group_blocks = 0;
+    o.n_kgroups = 0;
+  }
+  return o;
+}
+ResolvedPlan resolve_plan(const AteniaMoeLayer* L, int T) {
+  ResolvedPlan r{};
+  r.plan = plan_batch(L, T);
+  const bool pg = r.plan.pg_prefill;
+  r.ffn_dtype = pg ? ATENIA_MOE_WEIGHT_BF16 : L->wdtype;
+  const WeightSet gate = dims_of(L, L->gate, pg), down = dims_of(L, L->down, pg);
+  const bool tiles_ok = tiled_supported(gate, r.ffn_dtype) && tiled_supported(down, r.ffn_dtype);
+  r.fam_up = r.plan.up == kFamTiled && !tiles_ok ? kFamStream : r.plan.up;
+  r.fam_down = r.plan.down == kFamTiled && !tiles_ok ? kFamStream : r.plan.down;
+  r.duo_up = r.fam_up == kFamTiled && r.plan.duo_up;
+  r.duo_down = r.fam_down == kFamTiled && r.plan.duo_down;
+  r.split_tail = r.fam_down == kFamTiled && !r.duo_down && tiled_down_splits_tail(down, r.ffn_dtype);
+  // bf16 layers on the bf16 tiled kernels leave the expert outputs as bf16 for the combine (half
+  // the bytes written and read back; the bf16 rounding of h already sets this path's error).
+  auto pipe = [&](const WeightSet& w) {
+    return r.ffn_dtype == ATENIA_MOE_WEIGHT_BF16 && w.k_pad % 64 == 0 && w.k_pad >= 128 &&
+           w.n_rows % 8 == 0;  // (a lane of the bf16 epilogue stores 8 columns at once)
+  };
+  r.y_bf16 = y_bf16_enabled() && L->wdtype == ATENIA_MOE_WEIGHT_BF16 && r.fam_down == kFamTiled &&
+             pipe(down);
+  r.s_fam_up = r.s_fam_down = -1;
+  if (L->fs > 0 && L->wdtype != ATENIA_MOE_WEIGHT_F32) {
+    FfnArgs fsd{};
+    fsd.gate = dims_of(L, L->s_gate, pg);
+    fsd.up = dims_of(L, L->s_up, pg);
+    fsd.down = dims_of(L, L->s_down, pg);
+    shared_family(fsd, r.fam_up, r.ffn_dtype);
+    r.s_fam_up = fsd.use_mid ? kFamMid : fsd.use_tiled ? kFamTiled : kFamStream;
+    shared_family(fsd, r.fam_down, r.ffn_dtype);
+    r.s_fam_down = fsd.use_mid ? kFamMid : fsd.use_tiled ? kFamTiled : kFamStream;
+    r.ys_bf16 = r.y_bf16 && fsd.use_tiled && pipe(fsd.down);
+  }
+  return r;
 }
 
 // `view`: the workspace to run on (nullptr = the handle's own).  no_alloc: fail instead of
@@ -824,12 +913,13 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   // keeps in registers; below that the weights are streamed once (HBM-bound).
   // (each phase has its own family; a tiled phase whose widths the tiled kernels do not take
   // falls back to the register-resident streaming kernel)
-  const bool tiles_ok = tiled_supported(fa.gate, ffn_dtype) && tiled_supported(fa.down, ffn_dtype);
-  const int fam_up = plan.up == kFamTiled && !tiles_ok ? kFamStream : plan.up;
-  const int fam_down = plan.down == kFamTiled && !tiles_ok ? kFamStream : plan.down;
+  const ResolvedPlan rp = resolve_plan(L, T);
+  const int fam_up = rp.fam_up, fam_down = rp.fam_down;
   const bool tiled = fam_up == kFamTiled;  // gate/up phase
   fa.use_tiled = fam_up == kFamTiled;
   fa.use_mid = fam_up == kFamMid;
+  fa.use_duo = rp.duo_up;
+  fa.tall_tiles = plan.tall_tiles;
   fa.tile_group = V.tile_group;
   fa.tile_m0 = V.tile_m0;
   fa.n_tiles = V.shared_desc + 4;
@@ -837,16 +927,23 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   fa.tile_li = V.tile_li;
   fa.max_row_tiles = (int)(((size_t)T * L->k + kTileM - 1) / kTileM +
                            std::min<long long>(L->E, (long long)T * L->k));
-  const bool split_tail = fam_down == kFamTiled && tiled_down_splits_tail(fa.down, ffn_dtype);
+  const bool duo_down = rp.duo_down;
+  const bool split_tail = rp.split_tail;
   fa.y_parts = split_tail ? std::min(kMaxYParts, V.y_parts) : 1;
   fa.y_part_stride = (size_t)T * L->k * L->d;
   fa.part_flags = split_tail ? V.part_flags : nullptr;
   fa.n_cus = device_cu_count();
   L->last_split = split_tail;
+  fa.y_bf16 = rp.y_bf16;
+  L->last_y_bf16 = fa.y_bf16;
+  L->last_ys_bf16 = false;
 
   FfnArgs fsd{};
   if (L->fs > 0) {
     fsd = fa;
+    fsd.y_bf16 = 0;
+    fsd.use_duo = 0;
+    fsd.tall_tiles = 0;  // the shared expert's rows are cut into whole 256-row tiles
     fsd.sel = InlineSelect{};
     const int32_t* sd = V.shared_desc;
     fsd.g.offsets = sd;
@@ -926,7 +1023,12 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   // the down phase may take another family than gate/up did
   fa.use_tiled = fam_down == kFamTiled;
   fa.use_mid = fam_down == kFamMid;
-  if (L->fs > 0) shared_family(fsd, fam_down, ffn_dtype);
+  fa.use_duo = duo_down;
+  if (L->fs > 0) {
+    shared_family(fsd, fam_down, ffn_dtype);
+    fsd.y_bf16 = rp.ys_bf16;
+    L->last_ys_bf16 = fsd.y_bf16;
+  }
   const bool fuse_shared_down = L->fs > 0 && ffn_stream_fuses_shared(fa, fsd, true);
   // One token, whole pipeline requested: the down launch covers the routed experts and the
   // shared one and finishes the combine as well (one launch instead of two or three).
@@ -972,7 +1074,9 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   ca.part_flags = fa.part_flags;
   ca.flag_cols = (L->d + 255) / 256;
   ca.y_part_stride = fa.y_part_stride;
+  ca.y_bf16 = fa.y_bf16;
   ca.y_shared = L->fs > 0 ? V.ys : nullptr;
+  ca.ys_bf16 = L->fs > 0 && fsd.y_bf16;
   ca.sgate = gated ? V.sgate : nullptr;
   ca.residual = d_residual;
   ca.out = d_out;
@@ -1694,28 +1798,60 @@ int atenia_moe_hip_layer_last_expert_outputs(AteniaMoeLayer* L, float* y_host,
     return fail(ATENIA_MOE_ERR_SYNC, "device synchronisation failed");
   const size_t P = (size_t)L->last_T * L->k;
   const WsView& V = L->cur;
+  // one buffer of expert outputs as f32, whatever it is stored as
+  auto fetch = [&](float* dst, const float* src, size_t n, bool bf16) -> int {
+    if (!bf16) {
+      HIP_TRY(hipMemcpy(dst, src, n * 4, hipMemcpyDeviceToHost));
+      return ATENIA_MOE_OK;
+    }
+    std::vector<uint16_t> bits(n);
+    HIP_TRY(hipMemcpy(bits.data(), src, n * 2, hipMemcpyDeviceToHost));
+    for (size_t i = 0; i < n; ++i) {
+      const uint32_t u = (uint32_t)bits[i] << 16;
+      memcpy(dst + i, &u, 4);
+    }
+    return ATENIA_MOE_OK;
+  };
   if (y_host) {
-    HIP_TRY(hipMemcpy(y_host, V.y, P * L->d * 4, hipMemcpyDeviceToHost));
+    const size_t n = P * L->d;
+    const size_t part_bytes = n * (L->last_y_bf16 ? 2 : 4);  // between the partial buffers
+    int rc = fetch(y_host, V.y, n, L->last_y_bf16);
+    if (rc) return rc;
     if (L->last_split) {  // add the partial buffers the down phase wrote for split tail tiles
       const int fc = (L->d + 255) / 256;
       std::vector<uint8_t> flags(P * fc);
       HIP_TRY(hipMemcpy(flags.data(), V.part_flags, flags.size(), hipMemcpyDeviceToHost));
-      std::vector<float> part(P * L->d);
+      std::vector<float> part(n);
       for (int i = 1; i < kMaxYParts; ++i) {
         bool any = false;
         for (uint8_t f : flags) any = any || f > i;
         if (!any) break;
-        HIP_TRY(hipMemcpy(part.data(), (const float*)V.y + (size_t)i * P * L->d, P * L->d * 4,
-                          hipMemcpyDeviceToHost));
+        if ((rc = fetch(part.data(), (const float*)((const uint8_t*)V.y + (size_t)i * part_bytes), n,
+                        L->last_y_bf16)))
+          return rc;
         for (size_t pr = 0; pr < P; ++pr)
           for (int c = 0; c < L->d; ++c)
             if (flags[pr * fc + c / 256] > i) y_host[pr * L->d + c] += part[pr * L->d + c];
       }
     }
   }
-  if (y_shared_host && L->fs > 0)
-    HIP_TRY(hipMemcpy(y_shared_host, V.ys, (size_t)L->last_T * L->d * 4,
-                      hipMemcpyDeviceToHost));
+  if (y_shared_host && L->fs > 0) {
+    int rc = fetch(y_shared_host, V.ys, (size_t)L->last_T * L->d, L->last_ys_bf16);
+    if (rc) return rc;
+  }
+  return ATENIA_MOE_OK;
+}
+
+int atenia_moe_hip_layer_last_down_split(AteniaMoeLayer* L, uint8_t* parts_host) {
+  if (!valid_handle(L)) return fail(ATENIA_MOE_ERR_HANDLE, "invalid layer handle");
+  if (!parts_host) return fail(ATENIA_MOE_ERR_DIM, "null pointer");
+  std::lock_guard<std::mutex> lock(L->mu);
+  if (L->last_T <= 0) return fail(ATENIA_MOE_ERR_DIM, "no forward has run on this handle");
+  if (hipDeviceSynchronize() != hipSuccess)
+    return fail(ATENIA_MOE_ERR_SYNC, "device synchronisation failed");
+  const size_t n = (size_t)L->last_T * L->k * ((L->d + 255) / 256);
+  if (L->last_split) HIP_TRY(hipMemcpy(parts_host, L->cur.part_flags, n, hipMemcpyDeviceToHost));
+  else memset(parts_host, 1, n);
   return ATENIA_MOE_OK;
 }
 
@@ -1774,27 +1910,75 @@ int atenia_moe_hip_layer_expert_kernels(const AteniaMoeLayer* L, int64_t n_token
     family[1] = L->fs > 0 ? ATENIA_MOE_KERNELS_F32 : -1;
     return ATENIA_MOE_OK;
   }
-  // the same decisions run_forward takes for the gate/up phase
-  const BatchPlan plan = plan_batch(L, T);
-  const int dt = plan.pg_prefill ? ATENIA_MOE_WEIGHT_BF16 : L->wdtype;
-  const WeightSet& g = plan.pg_prefill ? L->gate_b : L->gate;
-  const WeightSet& dn = plan.pg_prefill ? L->down_b : L->down;
-  const bool tiles_ok = tiled_supported(g, dt) && tiled_supported(dn, dt);
-  const int fam = plan.up == kFamTiled && !tiles_ok ? kFamStream : plan.up;
-  auto name = [](int f) {
-    return f == kFamMid ? ATENIA_MOE_KERNELS_MID
-           : f == kFamTiled ? ATENIA_MOE_KERNELS_TILED : ATENIA_MOE_KERNELS_STREAM;
+  const ResolvedPlan r = resolve_plan(L, T);  // the decisions run_forward takes
+  family[0] = family_name(r.fam_up);
+  family[1] = L->fs > 0 ? family_name(r.s_fam_up) : -1;
+  return ATENIA_MOE_OK;
+}
+
+int atenia_moe_hip_plan_batch(int num_experts, int top_k, int d_model, int d_ff, int d_ff_shared,
+                              int weight_dtype, int group_size, int64_t n_tokens,
+                              int32_t plan[8]) {
+  if (!plan) return fail(ATENIA_MOE_ERR_DIM, "null pointer");
+  if (num_experts < 1 || d_model < 1 || d_ff < 1 || d_ff_shared < 0)
+    return fail(ATENIA_MOE_ERR_DIM, "bad dimensions E=%d d=%d f=%d f_s=%d", num_experts, d_model,
+                d_ff, d_ff_shared);
+  if (top_k < 1 || top_k > num_experts)
+    return fail(ATENIA_MOE_ERR_K, "bad k=%d for %d experts", top_k, num_experts);
+  if (weight_dtype < 0 || weight_dtype > ATENIA_MOE_WEIGHT_INT8_PER_GROUP)
+    return fail(ATENIA_MOE_ERR_DIM, "unknown weight dtype %d", weight_dtype);
+  const bool per_group = weight_dtype == ATENIA_MOE_WEIGHT_INT8_PER_GROUP;
+  if (per_group && (group_size <= 0 || group_size % kKbInt8 != 0))
+    return fail(ATENIA_MOE_ERR_DIM, "per-group int8 needs group_size > 0 and a multiple of %d (got %d)",
+                kKbInt8, group_size);
+  if (n_tokens <= 0 || n_tokens > INT32_MAX) return fail(ATENIA_MOE_ERR_DIM, "n_tokens = %lld", (long long)n_tokens);
+  // a layer of these dimensions, as `create` fills them in (no device memory behind it)
+  AteniaMoeLayer L;
+  L.E = num_experts;
+  L.k = top_k;
+  L.d = d_model;
+  L.f = d_ff;
+  L.fs = d_ff_shared;
+  L.wdtype = per_group ? ATENIA_MOE_WEIGHT_INT8_W8A16 : weight_dtype;
+  L.group_size = per_group ? group_size : 0;
+  const bool f32w = L.wdtype == ATENIA_MOE_WEIGHT_F32;
+  const int KB = f32w ? 1 : kb_of(L.wdtype);
+  L.d_kpad = round_up(L.d, KB);
+  L.f_kpad = round_up(L.f, KB);
+  L.fs_kpad = round_up(L.fs, KB);
+  auto dims = [&](WeightSet& w, int n_rows, int k_cols) {
+    w.n_rows = n_rows;
+    w.k_cols = k_cols;
+    w.n_pad = f32w ? n_rows : round_up(n_rows, 16);
+    w.k_pad = f32w ? k_cols : round_up(k_cols, KB);
+    if (per_group) {
+      w.group_blocks = group_size / kKbInt8;
+      w.n_kgroups = (k_cols + group_size - 1) / group_size;
+    }
   };
-  family[0] = name(fam);
-  family[1] = -1;
-  if (L->fs > 0) {
-    FfnArgs fsd{};
-    fsd.gate = plan.pg_prefill ? L->s_gate_b : L->s_gate;
-    fsd.up = plan.pg_prefill ? L->s_up_b : L->s_up;
-    fsd.down = plan.pg_prefill ? L->s_down_b : L->s_down;
-    shared_family(fsd, fam, dt);
-    family[1] = name(fsd.use_mid ? kFamMid : fsd.use_tiled ? kFamTiled : kFamStream);
+  dims(L.gate, L.f, L.d);
+  dims(L.up, L.f, L.d);
+  dims(L.down, L.d, L.f);
+  if (L.fs > 0) {
+    dims(L.s_gate, L.fs, L.d);
+    dims(L.s_up, L.fs, L.d);
+    dims(L.s_down, L.d, L.fs);
   }
+  for (int i = 0; i < 8; ++i) plan[i] = 0;
+  if (f32w) {
+    plan[0] = plan[1] = ATENIA_MOE_KERNELS_F32;
+    plan[2] = plan[3] = L.fs > 0 ? ATENIA_MOE_KERNELS_F32 : -1;
+    return ATENIA_MOE_OK;
+  }
+  const ResolvedPlan r = resolve_plan(&L, (int)n_tokens);
+  plan[0] = family_name(r.fam_up);
+  plan[1] = family_name(r.fam_down);
+  plan[2] = L.fs > 0 ? family_name(r.s_fam_up) : -1;
+  plan[3] = L.fs > 0 ? family_name(r.s_fam_down) : -1;
+  plan[4] = r.y_bf16;
+  plan[5] = r.ys_bf16;
+  plan[6] = r.plan.tall_tiles;
+  plan[7] = (r.duo_up ? 1 : 0) | (r.duo_down ? 2 : 0);
   return ATENIA_MOE_OK;
 }
 

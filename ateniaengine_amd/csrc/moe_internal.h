@@ -144,6 +144,10 @@ struct FfnArgs {
   WeightSet down;
   float* y;            // f32 [rows, y_stride] indexed by PAIR id (token*pair_div+slot)
   int y_stride;
+  // bf16 pipelined / two-workgroup tiled down kernels only: y (and its partial buffers) holds
+  // bf16 values, rounded to nearest even, in the first half of the same allocation -- half the
+  // bytes written here and read back by the combine.  Element strides stay as they are.
+  int y_bf16;
   // Tiled down phase only: the tiles of a partly filled last round may be cut into up to
   // y_parts k ranges, range i writing its partial sums to y + i * y_part_stride; part_flags
   // [pairs, ceil(d / 256)] receives the number of buffers written per (pair, column tile) and
@@ -157,6 +161,12 @@ struct FfnArgs {
   int use_mid;
   // tiled kernels only
   int use_tiled;
+  // Tiled bf16 kernels: the form that runs two workgroups per compute unit (128-row slices of
+  // the 256-row tiles; for short K).  Needs tiles of at most 256 rows: tile_rows / tile_li null.
+  int use_duo;
+  // The row-tile list holds tiles of up to nine 32-row groups (PermuteArgs::max_tile_groups == 9);
+  // only the bf16 pipelined kernel reads such a list.
+  int tall_tiles;
   const int32_t* tile_group;
   const int32_t* tile_m0;
   const int32_t* n_tiles;
@@ -201,7 +211,9 @@ struct CombineArgs {
   const uint8_t* part_flags;
   int flag_cols;
   size_t y_part_stride;  // elements
+  int y_bf16;            // y and its partial buffers hold bf16 (see FfnArgs::y_bf16)
   const float* y_shared; // [T, y_stride] or null
+  int ys_bf16;           // the same for y_shared
   const float* sgate;    // [T] or null (scale 1)
   const float* residual; // [T, d] or null: out = residual + combine (one more f32 add); may be `out`
   float* out;            // [T, d]

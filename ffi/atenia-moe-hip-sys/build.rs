@@ -15,6 +15,7 @@ const SOURCES: &[&str] = &[
     "permute.hip",
     "ffn_stream.hip",
     "ffn_tiled.hip",
+    "ffn_tiled_duo.hip",
     "ffn_f32.hip",
     "combine.hip",
     "norm.hip",

@@ -216,6 +216,10 @@ unsafe extern "C" {
         y_host: *mut f32,
         y_shared_host: *mut f32,
     ) -> c_int;
+    pub fn atenia_moe_hip_layer_last_down_split(
+        layer: *mut AteniaMoeLayer,
+        parts_host: *mut u8,
+    ) -> c_int;
     pub fn atenia_moe_hip_layer_last_normed(layer: *mut AteniaMoeLayer, h2_host: *mut f32) -> c_int;
     pub fn atenia_moe_hip_layer_set_profiling(layer: *mut AteniaMoeLayer, enabled: c_int) -> c_int;
     pub fn atenia_moe_hip_layer_stage_ms(layer: *mut AteniaMoeLayer, ms: *mut f32) -> c_int;
@@ -229,6 +233,17 @@ unsafe extern "C" {
         layer: *const AteniaMoeLayer,
         n_tokens: i64,
         family: *mut i32,
+    ) -> c_int;
+    pub fn atenia_moe_hip_plan_batch(
+        num_experts: c_int,
+        top_k: c_int,
+        d_model: c_int,
+        d_ff: c_int,
+        d_ff_shared: c_int,
+        weight_dtype: c_int,
+        group_size: c_int,
+        n_tokens: i64,
+        plan: *mut i32,
     ) -> c_int;
     pub fn atenia_moe_quantize_per_row_i8(
         w: *const f32,
@@ -528,6 +543,15 @@ pub unsafe fn atenia_moe_hip_layer_last_expert_outputs(
 
 #[cfg(not(atenia_hip))]
 #[allow(unused_variables, clippy::missing_safety_doc)]
+pub unsafe fn atenia_moe_hip_layer_last_down_split(
+    layer: *mut AteniaMoeLayer,
+    parts_host: *mut u8,
+) -> c_int {
+    unreachable!("HIP symbol atenia_moe_hip_layer_last_down_split called in a build without atenia_hip")
+}
+
+#[cfg(not(atenia_hip))]
+#[allow(unused_variables, clippy::missing_safety_doc)]
 pub unsafe fn atenia_moe_hip_layer_last_normed(
     layer: *mut AteniaMoeLayer,
     h2_host: *mut f32,
@@ -582,6 +606,22 @@ pub unsafe fn atenia_moe_hip_layer_expert_kernels(
     family: *mut i32,
 ) -> c_int {
     unreachable!("HIP symbol atenia_moe_hip_layer_expert_kernels called in a build without atenia_hip")
+}
+
+#[cfg(not(atenia_hip))]
+#[allow(unused_variables, clippy::missing_safety_doc, clippy::too_many_arguments)]
+pub unsafe fn atenia_moe_hip_plan_batch(
+    num_experts: c_int,
+    top_k: c_int,
+    d_model: c_int,
+    d_ff: c_int,
+    d_ff_shared: c_int,
+    weight_dtype: c_int,
+    group_size: c_int,
+    n_tokens: i64,
+    plan: *mut i32,
+) -> c_int {
+    unreachable!("HIP symbol atenia_moe_hip_plan_batch called in a build without atenia_hip")
 }
 
 #[cfg(not(atenia_hip))]

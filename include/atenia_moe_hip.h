@@ -289,6 +289,15 @@ int atenia_moe_hip_layer_last_routing(AteniaMoeLayer* layer, int32_t* idx_host, 
 int atenia_moe_hip_layer_last_expert_outputs(AteniaMoeLayer* layer, float* y_host,
                                              float* y_shared_host);
 
+/* Parity tap next to the one above: into how many k ranges the last forward's down launch cut the
+ * tile behind each expert-output row and 256-column block, parts_host[n_tokens * top_k,
+ * ceil(d_model / 256)] (1 everywhere unless the matrix-core down launch split the tiles of its
+ * last, partly filled round; range i of S covers the 64-k stages [n*i/S, n*(i+1)/S) of the n =
+ * ceil(d_ff / 64) stages).  An expert output there is the sum, in range order, of its partial
+ * sums -- each rounded to bf16 first when the outputs travel as bf16 (atenia_moe_hip_plan_batch).
+ * No counterpart in the reference; tests use it to restate the kernels' arithmetic exactly. */
+int atenia_moe_hip_layer_last_down_split(AteniaMoeLayer* layer, uint8_t* parts_host);
+
 /* The rows the MoE layer saw in the most recent block forward: RMSNorm(x1) * gamma, [T, d] f32,
  * host buffer (the `h2` of src/moe/full_forward.rs:243). */
 int atenia_moe_hip_layer_last_normed(AteniaMoeLayer* layer, float* h2_host);
@@ -334,6 +343,19 @@ int atenia_moe_hip_layer_info(const AteniaMoeLayer* layer, int64_t info[8]);
 #define ATENIA_MOE_KERNELS_F32 3    /* f32 weights, f64 or f32 accumulation */
 int atenia_moe_hip_layer_expert_kernels(const AteniaMoeLayer* layer, int64_t n_tokens,
                                         int32_t family[2]);
+
+/* The same question without a layer or a device: which kernels a batch of `n_tokens` tokens takes
+ * on a layer of these dimensions (weight_dtype / group_size as in AteniaMoeLayerDesc).  A pure
+ * function of its arguments and of the tuning knobs in the environment.  plan[0] / plan[1]:
+ * family of the routed experts' gate/up and down phase (ATENIA_MOE_KERNELS_*); plan[2] / plan[3]:
+ * the same for the shared expert (-1 without one); plan[4] / plan[5]: 1 when the routed / shared
+ * expert outputs travel to the combine as bf16 instead of f32 (bf16 layers on the matrix-core
+ * kernels); plan[6]: 1 when row tiles may hold nine 32-row groups; plan[7]: bit 0 / bit 1 set when
+ * the gate/up / down phase takes the tiled form with two workgroups per compute unit.  No
+ * counterpart in the reference; hosts and tests use it to see where a batch size falls. */
+int atenia_moe_hip_plan_batch(int num_experts, int top_k, int d_model, int d_ff, int d_ff_shared,
+                              int weight_dtype, int group_size, int64_t n_tokens,
+                              int32_t plan[8]);
 
 /* Host-side weight preparation (load time, no GPU involved) ------------------------------ */
 

@@ -99,13 +99,31 @@ def bf16_rne(a):
 FLIP_WINDOW = 2.0 ** -18  # relative distance from a bf16 rounding midpoint that counts as fragile
 
 
-def emulate_bf16_kernels(oL, x, idx, w, with_slack=False):
+def _fragile_ulp(v, moved_by=0.0):
+    """Per element: one bf16 ulp of v where v (an f32 array) lies within FLIP_WINDOW (relative) plus
+    `moved_by` (absolute, per element) of the midpoint between two bf16 values -- there two
+    computations of v that differ by that much may round to different bf16 neighbours -- and 0
+    elsewhere."""
+    low = (v.view(np.uint32) & 0xFFFF).astype(np.float64)          # position between two bf16 values
+    expo = np.floor(np.log2(np.maximum(np.abs(v).astype(np.float64), 2.0 ** -126)))
+    window = FLIP_WINDOW * 2.0 ** 23 + np.asarray(moved_by, dtype=np.float64) / 2.0 ** (expo - 23)
+    fragile = np.abs(low - 0x8000) <= window
+    return np.where(fragile, 2.0 ** (expo - 7), 0.0)
+
+
+def emulate_bf16_kernels(oL, x, idx, w, with_slack=False, y_bf16=False, ys_bf16=False, split=None):
     """NumPy model of the bf16/int8 HIP path's arithmetic on the oracle layer's stored
     weights: exact products with wide accumulation, gate/up rounded to f32, h = silu(g)*u in
     f32 rounded to bf16 (nearest even), f32 combine with separate multiply and add.  The GPU
     result must sit within ~1e-3 of this model (difference: f32 accumulation order); the
     distance of either from the all-f64 reference is the bf16 rounding of h, ~2e-3 at real
     layer sizes.
+
+    `y_bf16` / `ys_bf16`: the routed / shared expert outputs travel to the combine as bf16 (what
+    `capi.plan_batch` reports for the batch): every expert output is rounded to bf16 (nearest even)
+    before it is weighted.  `split` ([T, k, ceil(d / 256)], `Layer.last_down_split`): where the
+    down launch cut a tile into S ranges of its 64-k stages, the output of that 256-column block is
+    the f32 sum, in range order, of S partial sums, each rounded on its own.
 
     One more difference cannot be bounded by a relative figure: where silu(g)*u lies within a
     few f32 ulps of the midpoint between two bf16 values, the kernel (hardware exp2 / rcp, another
@@ -115,12 +133,14 @@ def emulate_bf16_kernels(oL, x, idx, w, with_slack=False):
     differ there by 1.954e-3 of the token's largest output, the same figure the kernel showed.
     `with_slack` also returns, per token, the largest output change that flips of the fragile h
     elements (within FLIP_WINDOW of a midpoint, about 0.2 % of all) can cause:
-    sum over slots w * sum over fragile j max_n |W_d[n, j]| * ulp_bf16(h_j)."""
+    sum over slots w * sum over fragile j max_n |W_d[n, j]| * ulp_bf16(h_j); and, for outputs that
+    travel as bf16, of the fragile expert outputs themselves: max over n of the sum over slots of
+    w * ulp_bf16(y[n]) (y, or the partial sum of a split block, near a rounding midpoint)."""
     T, d = x.shape
     out = np.zeros((T, d), dtype=np.float32)
     slack = np.zeros(T, dtype=np.float64)
 
-    def expert(g, u, dn, xv):
+    def expert(g, u, dn, xv, round_y, parts):
         gg = (g.astype(np.float64) @ xv).astype(np.float32)
         uu = (u.astype(np.float64) @ xv).astype(np.float32)
         hv = (gg / (np.float32(1) + np.exp(-gg, dtype=np.float32))) * uu
@@ -128,23 +148,53 @@ def emulate_bf16_kernels(oL, x, idx, w, with_slack=False):
         low = (hv.view(np.uint32) & 0xFFFF).astype(np.int64)   # position between two bf16 values
         fragile = np.abs(low - 0x8000) <= FLIP_WINDOW * 2.0 ** 23
         bump = 0.0
+        h_ulp = np.zeros(hv.shape, dtype=np.float64)  # what a flip moves each fragile h by
         if fragile.any():
             ulp = 2.0 ** (np.floor(np.log2(np.abs(hv[fragile]).astype(np.float64))) - 7)
+            h_ulp[fragile] = ulp
             bump = float((np.abs(dn[:, fragile]).max(axis=0) * ulp).sum())
-        return (dn.astype(np.float64) @ h.astype(np.float64)).astype(np.float32), bump
+        h64 = h.astype(np.float64)
+        if not round_y:
+            return (dn.astype(np.float64) @ h64).astype(np.float32), bump, None
+        # bf16 outputs: per 256-column block, S partial sums over ranges of 64-k stages
+        f = h.shape[0]
+        nst = (f + 63) // 64
+        y = np.zeros(d, dtype=np.float32)
+        y_ulp = np.zeros(d, dtype=np.float64)
+        parts = np.ones((d + 255) // 256, dtype=np.int64) if parts is None else parts
+        for S_ in np.unique(parts):
+            cols = np.repeat(parts == S_, 256)[:d]
+            acc = np.zeros(int(cols.sum()), dtype=np.float32)
+            for i in range(int(S_)):
+                lo, hi = 64 * (nst * i // int(S_)), min(f, 64 * (nst * (i + 1) // int(S_)))
+                part = (dn[cols, lo:hi].astype(np.float64) @ h64[lo:hi]).astype(np.float32)
+                # (a flip of a fragile h moves the sum a little, which can carry it across a
+                # rounding midpoint of its own)
+                moved = np.abs(dn[cols, lo:hi]).astype(np.float64) @ h_ulp[lo:hi]
+                y_ulp[cols] += _fragile_ulp(part, moved)
+                acc = acc + bf16_rne(part)
+            y[cols] = acc
+        return y, bump, y_ulp
 
     for t in range(T):
         xv = x[t].astype(np.float64)
+        y_allow = np.zeros(d, dtype=np.float64)
         for s_, e in enumerate(idx[t]):
-            y, bump = expert(oL.w_gate[e], oL.w_up[e], oL.w_down[e], xv)
+            y, bump, y_ulp = expert(oL.w_gate[e], oL.w_up[e], oL.w_down[e], xv, y_bf16,
+                                    None if split is None else split[t, s_].astype(np.int64))
             out[t] = out[t] + w[t, s_] * y
             slack[t] += abs(float(w[t, s_])) * bump
+            if y_ulp is not None:
+                y_allow += abs(float(w[t, s_])) * y_ulp
         if oL.f_s:
             sc = np.float32(1.0)
             if oL.convention == 1 and oL.shared_gate is not None:
                 acc = float(oL.shared_gate.astype(np.float64) @ xv)
                 sc = np.float32(1.0 / (1.0 + np.exp(-acc)))
-            y, bump = expert(oL.s_gate, oL.s_up, oL.s_down, xv)
+            y, bump, y_ulp = expert(oL.s_gate, oL.s_up, oL.s_down, xv, ys_bf16, None)
             out[t] = out[t] + sc * y
             slack[t] += float(sc) * bump
+            if y_ulp is not None:
+                y_allow += float(sc) * y_ulp
+        slack[t] += float(y_allow.max())
     return (out, slack) if with_slack else out

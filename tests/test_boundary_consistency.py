@@ -20,7 +20,7 @@ C_TO_RUST = {
     "int": "c_int", "float": "f32", "double": "f64", "size_t": "usize", "int64_t": "i64",
     "const char*": "*const c_char", "const float*": "*const f32", "float*": "*mut f32",
     "const void*": "*const c_void", "void*": "*mut c_void", "int32_t*": "*mut i32",
-    "const int32_t*": "*const i32", "int8_t*": "*mut i8", "uint16_t*": "*mut u16",
+    "const int32_t*": "*const i32", "int8_t*": "*mut i8", "uint8_t*": "*mut u8", "uint16_t*": "*mut u16",
     "int64_t*": "*mut i64", "AteniaMoeLayer*": "*mut AteniaMoeLayer",
     "const AteniaMoeLayer*": "*const AteniaMoeLayer",
     "AteniaMoeLayer**": "*mut *mut AteniaMoeLayer",
@@ -72,7 +72,7 @@ def rust_bindings():
 
 def test_header_prototypes_parse():
     protos = header_prototypes()
-    assert len(protos) == 36
+    assert len(protos) == 38
     assert protos["atenia_moe_hip_layer_forward"] == (
         "c_int", ["*mut AteniaMoeLayer", "*const f32", "c_int", "*mut f32"])
 

@@ -308,7 +308,11 @@ def check_layer(ora, oL, gL, x, tol, sample=None, model=True):
     assert worst <= tol, f"layer output off by {worst:.3e} (bar {tol})"
     if model and gL.weight_dtype != capi.WEIGHT_F32:
         rows = np.array(list(rows))
-        em, slack = S.emulate_bf16_kernels(oL, x[rows], o_idx[rows], o_w[rows], with_slack=True)
+        plan = gL.plan(T)  # bf16 layers on the tiled kernels hand bf16 expert outputs to the combine
+        split = gL.last_down_split(T)[rows] if plan["y_bf16"] else None
+        em, slack = S.emulate_bf16_kernels(oL, x[rows], o_idx[rows], o_w[rows], with_slack=True,
+                                           y_bf16=bool(plan["y_bf16"]), ys_bf16=bool(plan["ys_bf16"]),
+                                           split=split)
         # per token: TOL_MODEL of its largest output, plus what a bf16 rounding flip of its
         # fragile h elements can move (zero for all but a few tokens; see synth.py)
         for i, t in enumerate(rows):
