@@ -701,7 +701,11 @@ __global__ __launch_bounds__(64 * NWV, 8 / NWV) void ffn_mid_kernel(StreamParams
   // Workgroups walk K from different first stages (and wrap around): launched together and
   // paced by the same memory system, they would otherwise all read the same offset of their
   // 2^n-byte-spaced strips at the same time, i.e. the same few memory channels.
-  const int rot = p.mid_rot ? (int)((blockIdx.x * 13u + blockIdx.y * 29u + blockIdx.z * 7u) % (unsigned)ns) : 0;
+  // The first stage depends on the strip block and the expert only, not on where the expert sits
+  // in the list of active ones or on the row block: the f32 sum of a (token, expert) pair is then
+  // added up in the same order whatever else the batch holds (and the row blocks of an expert
+  // walk K together, which lets the later ones find the weights in L2).
+  const int rot = p.mid_rot ? (int)((blockIdx.x * 13u + (sh ? 5u : (unsigned)e * 29u)) % (unsigned)ns) : 0;
   auto stage_of = [&](int st) {
     const int sc = min(st, ns - 1) + rot;
     return sc >= ns ? sc - ns : sc;

@@ -36,7 +36,8 @@ constexpr int kDuoNA = 2;       // A stages of 64 k
 constexpr int kDuoNB = 3;       // B stages of 32 k
 constexpr int kDuoStage = 1024; // uint4 per stage (A and B alike): 16 KiB
 
-template <bool UP>
+// YB (down phase only): y leaves as bf16 (TiledParams::out_bf16), staged through LDS.
+template <bool UP, bool YB = false>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void ffn_tiled_duo_kernel(TiledParams p) {
   constexpr int NA = kDuoNA, NB = kDuoNB;
@@ -272,6 +273,45 @@ void ffn_tiled_duo_kernel(TiledParams p) {
       if (mrow < rows_here && n < p.n_blocks * 16)
         *(uint4*)(h + (size_t)(base + tm0 + mrow) * p.out_stride + n) = v;
     }
+  } else if (YB) {
+    // y as bf16, staged through LDS like h above: the wave's 64 x 128 block goes to its own region
+    // with a row pitch of 272 bytes and is read back 16 lanes per row, 4 rows at a time, so that
+    // a row's 256 bytes leave as two full lines.
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    constexpr int kPitch = 272;
+    char* stage = (char*)S + wave * (64 * kPitch);
+    const int r4 = lane >> 4, c16 = lane & 15;
+    int pair_of[16];  // pair id of the rows this lane stores
+#pragma unroll
+    for (int it = 0; it < 16; ++it) {
+      const int m = wm * 64 + it * 4 + r4;
+      pair_of[it] = p.g.perm[base + tm0 + min(m, rows_here - 1)];
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {  // rows m and m + 1
+          const int m = i * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
+          const uint32_t hh = bf16_rne_pair(acc[i][j][r], acc[i][j][r + 1]);
+          char* dst = stage + m * kPitch + (j * 32 + l32) * 2;
+          *(uint16_t*)dst = (uint16_t)hh;
+          *(uint16_t*)(dst + kPitch) = (uint16_t)(hh >> 16);
+        }
+      }
+    }
+    uint16_t* yb = (uint16_t*)p.out;
+    const int n = nb0 * 16 + wn * 128 + c16 * 8;
+#pragma unroll
+    for (int it = 0; it < 16; ++it) {
+      const int m = it * 4 + r4;
+      const uint4 v = *(const uint4*)(stage + m * kPitch + c16 * 16);
+      if (wm * 64 + m < rows_here && n < p.n_rows)
+        *(uint4*)(yb + (size_t)pair_of[it] * p.out_stride + n) = v;
+    }
   } else {
     float* y = (float*)p.out;
     // The pair id of every row first, in one batch of loads (fetched next to the stores they
@@ -290,15 +330,6 @@ void ffn_tiled_duo_kernel(TiledParams p) {
       for (int r = 0; r < 16; ++r) {
         const int m = wm * 64 + i * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
         if (m >= rows_here) continue;
-        if (p.out_bf16) {
-          uint16_t* ybr = (uint16_t*)p.out + (size_t)pair_of[i][r] * p.out_stride;
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const int n = nb0 * 16 + (4 * wn + j) * 32 + l32;
-            if (n < p.n_rows) ybr[n] = (uint16_t)bf16_rne_pair(acc[i][j][r], 0.f);
-          }
-          continue;
-        }
         float* yr = y + (size_t)pair_of[i][r] * p.out_stride;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -327,7 +358,12 @@ hipError_t launch_duo(TiledParams p, int max_row_tiles, hipStream_t s) {
   p.stagger = p.n_cus > 0 ? (p.k_pad / 32) * duo_stagger_eighths() / 8 : 0;
   int n_wg = max_row_tiles * kDuoSub * p.n_col_tiles;
   n_wg = (n_wg + 7) / 8 * 8;
-  ffn_tiled_duo_kernel<UP><<<n_wg, kThreads, 0, s>>>(p);
+  if (!UP && p.out_bf16) {
+    if (p.n_rows % 8) return hipErrorInvalidValue;  // a lane stores 8 columns at once
+    ffn_tiled_duo_kernel<false, true><<<n_wg, kThreads, 0, s>>>(p);
+  } else {
+    ffn_tiled_duo_kernel<UP><<<n_wg, kThreads, 0, s>>>(p);
+  }
   return hipGetLastError();
 }
 

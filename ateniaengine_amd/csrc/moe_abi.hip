@@ -180,6 +180,7 @@ struct AteniaMoeLayer {
   hipEvent_t ev_fork = nullptr, ev_join = nullptr;
   hipStream_t done_stream = nullptr;
   bool done_valid = false;
+  bool done_recorded = false;  // `done` marks the end of the last forward on done_stream
 
   bool profiling = false;
   int policy = ATENIA_MOE_POLICY_CERTIFIED;  // expert arithmetic of f32 layers
@@ -584,24 +585,50 @@ MidBounds mid_bounds(const AteniaMoeLayer* L) {
   if (env_max_tokens > 0) b.max_tokens = env_max_tokens;
   return b;
 }
-BatchPlan plan_batch(const AteniaMoeLayer* L, int T) {
+// The measured cross-overs as they stand: family of each phase at batch size T.
+void rule_families(const AteniaMoeLayer* L, int T, int& up, int& down) {
   const bool int8w = L->wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
-  BatchPlan p;
   const bool base_streams = batch_streams(T, (long long)T * L->k, L->E, int8w ? 32 : 16);
   const double avg = (double)T * L->k / L->E;
-  p.up = p.down = base_streams ? kFamStream : kFamTiled;
+  up = down = base_streams ? kFamStream : kFamTiled;
   if (stream_max_tokens_override() == 0 &&
       ffn_mid_supported(L->gate, L->wdtype) && ffn_mid_supported(L->up, L->wdtype) &&
       ffn_mid_supported(L->down, L->wdtype)) {
     const MidBounds b = mid_bounds(L);
-    if (T >= b.min_tokens && T <= b.max_tokens && avg >= b.lo && avg <= b.hi) p.up = kFamMid;
+    if (T >= b.min_tokens && T <= b.max_tokens && avg >= b.lo && avg <= b.hi) up = kFamMid;
     if (b.hi > 0.0 && T >= b.down_min_tokens && avg <= b.down_hi)
-      p.down = kFamMid;
-    else if (p.up == kFamMid && T < b.down_min_tokens)
-      p.down = kFamStream;  // narrow experts: the register-resident down launch holds out longer
+      down = kFamMid;
+    else if (up == kFamMid && T < b.down_min_tokens)
+      down = kFamStream;  // narrow experts: the register-resident down launch holds out longer
     // a per-group layer runs the tiled kernels on a bf16 copy: both phases or neither
-    if (L->group_size > 0 && (p.up == kFamTiled) != (p.down == kFamTiled))
-      p.up = p.down = kFamTiled;
+    if (L->group_size > 0 && (up == kFamTiled) != (down == kFamTiled)) up = down = kFamTiled;
+  }
+}
+// The bounds above are fitted to the shapes that were measured; on other shapes they can cross
+// (few experts: the rows per expert pass the mid-batch form's upper bound while the batch is
+// still small enough to stream; a wide shared expert: the down phase would enter the mid-batch
+// form after the tiled kernels have already taken it).  A phase never goes back to a
+// smaller-batch family as T grows: it takes the largest family the rule names at any batch size
+// up to T.  The rule only changes at its bounds, so those are the batch sizes to look at.
+BatchPlan plan_batch(const AteniaMoeLayer* L, int T) {
+  BatchPlan p;
+  rule_families(L, T, p.up, p.down);
+  {
+    const MidBounds b = mid_bounds(L);
+    const double per = (double)L->E / L->k;  // tokens per row-per-expert
+    const double marks[] = {(double)kStreamMaxTokens, 16.0 * per, 32.0 * per, (double)b.min_tokens,
+                            (double)b.max_tokens, b.lo * per, b.hi * per, (double)b.down_min_tokens,
+                            b.down_hi * per, (double)stream_max_tokens_override()};
+    for (double mk : marks)
+      for (int dt = -1; dt <= 1; ++dt) {
+        const double c = std::floor(mk) + dt;
+        if (c < 1.0 || c >= (double)T) continue;
+        int u, dn;
+        rule_families(L, (int)c, u, dn);
+        p.up = std::max(p.up, u);      // kFamStream < kFamMid < kFamTiled
+        p.down = std::max(p.down, dn);
+      }
+    if (L->group_size > 0 && (p.up == kFamTiled) != (p.down == kFamTiled)) p.up = p.down = kFamTiled;
   }
   p.routed_streams = p.up != kFamTiled;
   p.routed_mid = p.up == kFamMid;
@@ -727,9 +754,31 @@ ResolvedPlan resolve_plan(const AteniaMoeLayer* L, int T) {
 
 // `view`: the workspace to run on (nullptr = the handle's own).  no_alloc: fail instead of
 // allocating anything.
+int run_forward_impl(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d_out,
+                     hipStream_t s, int first, int last, const float* d_residual,
+                     const WsView* view, bool no_alloc);
+
+// A stream that this library did not make and that is not one of the runtime's own (null, legacy,
+// per-thread): its owner may destroy it between two calls on the handle.
+bool caller_owned_stream(const AteniaMoeLayer* L, hipStream_t s) {
+  return (uintptr_t)s > 15 && s != L->stream && s != L->side;
+}
+
 int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d_out,
                 hipStream_t s, int first, int last, const float* d_residual = nullptr,
                 const WsView* view = nullptr, bool no_alloc = false) {
+  const int rc = run_forward_impl(L, d_x, x_dtype, T, d_out, s, first, last, d_residual, view, no_alloc);
+  // (see the ordering note in run_forward_impl; nothing is recorded into a graph being captured)
+  if (L->done_valid && L->done_stream == s && caller_owned_stream(L, s) && !stream_is_capturing(s)) {
+    if (hipEventRecord(L->done, s) == hipSuccess) L->done_recorded = true;
+    else (void)hipGetLastError();
+  }
+  return rc;
+}
+
+int run_forward_impl(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d_out,
+                     hipStream_t s, int first, int last, const float* d_residual,
+                     const WsView* view, bool no_alloc) {
   for (int st = 0; st < first; ++st)
     if (L->stage_T[st] != T)
       return fail(ATENIA_MOE_ERR_DIM, "stage %d has not run for %d tokens on this handle", st, T);
@@ -742,14 +791,19 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
   const WsView V = view ? *view : L->ws;
   L->cur = V;
   // A forward still running on another stream uses the same workspace: wait for it.  Nothing
-  // is recorded while calls stay on one stream (an event per forward would cost a decode step
-  // several microseconds); when the stream changes, the previous stream is marked now -- the
-  // mark covers everything submitted to it so far -- and the new one waits for the mark.  A
-  // previous stream that no longer exists cannot be marked; the device is drained instead.
+  // is recorded while calls stay on the null stream or the handle's own stream (an event per
+  // forward would cost a decode step several microseconds): those cannot go away, so when the
+  // stream changes the previous one is marked then -- the mark covers everything submitted to it
+  // so far -- and the new one waits for the mark.  A stream the caller made may be gone by the
+  // next call (and its handle value reused), so it is never touched again: run_forward marks it
+  // at the end of each forward it submits there (`done_recorded`), and the next stream waits for
+  // that mark.
   const bool capturing = stream_is_capturing(s);
   if (!capturing) {
     if (L->done_valid && L->done_stream != s) {
-      if (hipEventRecord(L->done, L->done_stream) == hipSuccess) {
+      if (L->done_recorded) {
+        HIP_TRY(hipStreamWaitEvent(s, L->done, 0));
+      } else if (hipEventRecord(L->done, L->done_stream) == hipSuccess) {
         HIP_TRY(hipStreamWaitEvent(s, L->done, 0));
       } else {
         (void)hipGetLastError();
@@ -758,6 +812,7 @@ int run_forward(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, float* d
     }
     L->done_valid = true;
     L->done_stream = s;
+    L->done_recorded = false;
   }
   StageTimer tm{L, s};
   for (int i = 0; i < ATENIA_MOE_N_STAGES; ++i) L->launches[i] = 0;

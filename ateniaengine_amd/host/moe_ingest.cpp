@@ -248,16 +248,19 @@ MoeDetection detect_moe(const std::vector<std::string>& names) {
 }
 
 std::string unsupported_message(const MoeDetection& det) {
-  // Same counted fields as the reference's message (src/moe/detect.rs:249-265); the advice is
-  // this library's: such a checkpoint goes through assemble_real_moe_layer, not a dense loader.
+  // The sentence a dense loader fails with, worded as the reference words it
+  // (src/moe/detect.rs:251-264; its own tests look for "MoE checkpoint detected", "not implemented
+  // yet" and the counted fields, detect.rs:425-428, tests/moe_loader_failloud_test.rs:47), followed
+  // by this library's advice: such a checkpoint goes through assemble_real_moe_layer instead.
   const auto n = det.implied_expert_count();
-  return "MoE checkpoint detected (experts=" +
+  return "MoE checkpoint detected, but MoE execution is not implemented yet (experts=" +
          (n ? std::to_string(*n) : std::string("unknown")) +
          ", expert_tensors=" + std::to_string(det.expert_tensor_count) +
          ", router_tensors=" + std::to_string(det.router_tensor_count) +
          ", shared_expert_tensors=" + std::to_string(det.shared_expert_tensor_count) +
-         "): a dense loader would drop the expert weights; bind it with MoeWeightMap::from_tensors "
-         "and assemble_real_moe_layer.";
+         "). Atenia can load and run dense models only; loading this checkpoint as dense would "
+         "silently drop the expert weights and produce a broken model. On the MI355X path bind it "
+         "with MoeWeightMap::from_tensors and assemble_real_moe_layer instead.";
 }
 
 // ---- weight map -------------------------------------------------------------------------------

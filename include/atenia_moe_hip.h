@@ -33,7 +33,11 @@
  * forwards behind its registry mutex (src/moe/graph_op.rs:304-316).  The asynchronous entry
  * points keep that promise on the device as well: a call whose stream differs from the stream
  * of the handle's previous call first waits (hipStreamWaitEvent) for that call's kernels, so
- * two streams never use one workspace at the same time.  The one exception is a stream that is
+ * two streams never use one workspace at the same time.  A stream may be destroyed as soon as
+ * the call that took it has returned: the handle marks the end of each forward on a stream the
+ * caller made with an event of its own and never touches that stream again (the null stream and
+ * the handle's own streams are marked only when the next call changes the stream: one event per
+ * forward costs a decode step microseconds).  The one exception is a stream that is
  * being captured into a HIP graph: no cross-stream wait is recorded there, and replays of graphs
  * that hold calls on one handle must be ordered by the caller.  Different handles may run
  * concurrently.  A layer with a shared expert owns a second stream (default priority): in

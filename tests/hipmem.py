@@ -18,6 +18,15 @@ def hip():
     return _hip
 
 
+def mem_free() -> int:
+    """Free device memory in bytes as the runtime reports it (hipMemGetInfo)."""
+    free, total = C.c_size_t(), C.c_size_t()
+    rc = hip().hipDeviceSynchronize() or hip().hipMemGetInfo(C.byref(free), C.byref(total))
+    if rc:
+        raise RuntimeError(f"hipMemGetInfo failed: {rc}")
+    return free.value
+
+
 class DeviceArray:
     """A device allocation with a NumPy dtype/shape; `.ptr` is the raw device pointer."""
 

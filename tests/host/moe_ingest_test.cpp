@@ -295,6 +295,10 @@ int main(int argc, char** argv) {
     const std::string msg = unsupported_message(d1);
     CHECK(msg.find("experts=8, expert_tensors=24, router_tensors=1, shared_expert_tensors=2") != std::string::npos,
           "%s", msg.c_str());
+    // the phrases the reference's own tests look for (src/moe/detect.rs:425-428,
+    // tests/moe_loader_failloud_test.rs:47)
+    CHECK(msg.find("MoE checkpoint detected") != std::string::npos &&
+              msg.find("not implemented yet") != std::string::npos, "%s", msg.c_str());
     // A router alone does not make a checkpoint MoE; one shared-expert tensor does.
     CHECK(!detect_moe({"model.layers.0.mlp.gate.weight"}).is_moe, "router only");
     MoeDetection d2 = detect_moe({"model.layers.0.mlp.shared_expert.up_proj.weight"});

@@ -565,6 +565,33 @@ def test_packed_gate_up_layout(ora):
         assert a.forward(x).tobytes() == b.forward(x).tobytes()
 
 
+@pytest.mark.parametrize("wd", [capi.WEIGHT_BF16, capi.WEIGHT_INT8_W8A16])
+def test_mid_batch_rows_do_not_depend_on_the_rest_of_the_batch(ora, wd):
+    """The reference's CPU path is a function of the row (src/moe/graph_op.rs:340-349 walks the rows
+    one by one).  Inside one kernel family the same holds here bit for bit: a token forwarded in
+    two mid-batch batches of different size, order and expert activity gives the same output bits
+    (the kernel's walk over K starts at a stage that depends on the strip and the expert only)."""
+    E, k, d, f = 8, 2, 384, 640
+    W = S.make_weights(941, E, d, f, f_s=128, gated=True, router_std=0.3 / np.sqrt(d),
+                       outlier_frac=0.01 if wd != capi.WEIGHT_BF16 else 0.0)
+    oL, gL = S.build_pair(ora, W, k, capi.CONVENTION_HUGGINGFACE_QWEN, wd)
+    with gL:
+        pool = S.make_tokens(942, 260, d)
+        a = pool[:100]
+        b = np.concatenate([pool[180:250], pool[:100][::-1], pool[120:140]])  # 190 tokens
+        for x in (a, b):
+            plan = gL.plan(x.shape[0])
+            assert plan["up"] == plan["down"] == capi.KERNELS_MID, plan
+        out_a = gL.forward(a)
+        ya, ysa = gL.last_expert_outputs(a.shape[0])
+        out_b = gL.forward(b)
+        yb, ysb = gL.last_expert_outputs(b.shape[0])
+        back = out_b[70:170][::-1]  # the tokens of `a`, in a's order
+        assert ya.tobytes() == yb[70:170][::-1].tobytes(), "expert outputs depend on the batch"
+        assert ysa.tobytes() == ysb[70:170][::-1].tobytes(), "shared expert outputs depend on the batch"
+        assert out_a.tobytes() == np.ascontiguousarray(back).tobytes(), "layer outputs depend on the batch"
+
+
 @pytest.mark.parametrize("wd", [capi.WEIGHT_F32, capi.WEIGHT_BF16, capi.WEIGHT_INT8_W8A16])
 @pytest.mark.parametrize("T,shared", [(1, False), (1, True), (37, True), (700, False)])
 def test_combine_is_bit_exact_given_expert_outputs(ora, wd, T, shared):

@@ -10,7 +10,7 @@ import pytest
 
 from ateniaengine_amd import capi
 from tests import synth as S
-from tests.hipmem import DeviceArray, Graph, Stream
+from tests.hipmem import DeviceArray, Graph, Stream, mem_free
 
 pytestmark = pytest.mark.gpu
 
@@ -20,7 +20,7 @@ def _need_gpu():
     assert capi.available(), "no gfx950 device: the HIP path cannot run (there is no fallback)"
 
 
-def _run(gL, x, noalloc, act=capi.ACT_F32, stream=0):
+def _run(gL, x, noalloc, act=capi.ACT_F32, stream=0, watch_memory=False):
     T, d = x.shape
     if act == capi.ACT_BF16:
         dx = DeviceArray.from_host(capi.f32_to_bf16_trunc(x))
@@ -28,7 +28,11 @@ def _run(gL, x, noalloc, act=capi.ACT_F32, stream=0):
         dx = DeviceArray.from_host(x)
     out = DeviceArray((T, d), np.float32, fill=0xFF)
     fn = gL.forward_device_noalloc if noalloc else gL.forward_device
+    before = mem_free() if watch_memory else 0
     fn(dx.ptr, act, T, out.ptr, stream)
+    if watch_memory:  # the call must not have allocated (or freed) device memory
+        after = mem_free()
+        assert after == before, f"free device memory moved by {after - before} bytes across the call"
     assert gL.status(stream)[0] == 0
     return out.to_host()
 
@@ -40,6 +44,9 @@ CASES = [
     ("bf16_plain", 8, 2, 256, 512, 0, False, 0, capi.WEIGHT_BF16),
     ("f32", 8, 2, 128, 256, 0, False, 0, capi.WEIGHT_F32),
     ("many_experts_bf16", 40, 2, 128, 96, 64, True, 1, capi.WEIGHT_BF16),  # logits scratch (E > 31)
+    # per-group scales: streaming / mid-batch forms on the int8 blocks, the tiled kernels on the
+    # layer's bf16 copy (made by the allocating call that runs first for each batch size)
+    ("int8_per_group", 8, 2, 256, 512, 128, True, 1, capi.WEIGHT_INT8_PER_GROUP),
 ]
 
 
@@ -58,7 +65,9 @@ def test_noalloc_equals_forward_device_twice_second_smaller(ora, name, E, k, d, 
         for T in (37, 9, 1, 120, 300):
             x = S.make_tokens(1000 + T, T, d, bf16=bf16_rows)
             want = _run(gL, x, noalloc=False)
-            got = _run(gL, x, noalloc=True)
+            _run(gL, x, noalloc=True)  # warm: one-time kernel attributes, lazily made copies
+            # whatever batch sizes were seen before, the call itself allocates nothing
+            got = _run(gL, x, noalloc=True, watch_memory=True)
             assert got.tobytes() == want.tobytes(), f"{name} T={T}: no-alloc output differs"
             idx, w, counts, offsets, perm = gL.last_routing(T)  # taps read the static buffer
             o_idx, _ = oL.route_tokens(x)
@@ -87,14 +96,18 @@ def test_noalloc_rejects_what_does_not_fit(ora):
         assert _run(gL, x, True).tobytes() == _run(gL, x, False).tobytes()
 
 
-def test_noalloc_call_can_be_captured_and_replayed(ora):
+@pytest.mark.parametrize("T", [8, 120, 300])
+def test_noalloc_call_can_be_captured_and_replayed(ora, T):
     """The call only launches kernels (its workspace is initialised by a kernel, not a memset),
     so it can sit in a HIP graph: every replay, with eager work in between, equals the eager
-    result for the input then in the buffer."""
+    result for the input then in the buffer.  Batch sizes: the register-resident streaming
+    kernels, the mid-batch kernel, the tiled kernels (with the split tail of their down launch)."""
     W = S.make_weights(314, 8, 256, 512)
     _, gL = S.build_pair(ora, W, 2, 0, capi.WEIGHT_BF16)
     with gL:
-        T, d = 8, 256
+        d = 256
+        want_family = {8: capi.KERNELS_STREAM, 120: capi.KERNELS_MID, 300: capi.KERNELS_TILED}[T]
+        assert gL.expert_kernels(T)[0] == want_family
         s = Stream()
         dx = DeviceArray((T, d), np.float32, fill=0)
         out = DeviceArray((T, d), np.float32, fill=0)
