@@ -12,6 +12,8 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <atomic>
+#include <thread>
 #include <mutex>
 #include <new>
 #include <string>
@@ -1204,9 +1206,68 @@ int ensure_host_staging(AteniaMoeLayer* L) {
   return ATENIA_MOE_OK;
 }
 
+// The staging copies (pageable caller memory <-> page-locked slots) are what the calling thread
+// would otherwise spend most of the call on: one core moves about half of what the copy engine
+// does.  For the length of a staged call a few helper threads take a slice of every chunk each
+// (tuning knob ATENIA_MOE_HOST_COPY_THREADS, read once: threads in all, 1 = the caller alone).
+class CopyCrew {
+ public:
+  explicit CopyCrew(int helpers) {
+    for (int i = 0; i < helpers; ++i) th_.emplace_back([this, i] { run(i + 1); });
+  }
+  ~CopyCrew() {
+    quit_ = true;
+    gen_.fetch_add(1, std::memory_order_release);
+    for (auto& t : th_) t.join();
+  }
+  void copy(void* dst, const void* src, size_t bytes) {
+    dst_ = (char*)dst;
+    src_ = (const char*)src;
+    bytes_ = bytes;
+    done_.store(0, std::memory_order_relaxed);
+    gen_.fetch_add(1, std::memory_order_release);
+    slice(0);
+    while (done_.load(std::memory_order_acquire) < (int)th_.size()) std::this_thread::yield();
+  }
+
+ private:
+  void slice(int i) {
+    const size_t n = th_.size() + 1;
+    const size_t per = ((bytes_ + n - 1) / n + 4095) & ~(size_t)4095;
+    const size_t lo = std::min(bytes_, (size_t)i * per), hi = std::min(bytes_, lo + per);
+    if (hi > lo) memcpy(dst_ + lo, src_ + lo, hi - lo);
+  }
+  void run(int i) {
+    int seen = 0;
+    for (;;) {
+      int g;
+      while ((g = gen_.load(std::memory_order_acquire)) == seen) std::this_thread::yield();
+      seen = g;
+      if (quit_) return;
+      slice(i);
+      done_.fetch_add(1, std::memory_order_release);
+    }
+  }
+  std::vector<std::thread> th_;
+  std::atomic<int> gen_{0}, done_{0};
+  std::atomic<bool> quit_{false};
+  char* dst_ = nullptr;
+  const char* src_ = nullptr;
+  size_t bytes_ = 0;
+};
+int host_copy_threads() {
+  static const int v = [] {
+    const char* e = getenv("ATENIA_MOE_HOST_COPY_THREADS");
+    const int n = e ? atoi(e) : 4;
+    return std::max(1, std::min(n, 16));
+  }();
+  return v;
+}
+
 int forward_host_staged(AteniaMoeLayer* L, const float* x_host, int T, float* out_host) {
   int rc = ensure_host_staging(L);
   if (rc) return rc;
+  CopyCrew crew(host_copy_threads() - 1);
   const size_t row = (size_t)L->d * 4;
   const int n_chunks = (T + kHostChunkTokens - 1) / kHostChunkTokens;
   auto tokens_of = [&](int c) { return std::min(kHostChunkTokens, T - c * kHostChunkTokens); };
@@ -1215,7 +1276,7 @@ int forward_host_staged(AteniaMoeLayer* L, const float* x_host, int T, float* ou
     const size_t off = (size_t)c * kHostChunkTokens * row, bytes = (size_t)tokens_of(c) * row;
     // the slot is free once the copy of chunk c - 2 has left it
     if (c >= 2) HIP_TRY(hipEventSynchronize(L->ev_h2d[slot]));
-    memcpy((char*)L->pin_in + slot * L->pin_bytes, (const char*)x_host + off, bytes);
+    crew.copy((char*)L->pin_in + slot * L->pin_bytes, (const char*)x_host + off, bytes);
     HIP_TRY(hipMemcpyAsync((char*)L->x_in.p + off, (char*)L->pin_in + slot * L->pin_bytes, bytes,
                            hipMemcpyHostToDevice, L->stream));
     HIP_TRY(hipEventRecord(L->ev_h2d[slot], L->stream));
@@ -1226,8 +1287,8 @@ int forward_host_staged(AteniaMoeLayer* L, const float* x_host, int T, float* ou
   auto drain = [&](int c) -> int {  // chunk c's output: staging -> caller
     const int slot = c & 1;
     HIP_TRY(hipEventSynchronize(L->ev_d2h[slot]));
-    memcpy((char*)out_host + (size_t)c * kHostChunkTokens * row,
-           (char*)L->pin_out + slot * L->pin_bytes, (size_t)tokens_of(c) * row);
+    crew.copy((char*)out_host + (size_t)c * kHostChunkTokens * row,
+              (char*)L->pin_out + slot * L->pin_bytes, (size_t)tokens_of(c) * row);
     return ATENIA_MOE_OK;
   };
   for (int c = 0; c < n_chunks; ++c) {

@@ -41,6 +41,13 @@ CONFIGS = {
                       zipf=False, unit_logits=True, sweep=(1, 16, 64, 128, 256, 8192)),
     "deepseek_bf16": dict(d=2048, E=64, k=6, f=1408, fs=2816, gated=False, conv=1, wd="bf16",
                           zipf=True, sweep=(1, 16, 64, 128, 1024, 16384)),
+    # Two shapes of the reference's model families (src/moe/family.rs) outside the benchmark list,
+    # kept to see how the kernel plan's bounds carry over: Mixtral-8x22B, and a layer of 128
+    # narrow experts with top-8 routing.
+    "mixtral22b_bf16": dict(d=6144, E=8, k=2, f=16384, fs=0, gated=False, conv=0, wd="bf16",
+                            zipf=False, sweep=(1, 64, 512, 4096)),
+    "narrow128_bf16": dict(d=2048, E=128, k=8, f=768, fs=0, gated=False, conv=1, wd="bf16",
+                           zipf=False, unit_logits=True, sweep=(1, 64, 512, 4096)),
     # DeepSeek-V3 router shape (256 experts in 8 groups, top-8 of the 4 best groups) in front of
     # narrow experts: times the sigmoid / group-limited routing path, not a checkpoint shape.
     "v3route_bf16": dict(d=7168, E=256, k=8, f=256, fs=256, gated=False, conv=1, wd="bf16",
