@@ -843,9 +843,17 @@ int run_forward_impl(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, flo
   ra.xb = need_xb ? V.xb : nullptr;
   ra.d_pad = L->d_kpad;
   ra.status = L->status.as<int32_t>();
-  // f32-valued operands almost never satisfy the exactness test of the per-token kernel, so
-  // f32 layers always take the sequential-order kernel.
-  ra.token_kernel_max_tokens = f32w ? 0 : router_token_max();
+  // f32 layers: the sums of f32-valued products are not exact in every order, but the per-token
+  // kernel's interval certificate settles all but about one sum in a thousand (those rows are
+  // recomputed in the reference's order inside the kernel), so small batches take it as well
+  // (router stage, d = 1024, 8 rows, per-token kernel / one sequential chain per (token, row):
+  // T = 1 9.6 / 18.5 us, 16 13.5 / 19.0, 64 15.5 / 19.4, 128 14.9 / 19.4, 256 19.9 / 19.4,
+  // 512 29.9 / 19.3).  Tuning knob ATENIA_MOE_ROUTER_TOKEN_MAX_F32 (read once).
+  static const int f32_token_max = [] {
+    const char* e = getenv("ATENIA_MOE_ROUTER_TOKEN_MAX_F32");
+    return e ? atoi(e) : 192;
+  }();
+  ra.token_kernel_max_tokens = f32w ? f32_token_max : router_token_max();
   PermuteArgs pa{};
   pa.idx = V.idx;
   pa.T = T;
