@@ -39,6 +39,19 @@ const HIPCC_FLAGS: &[&str] = &[
     "-packed-fp32-ops",
 ];
 
+// The hipcc release the kernels' generated code was validated with (HIPCC_VALIDATED of the
+// Makefile): the inline-assembly wait states of ffn_tiled.hip and the checks of
+// tests/test_isa_guards.py were read against this release's assembly.
+const HIPCC_VALIDATED: &str = "7.2";
+
+fn hipcc_release(hipcc: &Path) -> Option<String> {
+    let out = Command::new(hipcc).arg("--version").output().ok()?;
+    let text = String::from_utf8_lossy(&out.stdout).to_string();
+    let v = text.lines().find_map(|l| l.strip_prefix("HIP version: "))?;
+    let mut it = v.split('.');
+    Some(format!("{}.{}", it.next()?, it.next()?))
+}
+
 fn find_hipcc() -> Option<PathBuf> {
     let rocm = env::var("ROCM_PATH").unwrap_or_else(|_| "/opt/rocm".to_string());
     let p = Path::new(&rocm).join("bin").join("hipcc");
@@ -60,6 +73,14 @@ fn main() {
             return;
         }
     };
+    match hipcc_release(&hipcc) {
+        Some(v) if v == HIPCC_VALIDATED => {}
+        other => println!(
+            "cargo::warning=hipcc release {:?} differs from the validated {}: run tests/test_isa_guards.py \
+             against it before trusting the tiled kernels",
+            other, HIPCC_VALIDATED
+        ),
+    }
     let manifest = PathBuf::from(env::var("CARGO_MANIFEST_DIR").unwrap());
     let csrc = env::var("ATENIA_MOE_HIP_CSRC")
         .map(PathBuf::from)

@@ -39,7 +39,31 @@ def _assembly(tmp_path_factory, name):
     return [ln.strip() for ln in open(out).read().split("\n")]
 
 
-@pytest.fixture(scope="module", params=["ffn_stream.hip", "ffn_tiled.hip", "ffn_f32.hip"])
+def _validated_release():
+    """(Makefile, build.rs): the hipcc major.minor the generated code was validated with."""
+    mk = open(os.path.join(CSRC, "Makefile")).read()
+    rs = open(os.path.join(ROOT, "ffi", "atenia-moe-hip-sys", "build.rs")).read()
+    return (re.search(r"^HIPCC_VALIDATED\s*:=\s*(\S+)", mk, flags=re.M).group(1),
+            re.search(r'const HIPCC_VALIDATED: &str = "([^"]+)";', rs).group(1))
+
+
+def test_hipcc_is_the_release_the_generated_code_was_validated_with():
+    """The inline-assembly MFMAs of the nine-group tiles carry hand-counted wait states, and the
+    checks below were read against one compiler release's assembly.  Another major.minor fails
+    here, loudly, until somebody has read the new assembly and moved HIPCC_VALIDATED (Makefile and
+    build.rs) on purpose."""
+    if not os.path.exists(HIPCC):
+        pytest.skip("hipcc not found")
+    mk, rs = _validated_release()
+    assert mk == rs, f"Makefile says {mk}, build.rs says {rs}"
+    out = subprocess.run([HIPCC, "--version"], capture_output=True, text=True, timeout=120).stdout
+    m = re.search(r"HIP version: (\d+)\.(\d+)", out)
+    assert m, out[:300]
+    assert f"{m.group(1)}.{m.group(2)}" == mk, (
+        f"hipcc is release {m.group(1)}.{m.group(2)}, the kernels' assembly was validated with {mk}")
+
+
+@pytest.fixture(scope="module", params=["ffn_stream.hip", "ffn_tiled.hip", "ffn_tiled_duo.hip", "ffn_f32.hip"])
 def asm(request, tmp_path_factory):
     if not os.path.exists(HIPCC):
         pytest.skip("hipcc not found")
