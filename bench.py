@@ -479,7 +479,12 @@ def cpu_and_parity(torch, np, capi, ctx, x_head, out_head, tokens, cpu_tokens):
         sample_tokens=n)
     if margin:
         parity.update(margin)
-    parity.update(ora.numerical_metrics(got, ref))  # max_abs_diff, mean_abs_diff, rmse, argmax_match
+    # the reference's metric block (max_abs_diff, mean_abs_diff, rmse over the sample; its
+    # argmax check is made per output row, as it is made per logits vector there)
+    m = ora.numerical_metrics(got, ref)
+    rows = [ora.numerical_metrics(got[i], ref[i])["argmax_match"] for i in range(n)]
+    parity.update(max_abs_diff=m["max_abs_diff"], mean_abs_diff=m["mean_abs_diff"], rmse=m["rmse"],
+                  argmax_match_rows=int(sum(rows)), argmax_rows=n)
     return cpu, parity
 
 
