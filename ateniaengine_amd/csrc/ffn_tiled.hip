@@ -232,13 +232,14 @@ constexpr int kRingB = 3;  // B stages of 32 k (16 KiB each); a fourth measured 
 constexpr int kXaStage = 256;  // uint4 per stage
 
 // YB (down phase only): y leaves as bf16 (TiledParams::out_bf16), staged through LDS.
-template <bool UP, bool YB = false>
-__global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p) {
+// The tile of workgroup `bid` of a launch described by p.
+template <bool UP, bool YB>
+__device__ __forceinline__ void pipe_tile(const TiledParams& p, int bid) {
   constexpr int NA = kRingA, NB = kRingB;
   constexpr int XA0 = NA * 2048 + NB * 1024;            // first uint4 of the extra-rows ring
   __shared__ uint4 S[XA0 + NA * kXaStage];              // A ring, B ring, extra-rows ring
   int wid, n_parts, part;  // k range `part` of `n_parts` (1 unless this is a split tail tile)
-  if (!split_of_workgroup(p, p.k_pad / 64, wid, n_parts, part)) return;
+  if (!split_of_workgroup(p, bid, p.k_pad / 64, wid, n_parts, part)) return;
   int rt, ct;
   if (!tile_of_workgroup(p, wid, rt, ct)) return;
 
@@ -721,6 +722,46 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p)
   }
 }
 
+template <bool UP, bool YB = false>
+__global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p) {
+  pipe_tile<UP, YB>(p, (int)blockIdx.x);
+}
+
+// Gate/up launch of the routed experts and of a shared expert in one grid: workgroups below
+// n_first take the routed experts' tiles (p), the others the shared expert's (ps), in that order,
+// so the compute units that the last routed tiles leave idle start on the shared expert instead
+// of waiting for a second launch (each launch by itself ends on a partly filled round of tiles).
+// The parameter set is picked field by field with the workgroup-uniform condition: selecting a
+// reference to one of two by-value kernel arguments makes the compiler copy the struct to the stack.
+__device__ __forceinline__ TiledParams pick_params(const TiledParams& a, const TiledParams& b, bool second) {
+  TiledParams q;
+#define ATENIA_PICK(f) q.f = second ? b.f : a.f
+  ATENIA_PICK(wa); ATENIA_PICK(wb); ATENIA_PICK(sa); ATENIA_PICK(sb); ATENIA_PICK(w_stride_u4);
+  ATENIA_PICK(n_rows); ATENIA_PICK(n_blocks); ATENIA_PICK(nkb); ATENIA_PICK(k_pad); ATENIA_PICK(a);
+  ATENIA_PICK(a_stride); ATENIA_PICK(out); ATENIA_PICK(out_stride); ATENIA_PICK(out_bf16);
+  ATENIA_PICK(g.offsets); ATENIA_PICK(g.active); ATENIA_PICK(g.n_active); ATENIA_PICK(g.perm);
+  ATENIA_PICK(g.pair_div); ATENIA_PICK(g.idx1);
+  ATENIA_PICK(tile_group); ATENIA_PICK(tile_m0); ATENIA_PICK(n_tiles); ATENIA_PICK(tile_rows);
+  ATENIA_PICK(tile_li); ATENIA_PICK(n_col_tiles); ATENIA_PICK(max_parts); ATENIA_PICK(wg_upper);
+  ATENIA_PICK(n_cus); ATENIA_PICK(out_part_stride); ATENIA_PICK(part_flags); ATENIA_PICK(stagger);
+#undef ATENIA_PICK
+  return q;
+}
+__global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_up2_kernel(TiledParams p, TiledParams ps,
+                                                                      int n_first) {
+  const bool second = (int)blockIdx.x >= n_first;
+  const TiledParams q = pick_params(p, ps, second);
+  pipe_tile<true, false>(q, second ? (int)blockIdx.x - n_first : (int)blockIdx.x);
+}
+// The same for the down phase (the caller puts the parameter set with the longer K first).
+template <bool YB>
+__global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_down2_kernel(TiledParams p, TiledParams ps,
+                                                                        int n_first) {
+  const bool second = (int)blockIdx.x >= n_first;
+  const TiledParams q = pick_params(p, ps, second);
+  pipe_tile<false, YB>(q, second ? (int)blockIdx.x - n_first : (int)blockIdx.x);
+}
+
 // ---- INT8 W8A16 form of the pipelined kernel -----------------------------------------------
 // Same tiling, A ring and k16-unit pipeline.  Weights stay int8 all the way into LDS: a B stage
 // is 64 k = 16 stored blocks (16 KiB, one load instruction per block), so there is one barrier
@@ -740,7 +781,7 @@ __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_i8_kernel(TiledParams
   constexpr int NA = kRingA, NB = 4;          // 64-k stages: A 32 KiB, B 16 KiB
   __shared__ uint4 S[NA * 2048 + NB * 1024];  // A ring, then B ring
   int wid, n_parts, part;  // k range `part` of `n_parts` (1 unless this is a split tail tile)
-  if (!split_of_workgroup(p, p.k_pad / 64, wid, n_parts, part)) return;
+  if (!split_of_workgroup(p, (int)blockIdx.x, p.k_pad / 64, wid, n_parts, part)) return;
   int rt, ct;
   if (!tile_of_workgroup(p, wid, rt, ct)) return;
 
@@ -1044,7 +1085,8 @@ bool tiled_supported(const WeightSet& w, int wdtype) {
   return w.k_pad % TK == 0;
 }
 
-hipError_t launch_ffn_up_tiled(const FfnArgs& a, hipStream_t s) {
+namespace {
+TiledParams up_params(const FfnArgs& a) {
   const bool int8 = a.wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
   TiledParams p{};
   p.wa = (const uint4*)a.gate.w;
@@ -1068,6 +1110,35 @@ hipError_t launch_ffn_up_tiled(const FfnArgs& a, hipStream_t s) {
   p.tile_li = a.tile_li;
   p.n_col_tiles = (a.gate.n_pad + 127) / 128;
   p.max_parts = 1;
+  return p;
+}
+bool up_takes_pipe_bf16(const FfnArgs& a) {
+  return a.use_tiled && !a.use_duo && a.wdtype != ATENIA_MOE_WEIGHT_INT8_W8A16 &&
+         a.wdtype != ATENIA_MOE_WEIGHT_F32 && a.gate.group_blocks == 0 && a.gate.k_pad % 64 == 0 &&
+         a.gate.k_pad >= 128 && (!a.tall_tiles || (a.tile_rows && a.tile_li));
+}
+}  // namespace
+
+// Routed experts and a shared expert in one gate/up launch (ffn_tiled_pipe_up2_kernel): both on
+// the bf16 pipelined kernel.
+bool tiled_up_pair_supported(const FfnArgs& a, const FfnArgs& shared) {
+  return up_takes_pipe_bf16(a) && up_takes_pipe_bf16(shared);
+}
+hipError_t launch_ffn_up_tiled_pair(const FfnArgs& a, const FfnArgs& shared, hipStream_t s) {
+  if (!tiled_up_pair_supported(a, shared)) return hipErrorInvalidValue;
+  TiledParams p = up_params(a), ps = up_params(shared);
+  int n1 = a.max_row_tiles * p.n_col_tiles, n2 = shared.max_row_tiles * ps.n_col_tiles;
+  n1 = (n1 + 7) / 8 * 8;  // whole rounds over the 8 XCDs: the second part starts on XCD 0 again
+  n2 = (n2 + 7) / 8 * 8;
+  p.wg_upper = n1;
+  ps.wg_upper = n2;
+  ffn_tiled_pipe_up2_kernel<<<n1 + n2, kThreads, 0, s>>>(p, ps, n1);
+  return hipGetLastError();
+}
+
+hipError_t launch_ffn_up_tiled(const FfnArgs& a, hipStream_t s) {
+  const bool int8 = a.wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
+  TiledParams p = up_params(a);
   const bool pipe_bf16 = !int8 && p.k_pad % 64 == 0 && p.k_pad >= 128;
   // A list of nine-group tiles in any other kernel would lose the rows past 256 of such a tile.
   if (a.tall_tiles && (!pipe_bf16 || a.use_duo || !p.tile_rows || !p.tile_li)) return hipErrorInvalidValue;
@@ -1084,7 +1155,8 @@ hipError_t launch_ffn_up_tiled(const FfnArgs& a, hipStream_t s) {
               : launch_tiled<false, true>(p, a.max_row_tiles, s);
 }
 
-hipError_t launch_ffn_down_tiled(const FfnArgs& a, hipStream_t s) {
+namespace {
+TiledParams down_params(const FfnArgs& a) {
   const bool int8 = a.wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
   TiledParams p{};
   p.wa = (const uint4*)a.down.w;
@@ -1108,6 +1180,49 @@ hipError_t launch_ffn_down_tiled(const FfnArgs& a, hipStream_t s) {
   p.tile_li = a.tile_li;
   p.n_col_tiles = (a.down.n_pad + 255) / 256;
   p.max_parts = 1;
+  return p;
+}
+// k split of the tail round (pipelined kernels; see split_of_workgroup)
+void down_split_params(const FfnArgs& a, TiledParams& p) {
+  if (a.y_parts > 1 && a.part_flags && a.n_cus >= 8) {
+    p.max_parts = a.y_parts;
+    p.n_cus = a.n_cus / 8 * 8;
+    p.out_part_stride = a.y_part_stride;
+    p.part_flags = a.part_flags;
+  }
+}
+bool down_takes_pipe_bf16(const FfnArgs& a) {
+  return a.use_tiled && !a.use_duo && a.wdtype != ATENIA_MOE_WEIGHT_INT8_W8A16 &&
+         a.wdtype != ATENIA_MOE_WEIGHT_F32 && a.down.group_blocks == 0 && a.down.k_pad % 64 == 0 &&
+         a.down.k_pad >= 128 && (!a.tall_tiles || (a.tile_rows && a.tile_li)) &&
+         (!a.y_bf16 || a.down.n_rows % 8 == 0);
+}
+}  // namespace
+
+bool tiled_down_pair_supported(const FfnArgs& first, const FfnArgs& second) {
+  return down_takes_pipe_bf16(first) && down_takes_pipe_bf16(second) && !first.y_bf16 == !second.y_bf16;
+}
+hipError_t launch_ffn_down_tiled_pair(const FfnArgs& first, const FfnArgs& second, hipStream_t s) {
+  if (!tiled_down_pair_supported(first, second)) return hipErrorInvalidValue;
+  TiledParams p1 = down_params(first), p2 = down_params(second);
+  p1.out_bf16 = first.y_bf16;
+  p2.out_bf16 = second.y_bf16;
+  down_split_params(first, p1);
+  down_split_params(second, p2);
+  int n1 = first.max_row_tiles * p1.n_col_tiles, n2 = second.max_row_tiles * p2.n_col_tiles;
+  n1 = (n1 + 7) / 8 * 8;
+  n2 = (n2 + 7) / 8 * 8;
+  p1.wg_upper = n1;
+  p2.wg_upper = n2;
+  const int e1 = p1.max_parts > 1 ? p1.n_cus : 0, e2 = p2.max_parts > 1 ? p2.n_cus : 0;
+  if (first.y_bf16) ffn_tiled_pipe_down2_kernel<true><<<n1 + e1 + n2 + e2, kThreads, 0, s>>>(p1, p2, n1 + e1);
+  else ffn_tiled_pipe_down2_kernel<false><<<n1 + e1 + n2 + e2, kThreads, 0, s>>>(p1, p2, n1 + e1);
+  return hipGetLastError();
+}
+
+hipError_t launch_ffn_down_tiled(const FfnArgs& a, hipStream_t s) {
+  const bool int8 = a.wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16;
+  TiledParams p = down_params(a);
   const bool pipelined = int8 ? p.k_pad >= 128 : (p.k_pad % 64 == 0 && p.k_pad >= 128);
   const bool pipe_bf16 = !int8 && pipelined;
   if (a.tall_tiles && (!pipe_bf16 || a.use_duo || !p.tile_rows || !p.tile_li)) return hipErrorInvalidValue;
@@ -1121,12 +1236,7 @@ hipError_t launch_ffn_down_tiled(const FfnArgs& a, hipStream_t s) {
     p.n_cus = a.n_cus;
     return launch_tiled_duo_down(p, a.max_row_tiles, s);
   }
-  if (pipelined && a.y_parts > 1 && a.part_flags && a.n_cus >= 8) {
-    p.max_parts = a.y_parts;
-    p.n_cus = a.n_cus / 8 * 8;
-    p.out_part_stride = a.y_part_stride;
-    p.part_flags = a.part_flags;
-  }
+  if (pipelined) down_split_params(a, p);
   if (!int8 && p.k_pad % 64 == 0 && p.k_pad >= 128) return launch_tiled_dma<false>(p, a.max_row_tiles, s);
   if (int8 && p.k_pad >= 128) return launch_tiled_pipe_i8<false>(p, a.max_row_tiles, s);
   return int8 ? launch_tiled<true, false>(p, a.max_row_tiles, s)

@@ -212,9 +212,11 @@ __device__ inline bool tile_of_workgroup_sub(const TiledParams& p, int wid, int&
 // range i writes its partial sums to buffer i, and range 0 records S per (row, column tile) so
 // that the combine adds up exactly the buffers that were written.  Sets wid (the tile's
 // workgroup id for tile_of_workgroup), S and part; false = nothing to do.
-__device__ inline bool split_of_workgroup(const TiledParams& p, int n_stages, int& wid, int& S,
+// bid: the workgroup's id within its launch (blockIdx.x, or the id inside its own part of a launch
+// that carries two parameter sets).
+__device__ inline bool split_of_workgroup(const TiledParams& p, int bid, int n_stages, int& wid, int& S,
                                           int& part) {
-  wid = blockIdx.x;
+  wid = bid;
   S = 1;
   part = 0;
   if (p.max_parts <= 1) return true;
@@ -225,8 +227,8 @@ __device__ inline bool split_of_workgroup(const TiledParams& p, int n_stages, in
   int s_tail = 1;
   if (tail > 0 && 2 * tail <= p.n_cus) s_tail = min(min(p.max_parts, p.n_cus / tail), n_stages / 2);
   if (s_tail < 1) s_tail = 1;
-  if ((int)blockIdx.x >= p.wg_upper) {
-    const int x = blockIdx.x - p.wg_upper;
+  if (bid >= p.wg_upper) {
+    const int x = bid - p.wg_upper;
     if (s_tail == 1 || x >= tail * (s_tail - 1)) return false;
     part = 1 + x / tail;
     const int j = x - (part - 1) * tail;

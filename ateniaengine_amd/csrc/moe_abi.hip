@@ -668,6 +668,16 @@ bool y_bf16_enabled() {
   return on;
 }
 
+// Routed and shared experts' tiled launches of a phase as one launch where both are on the
+// caller's stream (tuning knob ATENIA_MOE_PAIR_LAUNCHES=0: always two; read once).
+bool pair_launches_enabled() {
+  static const bool on = [] {
+    const char* e = getenv("ATENIA_MOE_PAIR_LAUNCHES");
+    return !(e && atoi(e) == 0);
+  }();
+  return on;
+}
+
 bool side_stream_enabled() {
   static const bool on = [] {
     const char* e = getenv("ATENIA_MOE_SHARED_SIDE_STREAM");  // 0 = everything on the caller's stream
@@ -1061,9 +1071,25 @@ int run_forward_impl(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, flo
   // 8192 1360 / 1379, 16384 2546 / 2592.
   const long long shared_down_tiles =
       (long long)((T + kTileM - 1) / kTileM) * ((L->d + 255) / 256);
+  // Where both are on the bf16 pipelined kernel the routed and the shared expert's tiles of a
+  // phase are ONE launch instead (the shared expert's tiles behind the routed ones in the gate/up
+  // phase, in front of them in the down phase where its K is the longer one): the compute units
+  // that the last tiles of one part leave idle start on the other part at once, where each launch
+  // by itself ends on a partly filled round of tiles, and the two parts never compete for an
+  // XCD's L2.  One-stream stage times, two launches / one (us), gate/up and down: Qwen1.5-MoE
+  // shape T = 2048 271 / 238 and 213 / 149, 4096 429 / 386 and 272 / 222, 12288 1045 / 1002 and
+  // 613 / 560; DeepSeek-V2-Lite shape T = 4096 450 / 433 and 297 / 269, 12288 1092 / 1062 and
+  // 680 / 650.  Whole forward, second stream / paired launches (ms): Qwen T = 768 0.344 / 0.332,
+  // 1024 0.371 / 0.358, 2048 0.447 / 0.439, 3072 0.579 / 0.559, 4096 0.712 / 0.700, 6144
+  // 1.018 / 1.002; DeepSeek T = 768 0.369 / 0.359, 1024 0.416 / 0.405, 1536 0.444 / 0.446, 2048
+  // 0.509 / 0.495, 3072 0.670 / 0.657, 6144 1.104 / 1.091; two launches on one stream / paired:
+  // Qwen T = 8192 1.261 / 1.249, 12288 1.848 / 1.769; DeepSeek T = 8192 1.367 / 1.335, 16384
+  // 2.527 / 2.490.  The second stream stays for the layers that cannot pair (int8 tiles).
+  const bool pair_up = pair_launches_enabled() && L->fs > 0 && !fuse_shared_up &&
+                       tiled_up_pair_supported(fa, fsd);
   const bool side_run = side_stream_enabled() && L->fs > 0 && !fuse_shared_up && tiled && L->side &&
                         shared_down_tiles < fa.n_cus && first <= kStageFfn && !L->profiling &&
-                        !no_alloc && !stream_is_capturing(s);
+                        !no_alloc && !pair_up && !stream_is_capturing(s);
   bool side_open = false;
   if (first <= kStageFfn) {
     if (side_run) {
@@ -1071,11 +1097,16 @@ int run_forward_impl(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, flo
       HIP_TRY(hipStreamWaitEvent(L->side, L->ev_fork, 0));
       side_open = true;
     }
-    HIP_TRY(launch_ffn_up(fa, s, fuse_shared_up ? &fsd : nullptr));
-    L->launches[2] = 1;
-    if (L->fs > 0 && !fuse_shared_up) {
-      HIP_TRY(launch_ffn_up(fsd, side_run ? L->side : s));
-      L->launches[2] = 2;
+    if (pair_up) {
+      HIP_TRY(launch_ffn_up_tiled_pair(fa, fsd, s));
+      L->launches[2] = 1;
+    } else {
+      HIP_TRY(launch_ffn_up(fa, s, fuse_shared_up ? &fsd : nullptr));
+      L->launches[2] = 1;
+      if (L->fs > 0 && !fuse_shared_up) {
+        HIP_TRY(launch_ffn_up(fsd, side_run ? L->side : s));
+        L->launches[2] = 2;
+      }
     }
   }
   auto side_join = [&]() -> hipError_t {  // the caller's stream waits for the side stream's work
@@ -1099,6 +1130,7 @@ int run_forward_impl(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, flo
   // shared one and finishes the combine as well (one launch instead of two or three).
   const bool fuse1 = first <= kStageFfn && last >= kStageCombine && L->group_size == 0 &&
                      ffn_down_decode1_supported(T, fa, L->k, tiled, L->fs > 0 ? &fsd : nullptr);
+  bool pair_down = false;
   if (first <= kStageFfn) {
     if (fuse1) {
       fa.fuse_w = V.w;
@@ -1109,10 +1141,14 @@ int run_forward_impl(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, flo
       HIP_TRY(launch_ffn_down_decode1(fa, s, L->fs > 0 ? &fsd : nullptr));
     } else {
       if (fuse_shared_down) HIP_TRY(side_join());  // the fused launch reads the shared expert's h
-      HIP_TRY(launch_ffn_down(fa, s, fuse_shared_down ? &fsd : nullptr));
+      // one launch for both, the shared expert's tiles (the longer K) first
+      pair_down = pair_launches_enabled() && L->fs > 0 && !fuse_shared_down && !side_open &&
+                  tiled_down_pair_supported(fsd, fa);
+      if (pair_down) HIP_TRY(launch_ffn_down_tiled_pair(fsd, fa, s));
+      else HIP_TRY(launch_ffn_down(fa, s, fuse_shared_down ? &fsd : nullptr));
     }
     L->launches[3] = 1;
-    if (L->fs > 0 && !fuse_shared_down && !fuse1) {
+    if (L->fs > 0 && !fuse_shared_down && !fuse1 && !pair_down) {
       HIP_TRY(launch_ffn_down(fsd, side_open ? L->side : s));
       L->launches[3] = 2;
     }

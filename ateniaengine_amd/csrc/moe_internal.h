@@ -190,6 +190,14 @@ bool ffn_mid_supported(const WeightSet& w, int wdtype);
 // True when the tiled down launch for these weights can split the k range of tail tiles.
 bool tiled_down_splits_tail(const WeightSet& down, int wdtype);
 hipError_t launch_ffn_up_tiled(const FfnArgs& a, hipStream_t s);
+// Gate/up of the routed experts and of a shared expert as one launch of the bf16 pipelined kernel
+// (routed tiles first): both argument sets must ask for that kernel (tiled_up_pair_supported).
+bool tiled_up_pair_supported(const FfnArgs& a, const FfnArgs& shared);
+hipError_t launch_ffn_up_tiled_pair(const FfnArgs& a, const FfnArgs& shared, hipStream_t s);
+// The same for the down phase, `first`'s tiles in front (the caller puts the longer K there);
+// both sets must store y in the same element type.
+bool tiled_down_pair_supported(const FfnArgs& first, const FfnArgs& second);
+hipError_t launch_ffn_down_tiled_pair(const FfnArgs& first, const FfnArgs& second, hipStream_t s);
 hipError_t launch_ffn_down_tiled(const FfnArgs& a, hipStream_t s);
 // `shared` (may be null): the shared expert's arguments; when ffn_stream_fuses_shared(a, *shared,
 // phase) holds, its work is done by the same launch and the caller must not launch it again.

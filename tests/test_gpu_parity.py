@@ -418,8 +418,10 @@ def test_mid_batch_kernel(ora, wd, T, d, f_s, skew):
 @pytest.mark.parametrize("wd", [capi.WEIGHT_BF16, capi.WEIGHT_INT8_W8A16])
 @pytest.mark.parametrize("E,T,f_s", [(8, 700, 256), (8, 1500, 128), (16, 700, 256)])
 def test_shared_expert_on_its_own_stream(ora, wd, E, T, f_s):
-    """Tiled family with a shared expert: its two launches run on a stream of the handle's own
-    beside the routed experts' (forked after the grouping, joined before the combine).  The result
+    """Tiled family with a shared expert, int8 weights: its two launches run on a stream of the
+    handle's own beside the routed experts' (forked after the grouping, joined before the combine;
+    bf16 layers carry the shared expert's tiles in the routed experts' launches instead,
+    tests/test_gpu_pair_launch.py, and only pass through here).  The result
     must be the oracle's, and bit for bit what the same kernels give one after the other on the
     caller's stream (stage profiling on keeps everything there) -- on repeated calls, so that a
     missing wait between the streams would show as a stale read.  With 16 experts the down phase
