@@ -58,19 +58,39 @@ __global__ __launch_bounds__(256) void ffn_f32_kernel(
 
   double acc_a[4] = {0, 0, 0, 0}, acc_b[4] = {0, 0, 0, 0};
   float facc_a[4] = {0.f, 0.f, 0.f, 0.f}, facc_b[4] = {0.f, 0.f, 0.f, 0.f};
+  // A thread stages elements (r, c) = (tid / 32 + 8 q, tid % 32), q = 0..3, of each 32 x 32 tile.
+  // The next tile's elements are fetched into registers before the current tile is multiplied,
+  // so a k tile does not start with a memory round trip (the sums and their order are untouched).
+  __syncthreads();  // sRow
+  float ra[4], rba[4], rbb[4];
+  auto fetch = [&](int k0) {
+    const int c = tid & 31, kk = k0 + c;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int r = (tid >> 5) + 8 * q;
+      const int src = sRow[r];
+      ra[q] = (src >= 0 && kk < k_cols) ? a[(size_t)src * a_stride + kk] : 0.f;
+      const int n = n0 + r;
+      const bool ok = n < n_rows && kk < k_cols;
+      rba[q] = ok ? wae[(size_t)n * k_cols + kk] : 0.f;
+      rbb[q] = (UP && ok) ? wbe[(size_t)n * k_cols + kk] : 0.f;
+    }
+  };
+  fetch(0);
   for (int k0 = 0; k0 < k_cols; k0 += kTile) {
     __syncthreads();
-    for (int j = tid; j < kTile * kTile; j += 256) {
-      int r = j >> 5, c = j & 31;
-      int kk = k0 + c;
-      int src = sRow[r];
-      sA[r * kLdT + c] = (src >= 0 && kk < k_cols) ? a[(size_t)src * a_stride + kk] : 0.f;
-      int n = n0 + r;
-      bool ok = n < n_rows && kk < k_cols;
-      sBa[r * kLdT + c] = ok ? wae[(size_t)n * k_cols + kk] : 0.f;
-      if (UP) sBb[r * kLdT + c] = ok ? wbe[(size_t)n * k_cols + kk] : 0.f;
+    {
+      const int c = tid & 31;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int r = (tid >> 5) + 8 * q;
+        sA[r * kLdT + c] = ra[q];
+        sBa[r * kLdT + c] = rba[q];
+        if (UP) sBb[r * kLdT + c] = rbb[q];
+      }
     }
     __syncthreads();
+    if (k0 + kTile < k_cols) fetch(k0 + kTile);
     if (F32ACC) {
       // tile columns past k_cols hold +0.0: acc + 0 * 0 leaves every sum as it was (a sum that
       // starts at +0.0 never becomes -0.0)

@@ -668,6 +668,15 @@ def main():
                 xo = (x_t, out_t, t)
             _, parities[name] = cpu_and_parity(torch, np, capi, ctx, xo[0], xo[1], xo[2],
                                                min(xo[2], 64))
+            if CONFIGS[name]["wd"] == "f32":
+                # the reference's other expert arithmetic for f32 layers (NumericPolicy::Strict,
+                # and what Fast falls back to: f32 accumulation, numeric_policy.rs:36-75)
+                ctx["layer"].set_numeric_policy(capi.POLICY_STRICT)
+                r, _, _ = measure(torch, np, capi, ctx["layer"], ts[-1], max(a.steps, 50), a.warmup, a.seed)
+                e = compact(name, r)
+                e["numeric_policy"] = "strict"
+                entries.append(e)
+                ctx["layer"].set_numeric_policy(capi.POLICY_CERTIFIED)
             ctx["layer"].close()
             del ctx, xo
         line["configs"] = entries
