@@ -303,14 +303,8 @@ bool mfma_f64_ok(const FfnArgs& a, bool up) {
   return !a.f32_accumulate && k % 8 == 0 && stride % 4 == 0 && ((uintptr_t)act & 15) == 0;
 }
 
-// Four waves on one strip's K, or one strip per wave (tuning knob ATENIA_MOE_F32_KSPLIT = 0 / 1,
-// read once per process; default: split unless K is a few steps only).
+// Four waves on one strip's K, or one strip per wave: split unless K is a few steps only.
 bool mfma_f64_splits_k(int n_rows, int k_cols) {
-  static const int forced = [] {
-    const char* e = getenv("ATENIA_MOE_F32_KSPLIT");
-    return e ? atoi(e) : -1;
-  }();
-  if (forced >= 0) return forced != 0;
   (void)n_rows;
   return k_cols >= 128;  // measured at d = 1024, f = 2048, T = 64: gate/up 53 against 59 us, down 32 against 69
 }

@@ -934,11 +934,8 @@ hipError_t launch_stream(const StreamParams& p, int n_groups, int rows_max, hipS
     // (two row tiles, two strips per workgroup) 36.1 -> 29.6 and 59.0 -> 46.2; two
     // slices are slower again (T = 2 17.5 against 15.9 us).  A single token keeps eight: its
     // fused down + combine launch adds the slices up in that order, and the two must agree bit
-    // for bit.  ATENIA_MOE_DOWN_W4_BELOW moves the bound (0 = never).
-    static const int w4_below = [] {
-      const char* e = getenv("ATENIA_MOE_DOWN_W4_BELOW");
-      return e ? atoi(e) : 64;
-    }();
+    // for bit.
+    constexpr int w4_below = 64;
     if (p.nkb < w4_below && rows_max > 1) {
       if (mt == 1 && two)
         ffn_stream_kernel<1, INT8, false, 4, false, 2><<<grid, 256, 0, s>>>(p, ps, shared_y);
@@ -1023,7 +1020,7 @@ StreamParams stream_params_down(const FfnArgs& a) {
 // T = 2 18.5 against 22.9 us as two launches, T = 16 52.2 / 60.1, T = 48 72.8 / 77.5; from
 // 64 rows on, where its T rows take several passes over its weights, a shared expert more than
 // twice as wide is faster in a launch of its own (T = 64 81.3 / 79.0, T = 128 100.9 / 85.5).
-// ATENIA_MOE_WIDE_SHARED_ROWS moves the bound (default 48).
+// The bound used is 48 rows.
 bool can_fuse_shared(const FfnArgs& a, const FfnArgs* sh, bool down_phase) {
   if (!(sh && a.wdtype != ATENIA_MOE_WEIGHT_F32 && sh->wdtype == a.wdtype && !a.use_tiled &&
         !sh->use_tiled && sh->rows_max == a.rows_max &&
@@ -1033,16 +1030,9 @@ bool can_fuse_shared(const FfnArgs& a, const FfnArgs* sh, bool down_phase) {
   // (the mid-batch launch starts all of the shared expert's workgroups first, which hides a
   // wider one: measured on the Qwen1.5-MoE shape, whole forward fused / a launch of its own
   // beyond 384 rows: T = 512 312 / 336 us, T = 768 339 / 365, T = 1024 363 / 386, T = 1280
-  // 420 / 430.  ATENIA_MOE_MID_SHARED_ROWS sets a bound.)
-  static const int mid_rows = [] {
-    const char* e = getenv("ATENIA_MOE_MID_SHARED_ROWS");
-    return e ? atoi(e) : 1 << 30;
-  }();
-  if (a.use_mid && a.rows_max <= mid_rows) return true;
-  static const int wide_rows = [] {
-    const char* e = getenv("ATENIA_MOE_WIDE_SHARED_ROWS");
-    return e ? atoi(e) : 48;
-  }();
+  // 420 / 430: at every batch size.)
+  if (a.use_mid) return true;
+  constexpr int wide_rows = 48;
   if (!a.use_mid && down_phase && a.rows_max > 1 && a.rows_max <= wide_rows) return true;  // first in the grid
   return !down_phase || sh->down.k_pad <= 2 * a.down.k_pad;
 }

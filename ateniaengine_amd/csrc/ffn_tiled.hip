@@ -743,7 +743,7 @@ __device__ __forceinline__ TiledParams pick_params(const TiledParams& a, const T
   ATENIA_PICK(g.pair_div); ATENIA_PICK(g.idx1);
   ATENIA_PICK(tile_group); ATENIA_PICK(tile_m0); ATENIA_PICK(n_tiles); ATENIA_PICK(tile_rows);
   ATENIA_PICK(tile_li); ATENIA_PICK(n_col_tiles); ATENIA_PICK(max_parts); ATENIA_PICK(wg_upper);
-  ATENIA_PICK(n_cus); ATENIA_PICK(out_part_stride); ATENIA_PICK(part_flags); ATENIA_PICK(stagger);
+  ATENIA_PICK(n_cus); ATENIA_PICK(out_part_stride); ATENIA_PICK(part_flags);
 #undef ATENIA_PICK
   return q;
 }

@@ -39,9 +39,6 @@ struct TiledParams {
   int n_cus;
   size_t out_part_stride;     // elements between the partial output buffers
   uint8_t* part_flags;        // [pairs, n_col_tiles] partial buffers written per (row, column tile)
-  // Two-workgroup form only: s_sleep 8 periods (512 cycles each) that a workgroup of the first
-  // round waits before its main loop when its waves sit in the second wave slot of their SIMDs.
-  int stagger;
 };
 
 // The form of the bf16 tiled kernels that runs two workgroups per compute unit (ffn_tiled_duo.hip).

@@ -222,16 +222,9 @@ void ffn_tiled_duo_kernel(TiledParams p) {
     }
     wait_vm_lgkm0<0>();
   };
-  // Two workgroups that start together on a compute unit would stay in step -- both in their main
-  // loops at half speed, then both in their epilogues with the matrix pipes idle -- and so would
-  // their successors.  In the first round the workgroup whose waves got the second wave slot of
-  // their SIMDs therefore waits about one main loop (its first stages are in flight meanwhile),
-  // after which one's main loop runs beside the other's epilogue and prologue.
-  if (p.stagger > 0 && (int)blockIdx.x < 2 * p.n_cus) {
-    const uint32_t slot = __builtin_amdgcn_s_getreg(4 | (0 << 6) | (3 << 11));  // HW_ID.wave_id
-    if (slot & 1)
-      for (int i = 0; i < p.stagger; ++i) __builtin_amdgcn_s_sleep(8);
-  }
+  // (Two workgroups that start together on a compute unit do not stay in step: delaying the one
+  // in the second wave slot of its SIMDs by 0 to 1.5 main loops in the first round measured the
+  // same to 0.5 %, so nothing is staggered.)
   if (my_rows > 32) run(integral_constant<int, 2>{});
   else if (my_rows > 0) run(integral_constant<int, 1>{});
   else run(integral_constant<int, 0>{});
@@ -341,21 +334,9 @@ void ffn_tiled_duo_kernel(TiledParams p) {
   }
 }
 
-// Stagger of the first round in eighths of a main loop (tuning knob ATENIA_MOE_DUO_STAGGER, read
-// once; 0 = none).
-int duo_stagger_eighths() {
-  static const int v = [] {
-    const char* e = getenv("ATENIA_MOE_DUO_STAGGER");
-    return e ? atoi(e) : 8;
-  }();
-  return v;
-}
-
 template <bool UP>
 hipError_t launch_duo(TiledParams p, int max_row_tiles, hipStream_t s) {
   if (!tiled_duo_supported(p)) return hipErrorInvalidValue;
-  // a main loop alone on its SIMDs: 16 matrix instructions of 32 cycles per 32-k step
-  p.stagger = p.n_cus > 0 ? (p.k_pad / 32) * duo_stagger_eighths() / 8 : 0;
   int n_wg = max_row_tiles * kDuoSub * p.n_col_tiles;
   n_wg = (n_wg + 7) / 8 * 8;
   if (!UP && p.out_bf16) {

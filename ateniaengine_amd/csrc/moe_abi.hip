@@ -580,11 +580,6 @@ MidBounds mid_bounds(const AteniaMoeLayer* L) {
   if (env_lo >= 0.0) b.lo = env_lo;
   if (env_hi >= 0.0) b.hi = b.down_hi = env_hi;
   if (env_min_tokens > 0) b.min_tokens = b.down_min_tokens = env_min_tokens;
-  static const int env_max_tokens = [] {
-    const char* e = getenv("ATENIA_MOE_MID_MAX_TOKENS");
-    return e ? atoi(e) : 0;
-  }();
-  if (env_max_tokens > 0) b.max_tokens = env_max_tokens;
   return b;
 }
 // The measured cross-overs as they stand: family of each phase at batch size T.

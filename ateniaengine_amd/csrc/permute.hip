@@ -351,12 +351,7 @@ hipError_t launch_permute(const PermuteArgs& a, hipStream_t s, int* n_launches) 
     return hipGetLastError();
   }
   const int nblk = (P + kPermuteBlock - 1) / kPermuteBlock;
-  static const int multi_max = [] {
-    const char* e = getenv("ATENIA_MOE_PERMUTE_MULTI_BLOCKS");  // tuning knob: 0 = three launches
-    const int n = e ? atoi(e) : kMultiBlocks;
-    return n < 0 ? 0 : n > 64 ? 64 : n;
-  }();
-  if (nblk <= multi_max) {
+  if (nblk <= kMultiBlocks) {
     size_t sm = ((size_t)kWaves * E + 4 * (size_t)E + 1) * sizeof(int32_t);
     permute_multi_kernel<<<nblk, kPermuteBlock, sm, s>>>(a.idx, P, E, a.T, a.counts, a.offsets,
                                                          a.perm, a.inv, a.active, a.n_active,

@@ -974,17 +974,11 @@ bool router_mfma_ok(const RouterArgs& a, int R) {
   }();
   // Against the sequential kernel (route stage, us): 8 rows, d = 4096: T = 4096 32 / 57-75,
   // 8192 48 / 89, 16384 89 / 160; 61-64 rows, d = 2048: T = 4096 59 / 92-97, 8192 86 / 87,
-  // 12288 127 / 178, 16384 155 / 180.  ATENIA_MOE_ROUTER_MFMA_MAX_T sets an upper bound on the
-  // batch (none by default).
+  // 12288 127 / 178, 16384 155 / 180: at every batch size.
   // Only with operands that make the exactness test pass -- bf16 activations and router rows whose
   // f32 values fit bf16: otherwise every sum the interval test flags (one in a thousand) costs a
   // sequential chain in its workgroup, and the launch lasts as long as the slowest of them.
-  static const int max_t = [] {
-    const char* e = getenv("ATENIA_MOE_ROUTER_MFMA_MAX_T");
-    return e ? atoi(e) : 0;
-  }();
-  const int t_max = max_t > 0 ? max_t : 0x7fffffff;
-  const bool operands = !off && a.T <= t_max && a.d % 8 == 0 && !a.xb && a.x_is_bf16 &&
+  const bool operands = !off && a.d % 8 == 0 && !a.xb && a.x_is_bf16 &&
                         a.w_fits_bf16 && a.E >= a.k;
   if (R < 0) return operands;  // the form that deals the rows to workgroups takes any row count
   return operands && R <= 80 && !a.logits_out;
@@ -996,17 +990,9 @@ bool router_mfma_ok(const RouterArgs& a, int R) {
 // 4096 37 / 32; 48 rows, d = 4096, T = 2048 54 / 81.  Against the per-token kernel below 512
 // tokens (64 rows): T = 16 23 / 15, 32 24 / 19, 48 24 / 23, 56 24 / 27, 64 24 / 29, 128 24 / 28,
 // 256 24 / 32, 384 25 / 47, 512 25 / 50; 32 rows: T = 128 23 / 20, 512 23 / 35.
-// ATENIA_MOE_ROUTER_SPLIT_MIN_T / _MAX_T move the bounds (a maximum of 0 switches it off).
 bool router_mfma_split_wanted(const RouterArgs& a, int R) {
-  static const int max_t = [] {
-    const char* e = getenv("ATENIA_MOE_ROUTER_SPLIT_MAX_T");
-    return e ? atoi(e) : 2048;
-  }();
-  static const int min_t = [] {
-    const char* e = getenv("ATENIA_MOE_ROUTER_SPLIT_MIN_T");
-    return e ? atoi(e) : -1;
-  }();
-  const int lo = min_t >= 0 ? min_t : R > 32 ? 52 : 192;
+  constexpr int max_t = 2048;
+  const int lo = R > 32 ? 52 : 192;
   if (R <= 16 || a.T < lo || !router_mfma_ok(a, -1)) return false;
   // The raw logits are wanted (another launch routes), or more rows than one workgroup holds:
   // no other form on the matrix cores, so at every batch size.  DeepSeek-V3 router shape (256
@@ -1039,13 +1025,9 @@ hipError_t dispatch_router_batch(const RouterArgs& a, int R, hipStream_t s) {
   // Many rows and many tokens: a thread takes two tokens as well (each w value read from LDS
   // serves two chains, eight independent f64 chains per thread) while the grid still covers
   // the chip.
-  static const int forced = [] {
-    const char* e = getenv("ATENIA_MOE_ROUTER_TPT");  // tuning knob: tokens per thread (1, 2)
-    return e ? atoi(e) : 0;
-  }();
   // measured on MI355X at 64 rows, d = 2048: two tokens per thread pay from 8192 tokens on
   const long long work = (long long)a.T * ((R + 63) / 64);  // row blocks count like more tokens
-  const int tpt = forced ? forced : (work >= 8192 ? 2 : 1);
+  const int tpt = work >= 8192 ? 2 : 1;
   if (tpt >= 2) return launch_router_batch<XT, 4, 2, 64>(a, s);
   return launch_router_batch<XT, 4, 1, 64>(a, s);
 }
