@@ -15,9 +15,11 @@ pytestmark = pytest.mark.gpu
 @pytest.mark.parametrize("wd,T,k,shared", [(capi.WEIGHT_BF16, 1, 2, False), (capi.WEIGHT_BF16, 8, 3, True),
                                            (capi.WEIGHT_INT8_W8A16, 1, 2, False), (capi.WEIGHT_BF16, 300, 2, False),
                                            (capi.WEIGHT_BF16, 100, 2, True), (capi.WEIGHT_INT8_W8A16, 150, 2, False),
-                                           # tiled kernels with a shared expert: eager calls put its launches
-                                           # on the handle's second stream, a captured one must not
-                                           (capi.WEIGHT_BF16, 700, 2, True)])
+                                           # tiled kernels with a shared expert: a bf16 layer carries its
+                                           # tiles in the routed experts' launches; an int8 layer's eager calls
+                                           # put its launches on the handle's second stream, a captured one
+                                           # must not
+                                           (capi.WEIGHT_BF16, 700, 2, True), (capi.WEIGHT_INT8_W8A16, 700, 2, True)])
 def test_forward_replays_from_a_graph(ora, wd, T, k, shared):
     d = 256
     W = S.make_weights(40 + T, 8, d, 512, f_s=128 if shared else 0, gated=shared, router_std=1.0 / 16.0)
