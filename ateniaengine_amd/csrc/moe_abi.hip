@@ -15,6 +15,7 @@
 #include <atomic>
 #include <thread>
 #include <mutex>
+#include <memory>
 #include <new>
 #include <string>
 #include <vector>
@@ -1247,12 +1248,21 @@ int ensure_host_staging(AteniaMoeLayer* L) {
 
 // The staging copies (pageable caller memory <-> page-locked slots) are what the calling thread
 // would otherwise spend most of the call on: one core moves about half of what the copy engine
-// does.  For the length of a staged call a few helper threads take a slice of every chunk each
-// (tuning knob ATENIA_MOE_HOST_COPY_THREADS, read once: threads in all, 1 = the caller alone).
+// does.  For each of the two copy phases of a staged call (input in, output out -- not while the
+// forward itself runs, during which helpers would only spin) a few helper threads take a slice
+// of every chunk each (tuning knob ATENIA_MOE_HOST_COPY_THREADS, read once: threads in all,
+// 1 = the caller alone).  A thread that cannot be started is done without.
 class CopyCrew {
  public:
   explicit CopyCrew(int helpers) {
-    for (int i = 0; i < helpers; ++i) th_.emplace_back([this, i] { run(i + 1); });
+    th_.reserve(helpers > 0 ? helpers : 0);
+    for (int i = 0; i < helpers; ++i) {
+      try {
+        th_.emplace_back([this, i] { run(i + 1); });
+      } catch (...) {  // no exception may cross the C boundary: copy with the threads there are
+        break;
+      }
+    }
   }
   ~CopyCrew() {
     quit_ = true;
@@ -1306,28 +1316,34 @@ int host_copy_threads() {
 int forward_host_staged(AteniaMoeLayer* L, const float* x_host, int T, float* out_host) {
   int rc = ensure_host_staging(L);
   if (rc) return rc;
-  CopyCrew crew(host_copy_threads() - 1);
   const size_t row = (size_t)L->d * 4;
   const int n_chunks = (T + kHostChunkTokens - 1) / kHostChunkTokens;
   auto tokens_of = [&](int c) { return std::min(kHostChunkTokens, T - c * kHostChunkTokens); };
-  for (int c = 0; c < n_chunks; ++c) {
-    const int slot = c & 1;
-    const size_t off = (size_t)c * kHostChunkTokens * row, bytes = (size_t)tokens_of(c) * row;
-    // the slot is free once the copy of chunk c - 2 has left it
-    if (c >= 2) HIP_TRY(hipEventSynchronize(L->ev_h2d[slot]));
-    crew.copy((char*)L->pin_in + slot * L->pin_bytes, (const char*)x_host + off, bytes);
-    HIP_TRY(hipMemcpyAsync((char*)L->x_in.p + off, (char*)L->pin_in + slot * L->pin_bytes, bytes,
-                           hipMemcpyHostToDevice, L->stream));
-    HIP_TRY(hipEventRecord(L->ev_h2d[slot], L->stream));
+  {
+    CopyCrew crew(host_copy_threads() - 1);
+    for (int c = 0; c < n_chunks; ++c) {
+      const int slot = c & 1;
+      const size_t off = (size_t)c * kHostChunkTokens * row, bytes = (size_t)tokens_of(c) * row;
+      // the slot is free once the copy of chunk c - 2 has left it
+      if (c >= 2) HIP_TRY(hipEventSynchronize(L->ev_h2d[slot]));
+      crew.copy((char*)L->pin_in + slot * L->pin_bytes, (const char*)x_host + off, bytes);
+      HIP_TRY(hipMemcpyAsync((char*)L->x_in.p + off, (char*)L->pin_in + slot * L->pin_bytes, bytes,
+                             hipMemcpyHostToDevice, L->stream));
+      HIP_TRY(hipEventRecord(L->ev_h2d[slot], L->stream));
+    }
   }
   rc = run_forward(L, L->x_in.p, ATENIA_MOE_ACT_F32, T, L->out.as<float>(), L->stream,
                    kStageRouter, kStageCombine);
   if (rc) return rc;
+  std::unique_ptr<CopyCrew> crew;  // started when the first output chunk has arrived
   auto drain = [&](int c) -> int {  // chunk c's output: staging -> caller
     const int slot = c & 1;
     HIP_TRY(hipEventSynchronize(L->ev_d2h[slot]));
-    crew.copy((char*)out_host + (size_t)c * kHostChunkTokens * row,
-              (char*)L->pin_out + slot * L->pin_bytes, (size_t)tokens_of(c) * row);
+    if (!crew) crew.reset(new (std::nothrow) CopyCrew(host_copy_threads() - 1));
+    void* dst = (char*)out_host + (size_t)c * kHostChunkTokens * row;
+    const void* src = (char*)L->pin_out + slot * L->pin_bytes;
+    if (crew) crew->copy(dst, src, (size_t)tokens_of(c) * row);
+    else memcpy(dst, src, (size_t)tokens_of(c) * row);
     return ATENIA_MOE_OK;
   };
   for (int c = 0; c < n_chunks; ++c) {
