@@ -332,7 +332,7 @@ def measure_dequant(torch, capi, steps, warmup, seed):
 
 
 # Batch sizes the benchmark list names per configuration (decode and prefill points).
-BASELINE_SWEEPS = {
+BENCHMARK_SWEEPS = {
     "tiny_f32": (64,),
     "mixtral_bf16": (1, 16, 128, 512, 4096),
     "mixtral_int8": (1, 16, 4096),
@@ -655,10 +655,10 @@ def main():
         parities = {a.config: parity}
         layer.close()
         del ctx, layer, x_head, out_head
-        for name in BASELINE_SWEEPS:
+        for name in BENCHMARK_SWEEPS:
             if name == a.config:
                 continue
-            ts = BASELINE_SWEEPS[name]
+            ts = BENCHMARK_SWEEPS[name]
             ctx = build_config(torch, np, capi, name, a.seed, max(ts))
             xo = None
             for t in ts:
