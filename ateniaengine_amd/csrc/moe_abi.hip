@@ -140,6 +140,9 @@ struct AteniaMoeLayer {
   DevBuf w_router, router_bias, shared_gate;
   bool router_fits_bf16 = false;  // every router / gate value is exactly a bf16 value
   DevBuf router_lsb;              // [E + 1] i32: lowest last-bit exponent of each router row / the gate
+  DevBuf router_t8;               // bf16 [ceil(d / 32) * 4][router_rows_pad][8]: RouterArgs::w_t8
+  DevBuf router_norm2;            // f64 [router_rows_pad]: squared norms of the stacked rows
+  int router_rows_pad = 0;
   DevBuf wg, wu, wd, sg, su, sd;        // routed experts
   DevBuf swg, swu, swd, ssg, ssu, ssd;  // shared expert
   WeightSet gate{}, up{}, down{}, s_gate{}, s_up{}, s_down{};
@@ -839,6 +842,9 @@ int run_forward_impl(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, flo
   ra.w_router = L->w_router.as<float>();
   ra.w_fits_bf16 = L->router_fits_bf16;
   ra.w_lsb_min = L->router_lsb.as<int32_t>();
+  ra.w_t8 = L->router_t8.as<uint16_t>();
+  ra.w_rows_pad = L->router_rows_pad;
+  ra.w_norm2 = L->router_norm2.as<double>();
   ra.router_bias = L->router_bias.as<float>();
   const bool gated = L->fs > 0 && L->conv == ATENIA_MOE_CONVENTION_HUGGINGFACE_QWEN &&
                      L->shared_gate.p != nullptr && L->v3_n_group == 0;
@@ -1479,6 +1485,32 @@ int atenia_moe_hip_layer_create(const AteniaMoeLayerDesc* D, AteniaMoeLayer** ou
     if ((rc = L->router_lsb.ensure(lsb.size() * 4))) return bail(rc);
     if (hipMemcpy(L->router_lsb.p, lsb.data(), lsb.size() * 4, hipMemcpyHostToDevice) != hipSuccess)
       return bail(fail(ATENIA_MOE_ERR_LAUNCH, "upload of the router row table failed"));
+    if (L->router_fits_bf16 && d % 8 == 0) {
+      // The copy the matrix-core router streams: bf16 (exact: the values fit), eight columns
+      // of all rows side by side, zero rows up to a multiple of 16 and zero chunks up to a
+      // multiple of 32 columns; and |row|^2 for its bound on sum|p|.
+      const size_t R = E + (D->shared_gate ? 1 : 0), Rp = (R + 15) / 16 * 16;
+      const size_t chunks = (d + 31) / 32 * 4;
+      std::vector<uint16_t> t8(chunks * Rp * 8, 0);
+      std::vector<double> n2(Rp, 0.0);
+      for (size_t r = 0; r < R; ++r) {
+        const float* row = r < E ? D->w_router + r * d : D->shared_gate;
+        double acc = 0.0;
+        for (size_t c = 0; c < d; ++c) {
+          uint32_t u;
+          memcpy(&u, row + c, 4);
+          t8[((c / 8) * Rp + r) * 8 + c % 8] = (uint16_t)(u >> 16);
+          acc += (double)row[c] * (double)row[c];
+        }
+        n2[r] = acc;
+      }
+      if ((rc = L->router_t8.ensure(t8.size() * 2)) || (rc = L->router_norm2.ensure(n2.size() * 8)))
+        return bail(rc);
+      if (hipMemcpy(L->router_t8.p, t8.data(), t8.size() * 2, hipMemcpyHostToDevice) != hipSuccess ||
+          hipMemcpy(L->router_norm2.p, n2.data(), n2.size() * 8, hipMemcpyHostToDevice) != hipSuccess)
+        return bail(fail(ATENIA_MOE_ERR_LAUNCH, "upload of the router's bf16 copy failed"));
+      L->router_rows_pad = (int)Rp;
+    }
   }
 
   DevBuf staging;

@@ -65,6 +65,12 @@ struct RouterArgs {
   const float* w_router;     // [E, d]
   int w_fits_bf16;           // every value of w_router and shared_gate is exactly a bf16 value
   const int32_t* w_lsb_min;  // [E + 1] lowest last-bit exponent of each router row / the gate (or null)
+  // bf16 copy of [w_router ; shared_gate] in chunk-major order [ceil(d / 32) * 4][w_rows_pad][8]
+  // (rows past the last one and columns past d are zeros) and the squared norm of each of its
+  // rows; both null unless w_fits_bf16 and d % 8 == 0.  What the matrix-core router reads.
+  const uint16_t* w_t8;
+  int w_rows_pad;         // multiple of 16
+  const double* w_norm2;  // [w_rows_pad]
   const float* router_bias;  // [E] or null
   const float* shared_gate;  // [d] or null
   int32_t* idx;              // [T, k]

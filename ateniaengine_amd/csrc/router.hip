@@ -515,9 +515,9 @@ hipError_t launch_router_batch(const RouterArgs& a, hipStream_t s) {
 // so the result differs from the reference's c-ascending sum only by the order of the f64
 // additions.  That is accepted only under the same two certificates as in router_token_kernel:
 //   interval : any order lands within g = d 2^-53 sum|p| of the true sum, and sum|p| is bounded
-//              here by |w_r| |x_t| (Cauchy-Schwarz; both norms are accumulated next to the
-//              matrix instructions); if [acc - 2g, acc + 2g] rounds to one f32 (one f32 sigmoid
-//              for the gate row) that value is the reference's;
+//              here by |w_r| |x_t| (Cauchy-Schwarz; |x_t|^2 is accumulated next to the matrix
+//              instructions, |w_r|^2 comes with the layer); if [acc - 2g, acc + 2g] rounds to
+//              one f32 (one f32 sigmoid for the gate row) that value is the reference's;
 //   exactness: for the few sums that fail it, one wave checks that every product is a multiple
 //              of 2^q and sum|p| < 2^(q+53), which makes every order exact (bf16-valued
 //              operands pass);
@@ -551,7 +551,26 @@ template <> struct XChunk<uint16_t> {
       f[2 * i + 1] = __uint_as_float(u[i] & 0xffff0000u);
     }
   }
+  // min(key, |bits| - 1 of each of the eight values) as unsigned numbers: magnitudes order like
+  // their bit patterns, and a zero wraps to the largest key, so the result names the smallest
+  // non-zero magnitude seen (bf16_key_lsb below turns it into a last-bit exponent).
+  __device__ inline uint32_t min_key(uint32_t key) const {
+    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      key = min(key, min((u[i] & 0x7fffu) - 1u, ((u[i] >> 16) & 0x7fffu) - 1u));
+    return key;
+  }
 };
+// A bf16 value with exponent field e is a multiple of 2^(e - 134) (2^-133 for a denormal), so
+// the exponent field of the smallest non-zero magnitude among some values bounds the last-bit
+// exponent of every one of them from below: cheaper to follow than the exact last set bit, and
+// the exactness test it feeds has bits to spare.  kNoLsb: every value was zero.  (An inf or a
+// NaN is not seen here; it makes the norm that the same test compares infinite or NaN.)
+constexpr uint32_t kNoKey = 0xffffffffu;
+__device__ inline int bf16_key_lsb(uint32_t key) {
+  return key == kNoKey ? kNoLsb : (int)((key + 1u) >> 7) - 134;
+}
 
 // Softmax + top-k from logits that another launch left in HBM, one wavefront per token (up to 64
 // experts; wave_select_token in select_wave.h).
@@ -571,7 +590,8 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
     const float* __restrict__ w_router, const float* __restrict__ bias,
     const float* __restrict__ gate_vec, int32_t* __restrict__ idx_out,
     float* __restrict__ w_out, float* __restrict__ sgate_out, int32_t* __restrict__ status,
-    float* __restrict__ logits_out, const int32_t* __restrict__ w_lsb) {
+    float* __restrict__ logits_out, const int32_t* __restrict__ w_lsb,
+    const uint16_t* __restrict__ w_t8, int Rp, const double* __restrict__ w_norm2) {
   // gridDim.y > 1 (only with logits_out): this workgroup owns the rows row0 .. row0 + R - 1 of
   // the stacked matrix [W_r ; gate] and leaves the logits to another launch; otherwise all rows.
   constexpr int TT = 16;
@@ -587,26 +607,33 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
   constexpr int NT = 64 * NWV;                    // NWV waves split k
   double* sPart = smem_m;                         // [NWV][RB][4][64] partial sums
   double* sXsq = sPart + NWV * RB * 4 * 64;       // [NWV][16]  partial |x_t|^2
-  double* sWsq = sXsq + NWV * 16;                 // [NWV][RB][16] partial |w_r|^2
-  double* sAcc = sWsq + NWV * RB * 16;            // [16][R]
+  double* sAcc = sXsq + NWV * 16;                 // [16][R]
   double* sXn2 = sAcc + 16 * R;                   // [16]
   double* sWn2 = sXn2 + 16;                       // [R]
   float* sLogit = (float*)(sWn2 + R);             // [16][R]
-  int* sXq = (int*)(sLogit + 16 * R);             // [NWV][16] lowest last-bit exponent of x_t (partial)
+  uint32_t* sXq = (uint32_t*)(sLogit + 16 * R);   // [NWV][16] key of the smallest |x_t| (partial)
   uint8_t* sFlag = (uint8_t*)(sXq + NWV * 16);    // [16][R] 1 = the interval certificate failed
-  // Several row blocks: the matrix instructions of a step leave the VALU time to follow the
-  // lowest last-bit exponent of the token's activations as well (with one block they would not).
+  // A lower bound of the last-bit exponent of the token's activations is followed beside the
+  // matrix instructions when there are several row blocks.  f64 matrix instructions and vector
+  // instructions do not overlap on this chip (a step costs the sum of both), and with one block
+  // of 8 matrix instructions per step the extra ones cost more than the second looks they
+  // save: 25.8 -> 27.6 us on 8 rows, d = 4096.
   constexpr bool kTrackLsb = RB >= 2;
-  int xq = kNoLsb;
+  static_assert(sizeof(XT) == 2, "the last-bit bound below reads bf16 bit patterns");
+  uint32_t xq = kNoKey;
 
   const int tok = min(t0 + r16, T - 1);  // rows past T repeat the last token; never written out
   const XT* px = x + (size_t)tok * d + 8 * q;
-  const float* pw[RB];
+  // The stacked matrix comes from its bf16 copy in chunk-major order [d / 8][Rp][8] (made when
+  // the layer is created; rows past the last one and chunks past d are zeros): the 16 rows of a
+  // block lie side by side, so a load instruction reads 4 x 256 contiguous bytes instead of 64
+  // bytes from each of 16 rows -- the row-major f32 matrix cost the load path a fifth of the
+  // loop -- and neither a clamp nor a select is needed.
+  const uint16_t* pw[RB];
 #pragma unroll
-  for (int b = 0; b < RB; ++b) {
-    const int r = row0 + min(16 * b + r16, R - 1);
-    pw[b] = (r < E ? w_router + (size_t)r * d : gate_vec) + 8 * q;
-  }
+  for (int b = 0; b < RB; ++b) pw[b] = w_t8 + ((size_t)q * Rp + row0 + 16 * b + r16) * 8;
+  const size_t w_step = (size_t)32 * Rp;  // four chunks
+  if (tid < R) sWn2[tid] = w_norm2[row0 + tid];  // |w_r|^2, read after the barriers below
   // k in steps of 32 (8 per lane), the steps dealt to the four waves in contiguous runs
   const int nsteps = (d + 31) / 32;
   const int per = (nsteps + NWV - 1) / NWV;
@@ -622,12 +649,10 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
   for (int b = 0; b < RB; ++b)
 #pragma unroll
     for (int n = 0; n < NACC; ++n) acc[b][n] = f64x4_t{0.0, 0.0, 0.0, 0.0};
-  double xsq = 0.0, wsq[RB];
-#pragma unroll
-  for (int b = 0; b < RB; ++b) wsq[b] = 0.0;
+  double xsq = 0.0;
 
   XChunk<XT> xc[NBUF];
-  XChunk<float> wc[NBUF][RB];
+  XChunk<uint16_t> wc[NBUF][RB];
   // Every step issues the same loads whatever the lane or the step: a chunk past d is fetched
   // from the row's first columns and zeroed with selects, a step past the wave's range repeats
   // its last one.  With a branch around a load the compiler can no longer count the loads in
@@ -640,20 +665,17 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
     xc[buf].load(px + off);
     xc[buf].keep(in);
 #pragma unroll
-    for (int b = 0; b < RB; ++b) {
-      wc[buf][b].load(pw[b] + off);
-      wc[buf][b].keep(in);
-    }
+    for (int b = 0; b < RB; ++b) wc[buf][b].load(pw[b] + (size_t)st * w_step);
   };
   auto multiply = [&](int buf) {
     float xf[8];
     xc[buf].get(xf);
+    if (kTrackLsb) xq = xc[buf].min_key(xq);
     double xd[8];
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
       xd[t] = (double)xf[t];
       xsq = fma(xd[t], xd[t], xsq);
-      if (kTrackLsb) xq = min(xq, lsb_exponent(xf[t]));
     }
 #pragma unroll
     for (int b = 0; b < RB; ++b) {
@@ -662,7 +684,6 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
 #pragma unroll
       for (int t = 0; t < 8; ++t) {
         const double wd = (double)wf[t];
-        wsq[b] = fma(wd, wd, wsq[b]);
         acc[b][t % NACC] = __builtin_amdgcn_mfma_f64_16x16x4f64(wd, xd[t], acc[b][t % NACC], 0, 0, 0);
       }
     }
@@ -685,10 +706,6 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
 #pragma unroll
     for (int r = 0; r < 4; ++r)
       sPart[((wave * RB + b) * 4 + r) * 64 + lane] = NACC == 2 ? acc[b][0][r] + acc[b][NACC - 1][r] : acc[b][0][r];
-    double v = wsq[b];
-    v += __shfl_xor(v, 16);
-    v += __shfl_xor(v, 32);
-    if (q == 0) sWsq[(wave * RB + b) * 16 + r16] = v;
   }
   {
     double v = xsq;
@@ -711,19 +728,18 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
   if (rr == 0) sXn2[t] = xn2;
   int xq_t = kNoLsb;
   if (kTrackLsb) {
+    uint32_t key = kNoKey;
 #pragma unroll
-    for (int w = 0; w < NWV; ++w) xq_t = min(xq_t, sXq[w * 16 + t]);
+    for (int w = 0; w < NWV; ++w) key = min(key, sXq[w * 16 + t]);
+    xq_t = bf16_key_lsb(key);
   }
   const double gfac = (double)(2 * d + 4) * 1.1102230246251565e-16 * 1.001;
   for (int r = rr; r < R; r += NT / 16) {
     const int b = r >> 4, rho = r & 15, reg = rho >> 2, qq = rho & 3;
-    double a = 0.0, wn2 = 0.0;
+    double a = 0.0;
 #pragma unroll
-    for (int w = 0; w < NWV; ++w) {
-      a += sPart[((w * RB + b) * 4 + reg) * 64 + qq * 16 + t];
-      wn2 += sWsq[(w * RB + b) * 16 + rho];
-    }
-    if (t == 0) sWn2[r] = wn2;
+    for (int w = 0; w < NWV; ++w) a += sPart[((w * RB + b) * 4 + reg) * 64 + qq * 16 + t];
+    const double wn2 = sWn2[r];
     // sum|p| <= |w_r| |x_t|; the factor 1.001 covers the roundings of the norms and the root
     const double e = sqrt(xn2 * wn2) * gfac;
     const double lo = a - e, hi = a + e;
@@ -882,9 +898,8 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
     for (int j = 0; j < TPW; ++j) {
       const int tk = wave + j * NWV;
       const float my = on ? sLogit[tk * R + lane] : -INFINITY;
-      float mx = fmaxf(-INFINITY, my);  // a NaN logit is skipped, as f32::max skips it
-#pragma unroll
-      for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+      // a NaN logit is skipped, as f32::max skips it
+      const float mx = wave_max_f32(fmaxf(-INFINITY, my));
       ex[j] = on ? exp((double)(my - mx)) : 0.0;  // f32 subtraction, then f64 exp
       sExp[tk * 64 + lane] = ex[j];
     }
@@ -899,17 +914,21 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
       sInv[tid] = sum > 0.0 ? 1.0 / sum : 0.0;
     }
     __syncthreads();
+    float wt[TPW];
+    int token[TPW];
+    bool valid[TPW];
 #pragma unroll
     for (int j = 0; j < TPW; ++j) {
       const int tk = wave + j * NWV;
-      if (t0 + tk >= T) break;  // wave-uniform
-      const float wt = (float)(ex[j] * sInv[tk]);
-      if (on && (!isfinite(wt) || wt < 0.f)) {
+      token[j] = t0 + tk;
+      valid[j] = token[j] < T;  // wave-uniform
+      wt[j] = (float)(ex[j] * sInv[tk]);
+      if (valid[j] && on && (!isfinite(wt[j]) || wt[j] < 0.f)) {
         atomicMin(&status[0], -3);
-        atomicMin(&status[1], ((t0 + tk) << 10) | lane);
+        atomicMin(&status[1], (token[j] << 10) | lane);
       }
-      wave_topk_write(wt, on, lane, k, renorm, t0 + tk, idx_out, w_out);
     }
+    wave_topk_write_n<TPW>(wt, on, lane, k, renorm, token, valid, idx_out, w_out);
     return;
   }
   // the partial-sum area is free now: softmax scratch
@@ -923,12 +942,15 @@ __global__ __launch_bounds__(64 * NWV) void router_mfma_kernel(
 
 template <typename XT, int RB, int NBUF, int NWV>
 hipError_t launch_router_mfma_rb(const RouterArgs& a, int R, hipStream_t s) {
-  const size_t smem = ((size_t)NWV * RB * 4 * 64 + NWV * 16 + (size_t)NWV * RB * 16 + (size_t)16 * R + 16 + R) * 8 +
+  const size_t smem = ((size_t)NWV * RB * 4 * 64 + NWV * 16 + (size_t)16 * R + 16 + R) * 8 +
                       (size_t)16 * R * 4 + (size_t)NWV * 16 * 4 + (size_t)16 * R + 16;
-  if (smem > 64 * 1024) return hipErrorInvalidValue;
+  if (smem > 64 * 1024 || 16 * RB > a.w_rows_pad) return hipErrorInvalidValue;
+  // (The selection stays inside this kernel, four tokens per wave: with the logits in HBM and a
+  // second launch that gives every token a wave of its own the route stage measured 3-8 us
+  // longer at 8192-16384 tokens.)
   router_mfma_kernel<XT, RB, NBUF, NWV><<<(a.T + 15) / 16, 64 * NWV, smem, s>>>(
       (const XT*)a.x, a.T, a.d, a.E, a.k, a.renorm, a.w_router, a.router_bias, a.shared_gate,
-      a.idx, a.w, a.sgate, a.status, nullptr, a.w_lsb_min);
+      a.idx, a.w, a.sgate, a.status, nullptr, a.w_lsb_min, a.w_t8, a.w_rows_pad, a.w_norm2);
   return hipGetLastError();
 }
 
@@ -946,11 +968,13 @@ __global__ __launch_bounds__(kSelectThreads) void softmax_select_kernel(
 template <typename XT>
 hipError_t launch_router_mfma_split(const RouterArgs& a, int R, hipStream_t s) {
   constexpr int NWV = 8, RB = 1, RL = 16;
-  const size_t smem = ((size_t)NWV * RB * 4 * 64 + NWV * 16 + (size_t)NWV * RB * 16 + (size_t)16 * RL + 16 + RL) * 8 +
+  const size_t smem = ((size_t)NWV * RB * 4 * 64 + NWV * 16 + (size_t)16 * RL + 16 + RL) * 8 +
                       (size_t)16 * RL * 4 + (size_t)NWV * 16 * 4 + (size_t)16 * RL + 16;
+  if ((R + 15) / 16 * 16 > a.w_rows_pad) return hipErrorInvalidValue;
   router_mfma_kernel<XT, RB, 4, NWV><<<dim3((a.T + 15) / 16, (R + 15) / 16), 64 * NWV, smem, s>>>(
       (const XT*)a.x, a.T, a.d, a.E, a.k, a.renorm, a.w_router, a.router_bias, a.shared_gate,
-      a.idx, a.w, a.sgate, a.status, a.logits_out ? a.logits_out : a.logits_tmp, a.w_lsb_min);
+      a.idx, a.w, a.sgate, a.status, a.logits_out ? a.logits_out : a.logits_tmp, a.w_lsb_min,
+      a.w_t8, a.w_rows_pad, a.w_norm2);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || a.logits_out) return e;  // the caller's own launch routes from the logits
   if (a.E <= 64) {
@@ -979,7 +1003,7 @@ bool router_mfma_ok(const RouterArgs& a, int R) {
   // f32 values fit bf16: otherwise every sum the interval test flags (one in a thousand) costs a
   // sequential chain in its workgroup, and the launch lasts as long as the slowest of them.
   const bool operands = !off && a.d % 8 == 0 && !a.xb && a.x_is_bf16 &&
-                        a.w_fits_bf16 && a.E >= a.k;
+                        a.w_fits_bf16 && a.w_t8 && a.w_norm2 && a.E >= a.k;
   if (R < 0) return operands;  // the form that deals the rows to workgroups takes any row count
   return operands && R <= 80 && !a.logits_out;
 }
@@ -1275,8 +1299,7 @@ hipError_t launch_router(const RouterArgs& a, hipStream_t s, int* fused_permute)
   // (row blocks, logits mode) that only pays for a handful of tokens.
   const bool mfma = router_mfma_ok(a, R);
   if (router_mfma_split_wanted(a, R))
-    return a.x_is_bf16 ? launch_router_mfma_split<uint16_t>(a, R, s)
-                       : launch_router_mfma_split<float>(a, R, s);
+    return launch_router_mfma_split<uint16_t>(a, R, s);  // bf16 activations only (router_mfma_ok)
   const bool token_ok = a.T <= a.token_kernel_max_tokens &&
                         (R <= 64 || (long long)a.T * R * a.d <= (16ll << 20));
   if (token_ok) {
@@ -1334,7 +1357,7 @@ hipError_t launch_router(const RouterArgs& a, hipStream_t s, int* fused_permute)
     }
   }
   if (mfma)
-    return a.x_is_bf16 ? launch_router_mfma<uint16_t>(a, R, s) : launch_router_mfma<float>(a, R, s);
+    return launch_router_mfma<uint16_t>(a, R, s);
   // Up to 64 rows per workgroup; more rows only when the logits leave the kernel (row blocks).
   if ((R <= 64 || a.logits_out) && a.d % 4 == 0 && (!a.xb || a.d_pad % 4 == 0)) {
     return a.x_is_bf16 ? dispatch_router_batch<uint16_t>(a, R, s)

@@ -120,6 +120,61 @@ __device__ inline void wave_topk_write(float wt, bool on, int lane, int k, int r
   }
 }
 
+// The same for N tokens of one wave at once (lane r = expert r of each): the N selections are
+// independent chains of cross-lane steps, and run interleaved they hide each other's latency.
+// Token j is written only when valid[j].  Same results as N calls of wave_topk_write.
+template <int N>
+__device__ inline void wave_topk_write_n(const float (&wt)[N], bool on, int lane, int k, int renorm,
+                                         const int (&token)[N], const bool (&valid)[N],
+                                         int32_t* __restrict__ idx_out, float* __restrict__ w_out) {
+  int wbits[N];
+  unsigned long long avail[N], mask[N];
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    wbits[j] = on ? __float_as_int(wt[j]) : -1;
+    avail[j] = ~0ull;
+    mask[j] = 0ull;
+  }
+  for (int r = 0; r < k; ++r) {
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+      const int v = (avail[j] >> lane) & 1ull ? wbits[j] : -1;
+      const int m = wave_max_i32(v);
+      const unsigned long long cand = __ballot(v == m && m >= 0);
+      const unsigned long long win = cand & (~cand + 1ull);  // nothing left: no bit, no change
+      mask[j] |= win;
+      avail[j] &= ~win;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    if (!valid[j]) continue;  // wave-uniform
+    const bool selected = (mask[j] >> lane) & 1ull;
+    const int slot = __popcll(mask[j] & ((1ull << lane) - 1ull));
+    double ssum = 0.0;
+    for (unsigned long long m = mask[j]; m; m &= m - 1)
+      ssum += (double)readlane_f32(wt[j], __ffsll((long long)m) - 1);
+    const double scale = renorm ? 1.0 / ssum : 1.0;
+    if (selected && slot < k) {
+      const size_t o = (size_t)token[j] * k + slot;
+      idx_out[o] = lane;
+      w_out[o] = (float)((double)wt[j] * scale);
+    }
+  }
+}
+
+// Largest of 64 non-NaN floats, in every lane (the steps of wave_max_i32).
+__device__ inline float wave_max_f32(float f) {
+  int v = __float_as_int(f);
+  auto mx = [](int a, int b) { return __float_as_int(fmaxf(__int_as_float(a), __int_as_float(b))); };
+  v = mx(v, __builtin_amdgcn_update_dpp(v, v, 0xB1, 0xf, 0xf, false));
+  v = mx(v, __builtin_amdgcn_update_dpp(v, v, 0x4E, 0xf, 0xf, false));
+  v = mx(v, __builtin_amdgcn_update_dpp(v, v, 0x141, 0xf, 0xf, false));
+  v = mx(v, __builtin_amdgcn_update_dpp(v, v, 0x140, 0xf, 0xf, false));
+  return fmaxf(fmaxf(readlane_f32(__int_as_float(v), 0), readlane_f32(__int_as_float(v), 16)),
+               fmaxf(readlane_f32(__int_as_float(v), 32), readlane_f32(__int_as_float(v), 48)));
+}
+
 // Softmax + top-k of token t from its logits row in memory, by one wavefront (up to 64 experts).
 // Same arithmetic, casts and order as softmax_topk in router.hip; the sequential fold of the
 // exponentials runs over v_readlane values.  Every lane of the wave must call.

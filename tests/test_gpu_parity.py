@@ -230,6 +230,38 @@ def test_router_matrix_core_kernel(ora, E, k, d, T, gated, bias, bf16_router, wi
         assert ulp_diff(w, o_w).max() <= 1
 
 
+@pytest.mark.parametrize("E,k,d,T,gated", [(60, 4, 512, 2300, True), (20, 3, 256, 2100, False),
+                                           (64, 6, 1024, 300, False), (8, 2, 512, 700, False)])
+def test_router_matrix_core_kernel_zeros_and_denormals(ora, E, k, d, T, gated):
+    """The bound that settles most flagged sums is taken from the exponent of a token's smallest
+    non-zero activation: exact zeros (half of all values here, and whole tokens) must not count,
+    and bf16 denormals (a multiple of 2^-133 each) must -- the routing stays the reference's."""
+    W = S.make_weights(140 + E, E, d, 32, f_s=32 if gated else 0, gated=gated,
+                       router_std=1.0 / np.sqrt(d))
+    W["w_router"] = S.bf16_round_trip(W["w_router"])[1]
+    if gated:
+        W["shared_gate"] = S.bf16_round_trip(W["shared_gate"])[1]
+    conv = capi.CONVENTION_HUGGINGFACE_QWEN if gated else capi.CONVENTION_ATENIA
+    oL, gL = S.build_pair(ora, W, k, conv, capi.WEIGHT_BF16)
+    rng = np.random.default_rng(150 + T)
+    bits = (S.make_tokens(160 + T, T, d, bf16=True).view(np.uint32) >> 16).astype(np.uint16)
+    bits[rng.random((T, d)) < 0.5] = 0
+    den = rng.random((T, d)) < 0.01
+    bits[den] = (rng.integers(1, 128, size=int(den.sum())) |
+                 (rng.integers(0, 2, size=int(den.sum())) << 15)).astype(np.uint16)
+    bits[5] = 0
+    bits[T - 1] = 0x8000  # a token of negative zeros
+    x = (bits.astype(np.uint32) << 16).view(np.float32)
+    with gL:
+        dx = DeviceArray.from_host(bits)
+        out = DeviceArray((T, d), np.float32, fill=0)
+        gL.forward_device(dx.ptr, capi.ACT_BF16, T, out.ptr)
+        idx, w, *_ = gL.last_routing(T)
+        o_idx, o_w = oL.route_tokens(x)
+        assert (idx == o_idx).all(), f"{(idx != o_idx).any(axis=1).sum()} tokens routed differently"
+        assert ulp_diff(w, o_w).max() <= 1
+
+
 def test_router_engineered_ties(ora):
     """Duplicate router rows give exactly equal weights; the lower index must win."""
     E, k, d, T = 8, 2, 64, 40
