@@ -223,10 +223,15 @@ def plan_batch(E: int, k: int, d: int, f: int, f_s: int, weight_dtype: int, T: i
                group_size: int = 0) -> dict:
     """Which kernels a T-token batch takes on a layer of these dimensions (no device needed):
     kernel family per phase for the routed and the shared expert (KERNELS_*; -1 = none), whether
-    the expert outputs reach the combine as bf16, tall row tiles, two-workgroup form per phase."""
+    the expert outputs reach the combine as bf16, tall row tiles, two-workgroup form per phase
+    (`duo`, bits 0 and 1), and `int8_copy`: a W8A16 layer's tiled phases on the bf16 copy of its
+    int8 values."""
     v = np.zeros(8, dtype=np.int32)
     _check(lib().atenia_moe_hip_plan_batch(E, k, d, f, f_s, weight_dtype, group_size, T, _ptr(v)))
-    return dict(zip(PLAN_KEYS, (int(i) for i in v)))
+    plan = dict(zip(PLAN_KEYS, (int(i) for i in v)))
+    plan["int8_copy"] = (plan["duo"] >> 2) & 1
+    plan["duo"] &= 3
+    return plan
 
 
 def f32_to_bf16_trunc(a) -> np.ndarray:

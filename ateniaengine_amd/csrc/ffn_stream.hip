@@ -1211,7 +1211,8 @@ __global__ void dequant_group_blocks_kernel(const uint4* __restrict__ q,
   const int nb = (int)(strip % (n_pad / 16));
   const size_t g = strip / (n_pad / 16);
   const int row = nb * 16 + (lane & 15), q4 = lane >> 4;
-  const float sc = scales[(g * n_kgroups + kb / group_blocks) * n_pad + row];
+  // no scales: the int8 values themselves (every one is a bf16 value)
+  const float sc = scales ? scales[(g * n_kgroups + kb / group_blocks) * n_pad + row] : 1.f;
   const uint4 v = q[slot];
   const uint32_t w[4] = {v.x, v.y, v.z, v.w};
   uint32_t o[8];

@@ -233,8 +233,11 @@ constexpr int kXaStage = 256;  // uint4 per stage
 
 // YB (down phase only): y leaves as bf16 (TiledParams::out_bf16), staged through LDS.
 // The tile of workgroup `bid` of a launch described by p.
-template <bool UP, bool YB>
+// SC: the weights are the int8 values of a W8A16 layer widened to bf16 (exactly), and the f32
+// accumulators are multiplied by the per-row scales p.sa / p.sb [E, n_rows] on their way out.
+template <bool UP, bool YB, bool SC = false>
 __device__ __forceinline__ void pipe_tile(const TiledParams& p, int bid) {
+  static_assert(!(SC && YB), "scaled outputs are stored as f32");
   constexpr int NA = kRingA, NB = kRingB;
   constexpr int XA0 = NA * 2048 + NB * 1024;            // first uint4 of the extra-rows ring
   __shared__ uint4 S[XA0 + NA * kXaStage];              // A ring, B ring, extra-rows ring
@@ -569,18 +572,31 @@ __device__ __forceinline__ void pipe_tile(const TiledParams& p, int bid) {
     if (UP) {  // gate in accx[0], up in accx[1], this wave's 32 x 32 block
       uint16_t* h = (uint16_t*)p.out;
       const int n = nb0 * 16 + (2 * wn + wm) * 32 + l32;
+      float sg = 1.f, su = 1.f;
+      if (SC) {
+        const size_t at = (size_t)e * p.n_rows + min(n, p.n_rows - 1);
+        sg = p.sa[at];
+        su = p.sb[at];
+      }
       if (n < p.n_blocks * 16) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int mrow = TM + 8 * (r >> 2) + 4 * kh + (r & 3);
           if (mrow < rows_here)
-            h[(size_t)(base + tm0 + mrow) * p.out_stride + n] =
-                (uint16_t)bf16_rne_pair(swiglu_fast(accx[0][r], accx[1][r]), 0.f);
+            h[(size_t)(base + tm0 + mrow) * p.out_stride + n] = (uint16_t)bf16_rne_pair(
+                SC ? swiglu_fast(accx[0][r] * sg, accx[1][r] * su) : swiglu_fast(accx[0][r], accx[1][r]), 0.f);
         }
       }
     } else {  // column groups 4 wn + 2 wm, + 1 of this wave
       float* y = (float*)p.out + (size_t)part * p.out_part_stride;
       uint16_t* yb = (uint16_t*)p.out + (size_t)part * p.out_part_stride;
+      float sx[2] = {1.f, 1.f};
+      if (SC) {
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj)
+          sx[jj] = p.sa[(size_t)e * p.n_rows +
+                        min(nb0 * 16 + (4 * wn + 2 * wm + jj) * 32 + l32, p.n_rows - 1)];
+      }
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int m = TM + 8 * (r >> 2) + 4 * kh + (r & 3);
@@ -595,7 +611,7 @@ __device__ __forceinline__ void pipe_tile(const TiledParams& p, int bid) {
           const int n = nb0 * 16 + (4 * wn + 2 * wm + jj) * 32 + l32;
           if (n < p.n_rows) {
             if (YB) ybr[n] = (uint16_t)bf16_rne_pair(accx[jj][r], 0.f);
-            else yr[n] = accx[jj][r];
+            else yr[n] = SC ? accx[jj][r] * sx[jj] : accx[jj][r];
           }
         }
       }
@@ -620,13 +636,22 @@ __device__ __forceinline__ void pipe_tile(const TiledParams& p, int bid) {
     char* stage = (char*)S + wave * (128 * kPitch);
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
+      float sg = 1.f, su = 1.f;
+      if (SC) {
+        const size_t at = (size_t)e * p.n_rows + min(nb0 * 16 + (2 * wn + j) * 32 + l32, p.n_rows - 1);
+        sg = p.sa[at];
+        su = p.sb[at];
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
 #pragma unroll
         for (int r = 0; r < 16; r += 2) {  // rows m and m + 1
           const int m = i * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
-          const uint32_t hh = bf16_rne_pair(swiglu_fast(acc[i][j][r], acc[i][j + 2][r]),
-                                            swiglu_fast(acc[i][j][r + 1], acc[i][j + 2][r + 1]));
+          const uint32_t hh =
+              SC ? bf16_rne_pair(swiglu_fast(acc[i][j][r] * sg, acc[i][j + 2][r] * su),
+                                 swiglu_fast(acc[i][j][r + 1] * sg, acc[i][j + 2][r + 1] * su))
+                 : bf16_rne_pair(swiglu_fast(acc[i][j][r], acc[i][j + 2][r]),
+                                 swiglu_fast(acc[i][j][r + 1], acc[i][j + 2][r + 1]));
           char* dst = stage + m * kPitch + (j * 32 + l32) * 2;
           *(uint16_t*)dst = (uint16_t)hh;
           *(uint16_t*)(dst + kPitch) = (uint16_t)(hh >> 16);
@@ -694,6 +719,12 @@ __device__ __forceinline__ void pipe_tile(const TiledParams& p, int bid) {
     // The pair id of every row first, in one batch of loads: fetched next to the stores they
     // address, each would wait out its own L2 round trip (the compiler cannot move a load of
     // perm above a store to y).
+    float sd[4] = {1.f, 1.f, 1.f, 1.f};
+    if (SC) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        sd[j] = p.sa[(size_t)e * p.n_rows + min(nb0 * 16 + (4 * wn + j) * 32 + l32, p.n_rows - 1)];
+    }
     int pair_of[4][16];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -715,16 +746,16 @@ __device__ __forceinline__ void pipe_tile(const TiledParams& p, int bid) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const int n = nb0 * 16 + (4 * wn + j) * 32 + l32;
-          if (n < p.n_rows) yr[n] = acc[i][j][r];
+          if (n < p.n_rows) yr[n] = SC ? acc[i][j][r] * sd[j] : acc[i][j][r];
         }
       }
     }
   }
 }
 
-template <bool UP, bool YB = false>
+template <bool UP, bool YB = false, bool SC = false>
 __global__ __launch_bounds__(kThreads) void ffn_tiled_pipe_kernel(TiledParams p) {
-  pipe_tile<UP, YB>(p, (int)blockIdx.x);
+  pipe_tile<UP, YB, SC>(p, (int)blockIdx.x);
 }
 
 // Gate/up launch of the routed experts and of a shared expert in one grid: workgroups below
@@ -1049,7 +1080,10 @@ hipError_t launch_tiled_dma(TiledParams p, int max_row_tiles, hipStream_t s) {
   n_wg = (n_wg + 7) / 8 * 8;
   p.wg_upper = n_wg;
   const int extra = p.max_parts > 1 ? p.n_cus : 0;  // room for the extra k ranges of a tail round
-  if (!UP && p.out_bf16) {
+  if (p.sa) {  // int8 values widened to bf16: scaled f32 results
+    if (p.out_bf16 || (UP && !p.sb)) return hipErrorInvalidValue;
+    ffn_tiled_pipe_kernel<UP, false, true><<<n_wg + extra, kThreads, 0, s>>>(p);
+  } else if (!UP && p.out_bf16) {
     if (p.n_rows % 8) return hipErrorInvalidValue;  // a lane stores 8 columns at once
     ffn_tiled_pipe_kernel<false, true><<<n_wg + extra, kThreads, 0, s>>>(p);
   } else {
@@ -1115,7 +1149,7 @@ TiledParams up_params(const FfnArgs& a) {
 bool up_takes_pipe_bf16(const FfnArgs& a) {
   return a.use_tiled && !a.use_duo && a.wdtype != ATENIA_MOE_WEIGHT_INT8_W8A16 &&
          a.wdtype != ATENIA_MOE_WEIGHT_F32 && a.gate.group_blocks == 0 && a.gate.k_pad % 64 == 0 &&
-         a.gate.k_pad >= 128 && (!a.tall_tiles || (a.tile_rows && a.tile_li));
+         a.gate.k_pad >= 128 && (!a.tall_tiles || (a.tile_rows && a.tile_li)) && !a.gate.scale;
 }
 }  // namespace
 
@@ -1143,13 +1177,14 @@ hipError_t launch_ffn_up_tiled(const FfnArgs& a, hipStream_t s) {
   // A list of nine-group tiles in any other kernel would lose the rows past 256 of such a tile.
   if (a.tall_tiles && (!pipe_bf16 || a.use_duo || !p.tile_rows || !p.tile_li)) return hipErrorInvalidValue;
   if (a.use_duo) {
-    if (!pipe_bf16) return hipErrorInvalidValue;
+    if (!pipe_bf16 || p.sa) return hipErrorInvalidValue;
     p.tile_rows = nullptr;
     p.tile_li = nullptr;
     p.n_cus = a.n_cus;
     return launch_tiled_duo_up(p, a.max_row_tiles, s);
   }
   if (pipe_bf16) return launch_tiled_dma<true>(p, a.max_row_tiles, s);
+  if (!int8 && p.sa) return hipErrorInvalidValue;  // scaled bf16 values: that kernel only
   if (int8 && p.k_pad >= 128) return launch_tiled_pipe_i8<true>(p, a.max_row_tiles, s);
   return int8 ? launch_tiled<true, true>(p, a.max_row_tiles, s)
               : launch_tiled<false, true>(p, a.max_row_tiles, s);
@@ -1195,7 +1230,7 @@ bool down_takes_pipe_bf16(const FfnArgs& a) {
   return a.use_tiled && !a.use_duo && a.wdtype != ATENIA_MOE_WEIGHT_INT8_W8A16 &&
          a.wdtype != ATENIA_MOE_WEIGHT_F32 && a.down.group_blocks == 0 && a.down.k_pad % 64 == 0 &&
          a.down.k_pad >= 128 && (!a.tall_tiles || (a.tile_rows && a.tile_li)) &&
-         (!a.y_bf16 || a.down.n_rows % 8 == 0);
+         (!a.y_bf16 || a.down.n_rows % 8 == 0) && !a.down.scale;
 }
 }  // namespace
 
@@ -1230,7 +1265,7 @@ hipError_t launch_ffn_down_tiled(const FfnArgs& a, hipStream_t s) {
   p.out_bf16 = a.y_bf16;
   if (a.use_duo) {
     // no k split of tail tiles in this form: the caller passes y_parts <= 1
-    if (!pipe_bf16 || (a.y_parts > 1 && a.part_flags)) return hipErrorInvalidValue;
+    if (!pipe_bf16 || p.sa || (a.y_parts > 1 && a.part_flags)) return hipErrorInvalidValue;
     p.tile_rows = nullptr;
     p.tile_li = nullptr;
     p.n_cus = a.n_cus;
@@ -1238,6 +1273,7 @@ hipError_t launch_ffn_down_tiled(const FfnArgs& a, hipStream_t s) {
   }
   if (pipelined) down_split_params(a, p);
   if (!int8 && p.k_pad % 64 == 0 && p.k_pad >= 128) return launch_tiled_dma<false>(p, a.max_row_tiles, s);
+  if (!int8 && p.sa) return hipErrorInvalidValue;  // scaled bf16 values: that kernel only
   if (int8 && p.k_pad >= 128) return launch_tiled_pipe_i8<false>(p, a.max_row_tiles, s);
   return int8 ? launch_tiled<true, false>(p, a.max_row_tiles, s)
               : launch_tiled<false, false>(p, a.max_row_tiles, s);

@@ -315,19 +315,23 @@ int upload_group_scales(const float* host, int G, int n_rows, int k_cols, int gr
   return ATENIA_MOE_OK;
 }
 
-// bf16 copy of a per-group int8 family (made on the first batch that takes the MFMA-tiled
-// kernels): same rows and K padding, bf16 blocks, value = bf16(q * scale of its group).
+// bf16 copy of an int8 family (made on the first batch that takes the MFMA-tiled kernels on it):
+// same rows and K padding, bf16 blocks.  Per-group scales: value = bf16(q * scale of its group),
+// no scales left.  One scale per row: value = q itself (exact in bf16), and the copy keeps the
+// row scales for the kernel's epilogue.
 int make_bf16_copy(const WeightSet& q, int G, DevBuf& dst, WeightSet& out) {
+  const bool per_group = q.group_blocks > 0;
   out = q;
-  out.scale = nullptr;
+  out.scale = per_group ? nullptr : q.scale;
   out.group_blocks = 0;
   out.n_kgroups = 0;
   out.expert_stride = (int64_t)q.n_pad * q.k_pad * 2;  // bytes
   int rc = dst.ensure((size_t)G * out.expert_stride);
   if (rc) return rc;
   out.w = dst.p;
-  HIP_TRY(launch_dequant_group_blocks(q.w, q.scale, dst.p, G, q.n_pad, q.k_pad, q.group_blocks,
-                                      q.n_kgroups, nullptr));
+  HIP_TRY(launch_dequant_group_blocks(q.w, per_group ? q.scale : nullptr, dst.p, G, q.n_pad, q.k_pad,
+                                      per_group ? q.group_blocks : 1, per_group ? q.n_kgroups : 1,
+                                      nullptr));
   return ATENIA_MOE_OK;
 }
 
@@ -478,6 +482,8 @@ struct BatchPlan {
   bool routed_streams;  // gate/up phase: weight-streaming kernels (either form), not the tiled ones
   bool routed_mid;      // gate/up phase in the mid-batch form (token rows shared through LDS)
   bool pg_prefill;      // per-group int8 layer running the tiled kernels on its bf16 copy
+  bool q_copy;          // W8A16 layer running the bf16 tiled kernels on a bf16 copy of its int8
+                        // values (exact), row scales applied to the f32 results
   bool tall_tiles;      // row tiles of up to nine 32-row groups (bf16 pipelined kernels only)
   bool duo_up, duo_down;  // tiled phase on the two-workgroups-per-compute-unit form (short K)
 };
@@ -487,6 +493,15 @@ int duo_max_k() {
   static const int v = [] {
     const char* e = getenv("ATENIA_MOE_DUO_MAX_K");
     return e ? atoi(e) : 0;
+  }();
+  return v;
+}
+// Rows per expert on average from which a W8A16 layer's tiled phases run on the bf16 copy of its
+// int8 values (tuning knob ATENIA_MOE_INT8_COPY_MIN_ROWS, read once; 0 = never, no copy is made).
+int int8_copy_min_rows() {
+  static const int v = [] {
+    const char* e = getenv("ATENIA_MOE_INT8_COPY_MIN_ROWS");
+    return e ? atoi(e) : 256;
   }();
   return v;
 }
@@ -636,7 +651,19 @@ BatchPlan plan_batch(const AteniaMoeLayer* L, int T) {
   p.pg_prefill = L->group_size > 0 && p.up == kFamTiled && L->d_kpad % 64 == 0 &&
                  L->f_kpad % 64 == 0 && (L->fs == 0 || L->fs_kpad % 64 == 0);
   // the routed experts on the bf16 pipelined kernel (K a multiple of 64, >= 128)
-  const bool bf16_tiles = L->wdtype == ATENIA_MOE_WEIGHT_BF16 || p.pg_prefill;
+  // W8A16: the int8 tiled kernel widens every weight in the VALU next to the matrix
+  // instructions and has no tiles of nine row groups; once a batch is bound by the matrix cores
+  // rather than by the weight stream (from int8_copy_min_rows() rows per expert on average) the
+  // bf16 kernel on a bf16 copy of the int8 values is the faster one, for three times the
+  // layer's footprint.  Both phases or neither (the row-tile lists differ), and only where the
+  // shared expert's widths fit the same kernel.
+  const bool dims64 = L->d_kpad % 64 == 0 && L->d_kpad >= 128 && L->f_kpad % 64 == 0 && L->f_kpad >= 128 &&
+                      (L->fs == 0 || (L->fs_kpad % 64 == 0 && L->fs_kpad >= 128));
+  p.q_copy = L->wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16 && L->group_size == 0 && p.up == kFamTiled &&
+             p.down == kFamTiled &&
+             dims64 && int8_copy_min_rows() > 0 &&
+             (double)T * L->k / L->E >= (double)int8_copy_min_rows();
+  const bool bf16_tiles = L->wdtype == ATENIA_MOE_WEIGHT_BF16 || p.pg_prefill || p.q_copy;
   const bool pipe_ok = bf16_tiles && L->d_kpad % 64 == 0 && L->d_kpad >= 128 && L->f_kpad % 64 == 0 &&
                        L->f_kpad >= 128;
   static const int duo_phases = [] {
@@ -732,7 +759,8 @@ ResolvedPlan resolve_plan(const AteniaMoeLayer* L, int T) {
   ResolvedPlan r{};
   r.plan = plan_batch(L, T);
   const bool pg = r.plan.pg_prefill;
-  r.ffn_dtype = pg ? ATENIA_MOE_WEIGHT_BF16 : L->wdtype;
+  // (a W8A16 layer's copy keeps its row scales and has the int8 blocks' dimensions)
+  r.ffn_dtype = pg || r.plan.q_copy ? ATENIA_MOE_WEIGHT_BF16 : L->wdtype;
   const WeightSet gate = dims_of(L, L->gate, pg), down = dims_of(L, L->down, pg);
   const bool tiles_ok = tiled_supported(gate, r.ffn_dtype) && tiled_supported(down, r.ffn_dtype);
   r.fam_up = r.plan.up == kFamTiled && !tiles_ok ? kFamStream : r.plan.up;
@@ -942,11 +970,13 @@ int run_forward_impl(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, flo
   // nearest bf16 (the reference's GPU dequantiser truncates instead,
   // src/cuda/int8_to_bf16.cu:91-110; rounding halves the error against the q * scale the
   // reference's CPU path multiplies with).  Decode batches stream the int8 weights themselves.
+  // A W8A16 layer does the same from int8_copy_min_rows() rows per expert on, with the int8
+  // values themselves in the copy (exact) and the row scales applied to the f32 results.
   const BatchPlan plan = plan_batch(L, T);
-  const bool pg_prefill = plan.pg_prefill;
+  const bool pg_prefill = plan.pg_prefill || plan.q_copy;
   if (pg_prefill && !L->pg_ready && no_alloc)
     return fail(ATENIA_MOE_ERR_UNSUPPORTED,
-                "per-group int8: a batch of %d tokens needs the layer's bf16 copy, which is made by "
+                "int8 layer: a batch of %d tokens needs the layer's bf16 copy, which is made by "
                 "the first such batch through an allocating entry point", T);
   if (pg_prefill && !L->pg_ready) {
     int rc = ensure_pg_copy(L);
@@ -1589,7 +1619,8 @@ int atenia_moe_hip_layer_create(const AteniaMoeLayerDesc* D, AteniaMoeLayer** ou
   if ((rc = resolve_static_scratch(L->device, nullptr))) return bail(rc);
   if (D->max_tokens_hint > 0) {
     if ((rc = ensure_workspace(L, D->max_tokens_hint))) return bail(rc);
-    if (plan_batch(L, D->max_tokens_hint).pg_prefill && (rc = ensure_pg_copy(L))) return bail(rc);
+    const BatchPlan hp = plan_batch(L, D->max_tokens_hint);
+    if ((hp.pg_prefill || hp.q_copy) && (rc = ensure_pg_copy(L))) return bail(rc);
   }
   if (hipDeviceSynchronize() != hipSuccess)
     return bail(fail(ATENIA_MOE_ERR_SYNC, "device synchronisation failed after upload"));
@@ -2181,7 +2212,7 @@ int atenia_moe_hip_plan_batch(int num_experts, int top_k, int d_model, int d_ff,
   plan[4] = r.y_bf16;
   plan[5] = r.ys_bf16;
   plan[6] = r.plan.tall_tiles;
-  plan[7] = (r.duo_up ? 1 : 0) | (r.duo_down ? 2 : 0);
+  plan[7] = (r.duo_up ? 1 : 0) | (r.duo_down ? 2 : 0) | (r.plan.q_copy ? 4 : 0);
   return ATENIA_MOE_OK;
 }
 

@@ -355,8 +355,10 @@ int atenia_moe_hip_layer_expert_kernels(const AteniaMoeLayer* layer, int64_t n_t
  * the same for the shared expert (-1 without one); plan[4] / plan[5]: 1 when the routed / shared
  * expert outputs travel to the combine as bf16 instead of f32 (bf16 layers on the matrix-core
  * kernels); plan[6]: 1 when row tiles may hold nine 32-row groups; plan[7]: bit 0 / bit 1 set when
- * the gate/up / down phase takes the tiled form with two workgroups per compute unit.  No
- * counterpart in the reference; hosts and tests use it to see where a batch size falls. */
+ * the gate/up / down phase takes the tiled form with two workgroups per compute unit, bit 2 when
+ * a W8A16 layer's tiled phases run on a bf16 copy of its int8 values (which the first such batch
+ * makes: twice the int8 bytes again).  No counterpart in the reference; hosts and tests use it to
+ * see where a batch size falls. */
 int atenia_moe_hip_plan_batch(int num_experts, int top_k, int d_model, int d_ff, int d_ff_shared,
                               int weight_dtype, int group_size, int64_t n_tokens,
                               int32_t plan[8]);

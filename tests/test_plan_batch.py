@@ -65,7 +65,15 @@ def test_plan_is_defined_and_ordered_in_the_batch_size(E, k, d, f, fs, wd):
         if p["ys_bf16"]:
             assert p["y_bf16"] and p["shared_down"] == capi.KERNELS_TILED, (T, p)
         if p["tall_tiles"]:
-            assert capi.KERNELS_TILED in (p["up"], p["down"]) and wd != capi.WEIGHT_INT8_W8A16, (T, p)
+            assert capi.KERNELS_TILED in (p["up"], p["down"]), (T, p)
+            # a W8A16 layer has them on the bf16 copy of its int8 values only
+            assert wd != capi.WEIGHT_INT8_W8A16 or p["int8_copy"], (T, p)
+        if p["int8_copy"]:
+            assert wd == capi.WEIGHT_INT8_W8A16 and p["up"] == p["down"] == capi.KERNELS_TILED, (T, p)
+            assert fs == 0 or p["shared_up"] == p["shared_down"] == capi.KERNELS_TILED, (T, p)
+            assert not p["y_bf16"], (T, p)
+        if prev is not None and prev[1]["int8_copy"]:
+            assert p["int8_copy"], f"back from the bf16 copy at T={T}"
         assert p["duo"] == 0, "the two-workgroup form is off unless ATENIA_MOE_DUO_MAX_K asks for it"
         if prev is not None:
             for phase in ("up", "down"):
