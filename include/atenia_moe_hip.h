@@ -180,8 +180,8 @@ int atenia_moe_hip_layer_forward_device(AteniaMoeLayer* layer, const void* d_x, 
  * n_tokens was seen before.  A batch whose workspace does not fit (about T * top_k * (2 * d_ff +
  * 4 * d_model) bytes for the streaming kernels that serve decode batches; the Mixtral shape fits
  * up to 85 tokens, i.e. every batch those kernels take) is refused with ATENIA_MOE_ERR_UNSUPPORTED and a message that names both sizes; so
- * is a per-group int8 batch large enough to need the layer's bf16 copy before an allocating
- * call has made it.  All handles on one GPU share that GPU's buffer, which keeps the previous
+ * is an int8 batch large enough to need the layer's bf16 copy (per-group scales: any batch for
+ * the tiled kernels; W8A16: from 256 rows per expert) before an allocating call has made it.  All handles on one GPU share that GPU's buffer, which keeps the previous
  * call's contents: the call rewrites what must start from a known state with a small kernel on
  * `stream` (no memset nodes), and calls that overlap in time on one GPU -- different handles
  * included -- race on it; order them on one stream or with events.  The status word of
