@@ -162,6 +162,7 @@ struct AteniaMoeLayer {
   DevBuf pg_wg, pg_wu, pg_wd, pg_swg, pg_swu, pg_swd;
   WeightSet gate_b{}, up_b{}, down_b{}, s_gate_b{}, s_up_b{}, s_down_b{};
   bool pg_ready = false;
+  bool q_copy_off = false;  // W8A16: the copy could not be allocated once; int8 tiled kernels from then on
   int normed_T = 0;     // rows of xn the last block forward wrote
   int last_T = 0;
   int stage_T[4] = {-1, -1, -1, -1};  // token count each pipeline stage last completed for
@@ -461,6 +462,20 @@ enum { kStageRouter = 0, kStagePermute = 1, kStageFfn = 2, kStageCombine = 3 };
 // Made at `create` when max_tokens_hint announces such batches, else by the first such batch.
 int ensure_pg_copy(AteniaMoeLayer* L) {
   if (L->pg_ready) return ATENIA_MOE_OK;
+  if (L->group_size == 0) {
+    // W8A16: the copy is optional; a cap on its size keeps a layer on the int8 kernels (tuning
+    // knob ATENIA_MOE_INT8_COPY_MAX_MB, read once; unset = no cap).
+    static const long long cap_mb = [] {
+      const char* e = getenv("ATENIA_MOE_INT8_COPY_MAX_MB");
+      return e ? atoll(e) : -1ll;
+    }();
+    auto bytes_of = [](const WeightSet& w, int G) { return (long long)G * w.n_pad * w.k_pad * 2; };
+    long long need = bytes_of(L->gate, L->E) + bytes_of(L->up, L->E) + bytes_of(L->down, L->E);
+    if (L->fs > 0) need += bytes_of(L->s_gate, 1) + bytes_of(L->s_up, 1) + bytes_of(L->s_down, 1);
+    if (cap_mb >= 0 && need > (cap_mb << 20))
+      return fail(ATENIA_MOE_ERR_UNSUPPORTED, "bf16 copy of %lld bytes is over the cap of %lld MiB",
+                  need, cap_mb);
+  }
   int rc = make_bf16_copy(L->gate, L->E, L->pg_wg, L->gate_b);
   if (!rc) rc = make_bf16_copy(L->up, L->E, L->pg_wu, L->up_b);
   if (!rc) rc = make_bf16_copy(L->down, L->E, L->pg_wd, L->down_b);
@@ -473,6 +488,11 @@ int ensure_pg_copy(AteniaMoeLayer* L) {
   HIP_TRY(hipDeviceSynchronize());
   L->pg_ready = true;
   return ATENIA_MOE_OK;
+}
+void release_pg_copy(AteniaMoeLayer* L) {
+  for (DevBuf* b : {&L->pg_wg, &L->pg_wu, &L->pg_wd, &L->pg_swg, &L->pg_swu, &L->pg_swd}) b->release();
+  L->gate_b = L->up_b = L->down_b = L->s_gate_b = L->s_up_b = L->s_down_b = WeightSet{};
+  L->pg_ready = false;
 }
 
 // Which expert kernels a batch of T tokens takes (a pure function of the layer and T).
@@ -661,7 +681,7 @@ BatchPlan plan_batch(const AteniaMoeLayer* L, int T) {
                       (L->fs == 0 || (L->fs_kpad % 64 == 0 && L->fs_kpad >= 128));
   p.q_copy = L->wdtype == ATENIA_MOE_WEIGHT_INT8_W8A16 && L->group_size == 0 && p.up == kFamTiled &&
              p.down == kFamTiled &&
-             dims64 && int8_copy_min_rows() > 0 &&
+             dims64 && int8_copy_min_rows() > 0 && !L->q_copy_off &&
              (double)T * L->k / L->E >= (double)int8_copy_min_rows();
   const bool bf16_tiles = L->wdtype == ATENIA_MOE_WEIGHT_BF16 || p.pg_prefill || p.q_copy;
   const bool pipe_ok = bf16_tiles && L->d_kpad % 64 == 0 && L->d_kpad >= 128 && L->f_kpad % 64 == 0 &&
@@ -827,6 +847,15 @@ int run_forward_impl(AteniaMoeLayer* L, const void* d_x, int x_dtype, int T, flo
     return fail(ATENIA_MOE_ERR_UNSUPPORTED, "f32 weights need f32 activations");
   if (first > kStageRouter && view == nullptr && L->cur.idx != L->ws.idx)
     return fail(ATENIA_MOE_ERR_DIM, "the earlier stages ran on another workspace");
+  // A W8A16 layer's bf16 copy only makes large batches faster: when it cannot be made (no room
+  // left for twice the int8 bytes) the layer keeps the int8 tiled kernels from then on.  Decided
+  // here, before the grouping stage lays out row tiles for either kernel.
+  if (!f32w && !no_alloc && !L->pg_ready && !L->q_copy_off && plan_batch(L, T).q_copy &&
+      ensure_pg_copy(L) != ATENIA_MOE_OK) {
+    release_pg_copy(L);
+    (void)hipGetLastError();
+    L->q_copy_off = true;
+  }
   const WsView V = view ? *view : L->ws;
   L->cur = V;
   // A forward still running on another stream uses the same workspace: wait for it.  Nothing

@@ -114,3 +114,47 @@ def test_noalloc_entry_needs_the_copy_to_exist(ora):
         assert gL.status()[0] == 0
         ha, hb = a.to_host(), b.to_host()
         assert hashlib.sha256(ha.tobytes()).hexdigest() == hashlib.sha256(hb.tobytes()).hexdigest()
+
+
+CAPPED = r"""
+import numpy as np
+from ateniaengine_amd import capi
+from oracle import moe_oracle as ora
+from tests import synth as S
+from tests.test_gpu_int8_copy import CASES, _layer
+from tests.test_gpu_parity import TOL_BF16_TOY, check_layer
+ora.build()
+for case in (CASES[0], CASES[2]):
+    E, k, d, f, fs, gated, T, _ = case
+    oL, gL = _layer(ora, case)
+    with gL:
+        assert gL.plan(T)["int8_copy"] == 1  # what the dimensions alone say
+        x = S.make_tokens(8500 + T, T, d)
+        out, _ = check_layer(ora, oL, gL, x, TOL_BF16_TOY, sample=range(0, T, 37))
+        assert gL.expert_kernels(T)[0] == capi.KERNELS_TILED
+        np.save(f"{OUT}/capped_{T}.npy", out)
+        check_layer(ora, oL, gL, S.make_tokens(8600, 40, d), TOL_BF16_TOY)
+        out2, _ = check_layer(ora, oL, gL, x, TOL_BF16_TOY, sample=range(0, T, 37))
+        assert out2.tobytes() == out.tobytes()
+print("child ok")
+"""
+
+
+def test_layer_keeps_the_int8_kernels_when_the_copy_cannot_be_made(ora, tmp_path):
+    """The copy is an optimisation: when it cannot be made (here: a cap of 0 MiB on its size, the
+    same path an allocation failure takes) the forward still runs, on the int8 tiled kernels, with
+    their results -- in that call and in every later one."""
+    env = dict(os.environ, ATENIA_MOE_INT8_COPY_MAX_MB="0", PYTHONPATH=ROOT)
+    r = subprocess.run([sys.executable, "-u", "-c", f"OUT = {str(tmp_path)!r}\n" + CAPPED], cwd=ROOT,
+                       env=env, capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0 and "child ok" in r.stdout, (r.stdout[-3000:], r.stderr[-3000:])
+    env0 = dict(os.environ, ATENIA_MOE_INT8_COPY_MIN_ROWS="0", PYTHONPATH=ROOT)
+    r0 = subprocess.run([sys.executable, "-u", "-c",
+                         f"OUT = {str(tmp_path)!r}\n" + CAPPED.replace("capped_", "int8_").replace(
+                             'assert gL.plan(T)["int8_copy"] == 1', 'assert gL.plan(T)["int8_copy"] == 0')],
+                        cwd=ROOT, env=env0, capture_output=True, text=True, timeout=900)
+    assert r0.returncode == 0 and "child ok" in r0.stdout, (r0.stdout[-3000:], r0.stderr[-3000:])
+    for case in (CASES[0], CASES[2]):
+        T = case[6]
+        a, b = np.load(tmp_path / f"capped_{T}.npy"), np.load(tmp_path / f"int8_{T}.npy")
+        assert a.tobytes() == b.tobytes(), "not the int8 tiled kernels' result"
