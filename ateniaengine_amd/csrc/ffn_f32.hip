@@ -30,8 +30,8 @@ constexpr int kLdT = kTile + 1;
 template <bool UP, bool F32ACC>
 __global__ __launch_bounds__(256) void ffn_f32_kernel(
     const float* __restrict__ wa, const float* __restrict__ wb, int64_t w_stride, int n_rows,
-    int k_cols, const float* __restrict__ a, int a_stride, float* __restrict__ out,
-    int out_stride, GroupDesc g) {
+    int k_cols, int n_pad, int k_pad, const float* __restrict__ a, int a_stride,
+    float* __restrict__ out, int out_stride, GroupDesc g) {
   const int u = blockIdx.y;
   if (u >= *g.n_active) return;
   const int e = g.active[u];
@@ -55,6 +55,12 @@ __global__ __launch_bounds__(256) void ffn_f32_kernel(
   }
   const float* wae = wa + (size_t)e * w_stride;
   const float* wbe = UP ? wb + (size_t)e * w_stride : nullptr;
+  // The 32 x 32 weight tile is four 1 KiB blocks (two strips of 16 rows x two blocks of 16 k): a
+  // thread fetches one lane slot, 4 consecutive k of one row, as one 16-byte load.
+  const int w_strip = n0 / 16 + (tid >> 7), w_kb2 = (tid >> 6) & 1, w_slot = tid & 63;
+  const int w_r = 16 * (tid >> 7) + (w_slot & 15), w_c = 16 * w_kb2 + 4 * (w_slot >> 4);
+  const int nkb = k_pad / kKbF32;
+  const bool w_row_ok = w_strip < n_pad / 16;
 
   double acc_a[4] = {0, 0, 0, 0}, acc_b[4] = {0, 0, 0, 0};
   float facc_a[4] = {0.f, 0.f, 0.f, 0.f}, facc_b[4] = {0.f, 0.f, 0.f, 0.f};
@@ -62,7 +68,8 @@ __global__ __launch_bounds__(256) void ffn_f32_kernel(
   // The next tile's elements are fetched into registers before the current tile is multiplied,
   // so a k tile does not start with a memory round trip (the sums and their order are untouched).
   __syncthreads();  // sRow
-  float ra[4], rba[4], rbb[4];
+  float ra[4];
+  float4 rba, rbb;
   auto fetch = [&](int k0) {
     const int c = tid & 31, kk = k0 + c;
 #pragma unroll
@@ -70,11 +77,12 @@ __global__ __launch_bounds__(256) void ffn_f32_kernel(
       const int r = (tid >> 5) + 8 * q;
       const int src = sRow[r];
       ra[q] = (src >= 0 && kk < k_cols) ? a[(size_t)src * a_stride + kk] : 0.f;
-      const int n = n0 + r;
-      const bool ok = n < n_rows && kk < k_cols;
-      rba[q] = ok ? wae[(size_t)n * k_cols + kk] : 0.f;
-      rbb[q] = (UP && ok) ? wbe[(size_t)n * k_cols + kk] : 0.f;
     }
+    const int kb = k0 / kKbF32 + w_kb2;  // rows past n_rows and columns past k_cols hold zeros
+    const bool ok = w_row_ok && kb < nkb;
+    const size_t at = ((size_t)w_strip * nkb + kb) * 256 + w_slot * 4;
+    rba = ok ? *(const float4*)(wae + at) : float4{0.f, 0.f, 0.f, 0.f};
+    rbb = (UP && ok) ? *(const float4*)(wbe + at) : float4{0.f, 0.f, 0.f, 0.f};
   };
   fetch(0);
   for (int k0 = 0; k0 < k_cols; k0 += kTile) {
@@ -82,11 +90,12 @@ __global__ __launch_bounds__(256) void ffn_f32_kernel(
     {
       const int c = tid & 31;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int r = (tid >> 5) + 8 * q;
-        sA[r * kLdT + c] = ra[q];
-        sBa[r * kLdT + c] = rba[q];
-        if (UP) sBb[r * kLdT + c] = rbb[q];
+      for (int q = 0; q < 4; ++q) sA[((tid >> 5) + 8 * q) * kLdT + c] = ra[q];
+      const float va[4] = {rba.x, rba.y, rba.z, rba.w}, vb[4] = {rbb.x, rbb.y, rbb.z, rbb.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        sBa[w_r * kLdT + w_c + j] = va[j];
+        if (UP) sBb[w_r * kLdT + w_c + j] = vb[j];
       }
     }
     __syncthreads();
@@ -151,10 +160,13 @@ __global__ __launch_bounds__(256) void ffn_f32_kernel(
 //
 // A workgroup owns a strip of 16 weight rows (gate and up strips in the gate/up phase) of one
 // expert and up to MT * 16 of its token rows; its four waves split K and add their partial sums
-// in wave order through LDS.  A lane loads 8 consecutive k of "its" row per step (rows l % 16,
-// k chunk l / 16: four lanes cover one full 128-byte line of the row) for both operands; MFMA t
-// of the step contracts element t of every lane's chunk, i.e. k = k0 + 8 * (l / 16) + t -- any
-// partition of k into groups of four is as good as another as long as A and B agree.
+// in wave order through LDS.  A lane holds 8 k of "its" row per step (row l % 16; two quads of 4
+// consecutive k, the lane's slots of two weight blocks) for both operands; MFMA t of the step
+// contracts element t of every lane's eight, i.e. k = k0 + 4 * (l / 16) + t for t < 4 and
+// k0 + 16 + 4 * (l / 16) + t - 4 beyond -- any partition of k into groups of four is as good as
+// another as long as A and B agree.  The weights come in 1 KiB blocks (moe_internal.h): read
+// row-major, 16 lanes of a load touched 16 different rows, and the launch moved its bytes at
+// 3 TB/s.
 typedef __attribute__((__vector_size__(4 * sizeof(double)))) double f64x4;
 
 // KS: waves that share one strip's K (4: one strip per workgroup, partial sums meet in LDS;
@@ -162,7 +174,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(double)))) double f64x4;
 template <bool UP, int MT, int KS>
 __global__ __launch_bounds__(256) void ffn_f32_mfma_kernel(
     const float* __restrict__ wa, const float* __restrict__ wb, int64_t w_stride, int n_rows,
-    int k_cols, const float* __restrict__ a, int a_stride, float* __restrict__ out,
+    int k_cols, int k_pad, const float* __restrict__ a, int a_stride, float* __restrict__ out,
     int out_stride, GroupDesc g) {
   const int u = blockIdx.y;
   if (u >= *g.n_active) return;
@@ -179,17 +191,20 @@ __global__ __launch_bounds__(256) void ffn_f32_mfma_kernel(
   const int r16 = lane & 15, q = lane >> 4;
   constexpr int NACC = UP ? 2 : 1;
 
-  // weight row of this lane (clamped: rows past n_rows are computed and never stored)
-  const int nrow = min(n0 + r16, n_rows - 1);
-  const float* pa = wa + (size_t)e * w_stride + (size_t)nrow * k_cols + 8 * q;
-  const float* pb = UP ? wb + (size_t)e * w_stride + (size_t)nrow * k_cols + 8 * q : nullptr;
+  // The strip's weights are 1 KiB blocks of 16 rows x 16 k, in k order: lane l's slot of a block
+  // is row l % 16, k = 16 kb + 4 (l / 16) .. + 3, so a wave reads a block as one contiguous KiB
+  // (rows past n_rows and columns past k_cols hold zeros).  A step takes two blocks: the lane's
+  // eight k are 32 st + 4 q + {0..3} and 32 st + 16 + 4 q + {0..3}, for the token rows too.
+  const int nkb = k_pad / kKbF32;
+  const float* pa = wa + (size_t)e * w_stride + (size_t)(n0 / 16) * nkb * 256 + lane * 4;
+  const float* pb = UP ? wb + (size_t)e * w_stride + (size_t)(n0 / 16) * nkb * 256 + lane * 4 : nullptr;
   const float* px[MT];
 #pragma unroll
   for (int i = 0; i < MT; ++i) {
     int pos = m0 + 16 * i + r16;
     if (pos >= cnt) pos = m0;  // an output column depends on its own token only; never stored
     const int row = UP ? g.perm[base + pos] / g.pair_div : base + pos;
-    px[i] = a + (size_t)row * a_stride + 8 * q;
+    px[i] = a + (size_t)row * a_stride + 4 * q;
   }
 
   // K in steps of 32 (8 per lane chunk), the steps dealt to the KS waves in contiguous runs
@@ -209,14 +224,26 @@ __global__ __launch_bounds__(256) void ffn_f32_mfma_kernel(
   // and waits for all of them before every use (one memory round trip per step).  A chunk past
   // the end of a row (k_cols is a multiple of 8: a chunk is whole or absent) is fetched from the
   // row's first columns and zeroed with selects; a step past the wave's range repeats its last.
+  auto keep = [](float4& v, bool in) {
+    v.x = in ? v.x : 0.f; v.y = in ? v.y : 0.f; v.z = in ? v.z : 0.f; v.w = in ? v.w : 0.f;
+  };
+  // token rows (row-major): the two quads of the step, each whole or absent (k_cols % 4 == 0)
   auto load8 = [&](const float* p, int st) {
     Chunk c;
-    const bool in = st * 32 + 8 * q < k_cols;
-    const size_t off = in ? (size_t)st * 32 : 0;
-    c.lo = *(const float4*)(p + off);
-    c.hi = *(const float4*)(p + off + 4);
-    c.lo.x = in ? c.lo.x : 0.f; c.lo.y = in ? c.lo.y : 0.f; c.lo.z = in ? c.lo.z : 0.f; c.lo.w = in ? c.lo.w : 0.f;
-    c.hi.x = in ? c.hi.x : 0.f; c.hi.y = in ? c.hi.y : 0.f; c.hi.z = in ? c.hi.z : 0.f; c.hi.w = in ? c.hi.w : 0.f;
+    const bool in_lo = st * 32 + 4 * q < k_cols, in_hi = st * 32 + 16 + 4 * q < k_cols;
+    c.lo = *(const float4*)(p + (in_lo ? (size_t)st * 32 : 0));
+    c.hi = *(const float4*)(p + (in_hi ? (size_t)st * 32 + 16 : 0));
+    keep(c.lo, in_lo);
+    keep(c.hi, in_hi);
+    return c;
+  };
+  // weights: blocks 2 st and 2 st + 1 of the strip (the second may lie past the last block)
+  auto load_w = [&](const float* p, int st) {
+    Chunk c;
+    const bool in_hi = 2 * st + 1 < nkb;
+    c.lo = *(const float4*)(p + (size_t)(2 * st) * 256);
+    c.hi = *(const float4*)(p + (size_t)(in_hi ? 2 * st + 1 : 0) * 256);
+    keep(c.hi, in_hi);
     return c;
   };
   auto elem = [](const Chunk& c, int t) {
@@ -226,8 +253,8 @@ __global__ __launch_bounds__(256) void ffn_f32_mfma_kernel(
   Chunk wA[2], wB[2], xs[2][MT] = {};
   auto load_step = [&](int buf, int st) {
     st = min(st, s1 - 1);
-    wA[buf] = load8(pa, st);
-    if (UP) wB[buf] = load8(pb, st);
+    wA[buf] = load_w(pa, st);
+    if (UP) wB[buf] = load_w(pb, st);
 #pragma unroll
     for (int i = 0; i < MT; ++i) xs[buf][i] = load8(px[i], st);  // rows past the end: clamped
   };
@@ -320,7 +347,7 @@ hipError_t launch_ffn_up_f32(const FfnArgs& a, hipStream_t s) {
     auto k = split ? (mt == 1 ? ffn_f32_mfma_kernel<true, 1, 4> : ffn_f32_mfma_kernel<true, 2, 4>)
                    : (mt == 1 ? ffn_f32_mfma_kernel<true, 1, 1> : ffn_f32_mfma_kernel<true, 2, 1>);
     k<<<grid, 256, 0, s>>>((const float*)a.gate.w, (const float*)a.up.w, a.gate.expert_stride,
-                           a.gate.n_rows, a.gate.k_cols, (const float*)a.x, a.x_stride,
+                           a.gate.n_rows, a.gate.k_cols, a.gate.k_pad, (const float*)a.x, a.x_stride,
                            (float*)a.h, a.h_stride, a.g);
     return hipGetLastError();
   }
@@ -328,8 +355,8 @@ hipError_t launch_ffn_up_f32(const FfnArgs& a, hipStream_t s) {
             (a.rows_max + kTile - 1) / kTile);
   auto k = a.f32_accumulate ? ffn_f32_kernel<true, true> : ffn_f32_kernel<true, false>;
   k<<<grid, 256, 0, s>>>((const float*)a.gate.w, (const float*)a.up.w, a.gate.expert_stride,
-                         a.gate.n_rows, a.gate.k_cols, (const float*)a.x, a.x_stride, (float*)a.h,
-                         a.h_stride, a.g);
+                         a.gate.n_rows, a.gate.k_cols, a.gate.n_pad, a.gate.k_pad, (const float*)a.x,
+                         a.x_stride, (float*)a.h, a.h_stride, a.g);
   return hipGetLastError();
 }
 
@@ -342,14 +369,16 @@ hipError_t launch_ffn_down_f32(const FfnArgs& a, hipStream_t s) {
     auto k = split ? (mt == 1 ? ffn_f32_mfma_kernel<false, 1, 4> : ffn_f32_mfma_kernel<false, 2, 4>)
                    : (mt == 1 ? ffn_f32_mfma_kernel<false, 1, 1> : ffn_f32_mfma_kernel<false, 2, 1>);
     k<<<grid, 256, 0, s>>>((const float*)a.down.w, nullptr, a.down.expert_stride, a.down.n_rows,
-                           a.down.k_cols, (const float*)a.h, a.h_stride, a.y, a.y_stride, a.g);
+                           a.down.k_cols, a.down.k_pad, (const float*)a.h, a.h_stride, a.y, a.y_stride,
+                           a.g);
     return hipGetLastError();
   }
   dim3 grid((a.down.n_rows + kTile - 1) / kTile, a.n_groups_max,
             (a.rows_max + kTile - 1) / kTile);
   auto k = a.f32_accumulate ? ffn_f32_kernel<false, true> : ffn_f32_kernel<false, false>;
   k<<<grid, 256, 0, s>>>((const float*)a.down.w, nullptr, a.down.expert_stride, a.down.n_rows,
-                         a.down.k_cols, (const float*)a.h, a.h_stride, a.y, a.y_stride, a.g);
+                         a.down.k_cols, a.down.n_pad, a.down.k_pad, (const float*)a.h, a.h_stride, a.y,
+                         a.y_stride, a.g);
   return hipGetLastError();
 }
 

@@ -256,31 +256,22 @@ int upload_family(const void* host, size_t host_stride_elems, int G, int n_rows,
   const size_t eb = elem_bytes_of(wdtype);
   ws.n_rows = n_rows;
   ws.k_cols = k_cols;
-  if (wdtype == ATENIA_MOE_WEIGHT_F32) {
-    ws.n_pad = n_rows;
-    ws.k_pad = k_cols;
-    ws.expert_stride = (int64_t)n_rows * k_cols;
-    int rc = dst.ensure((size_t)G * n_rows * k_cols * 4);
-    if (rc) return rc;
-    for (int g = 0; g < G; ++g)
-      HIP_TRY(hipMemcpy((float*)dst.p + (size_t)g * ws.expert_stride,
-                        (const float*)host + (size_t)g * host_stride_elems,
-                        (size_t)n_rows * k_cols * 4, hipMemcpyHostToDevice));
-    ws.w = dst.p;
-    return ATENIA_MOE_OK;
-  }
-  const int KB = kb_of(wdtype);
+  // f32: the same 1 KiB blocks with 16 k each (a lane slot = 4 consecutive k of one row), so a
+  // wave reads a strip of 16 rows in whole blocks; expert_stride stays in elements.
+  const bool f32w = wdtype == ATENIA_MOE_WEIGHT_F32;
+  const int KB = f32w ? kKbF32 : kb_of(wdtype);
   ws.n_pad = round_up(n_rows, 16);
   ws.k_pad = round_up(k_cols, KB);
-  ws.expert_stride = (int64_t)ws.n_pad * ws.k_pad * (int64_t)eb;  // bytes
-  int rc = dst.ensure((size_t)G * ws.expert_stride);
+  const int64_t expert_bytes = (int64_t)ws.n_pad * ws.k_pad * (int64_t)eb;
+  ws.expert_stride = f32w ? expert_bytes / 4 : expert_bytes;  // elements (f32) or bytes
+  int rc = dst.ensure((size_t)G * expert_bytes);
   if (rc) return rc;
   rc = staging.ensure((size_t)n_rows * k_cols * eb);
   if (rc) return rc;
   for (int g = 0; g < G; ++g) {
     HIP_TRY(hipMemcpy(staging.p, (const uint8_t*)host + (size_t)g * host_stride_elems * eb,
                       (size_t)n_rows * k_cols * eb, hipMemcpyHostToDevice));
-    HIP_TRY(launch_repack_blocks(staging.p, (uint8_t*)dst.p + (size_t)g * ws.expert_stride,
+    HIP_TRY(launch_repack_blocks(staging.p, (uint8_t*)dst.p + (size_t)g * expert_bytes,
                                  n_rows, k_cols, ws.n_pad, ws.k_pad, (int)eb, nullptr));
     HIP_TRY(hipDeviceSynchronize());
   }

@@ -25,6 +25,9 @@ constexpr int kTileM = 256;          // token rows per tile of the tiled expert 
 constexpr int kBlockBytes = 1024;
 constexpr int kKbBf16 = 32;
 constexpr int kKbInt8 = 64;
+// f32 expert matrices use the same blocks with KB = 16: a lane slot is 4 consecutive k of one row
+// (the chunk a lane of v_mfma_f64_16x16x4_f64 feeds one instruction at a time from).
+constexpr int kKbF32 = 16;
 
 static inline int round_up(int v, int m) { return (v + m - 1) / m * m; }
 
@@ -44,7 +47,7 @@ struct GroupDesc {
 
 // One expert projection family as stored on the device.
 struct WeightSet {
-  const void* w;            // blocks (bf16/int8) or row-major f32
+  const void* w;            // blocks (see above)
   const float* scale;       // int8: per output row, [G, N] (unpadded N stride = n_rows);
                             // per-group int8: [G][n_kgroups][n_pad] (see group_blocks)
   int group_blocks;         // per-group int8: 64-k blocks per scale group (0 = one scale per row)
